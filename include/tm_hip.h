@@ -1,0 +1,225 @@
+/*
+ * tm_hip.h — TuckCore <-> HIP narrow C ABI for the Q8_0 matrix-product path
+ * on MI355X (gfx950).
+ *
+ * This is the HIP counterpart of the reference's Metal ABI
+ * (native/metal/tm_metal.h): the same conventions, restricted to what the
+ * Q8_0 decode GEMV / prefill GEMM / embedding-row path needs. Every entry
+ * point names the reference declaration it stands in for.
+ *
+ * Conventions (native/metal/tm_metal.h:1-18, :32-40):
+ *   - One context owns one device, one HIP stream and the loaded kernels.
+ *   - Buffers are opaque handles with explicit lifetime, owned by exactly one
+ *     context; every call checks ownership and length before any device work.
+ *   - Dispatch is asynchronous; tm_hip_fence() waits for everything committed.
+ *     Host copies are ordered after all committed work.
+ *   - A context is used from one thread at a time (the caller serializes);
+ *     the counters are atomic and tm_hip_download_after may be called without
+ *     the caller's lock.
+ *   - Operations return 0 or a negative TM_HIP_ERR_* code and write a
+ *     NUL-terminated message into `err` (when non-NULL, `err_cap` bytes).
+ *   - Dimensions are uint32_t; x/y offsets are in f32 ELEMENTS; X is
+ *     [batch, cols] row-major, Y is [batch, rows] row-major (token-major).
+ *
+ * Q8_0 weights are `rows * cols/32` blocks of 34 bytes ([f16 d][i8 qs; 32],
+ * little endian), rows contiguous, exactly as stored in GGUF. Every Q8_0
+ * operation accepts a plain buffer holding those raw bytes. A buffer may
+ * additionally be sealed with tm_hip_q8_0_pack(), which re-lays it out on
+ * the device for coalesced loads; the same entry points then run their fast
+ * kernels. Results do not depend on which layout a buffer is in.
+ */
+#ifndef TM_HIP_H
+#define TM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tm_hip_ctx tm_hip_ctx;
+typedef struct tm_hip_buffer tm_hip_buffer;
+
+/* native/metal/tm_metal.h:32-40 */
+enum {
+    TM_HIP_OK = 0,
+    TM_HIP_ERR_NO_DEVICE = -1,   /* no usable HIP device */
+    TM_HIP_ERR_SOURCE = -2,      /* device code for this GPU is missing */
+    TM_HIP_ERR_ALLOC = -3,       /* buffer allocation failed */
+    TM_HIP_ERR_BOUNDS = -4,      /* size/range mismatch, zero length */
+    TM_HIP_ERR_UNSUPPORTED = -5, /* invalid arguments / mode */
+    TM_HIP_ERR_INTERNAL = -6     /* HIP runtime failure */
+};
+
+/* Largest batch of tm_hip_q8_0_gemm (native/metal/tm_metal.h:161-167;
+ * crates/metal/src/lib.rs:28-30 GEMM_MAX_BATCH). */
+#define TM_HIP_GEMM_MAX_BATCH 32u
+/* Largest batch of tm_hip_q8_0_gemm_mma (native/metal/tm_metal.h:170). */
+#define TM_HIP_GEMM_MMA_MAX_BATCH 512u
+/* Largest batch of tm_hip_q8_0_gemm_i8 / tm_hip_q8_0_quantize_act. */
+#define TM_HIP_GEMM_I8_MAX_BATCH 2048u
+
+/* 1 when a gfx950 device is visible (native/metal/tm_metal.h:43). */
+int tm_hip_available(void);
+
+/* One-line runtime description; always a valid static string
+ * (native/metal/tm_metal.h:47). */
+const char *tm_hip_runtime_info(void);
+
+/* Create a context on the current default device: stream, event pool and
+ * kernels. Returns NULL and fills `err` on failure. The Metal counterpart
+ * (native/metal/tm_metal.h:52) takes MSL source to compile; the HIP kernels
+ * are compiled ahead of time into this library, so there is no source
+ * argument. */
+tm_hip_ctx *tm_hip_create(char *err, size_t err_cap);
+
+/* Destroy the context after waiting for its work. Buffers created from it
+ * must have been freed first (native/metal/tm_metal.h:56). */
+void tm_hip_destroy(tm_hip_ctx *ctx);
+
+/* Allocate `bytes` (> 0) of device memory. `shared` buffers accept host
+ * copies; private (shared == 0) buffers refuse them, as on Metal. New
+ * buffers read as zero (native/metal/tm_metal.h:61-62). */
+tm_hip_buffer *tm_hip_buffer_new(tm_hip_ctx *ctx, size_t bytes, int shared, char *err,
+                                 size_t err_cap);
+
+/* Release a handle. Device memory that committed work still uses stays
+ * alive (and counted by tm_hip_in_flight_bytes) until that work completes
+ * (native/metal/tm_metal.h:66; lease rule native/metal/tm_metal.m:167-224). */
+void tm_hip_buffer_free(tm_hip_ctx *ctx, tm_hip_buffer *buffer);
+
+/* Length in bytes, 0 for an invalid handle (native/metal/tm_metal.h:73). */
+size_t tm_hip_buffer_len(const tm_hip_ctx *ctx, const tm_hip_buffer *buffer);
+
+/* Zero `len` bytes at byte offset `off` on the device, ordered with the
+ * context's other work (native/metal/tm_metal.h:78-79). */
+int tm_hip_buffer_zero(tm_hip_ctx *ctx, tm_hip_buffer *buffer, size_t off, size_t len,
+                       char *err, size_t err_cap);
+
+/* Host <-> device copies (shared buffers only). Both wait for every
+ * committed dispatch first and are refused while a group is open
+ * (native/metal/tm_metal.h:82-85; copy contract native/metal/tm_metal.m:569-609).
+ * Sealed (packed) weight buffers refuse them. */
+int tm_hip_upload(tm_hip_ctx *ctx, tm_hip_buffer *dst, size_t off, const void *src, size_t len,
+                  char *err, size_t err_cap);
+int tm_hip_download(tm_hip_ctx *ctx, tm_hip_buffer *src, size_t off, void *dst, size_t len,
+                    char *err, size_t err_cap);
+
+/* Copy a range once the first `completed_target` commits have completed,
+ * without waiting for later work (native/metal/tm_metal.h:295-300). */
+int tm_hip_download_after(tm_hip_ctx *ctx, tm_hip_buffer *src, size_t off, void *dst,
+                          size_t len, uint64_t completed_target, char *err, size_t err_cap);
+
+/* dst[dst_off + i] = src[src_off + i], i < n, f32 elements, bit-exact;
+ * usable inside a group (native/metal/tm_metal.h:108-113). */
+int tm_hip_copy_f32(tm_hip_ctx *ctx, tm_hip_buffer *src, uint32_t src_off, tm_hip_buffer *dst,
+                    uint32_t dst_off, uint32_t n, char *err, size_t err_cap);
+
+/* Grouped encoding: operations between begin and end are submitted as ONE
+ * commit at end_group; abort_group discards them unsubmitted. Copies and
+ * fence require no open group (native/metal/tm_metal.h:125-135). Inside a
+ * group, consecutive Q8_0 products whose buffers do not depend on each
+ * other are executed by a single kernel launch. */
+int tm_hip_begin_group(tm_hip_ctx *ctx, char *err, size_t err_cap);
+int tm_hip_end_group(tm_hip_ctx *ctx, char *err, size_t err_cap);
+int tm_hip_abort_group(tm_hip_ctx *ctx, char *err, size_t err_cap);
+
+/* Block until every commit has completed; refused while a group is open
+ * (native/metal/tm_metal.h:289-291). */
+int tm_hip_fence(tm_hip_ctx *ctx, char *err, size_t err_cap);
+
+/* ---- the Q8_0 products ---- */
+
+/* y[r] = dot(dequant_q8_0(w_row_r), x), r < rows. `cols` a positive multiple
+ * of 32; x holds cols f32, y rows f32 (native/metal/tm_metal.h:196-202;
+ * validation native/metal/tm_metal.m:962-980). */
+int tm_hip_q8_0_gemv(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                     uint32_t rows, uint32_t cols, char *err, size_t err_cap);
+
+/* Y[b, :] = W . X[b, :], b < batch (1..=TM_HIP_GEMM_MAX_BATCH), with the
+ * GEMV's per-token arithmetic: batch = 1 is bit-identical to
+ * tm_hip_q8_0_gemv, and every token's row equals the GEMV of that token
+ * (native/metal/tm_metal.h:161-167). */
+int tm_hip_q8_0_gemm(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                     uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off,
+                     uint32_t y_off, char *err, size_t err_cap);
+
+/* Same contract for batch 1..=TM_HIP_GEMM_MMA_MAX_BATCH on the MFMA matrix
+ * cores with f32 operand tiles (W dequantized exactly as d*q). Summation
+ * order differs from the GEMV: tolerance-qualified, not bit-identical
+ * (native/metal/tm_metal.h:172-178). */
+int tm_hip_q8_0_gemm_mma(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                         uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off,
+                         uint32_t y_off, char *err, size_t err_cap);
+
+/* out[out_off + i] = d * q of row `row`, i < cols; exact
+ * (native/metal/tm_metal.h:137-139). */
+int tm_hip_q8_0_row_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *out, uint32_t row,
+                        uint32_t cols, uint32_t out_off, char *err, size_t err_cap);
+
+/* out[i] = row ids[slot] of `w` dequantized to f32; an id >= rows writes
+ * zeros. Only type_id 8 (Q8_0) is built (native/metal/tm_metal.h:100-106). */
+int tm_hip_row_indirect_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t type_id, uint32_t rows,
+                            uint32_t cols, tm_hip_buffer *ids, uint32_t slot, tm_hip_buffer *out,
+                            char *err, size_t err_cap);
+
+/* ---- additions with no Metal counterpart ---- */
+
+/* Seal `w` (which holds the raw GGUF bytes of a rows x cols Q8_0 matrix) in
+ * the device layout: all int8 quants first ([rows][cols], 16-byte pieces
+ * aligned), then all f16 scales ([rows][cols/32]) — the same byte count, so
+ * the allocation ledger is unchanged. Called once after the staged upload
+ * that crates/tuckcore/src/engine/metal.rs:138-147 performs. After sealing,
+ * host copies and buffer_zero on `w` are refused, and Q8_0 operations must
+ * name the same rows/cols. No counterpart in the reference: Apple's unified
+ * memory has no use for it. */
+int tm_hip_q8_0_pack(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t rows, uint32_t cols, char *err,
+                     size_t err_cap);
+
+/* Quantize `batch` rows of `cols` f32 activations (at element offset x_off
+ * of `x`) to Q8_0 with the rule of crates/tuckcore/src/tensor.rs:184-206.
+ * `xq` receives batch*cols int8 quants (token-major) followed by
+ * batch*(cols/32) f32 scales (token-major; each the f32 value of the
+ * f16-rounded scale): batch * (cols + cols/32*4) bytes in all.
+ * Device form of the `llama-cpu` numerical profile's first step
+ * (crates/tuckcore/src/forward.rs:783-793). */
+int tm_hip_q8_0_quantize_act(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *xq, uint32_t cols,
+                             uint32_t batch, uint32_t x_off, char *err, size_t err_cap);
+
+/* Y[b, r] = sum over blocks of (d_w * d_x[b]) * (i32 block dot), the
+ * arithmetic of crates/tuckcore/src/kernels.rs:206-221, with `xq` produced
+ * by tm_hip_q8_0_quantize_act. The i32 block dots are exact; batch
+ * 1..=TM_HIP_GEMM_I8_MAX_BATCH. When `sumi` is non-NULL it receives the raw
+ * block dots as int32 [batch, rows, cols/32] (verification aid). */
+int tm_hip_q8_0_gemm_i8(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm_hip_buffer *y,
+                        tm_hip_buffer *sumi, uint32_t rows, uint32_t cols, uint32_t batch,
+                        uint32_t y_off, char *err, size_t err_cap);
+
+/* ---- measurement surface (native/metal/tm_metal.h:293-325) ---- */
+
+uint64_t tm_hip_committed_dispatches(const tm_hip_ctx *ctx);
+uint64_t tm_hip_completed_dispatches(const tm_hip_ctx *ctx);
+/* GPU milliseconds of the most recently completed commit (HIP events on the
+ * context's stream). */
+double tm_hip_last_gpu_ms(const tm_hip_ctx *ctx);
+/* Cumulative GPU nanoseconds over every completed commit. */
+uint64_t tm_hip_gpu_nanos_total(const tm_hip_ctx *ctx);
+/* Number of kernel launches issued so far (a group may issue fewer launches
+ * than it holds operations). */
+uint64_t tm_hip_kernel_launches(const tm_hip_ctx *ctx);
+/* Opt-in per-operator GPU time table; labels carry the shape
+ * ("q8_0_gemv:3072x1024"), a group is attributed to "group". */
+int tm_hip_profile_set(tm_hip_ctx *ctx, int enabled);
+int tm_hip_profile_read(tm_hip_ctx *ctx, uint32_t index, char *name, size_t name_cap,
+                        uint64_t *nanos, uint64_t *count);
+/* Live bytes in handles of this context. */
+uint64_t tm_hip_allocated_bytes(const tm_hip_ctx *ctx);
+/* Bytes leased by commits that have not completed yet. */
+uint64_t tm_hip_in_flight_bytes(const tm_hip_ctx *ctx);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TM_HIP_H */

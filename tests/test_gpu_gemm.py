@@ -1,0 +1,153 @@
+"""GPU parity: small-batch GEMM (GEMV arithmetic) and the MFMA prefill GEMM.
+
+Follows crates/metal/src/tests.rs:835-921 (batched GEMM, batch = 1 bit
+identity) and :1169-1247 (MMA GEMM: row tails, partial token tiles, offsets,
+batch 512, batch 513 refused).
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from tuckmill_amd import hip as H
+from tuckmill_amd import synth as S
+
+from q8util import bits, gemv, norm_err, ref_scale, require_gpu, upload_new, weights_buffer
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = require_gpu()
+    yield c
+    c.close()
+
+
+def run_gemm(ctx, fn, wb, x, rows, cols, batch, x_off=0, y_off=0):
+    xs = np.zeros(x_off + batch * cols, np.float32)
+    xs[x_off:] = x
+    xb = upload_new(ctx, xs)
+    yb = ctx.buffer((y_off + batch * rows) * 4)
+    fn(wb, xb, yb, rows, cols, batch, x_off, y_off)
+    ctx.fence()
+    out = yb.download_f32(0, y_off + batch * rows).copy()
+    xb.free()
+    yb.free()
+    return out
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("rows,cols,all_rows", [(32, 32, True), (64, 1024, True),
+                                                (2048, 1024, True), (3072, 1024, True),
+                                                (151_936, 1024, False)])
+def test_batched_gemm_matches_the_scalar_reference(ctx, rows, cols, all_rows, packed):
+    # crates/metal/src/tests.rs:835-892
+    w = O.boundary_weights(rows, cols, 101 + rows)
+    wb = weights_buffer(ctx, w, rows, cols, packed)
+    for batch in (1, 4, 8, 16):
+        xs = [O.boundary_input(cols, 200 + b) for b in range(batch)]
+        got = run_gemm(ctx, ctx.q8_0_gemm, wb, np.concatenate(xs), rows, cols, batch)
+        got = got.reshape(batch, rows)
+        check = np.arange(rows) if all_rows else np.array([0, 1, rows // 2, rows - 2, rows - 1])
+        for b, x in enumerate(xs):
+            if all_rows or b == 0:
+                cpu = O.gemv_q8_0_f32(w, rows, cols, x, threads=8)
+            scale = ref_scale(cpu)
+            if all_rows or b == 0:
+                assert np.max(np.abs(got[b][check] - cpu[check])) <= 1e-4 * scale
+    wb.free()
+
+
+def test_batch_one_gemm_is_bit_identical_to_gemv(ctx):
+    # crates/metal/src/tests.rs:895-921
+    rows, cols = 512, 1024
+    w = O.boundary_weights(rows, cols, 7)
+    x = O.boundary_input(cols, 9)
+    for packed in (False, True):
+        wb = weights_buffer(ctx, w, rows, cols, packed)
+        single = gemv(ctx, wb, x, rows, cols)
+        batch = run_gemm(ctx, ctx.q8_0_gemm, wb, x, rows, cols, 1)
+        assert np.array_equal(bits(single), bits(batch))
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(64, 1024, 32), (100, 1152, 7), (33, 96, 5),
+                                             (513, 2048, 13), (40, 6912, 3)])
+def test_every_token_of_the_small_gemm_equals_its_own_gemv(ctx, rows, cols, batch):
+    # Stronger than the reference's batch = 1 identity: the exact (speculative
+    # verify) path must reproduce decode for every token.
+    w = S.make_weights(rows, cols, 31 + rows)
+    x = S.make_activations(cols * batch, 77)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    got = run_gemm(ctx, ctx.q8_0_gemm, wb, x, rows, cols, batch).reshape(batch, rows)
+    want = O.gemm_q8_0_f32(w, rows, cols, x, batch)
+    assert norm_err(got, want) <= 1e-5
+    for b in range(batch):
+        single = gemv(ctx, wb, x[b * cols:(b + 1) * cols], rows, cols)
+        assert np.array_equal(bits(single), bits(got[b])), f"token {b}"
+
+
+def test_gemm_batch_limits(ctx):
+    wb, xb, yb = ctx.buffer(64), ctx.buffer(64), ctx.buffer(64)
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.q8_0_gemm(wb, xb, yb, 1, 32, H.GEMM_MAX_BATCH + 1, 0, 0)
+    assert e.value.abi_code == H.TM_HIP_ERR_UNSUPPORTED
+    with pytest.raises(H.TuckmillError):
+        ctx.q8_0_gemm(wb, xb, yb, 1, 32, 0, 0, 0)
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.q8_0_gemm(wb, xb, yb, 1, 32, 1, 16, 0)  # x range past the end
+    assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS
+
+
+MMA_SHAPES = [(16, 1024, 16), (40, 64, 3), (3584, 1024, 16), (3584, 1024, 32), (40, 64, 27),
+              (1024, 3584, 64), (100, 96, 77), (40, 64, 512), (1024, 3584, 7), (6144, 1024, 1)]
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("rows,cols,batch", MMA_SHAPES)
+def test_gemm_mma_matches_the_cpu_reference_within_tolerance(ctx, rows, cols, batch, packed):
+    # crates/metal/src/tests.rs:1169-1233
+    w = O.boundary_weights(rows, cols, 11)
+    x = O.boundary_input(cols * batch, 13)
+    wb = weights_buffer(ctx, w, rows, cols, packed)
+    x_off, y_off = 32, 8
+    got = run_gemm(ctx, ctx.q8_0_gemm_mma, wb, x, rows, cols, batch, x_off, y_off)
+    assert not got[:y_off].any(), "nothing before y_off"
+    got = got[y_off:].reshape(batch, rows)
+    cpu = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+    for b in range(batch):
+        assert np.max(np.abs(got[b] - cpu[b])) <= 1e-4 * ref_scale(cpu[b]), f"token {b}"
+    wb.free()
+
+
+def test_gemm_mma_refuses_batch_above_the_maximum(ctx):
+    # crates/metal/src/tests.rs:1234-1247
+    with pytest.raises(H.TuckmillError):
+        ctx.q8_0_gemm_mma(ctx.buffer(64), ctx.buffer(64), ctx.buffer(64), 1, 32,
+                          H.GEMM_MMA_MAX_BATCH + 1, 0, 0)
+
+
+@pytest.mark.parametrize("rows,cols", [(1024, 1024), (2048, 1024), (1024, 2048), (3072, 1024),
+                                       (1024, 3072)])
+def test_config2_prefill_gemm_m512_gaussian_within_1e5(ctx, rows, cols):
+    # BASELINE config 2: M = 512 against the Qwen3-0.6B projection shapes.
+    batch = 512
+    w = S.make_weights(rows, cols, S.tensor_seed(2, 0, f"{rows}x{cols}"))
+    x = S.make_activations(batch * cols, rows + cols)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    got = run_gemm(ctx, ctx.q8_0_gemm_mma, wb, x, rows, cols, batch).reshape(batch, rows)
+    want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+    assert norm_err(got, want) <= 1e-5
+    wb.free()
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(6912, 1152, 512), (1152, 6912, 512), (97, 1152, 33),
+                                             (6144, 2048, 64), (2048, 6144, 8), (70, 32, 2)])
+def test_gemm_mma_gemma_and_sweep_shapes_gaussian(ctx, rows, cols, batch):
+    # BASELINE configs 3 and 4 (K not a multiple of 256; 2B-class shapes).
+    w = S.make_weights(rows, cols, rows * 7 + cols)
+    x = S.make_activations(batch * cols, batch)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    got = run_gemm(ctx, ctx.q8_0_gemm_mma, wb, x, rows, cols, batch).reshape(batch, rows)
+    want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+    assert norm_err(got, want) <= 1e-5
+    wb.free()

@@ -1,0 +1,121 @@
+"""GPU parity: the int8-activation profile (device activation quantizer and
+int8 x int8 -> i32 MFMA block dots) against the CPU oracle's
+quantize_row_q8_0 / dot_q8_0_q8_0 (crates/tuckcore/src/tensor.rs:184-206,
+crates/tuckcore/src/kernels.rs:206-221).
+
+Bar: quantized activations bit-exact, every i32 block dot bit-exact, and the
+f32 result bit-exact as well (the kernel keeps the reference's unfused
+multiply, multiply, add in block order).
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from tuckmill_amd import hip as H
+from tuckmill_amd import synth as S
+
+from q8util import bits, require_gpu, upload_new, weights_buffer
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = require_gpu()
+    yield c
+    c.close()
+
+
+def quantize_on_gpu(ctx, x, cols, batch, x_off=0):
+    xs = np.zeros(x_off + batch * cols, np.float32)
+    xs[x_off:] = x
+    xb = upload_new(ctx, xs)
+    blocks = cols // 32
+    xq = ctx.buffer(batch * (cols + blocks * 4))
+    ctx.q8_0_quantize_act(xb, xq, cols, batch, x_off)
+    ctx.fence()
+    raw = xq.download(0, batch * (cols + blocks * 4))
+    qs = raw[:batch * cols].view(np.int8).reshape(batch, blocks, 32)
+    ds = raw[batch * cols:].view(np.float32).reshape(batch, blocks)
+    return xq, qs, ds
+
+
+def test_activation_quantizer_known_answer(ctx):
+    # crates/tuckcore/src/tensor.rs:373-392
+    x = np.zeros(32, np.float32)
+    x[0], x[1], x[2] = 127.0, -63.5, 1.0
+    _, qs, ds = quantize_on_gpu(ctx, x, 32, 1)
+    assert ds[0, 0] == 1.0
+    assert qs[0, 0, 0] == 127 and qs[0, 0, 1] == -64 and qs[0, 0, 2] == 1 and qs[0, 0, 3] == 0
+
+
+@pytest.mark.parametrize("cols,batch,scale", [(32, 1, 1.0), (1024, 7, 1.0), (1152, 33, 0.02),
+                                              (2048, 64, 37.5), (96, 5, 1e-6), (64, 3, 6e4)])
+def test_activation_quantizer_is_bit_exact(ctx, cols, batch, scale):
+    x = (S.make_activations(cols * batch, cols + batch) * np.float32(scale)).astype(np.float32)
+    x[:32] = 0.0  # an all-zero block
+    if x.size >= 96:
+        x[40], x[70] = np.nan, np.inf
+    _, qs, ds = quantize_on_gpu(ctx, x, cols, batch, x_off=4)
+    want_q, want_d = O.quantize_row_q8_0(x)
+    assert np.array_equal(qs.reshape(-1, 32), want_q)
+    assert np.array_equal(bits(ds.reshape(-1)), bits(want_d))
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("rows,cols,batch", [(16, 32, 1), (40, 64, 3), (100, 96, 77),
+                                             (1024, 1024, 16), (333, 1152, 40), (2048, 2048, 8)])
+def test_gemm_i8_block_dots_and_result_are_bit_exact(ctx, rows, cols, batch, packed):
+    blocks = cols // 32
+    w = S.make_weights(rows, cols, rows + cols)
+    if rows >= 40:  # extremes: q_w = -128 against q_x = +-127
+        wv = w.reshape(rows * blocks, 34)
+        wv[0, 2:] = 0x80
+        wv[blocks, 2:] = 0x80
+    x = S.make_activations(cols * batch, batch)
+    x[:32] = 5.0
+    if batch > 1:
+        x[cols:cols + 32] = -5.0
+    wb = weights_buffer(ctx, w, rows, cols, packed)
+    xq, qs, ds = quantize_on_gpu(ctx, x, cols, batch)
+    yb = ctx.buffer((3 + batch * rows) * 4)
+    sb = ctx.buffer(batch * rows * blocks * 4)
+    ctx.q8_0_gemm_i8(wb, xq, yb, rows, cols, batch, 3, sb)
+    ctx.fence()
+    out = yb.download_f32(0, 3 + batch * rows)
+    assert not out[:3].any()
+    got = out[3:].reshape(batch, rows)
+    sumi = sb.download(0, batch * rows * blocks * 4).view(np.int32).reshape(batch, rows, blocks)
+    want = O.gemm_q8_0_q8_0(w, rows, cols, x, batch, threads=8)
+    assert np.array_equal(bits(got), bits(want))
+    row_bytes = blocks * 34
+    wq = w.reshape(rows, blocks, 34)[:, :, 2:].view(np.int8).astype(np.int64)
+    for b in range(batch):
+        brute = np.einsum("rkl,kl->rk", wq, qs[b].astype(np.int64))
+        assert np.array_equal(sumi[b].astype(np.int64), brute)
+        if b == 0:
+            for r in (0, rows - 1):
+                one = O.block_sumi(w[r * row_bytes:(r + 1) * row_bytes], qs[b])
+                assert np.array_equal(sumi[b, r], one)
+    if rows >= 40:
+        assert sumi[0, 0, 0] == -128 * 127 * 32
+    # without the verification output
+    ctx.q8_0_gemm_i8(wb, xq, yb, rows, cols, batch, 3)
+    ctx.fence()
+    assert np.array_equal(bits(yb.download_f32(3, batch * rows)), bits(want.reshape(-1)))
+
+
+def test_i8_argument_refusals(ctx):
+    b = ctx.buffer(4096)
+    with pytest.raises(H.TuckmillError):
+        ctx.q8_0_quantize_act(b, b, 48, 1, 0)
+    with pytest.raises(H.TuckmillError):
+        ctx.q8_0_quantize_act(b, b, 32, H.GEMM_I8_MAX_BATCH + 1, 0)
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.q8_0_quantize_act(b, ctx.buffer(35), 32, 1, 0)
+    assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS
+    with pytest.raises(H.TuckmillError):
+        ctx.q8_0_gemm_i8(b, b, b, 0, 32, 1, 0)
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.q8_0_gemm_i8(b, b, b, 4, 32, 1, 0, ctx.buffer(8))
+    assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS

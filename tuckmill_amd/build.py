@@ -1,0 +1,46 @@
+"""Builds the HIP library in-tree for gfx950 (hipcc cross-compiles without a GPU)."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libtm_hip.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# -packed-fp32-ops is switched off on purpose: v_pk_*_f32 forms are not used
+# by this library (the flag is for the device pass; the host pass warns that
+# it does not know the feature, which is harmless).
+DEVICE_FLAGS = [
+    "--offload-arch=gfx950",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-ffp-contract=off",
+]
+
+
+def build_library(verbose: bool = False, extra: list[str] | None = None) -> str:
+    cmd = [HIPCC, "-x", "hip", "-std=c++17", "-O3", "-fPIC", "-shared",
+           "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
+           *DEVICE_FLAGS,
+           "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+           *(extra or []),
+           "-o", LIB, os.path.join(CSRC, "tm_hip.cpp")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    out = "\n".join(l for l in (res.stdout + res.stderr).splitlines()
+                    if "packed-fp32-ops" not in l and l.strip())
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
+    if verbose and out:
+        print(out)
+    return LIB
+
+
+if __name__ == "__main__":
+    build_library(verbose=True, extra=sys.argv[1:])
+    print("built", LIB)

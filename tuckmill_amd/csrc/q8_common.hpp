@@ -1,0 +1,142 @@
+// Shared device helpers for the Q8_0 kernels (gfx950, wave64).
+//
+// Two weight layouts are understood everywhere:
+//   RAW    — GGUF bytes: blocks of 34 bytes ([f16 d][i8 qs; 32]), rows
+//            contiguous (crates/manifest/src/ggml.rs:47).
+//   PACKED — the sealed device layout: int8 quants [rows][cols] first, then
+//            f16 scales [rows][cols/32]; same total byte count.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace q8 {
+
+constexpr int WAVE = 64;
+
+enum Layout : int { RAW = 0, PACKED = 1 };
+
+// binary16 -> binary32. v_cvt_f32_f16 is exact for every encoding, subnormals
+// included: kernels run with FP16 denormals enabled (the HSA default mode).
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+// binary32 -> binary16 bits with the rounding of
+// crates/tuckcore/src/tensor.rs:145-178: round to nearest even, overflow and
+// NaN both become +-inf, magnitudes below 2^-25 become +-0.
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float value) {
+    uint32_t bits = __float_as_uint(value);
+    uint32_t sign = (bits >> 16) & 0x8000u;
+    int32_t exp = (int32_t)((bits >> 23) & 0xffu) - 127 + 15;
+    uint32_t mant = bits & 0x7fffffu;
+    if (exp >= 0x1f) {
+        return sign | 0x7c00u;
+    }
+    if (exp <= 0) {
+        if (exp < -10) {
+            return sign;
+        }
+        uint32_t m = mant | 0x800000u;
+        uint32_t shift = (uint32_t)(14 - exp);
+        uint32_t half = (m >> shift) & 0x3ffu;
+        uint32_t rem = m & ((1u << shift) - 1u);
+        uint32_t halfway = 1u << (shift - 1u);
+        if (rem > halfway || (rem == halfway && (half & 1u))) {
+            half += 1u;
+        }
+        return sign | half;
+    }
+    uint32_t rounded = mant + 0x0fffu + ((mant >> 13) & 1u);
+    if (rounded & 0x800000u) {
+        exp += 1;
+        if (exp >= 0x1f) {
+            return sign | 0x7c00u;
+        }
+        return sign | ((uint32_t)exp << 10);
+    }
+    return sign | ((uint32_t)exp << 10) | (rounded >> 13);
+}
+
+// Signed byte `i` (0..3) of a dword as float.
+__device__ __forceinline__ float sbyte_to_float(uint32_t w, int i) {
+    return (float)(int)(int8_t)(w >> (8 * i));
+}
+
+// ---- weight views -------------------------------------------------------
+
+template <int L> struct WView;
+
+template <> struct WView<PACKED> {
+    const uint8_t *q;   // [rows][cols] int8
+    const uint16_t *s;  // [rows][blocks] f16 bits
+    uint32_t cols, blocks;
+    __device__ __forceinline__ WView(const uint8_t *base, uint32_t rows, uint32_t cols_)
+        : q(base), s((const uint16_t *)(base + (size_t)rows * cols_)), cols(cols_),
+          blocks(cols_ / 32u) {}
+    // NB consecutive quants of `row` starting at column `col` (col % NB == 0,
+    // the piece lies inside one block) into NB/4 dwords (low bytes first).
+    template <int NB>
+    __device__ __forceinline__ void load_quants(uint32_t row, uint32_t col, uint32_t *out) const {
+        const uint8_t *p = q + (size_t)row * cols + col;
+        if constexpr (NB == 16) {
+            uint4 v = *(const uint4 *)p;
+            out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+        } else if constexpr (NB == 8) {
+            uint2 v = *(const uint2 *)p;
+            out[0] = v.x; out[1] = v.y;
+        } else if constexpr (NB == 4) {
+            out[0] = *(const uint32_t *)p;
+        } else if constexpr (NB == 2) {
+            out[0] = *(const uint16_t *)p;
+        } else {
+            out[0] = *p;
+        }
+    }
+    __device__ __forceinline__ uint32_t scale_bits(uint32_t row, uint32_t block) const {
+        return s[(size_t)row * blocks + block];
+    }
+};
+
+template <> struct WView<RAW> {
+    const uint8_t *base;
+    uint32_t blocks;
+    size_t row_bytes;
+    __device__ __forceinline__ WView(const uint8_t *base_, uint32_t /*rows*/, uint32_t cols_)
+        : base(base_), blocks(cols_ / 32u), row_bytes((size_t)(cols_ / 32u) * 34u) {}
+    template <int NB>
+    __device__ __forceinline__ void load_quants(uint32_t row, uint32_t col, uint32_t *out) const {
+        // 34-byte blocks leave the quants only 2-byte aligned.
+        const uint8_t *p = base + (size_t)row * row_bytes + (size_t)(col >> 5) * 34u + 2u + (col & 31u);
+        if constexpr (NB >= 2) {
+            const uint16_t *h = (const uint16_t *)p;
+#pragma unroll
+            for (int i = 0; i < NB / 4; ++i) {
+                out[i] = (uint32_t)h[2 * i] | ((uint32_t)h[2 * i + 1] << 16);
+            }
+            if constexpr (NB == 2) {
+                out[0] = h[0];
+            }
+        } else {
+            out[0] = *p;
+        }
+    }
+    __device__ __forceinline__ uint32_t scale_bits(uint32_t row, uint32_t block) const {
+        return *(const uint16_t *)(base + (size_t)row * row_bytes + (size_t)block * 34u);
+    }
+};
+
+// Sum over the 64 lanes of a wave; every lane returns the same bits. The
+// pairing (xor 32, 16, 8, 4, 2, 1) is fixed: all kernels that must agree
+// bit for bit reduce through this one function.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += __shfl_xor(v, 32, WAVE);
+    v += __shfl_xor(v, 16, WAVE);
+    v += __shfl_xor(v, 8, WAVE);
+    v += __shfl_xor(v, 4, WAVE);
+    v += __shfl_xor(v, 2, WAVE);
+    v += __shfl_xor(v, 1, WAVE);
+    return v;
+}
+
+} // namespace q8

@@ -1,0 +1,192 @@
+// Q8_0 matrix-vector / small-batch matrix-matrix kernel (bandwidth-bound).
+//
+// One launch runs a LIST of products (a decode step issues ~200 of them, most
+// far too small to fill 256 CUs alone). A wave owns `rows_per_tile` consecutive
+// rows of one product and walks them R rows at a time:
+//
+//   columns are cut into chunks of 1024 (16 quants per lane, one 16-byte load
+//   per lane per row = 1 KiB contiguous per wave), then a tail of 512/256/128/
+//   64/32 columns (8/4/2/1/1 quants per lane). A lane's piece always lies in
+//   one Q8_0 block, so   acc += d_block * (sum of q*x over the piece)
+//   with the sum taken left to right in fused multiply-adds. The 64 lane
+//   partials are reduced by q8::wave_sum.
+//
+// Per-(row, token) arithmetic depends only on `cols`, never on R, TB,
+// rows_per_tile, the layout or which other products share the launch: this is
+// what makes gemm(batch = 1) bit-identical to gemv, and every token of the
+// small-batch gemm bit-identical to its own gemv
+// (contract: native/metal/tm_metal.h:161-164).
+#pragma once
+
+#include "q8_common.hpp"
+
+namespace q8 {
+
+struct GemvDesc {
+    const uint8_t *w;
+    const float *x;        // x_off already applied
+    float *y;              // y_off already applied
+    uint32_t rows, cols;
+    uint32_t batch;
+    uint32_t tile_begin;   // index of this product's first tile in the launch
+    uint32_t rows_per_tile;
+    uint32_t pad;
+};
+
+constexpr int GEMV_MAX_DESCS = 84; // 84 * 48 + 16 = 4048 bytes of kernel arguments
+
+struct GemvArgs {
+    uint32_t n;
+    uint32_t total_tiles;
+    uint32_t pad[2];
+    GemvDesc d[GEMV_MAX_DESCS];
+};
+
+template <int NB, bool XA>
+__device__ __forceinline__ void load_x(const float *p, float *out) {
+    if constexpr (XA && NB >= 4) {
+#pragma unroll
+        for (int i = 0; i < NB / 4; ++i) {
+            float4 v = ((const float4 *)p)[i];
+            out[4 * i] = v.x; out[4 * i + 1] = v.y; out[4 * i + 2] = v.z; out[4 * i + 3] = v.w;
+        }
+    } else if constexpr (XA && NB == 2) {
+        float2 v = *(const float2 *)p;
+        out[0] = v.x; out[1] = v.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            out[i] = p[i];
+        }
+    }
+}
+
+template <int NB>
+__device__ __forceinline__ float piece_dot(const uint32_t *q, const float *x) {
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+        s = __builtin_fmaf(sbyte_to_float(q[i / 4], i % 4), x[i], s);
+    }
+    return s;
+}
+
+// One chunk of 64*NB columns starting at `col0`, for R rows and TB tokens.
+// `active` is false only for the upper half-wave of a trailing 32-column
+// chunk; inactive lanes still execute (on clamped addresses) and add 0.
+template <int L, int R, int TB, int NB, bool XA>
+__device__ __forceinline__ void chunk(const WView<L> &wv, const float *x, uint32_t cols,
+                                      const uint32_t (&row)[R], const uint32_t (&tok)[TB],
+                                      uint32_t col0, uint32_t lane, bool active,
+                                      float (&acc)[R][TB]) {
+    const uint32_t col = col0 + (active ? lane * NB : 0u);
+    constexpr int ND = NB >= 4 ? NB / 4 : 1;
+    uint32_t q[R][ND];
+    uint32_t sb[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        wv.template load_quants<NB>(row[r], col, q[r]);
+        sb[r] = wv.scale_bits(row[r], col >> 5);
+    }
+#pragma unroll
+    for (int t = 0; t < TB; ++t) {
+        float xv[NB];
+        load_x<NB, XA>(x + (size_t)tok[t] * cols + col, xv);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float d = active ? f16_bits_to_f32(sb[r]) : 0.0f;
+            const float s = active ? piece_dot<NB>(q[r], xv) : 0.0f;
+            acc[r][t] = __builtin_fmaf(d, s, acc[r][t]);
+        }
+    }
+}
+
+template <int L, int R, int TB, bool XA>
+__global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t tile = blockIdx.x * 4u + wave;
+    if (tile >= args.total_tiles) {
+        return;
+    }
+    // Locate the product that owns this tile (tile_begin is increasing).
+    uint32_t lo = 0, hi = args.n;
+    while (hi - lo > 1u) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (args.d[mid].tile_begin <= tile) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    const GemvDesc &d = args.d[lo];
+    const uint32_t rows = d.rows, cols = d.cols, batch = d.batch;
+    const WView<L> wv(d.w, rows, cols);
+    const float *x = d.x;
+    float *y = d.y;
+    const uint32_t row_first = (tile - d.tile_begin) * d.rows_per_tile;
+    uint32_t row_end = row_first + d.rows_per_tile;
+    if (row_end > rows) {
+        row_end = rows;
+    }
+    const uint32_t full = cols >> 10;
+    const uint32_t tail0 = full << 10;
+
+    for (uint32_t t0 = 0; t0 < batch; t0 += TB) {
+        uint32_t tok[TB];
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+            tok[t] = (t0 + t < batch) ? t0 + t : batch - 1u;
+        }
+        for (uint32_t r0 = row_first; r0 < row_end; r0 += R) {
+            uint32_t row[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                row[r] = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+            }
+            float acc[R][TB];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+#pragma unroll
+                for (int t = 0; t < TB; ++t) {
+                    acc[r][t] = 0.0f;
+                }
+            }
+            for (uint32_t c = 0; c < full; ++c) {
+                chunk<L, R, TB, 16, XA>(wv, x, cols, row, tok, c << 10, lane, true, acc);
+            }
+            uint32_t col0 = tail0;
+            if (cols & 512u) {
+                chunk<L, R, TB, 8, XA>(wv, x, cols, row, tok, col0, lane, true, acc);
+                col0 += 512u;
+            }
+            if (cols & 256u) {
+                chunk<L, R, TB, 4, XA>(wv, x, cols, row, tok, col0, lane, true, acc);
+                col0 += 256u;
+            }
+            if (cols & 128u) {
+                chunk<L, R, TB, 2, XA>(wv, x, cols, row, tok, col0, lane, true, acc);
+                col0 += 128u;
+            }
+            if (cols & 64u) {
+                chunk<L, R, TB, 1, XA>(wv, x, cols, row, tok, col0, lane, true, acc);
+                col0 += 64u;
+            }
+            if (cols & 32u) {
+                chunk<L, R, TB, 1, XA>(wv, x, cols, row, tok, col0, lane, lane < 32u, acc);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+#pragma unroll
+                for (int t = 0; t < TB; ++t) {
+                    const float total = wave_sum(acc[r][t]);
+                    if (lane == 0u && r0 + r < row_end && t0 + t < batch) {
+                        y[(size_t)(t0 + t) * rows + (r0 + r)] = total;
+                    }
+                }
+            }
+        }
+    }
+}
+
+} // namespace q8

@@ -1,0 +1,1315 @@
+// tm_hip.cpp — host side of the C ABI declared in include/tm_hip.h.
+//
+// Mirrors the contract of the reference's Metal host
+// (native/metal/tm_metal.m): argument validation before any device work,
+// typed refusals, buffer leases held by pending commits, grouped encoding,
+// completion accounting. The execution model underneath is HIP's: one
+// non-blocking stream per context, one pair of HIP events per commit, and a
+// group that is scheduled at end_group (independent Q8_0 products coalesce
+// into one launch of the list kernel).
+#include "tm_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <deque>
+#include <mutex>
+#include <string>
+#include <unistd.h>
+#include <vector>
+
+#include "q8_gemm_i8.hpp"
+#include "q8_gemm_mma.hpp"
+#include "q8_gemv.hpp"
+#include "q8_misc.hpp"
+
+namespace {
+
+constexpr int kProfileSlots = 128;
+constexpr int kProfileName = 48;
+
+struct Alloc {
+    void *ptr = nullptr;
+    size_t len = 0;
+    std::atomic<int> refs{1};
+    bool packed = false;
+    uint32_t prows = 0, pcols = 0;
+};
+
+void alloc_release(Alloc *a) {
+    if (a != nullptr && a->refs.fetch_sub(1, std::memory_order_acq_rel) == 1) {
+        (void)hipFree(a->ptr);
+        delete a;
+    }
+}
+
+enum OpKind { OP_GEMV_LIST, OP_MMA, OP_ROW, OP_ROW_INDIRECT, OP_COPY, OP_PACK, OP_QUANT, OP_I8 };
+
+struct Op {
+    OpKind kind;
+    Alloc *a[4] = {nullptr, nullptr, nullptr, nullptr}; // a[0..] buffers touched; see writes_mask
+    int n_alloc = 0;
+    unsigned writes_mask = 0; // bit i: a[i] is written
+    uint32_t rows = 0, cols = 0, batch = 0, x_off = 0, y_off = 0, extra = 0;
+    bool packed = false;
+    char label[kProfileName] = {0};
+};
+
+struct Commit {
+    uint64_t seq = 0;
+    hipEvent_t start = nullptr, stop = nullptr;
+    std::vector<Alloc *> keep;
+    uint64_t leased = 0;
+    char label[kProfileName] = {0};
+};
+
+struct ProfileSlot {
+    char name[kProfileName];
+    uint64_t nanos;
+    uint64_t count;
+};
+
+} // namespace
+
+struct tm_hip_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipStream_t copy_stream = nullptr;
+    std::atomic<uint64_t> allocated{0};
+    std::atomic<uint64_t> leased{0};
+    std::atomic<uint64_t> committed{0};
+    std::atomic<uint64_t> completed{0};
+    std::atomic<uint64_t> last_gpu_nanos{0};
+    std::atomic<uint64_t> gpu_nanos_total{0};
+    std::atomic<uint64_t> launches{0};
+    std::atomic<int> profiling{0};
+    bool group_active = false;
+    std::vector<Op> group_ops;
+    std::mutex q_mu; // pending commits, event pool, profile table
+    std::mutex copy_mu;
+    std::deque<Commit> pending;
+    std::vector<hipEvent_t> event_pool;
+    ProfileSlot profile[kProfileSlots];
+    uint32_t profile_used = 0;
+};
+
+struct tm_hip_buffer {
+    tm_hip_ctx *owner;
+    Alloc *alloc;
+    size_t len;
+    int shared;
+};
+
+namespace {
+
+// ------------------------------------------------------------- errors ----
+
+int fail(char *err, size_t cap, int code, const char *fmt, ...) {
+    if (err != nullptr && cap > 0) {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(err, cap, fmt, ap);
+        va_end(ap);
+    }
+    return code;
+}
+
+int check_ctx(tm_hip_ctx *ctx, char *err, size_t cap, const char *what) {
+    if (ctx == nullptr) {
+        return fail(err, cap, TM_HIP_ERR_UNSUPPORTED, "%s: null context", what);
+    }
+    return TM_HIP_OK;
+}
+
+// native/metal/tm_metal.m:153-165: ownership first, then length.
+int check_buffer(tm_hip_ctx *ctx, tm_hip_buffer *b, size_t need, char *err, size_t cap,
+                 const char *name) {
+    if (b == nullptr || b->owner != ctx) {
+        return fail(err, cap, TM_HIP_ERR_UNSUPPORTED,
+                    "%s: buffer does not belong to this context (different context or null)", name);
+    }
+    if (need == 0 || b->len < need) {
+        return fail(err, cap, TM_HIP_ERR_BOUNDS, "%s: buffer holds %zu bytes but %zu are required",
+                    name, b->len, need);
+    }
+    return TM_HIP_OK;
+}
+
+int hip_fail(char *err, size_t cap, const char *what, hipError_t e) {
+    return fail(err, cap, TM_HIP_ERR_INTERNAL, "%s: %s", what, hipGetErrorString(e));
+}
+
+// ------------------------------------------------ completion accounting --
+
+hipEvent_t take_event(tm_hip_ctx *ctx) {
+    // q_mu held by the caller
+    if (!ctx->event_pool.empty()) {
+        hipEvent_t e = ctx->event_pool.back();
+        ctx->event_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) {
+        return nullptr;
+    }
+    return e;
+}
+
+void account_profile(tm_hip_ctx *ctx, const char *label, uint64_t nanos) {
+    // q_mu held by the caller
+    if (label[0] == '\0') {
+        return;
+    }
+    uint32_t slot = 0;
+    while (slot < ctx->profile_used && strcmp(ctx->profile[slot].name, label) != 0) {
+        slot++;
+    }
+    if (slot == ctx->profile_used && slot < kProfileSlots) {
+        snprintf(ctx->profile[slot].name, kProfileName, "%s", label);
+        ctx->profile[slot].nanos = 0;
+        ctx->profile[slot].count = 0;
+        ctx->profile_used++;
+    }
+    if (slot < kProfileSlots) {
+        ctx->profile[slot].nanos += nanos;
+        ctx->profile[slot].count += 1;
+    }
+}
+
+// Retire every commit whose stop event has been reached, in order. May be
+// called from any thread.
+void settle(tm_hip_ctx *ctx) {
+    std::vector<Alloc *> release;
+    {
+        std::lock_guard<std::mutex> g(ctx->q_mu);
+        while (!ctx->pending.empty()) {
+            Commit &c = ctx->pending.front();
+            if (hipEventQuery(c.stop) != hipSuccess) {
+                break;
+            }
+            float ms = 0.0f;
+            if (hipEventElapsedTime(&ms, c.start, c.stop) != hipSuccess || ms < 0.0f) {
+                ms = 0.0f;
+            }
+            const uint64_t nanos = (uint64_t)((double)ms * 1e6);
+            ctx->last_gpu_nanos.store(nanos, std::memory_order_relaxed);
+            ctx->gpu_nanos_total.fetch_add(nanos, std::memory_order_relaxed);
+            account_profile(ctx, c.label, nanos);
+            ctx->leased.fetch_sub(c.leased, std::memory_order_relaxed);
+            ctx->event_pool.push_back(c.start);
+            ctx->event_pool.push_back(c.stop);
+            release.insert(release.end(), c.keep.begin(), c.keep.end());
+            ctx->pending.pop_front();
+            ctx->completed.fetch_add(1, std::memory_order_release);
+        }
+    }
+    for (Alloc *a : release) {
+        alloc_release(a);
+    }
+}
+
+int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        return hip_fail(err, cap, "stream synchronize", e);
+    }
+    settle(ctx);
+    if (ctx->completed.load(std::memory_order_acquire) <
+        ctx->committed.load(std::memory_order_relaxed)) {
+        return fail(err, cap, TM_HIP_ERR_INTERNAL,
+                    "fence: stream drained but completion accounting did not settle");
+    }
+    return TM_HIP_OK;
+}
+
+// ------------------------------------------------------------ launches ---
+
+void add_unique(std::vector<Alloc *> &keep, Alloc *a) {
+    for (Alloc *k : keep) {
+        if (k == a) {
+            return;
+        }
+    }
+    keep.push_back(a);
+}
+
+struct GemvKey {
+    bool packed;
+    int tb;       // tokens per pass: 1 or 4
+    bool xalign;
+    bool operator==(const GemvKey &o) const {
+        return packed == o.packed && tb == o.tb && xalign == o.xalign;
+    }
+};
+
+GemvKey gemv_key(const Op &op) {
+    GemvKey k;
+    k.packed = op.packed;
+    k.tb = op.batch == 1 ? 1 : 4;
+    const uintptr_t xp = (uintptr_t)op.a[1]->ptr + (uintptr_t)op.x_off * 4u;
+    k.xalign = (xp % 16u == 0) && (op.batch == 1 || op.cols % 4u == 0);
+    return k;
+}
+
+uint32_t pick_rows_per_tile(uint32_t rows, uint32_t cols, uint32_t batch, int R) {
+    // Aim for about 16 KiB of weights per wave, at least one pass of R rows;
+    // small matrices get smaller tiles so that they still spread over CUs.
+    (void)batch;
+    uint32_t rpt = (16384u / cols);
+    if (rpt < (uint32_t)R) {
+        rpt = (uint32_t)R;
+    }
+    rpt = (rpt / (uint32_t)R) * (uint32_t)R;
+    while (rpt > (uint32_t)R && (rows + rpt - 1) / rpt < 2048u) {
+        rpt -= (uint32_t)R;
+    }
+    return rpt;
+}
+
+template <int L, int R, int TB, bool XA>
+hipError_t launch_gemv(tm_hip_ctx *ctx, const q8::GemvArgs &args) {
+    const uint32_t groups = (args.total_tiles + 3u) / 4u;
+    hipLaunchKernelGGL((q8::gemv_list_kernel<L, R, TB, XA>), dim3(groups), dim3(256), 0, ctx->stream,
+                       args);
+    ctx->launches.fetch_add(1, std::memory_order_relaxed);
+    return hipGetLastError();
+}
+
+constexpr int kGemvR1 = 4; // rows per pass at one token per pass
+constexpr int kGemvR4 = 2; // rows per pass at four tokens per pass
+
+hipError_t launch_gemv_list(tm_hip_ctx *ctx, const std::vector<const Op *> &ops, GemvKey key) {
+    q8::GemvArgs args;
+    memset(&args, 0, sizeof args);
+    const int R = key.tb == 1 ? kGemvR1 : kGemvR4;
+    uint32_t tiles = 0;
+    for (const Op *op : ops) {
+        q8::GemvDesc &d = args.d[args.n++];
+        d.w = (const uint8_t *)op->a[0]->ptr;
+        d.x = (const float *)op->a[1]->ptr + op->x_off;
+        d.y = (float *)op->a[2]->ptr + op->y_off;
+        d.rows = op->rows;
+        d.cols = op->cols;
+        d.batch = op->batch;
+        d.tile_begin = tiles;
+        d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, op->batch, R);
+        tiles += (op->rows + d.rows_per_tile - 1) / d.rows_per_tile;
+    }
+    args.total_tiles = tiles;
+#define TM_GEMV_CASE(P, T, A)                                                          \
+    if (key.packed == (P) && key.tb == (T) && key.xalign == (A)) {                     \
+        return launch_gemv<(P) ? q8::PACKED : q8::RAW, (T) == 1 ? kGemvR1 : kGemvR4, T, A>(ctx, args); \
+    }
+    TM_GEMV_CASE(true, 1, true)
+    TM_GEMV_CASE(true, 1, false)
+    TM_GEMV_CASE(true, 4, true)
+    TM_GEMV_CASE(true, 4, false)
+    TM_GEMV_CASE(false, 1, true)
+    TM_GEMV_CASE(false, 1, false)
+    TM_GEMV_CASE(false, 4, true)
+    TM_GEMV_CASE(false, 4, false)
+#undef TM_GEMV_CASE
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_single(tm_hip_ctx *ctx, const Op &op) {
+    const uint8_t *w = op.a[0] ? (const uint8_t *)op.a[0]->ptr : nullptr;
+    switch (op.kind) {
+    case OP_ROW: {
+        float *out = (float *)op.a[1]->ptr;
+        dim3 grid((op.cols + 255u) / 256u);
+        if (op.packed) {
+            hipLaunchKernelGGL(q8::row_kernel<q8::PACKED>, grid, dim3(256), 0, ctx->stream, w, out,
+                               op.rows, op.cols, op.extra, op.y_off);
+        } else {
+            hipLaunchKernelGGL(q8::row_kernel<q8::RAW>, grid, dim3(256), 0, ctx->stream, w, out,
+                               op.rows, op.cols, op.extra, op.y_off);
+        }
+        break;
+    }
+    case OP_ROW_INDIRECT: {
+        float *out = (float *)op.a[1]->ptr;
+        const uint32_t *ids = (const uint32_t *)op.a[2]->ptr;
+        dim3 grid((op.cols + 255u) / 256u);
+        if (op.packed) {
+            hipLaunchKernelGGL(q8::row_indirect_kernel<q8::PACKED>, grid, dim3(256), 0, ctx->stream,
+                               w, out, ids, op.extra, op.rows, op.cols);
+        } else {
+            hipLaunchKernelGGL(q8::row_indirect_kernel<q8::RAW>, grid, dim3(256), 0, ctx->stream, w,
+                               out, ids, op.extra, op.rows, op.cols);
+        }
+        break;
+    }
+    case OP_COPY: {
+        const float *src = (const float *)op.a[0]->ptr + op.x_off;
+        float *dst = (float *)op.a[1]->ptr + op.y_off;
+        hipLaunchKernelGGL(q8::copy_f32_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0,
+                           ctx->stream, src, dst, op.extra);
+        break;
+    }
+    case OP_PACK: {
+        const size_t nblocks = (size_t)op.rows * (op.cols / 32u);
+        hipLaunchKernelGGL(q8::pack_kernel, dim3((unsigned)((nblocks + 255u) / 256u)), dim3(256), 0,
+                           ctx->stream, w, (uint8_t *)op.a[1]->ptr, op.rows, op.cols);
+        break;
+    }
+    case OP_MMA: {
+        ctx->launches.fetch_add(1, std::memory_order_relaxed);
+        return q8::launch_gemm_mma(ctx->stream, op.packed, w,
+                                   (const float *)op.a[1]->ptr + op.x_off,
+                                   (float *)op.a[2]->ptr + op.y_off, op.rows, op.cols, op.batch);
+    }
+    case OP_QUANT: {
+        ctx->launches.fetch_add(1, std::memory_order_relaxed);
+        return q8::launch_quantize_act(ctx->stream, (const float *)op.a[0]->ptr + op.x_off,
+                                       (uint8_t *)op.a[1]->ptr, op.cols, op.batch);
+    }
+    case OP_I8: {
+        ctx->launches.fetch_add(1, std::memory_order_relaxed);
+        return q8::launch_gemm_i8(ctx->stream, op.packed, w, (const uint8_t *)op.a[1]->ptr,
+                                  (float *)op.a[2]->ptr + op.y_off,
+                                  op.a[3] ? (int32_t *)op.a[3]->ptr : nullptr, op.rows, op.cols,
+                                  op.batch);
+    }
+    default:
+        return hipErrorInvalidValue;
+    }
+    ctx->launches.fetch_add(1, std::memory_order_relaxed);
+    return hipGetLastError();
+}
+
+// Issue a sequence of recorded operations. Consecutive list-kernel products
+// that neither read nor overwrite each other's outputs share one launch.
+hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
+    std::vector<const Op *> batch;
+    GemvKey batch_key{};
+    auto flush = [&]() -> hipError_t {
+        if (batch.empty()) {
+            return hipSuccess;
+        }
+        hipError_t e = launch_gemv_list(ctx, batch, batch_key);
+        batch.clear();
+        return e;
+    };
+    for (const Op &op : ops) {
+        if (op.kind == OP_GEMV_LIST) {
+            const GemvKey key = gemv_key(op);
+            bool conflict = false;
+            for (const Op *b : batch) {
+                // a[0] = w (read), a[1] = x (read), a[2] = y (written)
+                if (op.a[2] == b->a[2] || op.a[2] == b->a[1] || op.a[2] == b->a[0] ||
+                    op.a[1] == b->a[2] || op.a[0] == b->a[2]) {
+                    conflict = true;
+                    break;
+                }
+            }
+            if (!batch.empty() &&
+                (conflict || !(key == batch_key) || (int)batch.size() == q8::GEMV_MAX_DESCS)) {
+                hipError_t e = flush();
+                if (e != hipSuccess) {
+                    return e;
+                }
+            }
+            batch_key = key;
+            batch.push_back(&op);
+        } else {
+            hipError_t e = flush();
+            if (e != hipSuccess) {
+                return e;
+            }
+            e = launch_single(ctx, op);
+            if (e != hipSuccess) {
+                return e;
+            }
+        }
+    }
+    return flush();
+}
+
+// Submit `ops` as one commit: start event, launches, stop event, leases.
+int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, char *err,
+               size_t cap) {
+    Commit c;
+    {
+        std::lock_guard<std::mutex> g(ctx->q_mu);
+        c.start = take_event(ctx);
+        c.stop = take_event(ctx);
+    }
+    if (c.start == nullptr || c.stop == nullptr) {
+        return fail(err, cap, TM_HIP_ERR_INTERNAL, "%s: event creation failed", label);
+    }
+    for (const Op &op : ops) {
+        for (int i = 0; i < op.n_alloc; ++i) {
+            if (op.a[i] != nullptr) {
+                add_unique(c.keep, op.a[i]);
+            }
+        }
+    }
+    for (Alloc *a : c.keep) {
+        a->refs.fetch_add(1, std::memory_order_relaxed);
+        c.leased += a->len;
+    }
+    if (ctx->profiling.load(std::memory_order_relaxed)) {
+        snprintf(c.label, sizeof c.label, "%s", label);
+    }
+    hipError_t e = hipEventRecord(c.start, ctx->stream);
+    if (e == hipSuccess) {
+        e = issue_ops(ctx, ops);
+    }
+    hipError_t e2 = hipEventRecord(c.stop, ctx->stream);
+    if (e == hipSuccess) {
+        e = e2;
+    }
+    c.seq = ctx->committed.fetch_add(1, std::memory_order_relaxed) + 1;
+    ctx->leased.fetch_add(c.leased, std::memory_order_relaxed);
+    {
+        std::lock_guard<std::mutex> g(ctx->q_mu);
+        ctx->pending.push_back(std::move(c));
+    }
+    settle(ctx);
+    if (e != hipSuccess) {
+        return hip_fail(err, cap, label, e);
+    }
+    return TM_HIP_OK;
+}
+
+// Either appends to the open group or commits on its own.
+int submit(tm_hip_ctx *ctx, Op &op, const char *label, char *err, size_t cap) {
+    snprintf(op.label, sizeof op.label, "%s", label);
+    if (ctx->group_active) {
+        ctx->group_ops.push_back(op);
+        return TM_HIP_OK;
+    }
+    std::vector<Op> one(1, op);
+    return commit_ops(ctx, one, label, err, cap);
+}
+
+struct DeviceProbe {
+    int available = 0;
+    int device = -1;
+    char info[256];
+};
+
+const DeviceProbe &probe() {
+    static DeviceProbe p = [] {
+        DeviceProbe r;
+        int n = 0;
+        if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            snprintf(r.info, sizeof r.info, "no HIP device available");
+            return r;
+        }
+        for (int i = 0; i < n; ++i) {
+            hipDeviceProp_t prop;
+            if (hipGetDeviceProperties(&prop, i) != hipSuccess) {
+                continue;
+            }
+            if (strncmp(prop.gcnArchName, "gfx950", 6) == 0) {
+                r.available = 1;
+                r.device = i;
+                snprintf(r.info, sizeof r.info, "%s %s (%d CUs, %llu MiB device memory)", prop.name,
+                         prop.gcnArchName, prop.multiProcessorCount,
+                         (unsigned long long)(prop.totalGlobalMem / (1024ull * 1024ull)));
+                return r;
+            }
+        }
+        snprintf(r.info, sizeof r.info, "no HIP device of architecture gfx950 (%d other device%s)", n,
+                 n == 1 ? "" : "s");
+        return r;
+    }();
+    return p;
+}
+
+// Shared argument checks of the three products
+// (native/metal/tm_metal.m:968-980, :1279-1290).
+int check_product(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                  uint32_t rows, uint32_t cols, uint32_t batch, uint32_t max_batch, uint32_t x_off,
+                  uint32_t y_off, char *err, size_t cap, const char *what) {
+    if (check_ctx(ctx, err, cap, what) != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (rows == 0 || cols == 0 || (cols % 32u) != 0u || batch == 0 || batch > max_batch) {
+        return fail(err, cap, TM_HIP_ERR_UNSUPPORTED,
+                    "%s: rows %u, cols %u (a positive multiple of 32), batch %u (1..=%u)", what,
+                    rows, cols, batch, max_batch);
+    }
+    const size_t w_need = (size_t)rows * ((size_t)cols / 32u) * 34u;
+    const size_t x_need = ((size_t)x_off + (size_t)batch * cols) * 4u;
+    const size_t y_need = ((size_t)y_off + (size_t)batch * rows) * 4u;
+    char name[64];
+    snprintf(name, sizeof name, "%s.weights", what);
+    int rc = check_buffer(ctx, w, w_need, err, cap, name);
+    if (rc != TM_HIP_OK) {
+        return rc == TM_HIP_ERR_BOUNDS ? TM_HIP_ERR_BOUNDS : rc;
+    }
+    snprintf(name, sizeof name, "%s.x", what);
+    if ((rc = check_buffer(ctx, x, x_need, err, cap, name)) != TM_HIP_OK) {
+        return rc;
+    }
+    snprintf(name, sizeof name, "%s.y", what);
+    if ((rc = check_buffer(ctx, y, y_need, err, cap, name)) != TM_HIP_OK) {
+        return rc;
+    }
+    if (w->alloc->packed && (w->alloc->prows != rows || w->alloc->pcols != cols)) {
+        return fail(err, cap, TM_HIP_ERR_UNSUPPORTED,
+                    "%s: weights were sealed as %ux%u but the call names %ux%u", what,
+                    w->alloc->prows, w->alloc->pcols, rows, cols);
+    }
+    if (x->alloc->packed || y->alloc->packed) {
+        return fail(err, cap, TM_HIP_ERR_UNSUPPORTED, "%s: x/y must not be sealed weight buffers",
+                    what);
+    }
+    return TM_HIP_OK;
+}
+
+} // namespace
+
+// ================================================================ ABI =====
+
+extern "C" {
+
+int tm_hip_available(void) { return probe().available; }
+
+const char *tm_hip_runtime_info(void) { return probe().info; }
+
+tm_hip_ctx *tm_hip_create(char *err, size_t err_cap) {
+    const DeviceProbe &p = probe();
+    if (!p.available) {
+        fail(err, err_cap, TM_HIP_ERR_NO_DEVICE, "%s", p.info);
+        return nullptr;
+    }
+    hipError_t e = hipSetDevice(p.device);
+    if (e != hipSuccess) {
+        hip_fail(err, err_cap, "set device", e);
+        return nullptr;
+    }
+    tm_hip_ctx *ctx = new (std::nothrow) tm_hip_ctx();
+    if (ctx == nullptr) {
+        fail(err, err_cap, TM_HIP_ERR_INTERNAL, "context allocation failed");
+        return nullptr;
+    }
+    ctx->device = p.device;
+    e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) {
+        e = hipStreamCreateWithFlags(&ctx->copy_stream, hipStreamNonBlocking);
+    }
+    if (e != hipSuccess) {
+        hip_fail(err, err_cap, "stream creation", e);
+        tm_hip_destroy(ctx);
+        return nullptr;
+    }
+    // Fail at creation, not at first use, when the device code is missing.
+    hipFuncAttributes attr;
+    e = hipFuncGetAttributes(&attr, (const void *)q8::gemv_list_kernel<q8::PACKED, kGemvR1, 1, true>);
+    if (e != hipSuccess) {
+        fail(err, err_cap, TM_HIP_ERR_SOURCE, "kernels for this device are missing: %s",
+             hipGetErrorString(e));
+        tm_hip_destroy(ctx);
+        return nullptr;
+    }
+    return ctx;
+}
+
+void tm_hip_destroy(tm_hip_ctx *ctx) {
+    if (ctx == nullptr) {
+        return;
+    }
+    if (ctx->group_active) {
+        for (Op &op : ctx->group_ops) {
+            (void)op;
+        }
+        ctx->group_ops.clear();
+        ctx->group_active = false;
+    }
+    if (ctx->stream != nullptr) {
+        (void)hipStreamSynchronize(ctx->stream);
+    }
+    settle(ctx);
+    {
+        std::lock_guard<std::mutex> g(ctx->q_mu);
+        for (Commit &c : ctx->pending) { // only after a device error
+            for (Alloc *a : c.keep) {
+                alloc_release(a);
+            }
+            (void)hipEventDestroy(c.start);
+            (void)hipEventDestroy(c.stop);
+        }
+        ctx->pending.clear();
+        for (hipEvent_t e : ctx->event_pool) {
+            (void)hipEventDestroy(e);
+        }
+        ctx->event_pool.clear();
+    }
+    if (ctx->copy_stream != nullptr) {
+        (void)hipStreamDestroy(ctx->copy_stream);
+    }
+    if (ctx->stream != nullptr) {
+        (void)hipStreamDestroy(ctx->stream);
+    }
+    delete ctx;
+}
+
+tm_hip_buffer *tm_hip_buffer_new(tm_hip_ctx *ctx, size_t bytes, int shared, char *err,
+                                 size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "buffer_new") != TM_HIP_OK) {
+        return nullptr;
+    }
+    if (bytes == 0) {
+        fail(err, err_cap, TM_HIP_ERR_BOUNDS, "buffer_new: zero-length allocation");
+        return nullptr;
+    }
+    void *ptr = nullptr;
+    hipError_t e = hipMalloc(&ptr, bytes);
+    if (e != hipSuccess || ptr == nullptr) {
+        (void)hipGetLastError();
+        fail(err, err_cap, TM_HIP_ERR_ALLOC, "buffer_new: allocation of %zu bytes failed (%s)",
+             bytes, hipGetErrorString(e));
+        return nullptr;
+    }
+    e = hipMemsetAsync(ptr, 0, bytes, ctx->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(ptr);
+        hip_fail(err, err_cap, "buffer_new: zero fill", e);
+        return nullptr;
+    }
+    Alloc *a = new (std::nothrow) Alloc();
+    tm_hip_buffer *h = new (std::nothrow) tm_hip_buffer();
+    if (a == nullptr || h == nullptr) {
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipFree(ptr);
+        delete a;
+        delete h;
+        fail(err, err_cap, TM_HIP_ERR_ALLOC, "buffer_new: handle allocation failed");
+        return nullptr;
+    }
+    a->ptr = ptr;
+    a->len = bytes;
+    h->owner = ctx;
+    h->alloc = a;
+    h->len = bytes;
+    h->shared = shared ? 1 : 0;
+    ctx->allocated.fetch_add(bytes, std::memory_order_relaxed);
+    return h;
+}
+
+void tm_hip_buffer_free(tm_hip_ctx *ctx, tm_hip_buffer *buffer) {
+    if (ctx == nullptr || buffer == nullptr) {
+        return;
+    }
+    if (buffer->owner != ctx) {
+        fprintf(stderr, "tm_hip: buffer_free from a different context refused\n");
+        return;
+    }
+    ctx->allocated.fetch_sub(buffer->len, std::memory_order_relaxed);
+    Alloc *a = buffer->alloc;
+    buffer->alloc = nullptr;
+    buffer->owner = nullptr;
+    delete buffer;
+    settle(ctx);
+    if (a->refs.load(std::memory_order_acquire) == 1) {
+        // No commit leases it, but the zero fill of buffer_new or a host copy
+        // may still be queued on the stream.
+        (void)hipStreamSynchronize(ctx->stream);
+        settle(ctx);
+    }
+    alloc_release(a);
+}
+
+size_t tm_hip_buffer_len(const tm_hip_ctx *ctx, const tm_hip_buffer *buffer) {
+    if (ctx == nullptr || buffer == nullptr || buffer->owner != ctx) {
+        return 0;
+    }
+    return buffer->len;
+}
+
+int tm_hip_buffer_zero(tm_hip_ctx *ctx, tm_hip_buffer *buffer, size_t off, size_t len, char *err,
+                       size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "buffer_zero") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (buffer == nullptr || buffer->owner != ctx) {
+        return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "buffer_zero: foreign buffer");
+    }
+    if (len == 0) {
+        return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "buffer_zero: zero length");
+    }
+    if (off > buffer->len || len > buffer->len - off) {
+        return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "buffer_zero: range outside the buffer");
+    }
+    if (buffer->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "buffer_zero: buffer holds sealed Q8_0 weights");
+    }
+    hipError_t e = hipMemsetAsync((uint8_t *)buffer->alloc->ptr + off, 0, len, ctx->stream);
+    if (e != hipSuccess) {
+        return hip_fail(err, err_cap, "buffer_zero", e);
+    }
+    return TM_HIP_OK;
+}
+
+static int host_copy(tm_hip_ctx *ctx, tm_hip_buffer *buffer, size_t off, void *host, size_t len,
+                     int to_device, char *err, size_t err_cap, const char *what) {
+    if (check_ctx(ctx, err, err_cap, what) != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (buffer == nullptr || buffer->owner != ctx) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "%s: buffer does not belong to this context", what);
+    }
+    if (len == 0 || off > buffer->len || len > buffer->len - off) {
+        return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "%s: range %zu..%zu outside buffer", what, off,
+                    off + len);
+    }
+    if (host == nullptr) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "%s: null host pointer", what);
+    }
+    if (!buffer->shared) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "%s: private buffers have no host copy",
+                    what);
+    }
+    if (buffer->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "%s: buffer holds sealed Q8_0 weights (device layout)", what);
+    }
+    if (ctx->group_active) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "%s: close the open dispatch group first", what);
+    }
+    int rc = wait_pending(ctx, err, err_cap);
+    if (rc != TM_HIP_OK) {
+        return rc;
+    }
+    uint8_t *dev = (uint8_t *)buffer->alloc->ptr + off;
+    hipError_t e = to_device ? hipMemcpyAsync(dev, host, len, hipMemcpyHostToDevice, ctx->stream)
+                             : hipMemcpyAsync(host, dev, len, hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) {
+        e = hipStreamSynchronize(ctx->stream);
+    }
+    if (e != hipSuccess) {
+        return hip_fail(err, err_cap, what, e);
+    }
+    return TM_HIP_OK;
+}
+
+int tm_hip_upload(tm_hip_ctx *ctx, tm_hip_buffer *dst, size_t off, const void *src, size_t len,
+                  char *err, size_t err_cap) {
+    return host_copy(ctx, dst, off, (void *)src, len, 1, err, err_cap, "upload");
+}
+
+int tm_hip_download(tm_hip_ctx *ctx, tm_hip_buffer *src, size_t off, void *dst, size_t len,
+                    char *err, size_t err_cap) {
+    return host_copy(ctx, src, off, dst, len, 0, err, err_cap, "download");
+}
+
+int tm_hip_download_after(tm_hip_ctx *ctx, tm_hip_buffer *src, size_t off, void *dst, size_t len,
+                          uint64_t completed_target, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "download_after") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (src == nullptr || src->owner != ctx) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "download_after: buffer does not belong to this context");
+    }
+    if (len == 0 || off > src->len || len > src->len - off) {
+        return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "download_after: range %zu..%zu outside buffer",
+                    off, off + len);
+    }
+    if (dst == nullptr) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "download_after: null host pointer");
+    }
+    if (!src->shared || src->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "download_after: buffer has no host copy");
+    }
+    if (completed_target > ctx->committed.load(std::memory_order_relaxed)) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "download_after: target is beyond the committed dispatches");
+    }
+    // Commits complete in stream order; wait for the target only.
+    for (;;) {
+        settle(ctx);
+        if (ctx->completed.load(std::memory_order_acquire) >= completed_target) {
+            break;
+        }
+        usleep(20);
+    }
+    std::lock_guard<std::mutex> g(ctx->copy_mu);
+    hipError_t e = hipMemcpyAsync(dst, (const uint8_t *)src->alloc->ptr + off, len,
+                                  hipMemcpyDeviceToHost, ctx->copy_stream);
+    if (e == hipSuccess) {
+        e = hipStreamSynchronize(ctx->copy_stream);
+    }
+    if (e != hipSuccess) {
+        return hip_fail(err, err_cap, "download_after", e);
+    }
+    return TM_HIP_OK;
+}
+
+int tm_hip_copy_f32(tm_hip_ctx *ctx, tm_hip_buffer *src, uint32_t src_off, tm_hip_buffer *dst,
+                    uint32_t dst_off, uint32_t n, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "copy_f32") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (n == 0) {
+        return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "copy_f32: zero-length copy");
+    }
+    int rc;
+    if ((rc = check_buffer(ctx, src, ((size_t)src_off + n) * 4u, err, err_cap, "copy_f32.src")) !=
+            TM_HIP_OK ||
+        (rc = check_buffer(ctx, dst, ((size_t)dst_off + n) * 4u, err, err_cap, "copy_f32.dst")) !=
+            TM_HIP_OK) {
+        return rc;
+    }
+    if (src->alloc->packed || dst->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "copy_f32: sealed weight buffer");
+    }
+    Op op;
+    op.kind = OP_COPY;
+    op.a[0] = src->alloc;
+    op.a[1] = dst->alloc;
+    op.n_alloc = 2;
+    op.writes_mask = 2;
+    op.x_off = src_off;
+    op.y_off = dst_off;
+    op.extra = n;
+    return submit(ctx, op, "copy_f32", err, err_cap);
+}
+
+int tm_hip_begin_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "begin_group") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (ctx->group_active) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "begin_group: a dispatch group is already open");
+    }
+    ctx->group_ops.clear();
+    ctx->group_active = true;
+    return TM_HIP_OK;
+}
+
+int tm_hip_end_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "end_group") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (!ctx->group_active) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "end_group: no dispatch group is open");
+    }
+    ctx->group_active = false;
+    std::vector<Op> ops;
+    ops.swap(ctx->group_ops);
+    // An empty group still commits once, like an empty command buffer.
+    return commit_ops(ctx, ops, "group", err, err_cap);
+}
+
+int tm_hip_abort_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "abort_group") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (!ctx->group_active) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "abort_group: no dispatch group is open");
+    }
+    ctx->group_ops.clear();
+    ctx->group_active = false;
+    return TM_HIP_OK;
+}
+
+int tm_hip_fence(tm_hip_ctx *ctx, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "fence") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (ctx->group_active) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "fence: a dispatch group is open; end or abort it first");
+    }
+    return wait_pending(ctx, err, err_cap);
+}
+
+// ---------------------------------------------------------- products -----
+
+static int product_list(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                        uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off,
+                        uint32_t y_off, const char *what, char *err, size_t err_cap) {
+    Op op;
+    op.kind = OP_GEMV_LIST;
+    op.a[0] = w->alloc;
+    op.a[1] = x->alloc;
+    op.a[2] = y->alloc;
+    op.n_alloc = 3;
+    op.writes_mask = 4;
+    op.rows = rows;
+    op.cols = cols;
+    op.batch = batch;
+    op.x_off = x_off;
+    op.y_off = y_off;
+    op.packed = w->alloc->packed;
+    char label[kProfileName];
+    if (ctx->profiling.load(std::memory_order_relaxed)) {
+        snprintf(label, sizeof label, "%s:%ux%u", what, rows, cols);
+    } else {
+        snprintf(label, sizeof label, "%s", what);
+    }
+    return submit(ctx, op, label, err, err_cap);
+}
+
+int tm_hip_q8_0_gemv(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                     uint32_t rows, uint32_t cols, char *err, size_t err_cap) {
+    int rc = check_product(ctx, w, x, y, rows, cols, 1, 1, 0, 0, err, err_cap, "q8_0_gemv");
+    if (rc != TM_HIP_OK) {
+        return rc;
+    }
+    return product_list(ctx, w, x, y, rows, cols, 1, 0, 0, "q8_0_gemv", err, err_cap);
+}
+
+int tm_hip_q8_0_gemm(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                     uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off, uint32_t y_off,
+                     char *err, size_t err_cap) {
+    int rc = check_product(ctx, w, x, y, rows, cols, batch, TM_HIP_GEMM_MAX_BATCH, x_off, y_off, err,
+                           err_cap, "q8_0_gemm");
+    if (rc != TM_HIP_OK) {
+        return rc;
+    }
+    return product_list(ctx, w, x, y, rows, cols, batch, x_off, y_off, "q8_0_gemm", err, err_cap);
+}
+
+int tm_hip_q8_0_gemm_mma(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                         uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off,
+                         uint32_t y_off, char *err, size_t err_cap) {
+    int rc = check_product(ctx, w, x, y, rows, cols, batch, TM_HIP_GEMM_MMA_MAX_BATCH, x_off, y_off,
+                           err, err_cap, "q8_0_gemm_mma");
+    if (rc != TM_HIP_OK) {
+        return rc;
+    }
+    Op op;
+    op.kind = OP_MMA;
+    op.a[0] = w->alloc;
+    op.a[1] = x->alloc;
+    op.a[2] = y->alloc;
+    op.n_alloc = 3;
+    op.writes_mask = 4;
+    op.rows = rows;
+    op.cols = cols;
+    op.batch = batch;
+    op.x_off = x_off;
+    op.y_off = y_off;
+    op.packed = w->alloc->packed;
+    return submit(ctx, op, "q8_0_gemm_mma", err, err_cap);
+}
+
+int tm_hip_q8_0_row_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *out, uint32_t row,
+                        uint32_t cols, uint32_t out_off, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "q8_0_row") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (cols == 0 || (cols % 32u) != 0u) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "q8_0_row: cols must be a positive multiple of 32");
+    }
+    const size_t w_need = ((size_t)row + 1u) * ((size_t)cols / 32u) * 34u;
+    int rc;
+    if ((rc = check_buffer(ctx, w, w_need, err, err_cap, "q8_0_row.weights")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, out, ((size_t)out_off + cols) * 4u, err, err_cap, "q8_0_row.out")) !=
+            TM_HIP_OK) {
+        return rc;
+    }
+    if (w->alloc->packed && w->alloc->pcols != cols) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "q8_0_row: weights were sealed with cols %u but the call names %u",
+                    w->alloc->pcols, cols);
+    }
+    if (out->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "q8_0_row: out is a sealed weight buffer");
+    }
+    Op op;
+    op.kind = OP_ROW;
+    op.a[0] = w->alloc;
+    op.a[1] = out->alloc;
+    op.n_alloc = 2;
+    op.writes_mask = 2;
+    op.rows = w->alloc->packed ? w->alloc->prows : row + 1u;
+    op.cols = cols;
+    op.extra = row;
+    op.y_off = out_off;
+    op.packed = w->alloc->packed;
+    return submit(ctx, op, "q8_0_row", err, err_cap);
+}
+
+int tm_hip_row_indirect_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t type_id, uint32_t rows,
+                            uint32_t cols, tm_hip_buffer *ids, uint32_t slot, tm_hip_buffer *out,
+                            char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "row_indirect") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (!(type_id == 8u && cols > 0 && (cols % 32u) == 0u)) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "row_indirect: type %u with cols %u is unsupported (only Q8_0, type 8, with "
+                    "cols a positive multiple of 32)",
+                    type_id, cols);
+    }
+    const size_t w_need = (size_t)rows * ((size_t)cols / 32u) * 34u;
+    if (rows == 0) {
+        return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "row_indirect: zero rows");
+    }
+    int rc;
+    if ((rc = check_buffer(ctx, w, w_need, err, err_cap, "row_indirect.weights")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, ids, ((size_t)slot + 1u) * 4u, err, err_cap, "row_indirect.ids")) !=
+            TM_HIP_OK ||
+        (rc = check_buffer(ctx, out, (size_t)cols * 4u, err, err_cap, "row_indirect.out")) !=
+            TM_HIP_OK) {
+        return rc;
+    }
+    if (w->alloc->packed && (w->alloc->prows != rows || w->alloc->pcols != cols)) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "row_indirect: weights were sealed as %ux%u but the call names %ux%u",
+                    w->alloc->prows, w->alloc->pcols, rows, cols);
+    }
+    if (ids->alloc->packed || out->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "row_indirect: sealed weight buffer");
+    }
+    Op op;
+    op.kind = OP_ROW_INDIRECT;
+    op.a[0] = w->alloc;
+    op.a[1] = out->alloc;
+    op.a[2] = ids->alloc;
+    op.n_alloc = 3;
+    op.writes_mask = 2;
+    op.rows = rows;
+    op.cols = cols;
+    op.extra = slot;
+    op.packed = w->alloc->packed;
+    return submit(ctx, op, "row_indirect", err, err_cap);
+}
+
+// ---------------------------------------------------------- additions ----
+
+int tm_hip_q8_0_pack(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t rows, uint32_t cols, char *err,
+                     size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "q8_0_pack") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (rows == 0 || cols == 0 || (cols % 32u) != 0u) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "q8_0_pack: rows %u, cols %u (cols must be a positive multiple of 32)", rows,
+                    cols);
+    }
+    const size_t need = (size_t)rows * ((size_t)cols / 32u) * 34u;
+    int rc = check_buffer(ctx, w, need, err, err_cap, "q8_0_pack.weights");
+    if (rc != TM_HIP_OK) {
+        return rc;
+    }
+    if (w->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "q8_0_pack: buffer is already sealed");
+    }
+    if (ctx->group_active) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "q8_0_pack: close the open dispatch group first");
+    }
+    void *ptr = nullptr;
+    hipError_t e = hipMalloc(&ptr, w->len);
+    if (e != hipSuccess || ptr == nullptr) {
+        (void)hipGetLastError();
+        return fail(err, err_cap, TM_HIP_ERR_ALLOC,
+                    "q8_0_pack: allocation of %zu bytes for the sealed copy failed (%s)", w->len,
+                    hipGetErrorString(e));
+    }
+    Alloc *fresh = new (std::nothrow) Alloc();
+    if (fresh == nullptr) {
+        (void)hipFree(ptr);
+        return fail(err, err_cap, TM_HIP_ERR_ALLOC, "q8_0_pack: handle allocation failed");
+    }
+    fresh->ptr = ptr;
+    fresh->len = w->len;
+    fresh->packed = true;
+    fresh->prows = rows;
+    fresh->pcols = cols;
+    if (w->len > need) {
+        e = hipMemcpyAsync((uint8_t *)ptr + need, (const uint8_t *)w->alloc->ptr + need,
+                           w->len - need, hipMemcpyDeviceToDevice, ctx->stream);
+        if (e != hipSuccess) {
+            alloc_release(fresh);
+            return hip_fail(err, err_cap, "q8_0_pack: tail copy", e);
+        }
+    }
+    Op op;
+    op.kind = OP_PACK;
+    op.a[0] = w->alloc;
+    op.a[1] = fresh;
+    op.n_alloc = 2;
+    op.writes_mask = 2;
+    op.rows = rows;
+    op.cols = cols;
+    std::vector<Op> one(1, op);
+    rc = commit_ops(ctx, one, "q8_0_pack", err, err_cap);
+    // The handle now names the sealed copy; the raw bytes stay leased by the
+    // commit above until the pack kernel has read them.
+    Alloc *old = w->alloc;
+    w->alloc = fresh;
+    alloc_release(old);
+    return rc;
+}
+
+int tm_hip_q8_0_quantize_act(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *xq, uint32_t cols,
+                             uint32_t batch, uint32_t x_off, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "q8_0_quantize_act") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (cols == 0 || (cols % 32u) != 0u || batch == 0 || batch > TM_HIP_GEMM_I8_MAX_BATCH) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "q8_0_quantize_act: cols %u (a positive multiple of 32), batch %u (1..=%u)", cols,
+                    batch, TM_HIP_GEMM_I8_MAX_BATCH);
+    }
+    const size_t x_need = ((size_t)x_off + (size_t)batch * cols) * 4u;
+    const size_t q_need = (size_t)batch * ((size_t)cols + (size_t)(cols / 32u) * 4u);
+    int rc;
+    if ((rc = check_buffer(ctx, x, x_need, err, err_cap, "q8_0_quantize_act.x")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, xq, q_need, err, err_cap, "q8_0_quantize_act.xq")) != TM_HIP_OK) {
+        return rc;
+    }
+    if (x->alloc->packed || xq->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "q8_0_quantize_act: sealed weight buffer");
+    }
+    Op op;
+    op.kind = OP_QUANT;
+    op.a[0] = x->alloc;
+    op.a[1] = xq->alloc;
+    op.n_alloc = 2;
+    op.writes_mask = 2;
+    op.cols = cols;
+    op.batch = batch;
+    op.x_off = x_off;
+    return submit(ctx, op, "q8_0_quantize_act", err, err_cap);
+}
+
+int tm_hip_q8_0_gemm_i8(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm_hip_buffer *y,
+                        tm_hip_buffer *sumi, uint32_t rows, uint32_t cols, uint32_t batch,
+                        uint32_t y_off, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "q8_0_gemm_i8") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (rows == 0 || cols == 0 || (cols % 32u) != 0u || batch == 0 ||
+        batch > TM_HIP_GEMM_I8_MAX_BATCH) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "q8_0_gemm_i8: rows %u, cols %u (a positive multiple of 32), batch %u (1..=%u)",
+                    rows, cols, batch, TM_HIP_GEMM_I8_MAX_BATCH);
+    }
+    const size_t blocks = cols / 32u;
+    const size_t w_need = (size_t)rows * blocks * 34u;
+    const size_t q_need = (size_t)batch * ((size_t)cols + blocks * 4u);
+    const size_t y_need = ((size_t)y_off + (size_t)batch * rows) * 4u;
+    int rc;
+    if ((rc = check_buffer(ctx, w, w_need, err, err_cap, "q8_0_gemm_i8.weights")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, xq, q_need, err, err_cap, "q8_0_gemm_i8.xq")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, y, y_need, err, err_cap, "q8_0_gemm_i8.y")) != TM_HIP_OK) {
+        return rc;
+    }
+    if (sumi != nullptr &&
+        (rc = check_buffer(ctx, sumi, (size_t)batch * rows * blocks * 4u, err, err_cap,
+                           "q8_0_gemm_i8.sumi")) != TM_HIP_OK) {
+        return rc;
+    }
+    if (w->alloc->packed && (w->alloc->prows != rows || w->alloc->pcols != cols)) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "q8_0_gemm_i8: weights were sealed as %ux%u but the call names %ux%u",
+                    w->alloc->prows, w->alloc->pcols, rows, cols);
+    }
+    if (xq->alloc->packed || y->alloc->packed || (sumi != nullptr && sumi->alloc->packed)) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "q8_0_gemm_i8: sealed weight buffer");
+    }
+    Op op;
+    op.kind = OP_I8;
+    op.a[0] = w->alloc;
+    op.a[1] = xq->alloc;
+    op.a[2] = y->alloc;
+    op.a[3] = sumi != nullptr ? sumi->alloc : nullptr;
+    op.n_alloc = 4;
+    op.writes_mask = 4 | 8;
+    op.rows = rows;
+    op.cols = cols;
+    op.batch = batch;
+    op.y_off = y_off;
+    op.packed = w->alloc->packed;
+    return submit(ctx, op, "q8_0_gemm_i8", err, err_cap);
+}
+
+// -------------------------------------------------------- measurement ----
+
+uint64_t tm_hip_committed_dispatches(const tm_hip_ctx *ctx) {
+    return ctx == nullptr ? 0 : ctx->committed.load(std::memory_order_relaxed);
+}
+
+uint64_t tm_hip_completed_dispatches(const tm_hip_ctx *ctx) {
+    if (ctx == nullptr) {
+        return 0;
+    }
+    settle(const_cast<tm_hip_ctx *>(ctx));
+    return ctx->completed.load(std::memory_order_acquire);
+}
+
+double tm_hip_last_gpu_ms(const tm_hip_ctx *ctx) {
+    if (ctx == nullptr) {
+        return 0.0;
+    }
+    settle(const_cast<tm_hip_ctx *>(ctx));
+    return (double)ctx->last_gpu_nanos.load(std::memory_order_relaxed) / 1e6;
+}
+
+uint64_t tm_hip_gpu_nanos_total(const tm_hip_ctx *ctx) {
+    if (ctx == nullptr) {
+        return 0;
+    }
+    settle(const_cast<tm_hip_ctx *>(ctx));
+    return ctx->gpu_nanos_total.load(std::memory_order_relaxed);
+}
+
+uint64_t tm_hip_kernel_launches(const tm_hip_ctx *ctx) {
+    return ctx == nullptr ? 0 : ctx->launches.load(std::memory_order_relaxed);
+}
+
+int tm_hip_profile_set(tm_hip_ctx *ctx, int enabled) {
+    if (ctx == nullptr) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    std::lock_guard<std::mutex> g(ctx->q_mu);
+    ctx->profile_used = 0;
+    ctx->profiling.store(enabled ? 1 : 0, std::memory_order_relaxed);
+    return TM_HIP_OK;
+}
+
+int tm_hip_profile_read(tm_hip_ctx *ctx, uint32_t index, char *name, size_t name_cap,
+                        uint64_t *nanos, uint64_t *count) {
+    if (ctx == nullptr) {
+        return 0;
+    }
+    settle(ctx);
+    std::lock_guard<std::mutex> g(ctx->q_mu);
+    if (index >= ctx->profile_used) {
+        return 0;
+    }
+    if (name != nullptr && name_cap > 0) {
+        snprintf(name, name_cap, "%s", ctx->profile[index].name);
+    }
+    if (nanos != nullptr) {
+        *nanos = ctx->profile[index].nanos;
+    }
+    if (count != nullptr) {
+        *count = ctx->profile[index].count;
+    }
+    return 1;
+}
+
+uint64_t tm_hip_allocated_bytes(const tm_hip_ctx *ctx) {
+    return ctx == nullptr ? 0 : ctx->allocated.load(std::memory_order_relaxed);
+}
+
+uint64_t tm_hip_in_flight_bytes(const tm_hip_ctx *ctx) {
+    if (ctx == nullptr) {
+        return 0;
+    }
+    settle(const_cast<tm_hip_ctx *>(ctx));
+    return ctx->leased.load(std::memory_order_relaxed);
+}
+
+} // extern "C"

@@ -1,0 +1,462 @@
+"""Typed handles over the ``tm_hip_*`` C ABI (``include/tm_hip.h``).
+
+The shape of this module follows the reference's Rust wrapper over its Metal
+ABI (``crates/metal/src/lib.rs``): ``HipContext`` / ``HipBuffer`` carry the
+same method names, argument meaning and error mapping as ``MetalContext`` /
+``MetalBuffer``, and ``Matrix`` is the projection abstraction of
+``crates/tuckcore/src/engine/metal.rs:106-226``.
+
+There is no CPU fallback: loading fails loudly when ``libtm_hip.so`` has not
+been built, and every operation runs on the GPU through the C ABI.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from dataclasses import dataclass
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtm_hip.so")
+
+ERR_CAP = 512  # crates/metal/src/lib.rs:32
+GEMM_MAX_BATCH = 32  # crates/metal/src/lib.rs:28-30
+GEMM_MMA_MAX_BATCH = 512
+GEMM_I8_MAX_BATCH = 2048
+STAGING_CHUNK_BYTES = 4 << 20  # crates/tuckcore/src/qwen35_gpu.rs:1176
+
+TM_HIP_ERR_NO_DEVICE = -1
+TM_HIP_ERR_SOURCE = -2
+TM_HIP_ERR_ALLOC = -3
+TM_HIP_ERR_BOUNDS = -4
+TM_HIP_ERR_UNSUPPORTED = -5
+TM_HIP_ERR_INTERNAL = -6
+
+
+class TuckmillError(Exception):
+    """``code`` carries the reference's ErrorCode name."""
+
+    def __init__(self, code: str, message: str, abi_code: int = 0):
+        super().__init__(f"{code}: {message}")
+        self.code = code
+        self.message = message
+        self.abi_code = abi_code
+
+
+def hip_error(abi_code: int, text: str, what: str) -> TuckmillError:
+    # crates/metal/src/lib.rs:732-745
+    if abi_code in (TM_HIP_ERR_BOUNDS, TM_HIP_ERR_UNSUPPORTED):
+        code = "InvalidRequest"
+    elif abi_code in (TM_HIP_ERR_NO_DEVICE, TM_HIP_ERR_ALLOC):
+        code = "Unavailable"
+    else:
+        code = "Internal"
+    return TuckmillError(code, f"hip {what}: {text}", abi_code)
+
+
+_lib = None
+_lib_lock = threading.Lock()
+
+_SIGS = {
+    # name: (restype, argtypes)
+    "tm_hip_available": (ctypes.c_int, []),
+    "tm_hip_runtime_info": (ctypes.c_char_p, []),
+    "tm_hip_create": (ctypes.c_void_p, [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_destroy": (None, [ctypes.c_void_p]),
+    "tm_hip_buffer_new": (ctypes.c_void_p, [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
+                                            ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_buffer_free": (None, [ctypes.c_void_p, ctypes.c_void_p]),
+    "tm_hip_buffer_len": (ctypes.c_size_t, [ctypes.c_void_p, ctypes.c_void_p]),
+    "tm_hip_buffer_zero": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                                          ctypes.c_size_t, ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_upload": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                                     ctypes.c_void_p, ctypes.c_size_t, ctypes.c_char_p,
+                                     ctypes.c_size_t]),
+    "tm_hip_download": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                                       ctypes.c_void_p, ctypes.c_size_t, ctypes.c_char_p,
+                                       ctypes.c_size_t]),
+    "tm_hip_download_after": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                                             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
+                                             ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_copy_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
+                                       ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32,
+                                       ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_begin_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_end_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_abort_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_fence": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_q8_0_gemv": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_uint32] * 2 +
+                         [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_q8_0_gemm": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_uint32] * 5 +
+                         [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_q8_0_gemm_mma": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_uint32] * 5 +
+                             [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_q8_0_row_f32": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_uint32] * 3 +
+                            [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_row_indirect_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
+                                               ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
+                                               ctypes.c_uint32, ctypes.c_void_p, ctypes.c_char_p,
+                                               ctypes.c_size_t]),
+    "tm_hip_q8_0_pack": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
+                                        ctypes.c_uint32, ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_q8_0_quantize_act": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_uint32] * 3 +
+                                 [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_q8_0_gemm_i8": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_uint32] * 4 +
+                            [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_committed_dispatches": (ctypes.c_uint64, [ctypes.c_void_p]),
+    "tm_hip_completed_dispatches": (ctypes.c_uint64, [ctypes.c_void_p]),
+    "tm_hip_last_gpu_ms": (ctypes.c_double, [ctypes.c_void_p]),
+    "tm_hip_gpu_nanos_total": (ctypes.c_uint64, [ctypes.c_void_p]),
+    "tm_hip_kernel_launches": (ctypes.c_uint64, [ctypes.c_void_p]),
+    "tm_hip_profile_set": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "tm_hip_profile_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_char_p,
+                                           ctypes.c_size_t, ctypes.POINTER(ctypes.c_uint64),
+                                           ctypes.POINTER(ctypes.c_uint64)]),
+    "tm_hip_allocated_bytes": (ctypes.c_uint64, [ctypes.c_void_p]),
+    "tm_hip_in_flight_bytes": (ctypes.c_uint64, [ctypes.c_void_p]),
+}
+
+ABI_SYMBOLS = tuple(_SIGS)
+
+
+def load_library() -> ctypes.CDLL:
+    """Loads ``libtm_hip.so``; raises when it has not been built."""
+    global _lib
+    with _lib_lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise TuckmillError(
+                    "Unavailable",
+                    f"{LIB_PATH} is missing: build it with `python -m tuckmill_amd.build` "
+                    "(there is no CPU fallback for the HIP path)")
+            lib = ctypes.CDLL(LIB_PATH)
+            for name, (restype, argtypes) in _SIGS.items():
+                fn = getattr(lib, name)
+                fn.restype = restype
+                fn.argtypes = argtypes
+            _lib = lib
+    return _lib
+
+
+@dataclass
+class Probe:
+    available: bool
+    info: str
+
+
+def probe() -> Probe:
+    """Cheap device probe (crates/metal/src/lib.rs ``probe``)."""
+    lib = load_library()
+    return Probe(bool(lib.tm_hip_available()), lib.tm_hip_runtime_info().decode())
+
+
+def _host_view(data):
+    """(address, nbytes, keepalive) of a bytes-like object or numpy array."""
+    if isinstance(data, np.ndarray):
+        arr = np.ascontiguousarray(data)
+        return arr.ctypes.data, arr.nbytes, arr
+    mv = memoryview(data).cast("B")
+    arr = np.frombuffer(mv, dtype=np.uint8)
+    return arr.ctypes.data, arr.nbytes, arr
+
+
+class _Inner:
+    def __init__(self, raw):
+        self.raw = raw
+        self.lock = threading.RLock()
+        self.live_buffers = 0
+
+    def close(self):
+        if self.raw:
+            load_library().tm_hip_destroy(self.raw)
+            self.raw = None
+
+
+class HipContext:
+    """One device context; every ABI call is serialized by one lock
+    (crates/metal/src/lib.rs:695-708, :983-1005)."""
+
+    def __init__(self, inner: _Inner):
+        self._inner = inner
+        self._lib = load_library()
+
+    @staticmethod
+    def open() -> "HipContext":
+        lib = load_library()
+        err = ctypes.create_string_buffer(ERR_CAP)
+        raw = lib.tm_hip_create(err, ERR_CAP)
+        if not raw:
+            raise hip_error(TM_HIP_ERR_NO_DEVICE, err.value.decode(), "create")
+        return HipContext(_Inner(raw))
+
+    def close(self):
+        self._inner.close()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    @property
+    def raw(self):
+        return self._inner.raw
+
+    def _operate(self, name: str, fn, *args):
+        with self._inner.lock:
+            err = ctypes.create_string_buffer(ERR_CAP)
+            code = fn(self._inner.raw, *args, err, ERR_CAP)
+        if code != 0:
+            raise hip_error(code, err.value.decode(), name)
+
+    def _check_owned(self, *buffers):
+        for b in buffers:
+            if b is not None and b._ctx is not self._inner:
+                raise TuckmillError("InvalidRequest",
+                                    "buffer belongs to a different context", TM_HIP_ERR_UNSUPPORTED)
+
+    # -- buffers ----------------------------------------------------------
+    def buffer(self, nbytes: int, shared: bool = True) -> "HipBuffer":
+        if nbytes == 0:
+            raise TuckmillError("InvalidRequest", "zero-length HIP buffers are refused "
+                                "(allocation must be explicit)", TM_HIP_ERR_BOUNDS)
+        with self._inner.lock:
+            err = ctypes.create_string_buffer(ERR_CAP)
+            raw = self._lib.tm_hip_buffer_new(self._inner.raw, nbytes, 1 if shared else 0, err,
+                                              ERR_CAP)
+        if not raw:
+            raise hip_error(TM_HIP_ERR_ALLOC, err.value.decode(), "buffer")
+        return HipBuffer(self._inner, raw)
+
+    # -- grouping / ordering ---------------------------------------------
+    def begin_group(self):
+        self._operate("begin_group", self._lib.tm_hip_begin_group)
+
+    def end_group(self):
+        self._operate("end_group", self._lib.tm_hip_end_group)
+
+    def abort_group(self):
+        self._operate("abort_group", self._lib.tm_hip_abort_group)
+
+    def fence(self):
+        self._operate("fence", self._lib.tm_hip_fence)
+
+    # -- the Q8_0 products -------------------------------------------------
+    def q8_0_gemv(self, w, x, y, rows: int, cols: int):
+        self._check_owned(w, x, y)
+        self._operate("q8_0_gemv", self._lib.tm_hip_q8_0_gemv, w.raw, x.raw, y.raw, rows, cols)
+
+    def q8_0_gemm(self, w, x, y, rows, cols, batch, x_off=0, y_off=0):
+        self._check_owned(w, x, y)
+        self._operate("q8_0_gemm", self._lib.tm_hip_q8_0_gemm, w.raw, x.raw, y.raw, rows, cols,
+                      batch, x_off, y_off)
+
+    def q8_0_gemm_mma(self, w, x, y, rows, cols, batch, x_off=0, y_off=0):
+        self._check_owned(w, x, y)
+        self._operate("q8_0_gemm_mma", self._lib.tm_hip_q8_0_gemm_mma, w.raw, x.raw, y.raw, rows,
+                      cols, batch, x_off, y_off)
+
+    def q8_0_row(self, w, out, row: int, cols: int, out_off: int = 0):
+        self._check_owned(w, out)
+        self._operate("q8_0_row", self._lib.tm_hip_q8_0_row_f32, w.raw, out.raw, row, cols, out_off)
+
+    def row_indirect_f32(self, w, type_id, rows, cols, ids, slot, out):
+        self._check_owned(w, ids, out)
+        self._operate("row_indirect", self._lib.tm_hip_row_indirect_f32, w.raw, type_id, rows, cols,
+                      ids.raw, slot, out.raw)
+
+    def copy_f32(self, src, src_off, dst, dst_off, n):
+        self._check_owned(src, dst)
+        self._operate("copy_f32", self._lib.tm_hip_copy_f32, src.raw, src_off, dst.raw, dst_off, n)
+
+    # -- additions ---------------------------------------------------------
+    def q8_0_pack(self, w, rows: int, cols: int):
+        self._check_owned(w)
+        self._operate("q8_0_pack", self._lib.tm_hip_q8_0_pack, w.raw, rows, cols)
+
+    def q8_0_quantize_act(self, x, xq, cols, batch, x_off=0):
+        self._check_owned(x, xq)
+        self._operate("q8_0_quantize_act", self._lib.tm_hip_q8_0_quantize_act, x.raw, xq.raw, cols,
+                      batch, x_off)
+
+    def q8_0_gemm_i8(self, w, xq, y, rows, cols, batch, y_off=0, sumi=None):
+        self._check_owned(w, xq, y, sumi)
+        self._operate("q8_0_gemm_i8", self._lib.tm_hip_q8_0_gemm_i8, w.raw, xq.raw, y.raw,
+                      sumi.raw if sumi is not None else None, rows, cols, batch, y_off)
+
+    # -- measurement -------------------------------------------------------
+    def committed_dispatches(self) -> int:
+        return int(self._lib.tm_hip_committed_dispatches(self._inner.raw))
+
+    def completed_dispatches(self) -> int:
+        return int(self._lib.tm_hip_completed_dispatches(self._inner.raw))
+
+    def last_gpu_ms(self) -> float:
+        return float(self._lib.tm_hip_last_gpu_ms(self._inner.raw))
+
+    def gpu_nanos_total(self) -> int:
+        return int(self._lib.tm_hip_gpu_nanos_total(self._inner.raw))
+
+    def kernel_launches(self) -> int:
+        return int(self._lib.tm_hip_kernel_launches(self._inner.raw))
+
+    def allocated_bytes(self) -> int:
+        return int(self._lib.tm_hip_allocated_bytes(self._inner.raw))
+
+    def in_flight_bytes(self) -> int:
+        return int(self._lib.tm_hip_in_flight_bytes(self._inner.raw))
+
+    def live_gpu_bytes(self) -> int:
+        return self.allocated_bytes() + self.in_flight_bytes()
+
+    def set_profiling(self, enabled: bool):
+        with self._inner.lock:
+            self._lib.tm_hip_profile_set(self._inner.raw, 1 if enabled else 0)
+
+    def profile_table(self):
+        out = []
+        index = 0
+        while True:
+            name = ctypes.create_string_buffer(64)
+            nanos = ctypes.c_uint64(0)
+            count = ctypes.c_uint64(0)
+            with self._inner.lock:
+                found = self._lib.tm_hip_profile_read(self._inner.raw, index, name, 64,
+                                                      ctypes.byref(nanos), ctypes.byref(count))
+            if not found:
+                break
+            out.append((name.value.decode(), int(nanos.value), int(count.value)))
+            index += 1
+        return out
+
+
+class HipBuffer:
+    """RAII-style handle; ``free()`` (or garbage collection) releases it."""
+
+    def __init__(self, ctx: _Inner, raw):
+        self._ctx = ctx
+        self.raw = raw
+        self._lib = load_library()
+
+    def __len__(self) -> int:
+        return self.len()
+
+    def len(self) -> int:
+        if not self.raw:
+            return 0
+        return int(self._lib.tm_hip_buffer_len(self._ctx.raw, self.raw))
+
+    def free(self):
+        if self.raw and self._ctx.raw:
+            with self._ctx.lock:
+                self._lib.tm_hip_buffer_free(self._ctx.raw, self.raw)
+        self.raw = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+    def _copy(self, name, fn, *args):
+        with self._ctx.lock:
+            err = ctypes.create_string_buffer(ERR_CAP)
+            code = fn(self._ctx.raw, self.raw, *args, err, ERR_CAP)
+        if code != 0:
+            raise hip_error(code, err.value.decode(), name)
+
+    def zero(self, offset: int, length: int):
+        self._copy("buffer_zero", self._lib.tm_hip_buffer_zero, offset, length)
+
+    def upload(self, offset: int, data):
+        addr, nbytes, keep = _host_view(data)
+        self._copy("upload", self._lib.tm_hip_upload, offset, addr, nbytes)
+        del keep
+
+    def download(self, offset: int, nbytes: int) -> np.ndarray:
+        out = np.empty(nbytes, dtype=np.uint8)
+        self._copy("download", self._lib.tm_hip_download, offset, out.ctypes.data, nbytes)
+        return out
+
+    def download_into(self, offset: int, out: np.ndarray):
+        self._copy("download", self._lib.tm_hip_download, offset, out.ctypes.data, out.nbytes)
+
+    def download_f32(self, offset_elems: int, n: int) -> np.ndarray:
+        return self.download(offset_elems * 4, n * 4).view(np.float32)
+
+    def download_after(self, offset: int, nbytes: int, completed_target: int) -> np.ndarray:
+        out = np.empty(nbytes, dtype=np.uint8)
+        # no lock, like crates/metal/src/lib.rs:2618-2633
+        err = ctypes.create_string_buffer(ERR_CAP)
+        code = self._lib.tm_hip_download_after(self._ctx.raw, self.raw, offset, out.ctypes.data,
+                                               nbytes, completed_target, err, ERR_CAP)
+        if code != 0:
+            raise hip_error(code, err.value.decode(), "download_after")
+        return out
+
+
+def q8_0_bytes(rows: int, cols: int) -> int:
+    return rows * (cols // 32) * 34
+
+
+class Matrix:
+    """A device projection matrix: the HIP form of the reference's ``Matrix``
+    (crates/tuckcore/src/engine/metal.rs:106-226) for Q8_0 weights."""
+
+    def __init__(self, buf: HipBuffer, type_id: int, in_dim: int, out_dim: int):
+        self.buf = buf
+        self.type_id = type_id
+        self.in_dim = in_dim
+        self.out_dim = out_dim
+
+    @staticmethod
+    def plan(in_dim: int, out_dim: int) -> int:
+        return q8_0_bytes(out_dim, in_dim)
+
+    @staticmethod
+    def load(ctx: HipContext, raw, in_dim: int, out_dim: int, type_id: int = 8,
+             seal: bool = True) -> "Matrix":
+        """Staged raw upload in 4 MiB slices (engine/metal.rs:138-147), then
+        the seal step that re-lays the weights out for the device."""
+        if out_dim <= 1:
+            raise TuckmillError("Internal", "1-D tensors use the f32 path")
+        if type_id != 8:
+            raise TuckmillError("UnsupportedQuantization",
+                                f"engine matrices on this path must be Q8_0; got type {type_id}")
+        raw = np.ascontiguousarray(np.frombuffer(raw, dtype=np.uint8) if not
+                                   isinstance(raw, np.ndarray) else raw).view(np.uint8).ravel()
+        total = Matrix.plan(in_dim, out_dim)
+        if raw.size != total:
+            raise TuckmillError("InvalidArtifact", f"tensor holds {raw.size} bytes, "
+                                f"expected {total}")
+        buf = ctx.buffer(total, True)
+        off = 0
+        while off < total:
+            n = min(STAGING_CHUNK_BYTES, total - off)
+            buf.upload(off, raw[off:off + n])
+            off += n
+        if seal:
+            ctx.q8_0_pack(buf, out_dim, in_dim)
+        return Matrix(buf, type_id, in_dim, out_dim)
+
+    def gemv(self, ctx: HipContext, x: HipBuffer, y: HipBuffer):
+        ctx.q8_0_gemv(self.buf, x, y, self.out_dim, self.in_dim)
+
+    def gemm(self, ctx: HipContext, x: HipBuffer, y: HipBuffer, batch: int, exact: bool):
+        rows, cols = self.out_dim, self.in_dim
+        if not exact and 2 <= batch <= GEMM_MMA_MAX_BATCH:
+            ctx.q8_0_gemm_mma(self.buf, x, y, rows, cols, batch, 0, 0)
+            return
+        t0 = 0
+        while t0 < batch:
+            n = min(batch - t0, GEMM_MAX_BATCH)
+            ctx.q8_0_gemm(self.buf, x, y, rows, cols, n, t0 * cols, t0 * rows)
+            t0 += n
+
+    def row_indirect(self, ctx: HipContext, ids: HipBuffer, slot: int, out: HipBuffer):
+        ctx.row_indirect_f32(self.buf, self.type_id, self.out_dim, self.in_dim, ids, slot, out)
+
+    def row_into(self, ctx: HipContext, row: int, out: HipBuffer, out_off: int):
+        ctx.q8_0_row(self.buf, out, row, self.in_dim, out_off)
