@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Benchmark of the Q8_0 matrix-product hot path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one pass of the hot path over one batch of synthetic input: the
+full Qwen3-0.6B-shaped decode step at M = 1 (28 layers x {q, k, v, o, gate,
+up, down} + lm_head = 197 Q8_0 GEMVs, 633 MB of weights), issued through the
+C ABI as one dispatch group per step by the native step runner. Inputs are
+resident in HBM before the timed region. One JSON line is printed:
+
+  value      whole-step achieved bandwidth, algorithmic bytes / wall time
+  roofline   the GEMV list kernel: algorithmic bytes per launch over its
+             average launch duration (HIP events on the library's stream)
+  gemm       the MFMA prefill GEMM at M = 512 on the seven projection shapes
+  cpu_baseline  the scalar CPU oracle timed on this host (reported only)
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from tuckmill_amd import hip as H  # noqa: E402
+from tuckmill_amd import synth as S  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E bandwidth
+MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X published dense f32 matrix rate
+MFMA_I8_PEAK_TOPS = 5000.0
+
+
+class tmh_product(ctypes.Structure):
+    _fields_ = [("w", ctypes.c_void_p), ("x", ctypes.c_void_p), ("y", ctypes.c_void_p),
+                ("rows", ctypes.c_uint32), ("cols", ctypes.c_uint32), ("batch", ctypes.c_uint32),
+                ("kind", ctypes.c_uint32)]
+
+
+class tmh_timing(ctypes.Structure):
+    _fields_ = [("wall_ms", ctypes.c_double), ("gpu_ms", ctypes.c_double),
+                ("launches", ctypes.c_uint64), ("commits", ctypes.c_uint64)]
+
+
+TMH_GEMV, TMH_GEMM, TMH_GEMM_MMA, TMH_GEMM_I8, TMH_QUANT = range(5)
+
+
+def load_host():
+    H.load_library()  # libtm_hip.so first, by absolute path
+    path = os.path.join(ROOT, "tuckmill_amd", "libtm_host.so")
+    if not os.path.exists(path):
+        raise SystemExit(f"{path} is missing: run `python -m tuckmill_amd.build` first")
+    lib = ctypes.CDLL(path)
+    lib.tmh_run_steps.restype = ctypes.c_int
+    lib.tmh_run_steps.argtypes = [ctypes.c_void_p, ctypes.POINTER(tmh_product), ctypes.c_uint32,
+                                  ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int,
+                                  ctypes.POINTER(tmh_timing), ctypes.c_char_p, ctypes.c_size_t]
+    return lib
+
+
+def run_steps(host, ctx, products, warmup, steps, grouped=True) -> tmh_timing:
+    arr = (tmh_product * len(products))(*products)
+    t = tmh_timing()
+    err = ctypes.create_string_buffer(H.ERR_CAP)
+    rc = host.tmh_run_steps(ctx.raw, arr, len(products), warmup, steps, 1 if grouped else 0,
+                            ctypes.byref(t), err, H.ERR_CAP)
+    if rc != 0:
+        raise SystemExit(f"step runner failed ({rc}): {err.value.decode()}")
+    return t
+
+
+def decode_step_tensors():
+    """(name, layer, rows, cols) of BASELINE config 1."""
+    out = []
+    for layer in range(S.QWEN3_0_6B_LAYERS):
+        for name, rows, cols in S.QWEN3_0_6B_LAYER:
+            out.append((name, layer, rows, cols))
+    name, rows, cols = S.QWEN3_0_6B_LM_HEAD
+    out.append((name, S.QWEN3_0_6B_LAYERS, rows, cols))
+    return out
+
+
+def build_decode_step(ctx, keep_host: bool):
+    tensors = decode_step_tensors()
+    products, keep, host_side = [], [], []
+    for name, layer, rows, cols in tensors:
+        seed = S.tensor_seed(1, layer, name)
+        raw = S.make_weights(rows, cols, seed)
+        x = S.make_activations(cols, seed)
+        m = H.Matrix.load(ctx, raw, cols, rows)
+        xb = ctx.buffer(cols * 4)
+        xb.upload(0, x)
+        yb = ctx.buffer(rows * 4)
+        keep += [m, xb, yb]
+        products.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, 1, TMH_GEMV))
+        if keep_host:
+            host_side.append((raw, x, rows, cols, yb))
+    return products, keep, host_side
+
+
+def cpu_baseline(host_side, budget_s: float):
+    """Times the scalar CPU oracle (single thread, like the reference's
+    matvec loop) on whole decode steps until about `budget_s` seconds are
+    spent, and checks the GPU's result of every product against it."""
+    import oracle as O
+
+    O.lib()
+    step_bytes = sum(S.gemv_bytes(r, c) for _, _, r, c, _ in host_side)
+    worst = 0.0
+    t0 = time.perf_counter()
+    for raw, x, rows, cols, yb in host_side:  # first pass doubles as the parity check
+        want = O.gemv_q8_0_f32(raw, rows, cols, x, threads=1)
+        got = yb.download_f32(0, rows)
+        worst = max(worst, float(np.max(np.abs(got - want)) / np.max(np.abs(want))))
+    one = time.perf_counter() - t0
+    reps = max(1, min(50, int(budget_s / max(one, 1e-3)) - 1))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        for raw, x, rows, cols, _ in host_side:
+            O.gemv_q8_0_f32(raw, rows, cols, x, threads=1)
+    t1 = (time.perf_counter() - t0) / reps
+    ncores = min(16, os.cpu_count() or 1)
+    t0 = time.perf_counter()
+    for raw, x, rows, cols, _ in host_side:
+        O.gemv_q8_0_f32(raw, rows, cols, x, threads=ncores)
+    tn = time.perf_counter() - t0
+    return {
+        "value": step_bytes / t1 / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"{reps} full decode steps (197 GEMVs, {step_bytes} algorithmic bytes each) "
+                  "through the scalar C restatement of kernels.rs:186-204, 1 thread",
+        "ms_per_step": t1 * 1e3,
+        "all_cores": {"value": step_bytes / tn / 1e9, "cores": ncores, "ms_per_step": tn * 1e3},
+        "max_norm_err_gpu_vs_cpu": worst,
+    }
+
+
+def bench_gemm(host, ctx, steps, warmup):
+    """BASELINE config 2: M = 512 against the seven projection matrices."""
+    M = 512
+    out = {"M": M, "shapes": []}
+    flops_total, ms_total = 0.0, 0.0
+    for name, rows, cols in S.QWEN3_0_6B_LAYER:
+        raw = S.make_weights(rows, cols, S.tensor_seed(2, 0, name))
+        m = H.Matrix.load(ctx, raw, cols, rows)
+        xb = ctx.buffer(M * cols * 4)
+        xb.upload(0, S.make_activations(M * cols, rows))
+        yb = ctx.buffer(M * rows * 4)
+        t = run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M,
+                                              TMH_GEMM_MMA)], warmup, steps, grouped=False)
+        ms = t.gpu_ms / steps
+        flops = 2.0 * M * rows * cols
+        out["shapes"].append({"name": name, "rows": rows, "cols": cols, "us": ms * 1e3,
+                              "tflops": flops / (ms * 1e-3) / 1e12})
+        flops_total += flops
+        ms_total += ms
+        for b in (m.buf, xb, yb):
+            b.free()
+    out["tflops"] = flops_total / (ms_total * 1e-3) / 1e12
+    out["mfma_f32_peak_tflops"] = MFMA_F32_PEAK_TFLOPS
+    out["frac"] = out["tflops"] / MFMA_F32_PEAK_TFLOPS
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0,
+                    help="budget of the CPU-baseline leg (0 skips it)")
+    ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--ungrouped", action="store_true",
+                    help="one commit per GEMV instead of one group per step")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one MI355X: this path runs on a single GPU "
+                         "(run with --gpus 1)")
+    p = H.probe()
+    if not p.available:
+        raise SystemExit(f"bench.py needs an MI355X: {p.info}")
+    host = load_host()
+    ctx = H.HipContext.open()
+
+    products, keep, host_side = build_decode_step(ctx, keep_host=args.cpu_seconds > 0)
+    step_bytes = sum(S.gemv_bytes(pr.rows, pr.cols) for pr in products)
+    ctx.fence()
+    t = run_steps(host, ctx, products, args.warmup, args.steps, grouped=not args.ungrouped)
+    ms_per_step = t.wall_ms / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    launches_per_step = t.launches / args.steps
+    launch_us = t.gpu_ms * 1e3 / t.launches
+    achieved = (step_bytes / launches_per_step) / (launch_us * 1e-6) / 1e9
+
+    line = {
+        "metric": "Q8_0 GEMV achieved HBM GB/s (% peak); Q8_0 GEMM TFLOP/s at M=512",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {
+            "workload": "Qwen3-0.6B-shaped decode step at M=1: 28 x {q,k,v,o,gate,up,down} + "
+                        "lm_head = 197 Q8_0 GEMVs, f32 activations (BASELINE config 1)",
+            "weights_bytes": sum(S.q8_0_bytes(pr.rows, pr.cols) for pr in products),
+            "algorithmic_bytes_per_step": step_bytes,
+            "issue": "one commit per GEMV" if args.ungrouped else "one dispatch group per step",
+            "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "kernel": "q8::gemv_list_kernel",
+            "launches_per_step": launches_per_step,
+            "avg_launch_us": launch_us,
+            "algorithmic_bytes_per_launch": step_bytes / launches_per_step,
+        },
+    }
+    if args.cpu_seconds > 0:
+        line["cpu_baseline"] = cpu_baseline(host_side, args.cpu_seconds)
+    for obj in keep:
+        (obj.buf if isinstance(obj, H.Matrix) else obj).free()
+    if not args.no_gemm:
+        line["gemm"] = bench_gemm(host, ctx, max(10, args.steps // 4), max(3, args.warmup // 4))
+    ctx.close()
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -20,7 +20,7 @@ def test_weight_quantizer_agrees_with_the_oracle_rule():
 
 
 def test_generator_is_seeded_and_shaped():
-    a = S.make_weights(50, 64, 7, chunk_rows=16)
+    a = S.make_weights(50, 64, 7, chunk_rows=16, threads=1)
     b = S.make_weights(50, 64, 7, chunk_rows=16)
     c = S.make_weights(50, 64, 8, chunk_rows=16)
     assert np.array_equal(a, b) and not np.array_equal(a, c)

@@ -41,6 +41,32 @@ def build_library(verbose: bool = False, extra: list[str] | None = None) -> str:
     return LIB
 
 
+HOST_LIB = os.path.join(HERE, "libtm_host.so")
+CXX = os.environ.get("CXX", "g++")
+
+
+def build_host(verbose: bool = False) -> str:
+    """The C++ host layer above the C ABI (typed handles + native step runner)."""
+    cmd = [CXX, "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wextra",
+           "-I", os.path.join(ROOT, "include"), "-I", os.path.join(HERE, "host"),
+           "-o", HOST_LIB, os.path.join(HERE, "host", "workloads.cpp"),
+           "-L", HERE, "-ltm_hip", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"host build failed ({res.returncode}):\n{res.stdout}{res.stderr}")
+    if verbose and (res.stdout or res.stderr):
+        print(res.stdout + res.stderr)
+    return HOST_LIB
+
+
+def build_all(verbose: bool = False) -> None:
+    build_library(verbose)
+    build_host(verbose)
+
+
 if __name__ == "__main__":
     build_library(verbose=True, extra=sys.argv[1:])
-    print("built", LIB)
+    build_host(verbose=True)
+    print("built", LIB, HOST_LIB)

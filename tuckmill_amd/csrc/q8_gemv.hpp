@@ -33,7 +33,10 @@ struct GemvDesc {
     uint32_t pad;
 };
 
-constexpr int GEMV_MAX_DESCS = 84; // 84 * 48 + 16 = 4048 bytes of kernel arguments
+// The list travels in the kernel-argument segment (read through the scalar
+// cache): 256 * 48 + 16 = 12304 bytes, enough for a whole decode step of a
+// 28-layer model (197 products) in one launch.
+constexpr int GEMV_MAX_DESCS = 256;
 
 struct GemvArgs {
     uint32_t n;

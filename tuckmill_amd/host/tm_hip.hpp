@@ -1,0 +1,349 @@
+// tm_hip.hpp — typed C++ handles over the tm_hip_* C ABI.
+//
+// The reference wraps its Metal ABI in Rust RAII types
+// (crates/metal/src/lib.rs: MetalContext :755-, MetalBuffer :2480-2650) and
+// builds the projection abstraction `Matrix` on them
+// (crates/tuckcore/src/engine/metal.rs:106-226). This header is the same
+// surface for the HIP ABI, for hosts written in C++: same method names,
+// argument meaning and error mapping. Header-only; link against libtm_hip.so.
+#pragma once
+
+#include <algorithm>
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "tm_hip.h"
+
+namespace tuckmill_hip {
+
+constexpr size_t ERR_CAP = 512;               // crates/metal/src/lib.rs:32
+constexpr uint32_t GEMM_MAX_BATCH = TM_HIP_GEMM_MAX_BATCH;
+constexpr uint32_t GEMM_MMA_MAX_BATCH = TM_HIP_GEMM_MMA_MAX_BATCH;
+constexpr size_t STAGING_CHUNK_BYTES = 4u << 20; // crates/tuckcore/src/qwen35_gpu.rs:1176
+
+enum class ErrorCode { InvalidRequest, Unavailable, Internal, UnsupportedQuantization, InvalidArtifact };
+
+class TuckmillError : public std::runtime_error {
+  public:
+    TuckmillError(ErrorCode code, const std::string &message, int abi_code = 0)
+        : std::runtime_error(message), code_(code), abi_code_(abi_code) {}
+    ErrorCode code() const { return code_; }
+    int abi_code() const { return abi_code_; }
+
+  private:
+    ErrorCode code_;
+    int abi_code_;
+};
+
+// crates/metal/src/lib.rs:732-745
+inline TuckmillError hip_error(int code, const char *text, const char *what) {
+    ErrorCode c = ErrorCode::Internal;
+    if (code == TM_HIP_ERR_BOUNDS || code == TM_HIP_ERR_UNSUPPORTED) {
+        c = ErrorCode::InvalidRequest;
+    } else if (code == TM_HIP_ERR_NO_DEVICE || code == TM_HIP_ERR_ALLOC) {
+        c = ErrorCode::Unavailable;
+    }
+    return TuckmillError(c, std::string("hip ") + what + ": " + text, code);
+}
+
+struct Probe {
+    bool available;
+    std::string info;
+};
+
+inline Probe probe() { return Probe{tm_hip_available() != 0, tm_hip_runtime_info()}; }
+
+struct ContextInner {
+    tm_hip_ctx *raw = nullptr;
+    std::mutex lock; // one ABI call at a time, crates/metal/src/lib.rs:695-708
+    bool owned = true;
+    ~ContextInner() {
+        if (raw != nullptr && owned) {
+            tm_hip_destroy(raw);
+        }
+    }
+};
+
+class HipContext;
+
+class HipBuffer {
+  public:
+    HipBuffer() = default;
+    HipBuffer(std::shared_ptr<ContextInner> ctx, tm_hip_buffer *raw, bool owned = true)
+        : ctx_(std::move(ctx)), raw_(raw), owned_(owned) {}
+    HipBuffer(const HipBuffer &) = delete;
+    HipBuffer &operator=(const HipBuffer &) = delete;
+    HipBuffer(HipBuffer &&o) noexcept : ctx_(std::move(o.ctx_)), raw_(o.raw_), owned_(o.owned_) {
+        o.raw_ = nullptr;
+    }
+    HipBuffer &operator=(HipBuffer &&o) noexcept {
+        if (this != &o) {
+            release();
+            ctx_ = std::move(o.ctx_);
+            raw_ = o.raw_;
+            owned_ = o.owned_;
+            o.raw_ = nullptr;
+        }
+        return *this;
+    }
+    ~HipBuffer() { release(); }
+
+    tm_hip_buffer *raw() const { return raw_; }
+    size_t len() const { return raw_ ? tm_hip_buffer_len(ctx_->raw, raw_) : 0; }
+    bool is_empty() const { return len() == 0; }
+
+    void zero(size_t offset, size_t length) const {
+        call("buffer_zero", [&](char *e) {
+            return tm_hip_buffer_zero(ctx_->raw, raw_, offset, length, e, ERR_CAP);
+        });
+    }
+    void upload(size_t offset, const void *data, size_t length) const {
+        call("upload", [&](char *e) {
+            return tm_hip_upload(ctx_->raw, raw_, offset, data, length, e, ERR_CAP);
+        });
+    }
+    void download(size_t offset, void *dst, size_t length) const {
+        call("download", [&](char *e) {
+            return tm_hip_download(ctx_->raw, raw_, offset, dst, length, e, ERR_CAP);
+        });
+    }
+    // No lock: the wait must not block encoding of later work
+    // (crates/metal/src/lib.rs:2618-2633).
+    void download_after(size_t offset, void *dst, size_t length, uint64_t completed_target) const {
+        char err[ERR_CAP] = {0};
+        int code = tm_hip_download_after(ctx_->raw, raw_, offset, dst, length, completed_target, err,
+                                         ERR_CAP);
+        if (code != 0) {
+            throw hip_error(code, err, "download_after");
+        }
+    }
+
+  private:
+    friend class HipContext;
+    template <class F> void call(const char *what, F f) const {
+        std::lock_guard<std::mutex> g(ctx_->lock);
+        char err[ERR_CAP] = {0};
+        int code = f(err);
+        if (code != 0) {
+            throw hip_error(code, err, what);
+        }
+    }
+    void release() {
+        if (raw_ != nullptr && owned_ && ctx_ && ctx_->raw != nullptr) {
+            std::lock_guard<std::mutex> g(ctx_->lock);
+            tm_hip_buffer_free(ctx_->raw, raw_);
+        }
+        raw_ = nullptr;
+    }
+    std::shared_ptr<ContextInner> ctx_;
+    tm_hip_buffer *raw_ = nullptr;
+    bool owned_ = true;
+};
+
+class HipContext {
+  public:
+    static HipContext open() {
+        char err[ERR_CAP] = {0};
+        tm_hip_ctx *raw = tm_hip_create(err, ERR_CAP);
+        if (raw == nullptr) {
+            throw hip_error(TM_HIP_ERR_NO_DEVICE, err, "create");
+        }
+        auto inner = std::make_shared<ContextInner>();
+        inner->raw = raw;
+        return HipContext(std::move(inner));
+    }
+    // Borrow a context created elsewhere (it is not destroyed here).
+    static HipContext borrow(tm_hip_ctx *raw) {
+        auto inner = std::make_shared<ContextInner>();
+        inner->raw = raw;
+        inner->owned = false;
+        return HipContext(std::move(inner));
+    }
+    HipBuffer borrow_buffer(tm_hip_buffer *raw) const { return HipBuffer(inner_, raw, false); }
+
+    HipBuffer buffer(size_t bytes, bool shared = true) const {
+        if (bytes == 0) {
+            throw TuckmillError(ErrorCode::InvalidRequest,
+                                "zero-length HIP buffers are refused (allocation must be explicit)",
+                                TM_HIP_ERR_BOUNDS);
+        }
+        std::lock_guard<std::mutex> g(inner_->lock);
+        char err[ERR_CAP] = {0};
+        tm_hip_buffer *raw = tm_hip_buffer_new(inner_->raw, bytes, shared ? 1 : 0, err, ERR_CAP);
+        if (raw == nullptr) {
+            throw hip_error(TM_HIP_ERR_ALLOC, err, "buffer");
+        }
+        return HipBuffer(inner_, raw);
+    }
+
+    void begin_group() const { operate("begin_group", [&](char *e) { return tm_hip_begin_group(raw(), e, ERR_CAP); }); }
+    void end_group() const { operate("end_group", [&](char *e) { return tm_hip_end_group(raw(), e, ERR_CAP); }); }
+    void abort_group() const { operate("abort_group", [&](char *e) { return tm_hip_abort_group(raw(), e, ERR_CAP); }); }
+    void fence() const { operate("fence", [&](char *e) { return tm_hip_fence(raw(), e, ERR_CAP); }); }
+
+    // Run `encode` inside one dispatch group; on any error the group is
+    // discarded without committing (crates/tuckcore/src/qwen35_gpu.rs:66-85).
+    template <class F> void grouped(F encode) const {
+        begin_group();
+        try {
+            encode();
+        } catch (...) {
+            try {
+                abort_group();
+            } catch (...) {
+            }
+            throw;
+        }
+        end_group();
+    }
+
+    void q8_0_gemv(const HipBuffer &w, const HipBuffer &x, const HipBuffer &y, uint32_t rows,
+                   uint32_t cols) const {
+        operate("q8_0_gemv", [&](char *e) {
+            return tm_hip_q8_0_gemv(raw(), w.raw(), x.raw(), y.raw(), rows, cols, e, ERR_CAP);
+        });
+    }
+    void q8_0_gemm(const HipBuffer &w, const HipBuffer &x, const HipBuffer &y, uint32_t rows,
+                   uint32_t cols, uint32_t batch, uint32_t x_off, uint32_t y_off) const {
+        operate("q8_0_gemm", [&](char *e) {
+            return tm_hip_q8_0_gemm(raw(), w.raw(), x.raw(), y.raw(), rows, cols, batch, x_off, y_off,
+                                    e, ERR_CAP);
+        });
+    }
+    void q8_0_gemm_mma(const HipBuffer &w, const HipBuffer &x, const HipBuffer &y, uint32_t rows,
+                       uint32_t cols, uint32_t batch, uint32_t x_off, uint32_t y_off) const {
+        operate("q8_0_gemm_mma", [&](char *e) {
+            return tm_hip_q8_0_gemm_mma(raw(), w.raw(), x.raw(), y.raw(), rows, cols, batch, x_off,
+                                        y_off, e, ERR_CAP);
+        });
+    }
+    void q8_0_row(const HipBuffer &w, const HipBuffer &out, uint32_t row, uint32_t cols,
+                  uint32_t out_off) const {
+        operate("q8_0_row", [&](char *e) {
+            return tm_hip_q8_0_row_f32(raw(), w.raw(), out.raw(), row, cols, out_off, e, ERR_CAP);
+        });
+    }
+    void row_indirect_f32(const HipBuffer &w, uint32_t type_id, uint32_t rows, uint32_t cols,
+                          const HipBuffer &ids, uint32_t slot, const HipBuffer &out) const {
+        operate("row_indirect", [&](char *e) {
+            return tm_hip_row_indirect_f32(raw(), w.raw(), type_id, rows, cols, ids.raw(), slot,
+                                           out.raw(), e, ERR_CAP);
+        });
+    }
+    void q8_0_pack(const HipBuffer &w, uint32_t rows, uint32_t cols) const {
+        operate("q8_0_pack",
+                [&](char *e) { return tm_hip_q8_0_pack(raw(), w.raw(), rows, cols, e, ERR_CAP); });
+    }
+    void q8_0_quantize_act(const HipBuffer &x, const HipBuffer &xq, uint32_t cols, uint32_t batch,
+                           uint32_t x_off) const {
+        operate("q8_0_quantize_act", [&](char *e) {
+            return tm_hip_q8_0_quantize_act(raw(), x.raw(), xq.raw(), cols, batch, x_off, e, ERR_CAP);
+        });
+    }
+    void q8_0_gemm_i8(const HipBuffer &w, const HipBuffer &xq, const HipBuffer &y, uint32_t rows,
+                      uint32_t cols, uint32_t batch, uint32_t y_off) const {
+        operate("q8_0_gemm_i8", [&](char *e) {
+            return tm_hip_q8_0_gemm_i8(raw(), w.raw(), xq.raw(), y.raw(), nullptr, rows, cols, batch,
+                                       y_off, e, ERR_CAP);
+        });
+    }
+
+    uint64_t committed_dispatches() const { return tm_hip_committed_dispatches(raw()); }
+    uint64_t completed_dispatches() const { return tm_hip_completed_dispatches(raw()); }
+    double last_gpu_ms() const { return tm_hip_last_gpu_ms(raw()); }
+    uint64_t gpu_nanos_total() const { return tm_hip_gpu_nanos_total(raw()); }
+    uint64_t kernel_launches() const { return tm_hip_kernel_launches(raw()); }
+    uint64_t allocated_bytes() const { return tm_hip_allocated_bytes(raw()); }
+    uint64_t in_flight_bytes() const { return tm_hip_in_flight_bytes(raw()); }
+    uint64_t live_gpu_bytes() const { return allocated_bytes() + in_flight_bytes(); }
+
+    tm_hip_ctx *raw() const { return inner_->raw; }
+
+  private:
+    explicit HipContext(std::shared_ptr<ContextInner> inner) : inner_(std::move(inner)) {}
+    template <class F> void operate(const char *what, F f) const {
+        std::lock_guard<std::mutex> g(inner_->lock);
+        char err[ERR_CAP] = {0};
+        int code = f(err);
+        if (code != 0) {
+            throw hip_error(code, err, what);
+        }
+    }
+    std::shared_ptr<ContextInner> inner_;
+};
+
+// A device projection matrix of Q8_0 weights
+// (crates/tuckcore/src/engine/metal.rs:106-226).
+class Matrix {
+  public:
+    static uint64_t plan(uint64_t in_dim, uint64_t out_dim) { return out_dim * (in_dim / 32u) * 34u; }
+
+    // Staged raw upload in 4 MiB slices (engine/metal.rs:138-147), then the
+    // seal step that re-lays the weights out for coalesced device loads.
+    static Matrix load(const HipContext &gpu, const uint8_t *raw, uint64_t in_dim, uint64_t out_dim,
+                       uint32_t type_id = 8, bool seal = true) {
+        if (out_dim <= 1) {
+            throw TuckmillError(ErrorCode::Internal, "1-D tensors use the f32 path");
+        }
+        if (type_id != 8) {
+            throw TuckmillError(ErrorCode::UnsupportedQuantization,
+                                "engine matrices on this path must be Q8_0");
+        }
+        const size_t total = (size_t)plan(in_dim, out_dim);
+        Matrix m;
+        m.buf = gpu.buffer(total, true);
+        for (size_t off = 0; off < total;) {
+            const size_t n = std::min(STAGING_CHUNK_BYTES, total - off);
+            m.buf.upload(off, raw + off, n);
+            off += n;
+        }
+        if (seal) {
+            gpu.q8_0_pack(m.buf, (uint32_t)out_dim, (uint32_t)in_dim);
+        }
+        m.type_id = type_id;
+        m.in_dim = in_dim;
+        m.out_dim = out_dim;
+        return m;
+    }
+
+    void gemv(const HipContext &gpu, const HipBuffer &x, const HipBuffer &y) const {
+        gpu.q8_0_gemv(buf, x, y, (uint32_t)out_dim, (uint32_t)in_dim);
+    }
+
+    // engine/metal.rs:171-196: batch 1 and `exact` keep the GEMV's per-row
+    // arithmetic in slices of GEMM_MAX_BATCH; other batches use the matrix cores.
+    void gemm(const HipContext &gpu, const HipBuffer &x, const HipBuffer &y, uint32_t batch,
+              bool exact) const {
+        const uint32_t rows = (uint32_t)out_dim, cols = (uint32_t)in_dim;
+        if (!exact && batch >= 2 && batch <= GEMM_MMA_MAX_BATCH) {
+            gpu.q8_0_gemm_mma(buf, x, y, rows, cols, batch, 0, 0);
+            return;
+        }
+        for (uint32_t t0 = 0; t0 < batch;) {
+            const uint32_t n = std::min(batch - t0, GEMM_MAX_BATCH);
+            gpu.q8_0_gemm(buf, x, y, rows, cols, n, t0 * cols, t0 * rows);
+            t0 += n;
+        }
+    }
+
+    void row_indirect(const HipContext &gpu, const HipBuffer &ids, uint32_t slot,
+                      const HipBuffer &out) const {
+        gpu.row_indirect_f32(buf, type_id, (uint32_t)out_dim, (uint32_t)in_dim, ids, slot, out);
+    }
+
+    void row_into(const HipContext &gpu, uint32_t row, const HipBuffer &out, uint32_t out_off) const {
+        gpu.q8_0_row(buf, out, row, (uint32_t)in_dim, out_off);
+    }
+
+    HipBuffer buf;
+    uint32_t type_id = 8;
+    uint64_t in_dim = 0, out_dim = 0;
+};
+
+} // namespace tuckmill_hip

@@ -1,0 +1,122 @@
+// workloads.cpp — native step runner above the C ABI.
+//
+// A "step" is one pass of the hot path: a list of Q8_0 products issued the
+// way the reference's engine issues a token step — one dispatch group per
+// step (crates/tuckcore/src/engine/metal.rs:2462, qwen35_gpu.rs:66-85) — or
+// one commit per product when `grouped` is 0. The loop lives in native code
+// so that the measured time is the library's, not an interpreter's.
+#include <chrono>
+#include <cstdio>
+#include <cstring>
+
+#include "tm_hip.hpp"
+
+using namespace tuckmill_hip;
+
+extern "C" {
+
+enum { TMH_GEMV = 0, TMH_GEMM = 1, TMH_GEMM_MMA = 2, TMH_GEMM_I8 = 3, TMH_QUANT = 4 };
+
+struct tmh_product {
+    tm_hip_buffer *w, *x, *y; // for TMH_GEMM_I8, x is the quantized activation buffer
+    uint32_t rows, cols, batch, kind;
+};
+
+struct tmh_timing {
+    double wall_ms;     // host clock around the timed steps, fence to fence
+    double gpu_ms;      // sum of the commits' HIP-event times on the context's stream
+    uint64_t launches;  // kernel launches issued by the timed steps
+    uint64_t commits;
+};
+
+static void issue(const HipContext &gpu, const tmh_product *p, uint32_t n) {
+    for (uint32_t i = 0; i < n; ++i) {
+        const tmh_product &q = p[i];
+        HipBuffer w = gpu.borrow_buffer(q.w), x = gpu.borrow_buffer(q.x), y = gpu.borrow_buffer(q.y);
+        switch (q.kind) {
+        case TMH_GEMV: gpu.q8_0_gemv(w, x, y, q.rows, q.cols); break;
+        case TMH_GEMM: gpu.q8_0_gemm(w, x, y, q.rows, q.cols, q.batch, 0, 0); break;
+        case TMH_GEMM_MMA: gpu.q8_0_gemm_mma(w, x, y, q.rows, q.cols, q.batch, 0, 0); break;
+        case TMH_GEMM_I8: gpu.q8_0_gemm_i8(w, x, y, q.rows, q.cols, q.batch, 0); break;
+        case TMH_QUANT: gpu.q8_0_quantize_act(x, y, q.cols, q.batch, 0); break;
+        default: throw TuckmillError(ErrorCode::InvalidRequest, "unknown product kind");
+        }
+    }
+}
+
+int tmh_run_steps(tm_hip_ctx *ctx, const tmh_product *products, uint32_t n, uint32_t warmup,
+                  uint32_t steps, int grouped, tmh_timing *out, char *err, size_t err_cap) {
+    try {
+        HipContext gpu = HipContext::borrow(ctx);
+        auto one_step = [&]() {
+            if (grouped) {
+                gpu.grouped([&]() { issue(gpu, products, n); });
+            } else {
+                issue(gpu, products, n);
+            }
+        };
+        for (uint32_t s = 0; s < warmup; ++s) {
+            one_step();
+        }
+        gpu.fence();
+        const uint64_t nanos0 = gpu.gpu_nanos_total();
+        const uint64_t launches0 = gpu.kernel_launches();
+        const uint64_t commits0 = gpu.committed_dispatches();
+        const auto t0 = std::chrono::steady_clock::now();
+        for (uint32_t s = 0; s < steps; ++s) {
+            one_step();
+        }
+        gpu.fence();
+        const auto t1 = std::chrono::steady_clock::now();
+        if (out != nullptr) {
+            out->wall_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+            out->gpu_ms = (double)(gpu.gpu_nanos_total() - nanos0) / 1e6;
+            out->launches = gpu.kernel_launches() - launches0;
+            out->commits = gpu.committed_dispatches() - commits0;
+        }
+        return 0;
+    } catch (const TuckmillError &e) {
+        if (err != nullptr && err_cap > 0) {
+            snprintf(err, err_cap, "%s", e.what());
+        }
+        return e.abi_code() != 0 ? e.abi_code() : TM_HIP_ERR_INTERNAL;
+    }
+}
+
+// Self-check of the C++ handles (Matrix::load with its staged upload and
+// seal, gemv, gemm slices, row lookup, ledger == plan). Returns 0 and the
+// outputs for the caller to compare with its oracle.
+int tmh_matrix_roundtrip(const uint8_t *raw, uint32_t rows, uint32_t cols, const float *x,
+                         uint32_t batch, int exact, float *y_out, float *row_out, uint32_t row,
+                         char *err, size_t err_cap) {
+    try {
+        HipContext gpu = HipContext::open();
+        const uint64_t before = gpu.allocated_bytes();
+        Matrix m = Matrix::load(gpu, raw, cols, rows);
+        if (gpu.allocated_bytes() - before != Matrix::plan(cols, rows)) {
+            throw TuckmillError(ErrorCode::Internal, "allocation ledger differs from the plan");
+        }
+        HipBuffer xb = gpu.buffer((size_t)batch * cols * 4);
+        HipBuffer yb = gpu.buffer((size_t)batch * rows * 4);
+        HipBuffer ob = gpu.buffer((size_t)cols * 4);
+        xb.upload(0, x, (size_t)batch * cols * 4);
+        gpu.grouped([&]() {
+            if (batch == 1) {
+                m.gemv(gpu, xb, yb);
+            } else {
+                m.gemm(gpu, xb, yb, batch, exact != 0);
+            }
+            m.row_into(gpu, row, ob, 0);
+        });
+        yb.download(0, y_out, (size_t)batch * rows * 4);
+        ob.download(0, row_out, (size_t)cols * 4);
+        return 0;
+    } catch (const TuckmillError &e) {
+        if (err != nullptr && err_cap > 0) {
+            snprintf(err, err_cap, "%s", e.what());
+        }
+        return e.abi_code() != 0 ? e.abi_code() : TM_HIP_ERR_INTERNAL;
+    }
+}
+
+} // extern "C"

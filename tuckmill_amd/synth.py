@@ -62,16 +62,34 @@ def quantize_q8_0(w: np.ndarray) -> np.ndarray:
     return out.reshape(-1)
 
 
+def _weights_chunk(args):
+    seed, chunk, n, cols, std = args
+    rng = np.random.default_rng([seed, chunk])
+    w = rng.standard_normal((n, cols), dtype=np.float32)
+    w *= np.float32(std)
+    return quantize_q8_0(w)
+
+
 def make_weights(rows: int, cols: int, seed: int, std: float = 0.02,
-                 chunk_rows: int = 16384) -> np.ndarray:
-    """Raw Q8_0 bytes of a [rows, cols] matrix drawn N(0, std), seeded."""
-    rng = np.random.default_rng(seed)
+                 chunk_rows: int = 4096, threads: int = 8) -> np.ndarray:
+    """Raw Q8_0 bytes of a [rows, cols] matrix drawn N(0, std), seeded. Row
+    chunk c is drawn from its own stream (seed, c), so the bytes do not depend
+    on the thread count."""
+    from concurrent.futures import ThreadPoolExecutor
+
     out = np.empty(q8_0_bytes(rows, cols), dtype=np.uint8)
     row_bytes = (cols // BLOCK) * BLOCK_BYTES
-    for r0 in range(0, rows, chunk_rows):
-        n = min(chunk_rows, rows - r0)
-        w = rng.standard_normal((n, cols), dtype=np.float32) * np.float32(std)
-        out[r0 * row_bytes:(r0 + n) * row_bytes] = quantize_q8_0(w)
+    jobs = [(seed, c, min(chunk_rows, rows - r0), cols, std)
+            for c, r0 in enumerate(range(0, rows, chunk_rows))]
+    if len(jobs) == 1 or threads <= 1:
+        parts = map(_weights_chunk, jobs)
+    else:
+        pool = ThreadPoolExecutor(max_workers=threads)
+        parts = pool.map(_weights_chunk, jobs)
+    r0 = 0
+    for job, part in zip(jobs, parts):
+        out[r0 * row_bytes:(r0 + job[2]) * row_bytes] = part
+        r0 += job[2]
     return out
 
 
