@@ -151,3 +151,28 @@ def test_gemm_mma_gemma_and_sweep_shapes_gaussian(ctx, rows, cols, batch):
     want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
     assert norm_err(got, want) <= 1e-5
     wb.free()
+
+
+def test_independent_mma_products_in_a_group_share_one_launch(ctx):
+    # q/k/v of a prefill chunk: same X, three weight matrices, one launch;
+    # the result of each product does not depend on what shares its launch.
+    cols, batch = 1024, 96
+    x = S.make_activations(batch * cols, 5)
+    xb = upload_new(ctx, x)
+    mats = []
+    for i, rows in enumerate((2048, 1024, 1024)):
+        w = S.make_weights(rows, cols, 40 + i)
+        mats.append((w, rows, weights_buffer(ctx, w, rows, cols, True), ctx.buffer(batch * rows * 4)))
+    launches = ctx.kernel_launches()
+    ctx.begin_group()
+    for w, rows, wb, yb in mats:
+        ctx.q8_0_gemm_mma(wb, xb, yb, rows, cols, batch, 0, 0)
+    ctx.end_group()
+    assert ctx.kernel_launches() == launches + 1
+    ctx.fence()
+    for w, rows, wb, yb in mats:
+        grouped = yb.download_f32(0, batch * rows).copy()
+        alone = run_gemm(ctx, ctx.q8_0_gemm_mma, wb, x, rows, cols, batch)
+        assert np.array_equal(bits(grouped), bits(alone))
+        want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+        assert norm_err(grouped.reshape(batch, rows), want) <= 1e-5

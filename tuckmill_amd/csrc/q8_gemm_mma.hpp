@@ -44,15 +44,59 @@ __device__ __forceinline__ void load_x16(const float *p, float (&out)[16]) {
     }
 }
 
+struct MmaDesc {
+    const uint8_t *w;
+    const float *x;      // x_off already applied
+    float *y;            // y_off already applied
+    uint32_t rows, cols, batch;
+    uint32_t tile_begin; // index of this product's first output tile in the launch
+    uint32_t tiles_t;    // token tiles per row tile
+    uint32_t pad;
+};
+
+constexpr int MMA_MAX_DESCS = 64;
+
+struct MmaArgs {
+    uint32_t n;
+    uint32_t total_tiles;
+    uint32_t chunk_wgs; // workgroups that share one weight row-tile (see the XCD mapping)
+    uint32_t pad;
+    MmaDesc d[MMA_MAX_DESCS];
+};
+
+// Operands of one Q8_0 block for a wave's TMW x TNW tiles, as loaded.
+template <int TMW, int TNW> struct MmaRaw {
+    uint32_t q[TNW][4];
+    uint32_t sb[TNW];
+    float xv[TMW][16];
+};
+
+template <int L, int TMW, int TNW, bool XA>
+__device__ __forceinline__ void mma_load_block(const WView<L> &wv, const float *x, uint32_t cols,
+                                               const uint32_t (&wrow)[TNW],
+                                               const uint32_t (&tok)[TMW], uint32_t kb,
+                                               uint32_t half, MmaRaw<TMW, TNW> &raw) {
+    const uint32_t col = (kb << 5) + (half << 4);
+#pragma unroll
+    for (int j = 0; j < TNW; ++j) {
+        wv.template load_quants<16>(wrow[j], col, raw.q[j]);
+        raw.sb[j] = wv.scale_bits(wrow[j], kb);
+    }
+#pragma unroll
+    for (int i = 0; i < TMW; ++i) {
+        load_x16<XA>(x + (size_t)tok[i] * cols + col, raw.xv[i]);
+    }
+}
+
+// One launch runs a list of products (the q/k/v or gate/up projections of a
+// prefill chunk share their input and do not depend on each other).
 // Workgroup = 4 waves = P slots x S k-slices. Slot p of workgroup g owns
-// output tile g*P + p; its S waves each take a contiguous share of the Q8_0
-// blocks and wave s = 0 adds the partial tiles of s = 1..S-1 in that order.
+// output tile g*P + p of the launch; its S waves each take a contiguous share
+// of the Q8_0 blocks and wave s = 0 adds the partial tiles of s = 1..S-1 in
+// that order. The k loop is software-pipelined: the operands of block kb+1
+// are requested before the 16*TMW*TNW MFMAs of block kb are issued.
 template <int L, int TMW, int TNW, int S, bool XA>
-__global__ __launch_bounds__(256) void gemm_mma_kernel(const uint8_t *__restrict__ w,
-                                                       const float *__restrict__ x,
-                                                       float *__restrict__ y, uint32_t rows,
-                                                       uint32_t cols, uint32_t batch,
-                                                       uint32_t tiles_t, uint32_t tiles_n) {
+__global__ __launch_bounds__(256) void gemm_mma_kernel(const MmaArgs args) {
     constexpr int P = 4 / S;
     constexpr int TILE_FLOATS = TMW * TNW * 16 * WAVE;
     extern __shared__ float red[]; // [P][S-1][TILE_FLOATS]
@@ -62,20 +106,42 @@ __global__ __launch_bounds__(256) void gemm_mma_kernel(const uint8_t *__restrict
     const uint32_t p = wave / S, s = wave % S;
     const uint32_t idx = lane & 31u, half = lane >> 5;
 
-    // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a
-    // contiguous range of tiles so that a weight tile lives in one L2.
+    // Workgroups are dealt round-robin to the 8 XCDs (workgroup g runs on XCD
+    // g % 8), each with its own L2. Tiles are numbered token-tile fastest, so
+    // `chunk_wgs` consecutive workgroups share one weight row-tile: hand whole
+    // chunks to the XCDs in turn. A weight tile then lives in one L2, and
+    // heavy products (large K) are spread over all XCDs instead of landing on
+    // the one that owns their index range.
     uint32_t g = blockIdx.x;
-    const uint32_t G = gridDim.x;
-    if ((G & 7u) == 0u) {
-        g = (g & 7u) * (G >> 3) + (g >> 3);
+    {
+        const uint32_t cw = args.chunk_wgs;
+        const uint32_t span = 8u * cw;
+        const uint32_t g_full = (gridDim.x / span) * span;
+        if (g < g_full) {
+            const uint32_t xcd = g & 7u, j = g >> 3;
+            g = ((j / cw) * 8u + xcd) * cw + (j % cw);
+        }
     }
     const uint32_t tile = g * P + p;
-    const bool valid = tile < tiles_t * tiles_n;
-    const uint32_t tn = valid ? tile / tiles_t : 0u;
-    const uint32_t tt = valid ? tile % tiles_t : 0u;
+    const bool valid = tile < args.total_tiles;
+    uint32_t lo = 0, hi = args.n;
+    while (hi - lo > 1u) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (args.d[mid].tile_begin <= tile) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    const MmaDesc &d = args.d[lo];
+    const uint32_t rows = d.rows, cols = d.cols, batch = d.batch;
+    const uint32_t local = valid ? tile - d.tile_begin : 0u;
+    const uint32_t tn = local / d.tiles_t, tt = local % d.tiles_t;
     const uint32_t t0 = tt * (32u * TMW), n0 = tn * (32u * TNW);
+    const float *x = d.x;
+    float *y = d.y;
 
-    const WView<L> wv(w, rows, cols);
+    const WView<L> wv(d.w, rows, cols);
     const uint32_t blocks = cols >> 5;
     const uint32_t kb_begin = (uint32_t)(((uint64_t)blocks * s) / S);
     const uint32_t kb_end = (uint32_t)(((uint64_t)blocks * (s + 1u)) / S);
@@ -104,29 +170,29 @@ __global__ __launch_bounds__(256) void gemm_mma_kernel(const uint8_t *__restrict
         }
     }
 
-    if (valid) {
+    if (valid && kb_begin < kb_end) {
+        MmaRaw<TMW, TNW> raw;
+        mma_load_block<L, TMW, TNW, XA>(wv, x, cols, wrow, tok, kb_begin, half, raw);
         for (uint32_t kb = kb_begin; kb < kb_end; ++kb) {
-            const uint32_t col = (kb << 5) + (half << 4);
-            uint32_t q[TNW][4];
-            uint32_t sb[TNW];
-            float xv[TMW][16];
+            float wf[TNW][16];
+            float xa[TMW][16];
 #pragma unroll
             for (int j = 0; j < TNW; ++j) {
-                wv.template load_quants<16>(wrow[j], col, q[j]);
-                sb[j] = wv.scale_bits(wrow[j], kb);
+                const float dsc = f16_bits_to_f32(raw.sb[j]);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    wf[j][e] = dsc * sbyte_to_float(raw.q[j][e / 4], e % 4);
+                }
             }
 #pragma unroll
             for (int i = 0; i < TMW; ++i) {
-                load_x16<XA>(x + (size_t)tok[i] * cols + col, xv[i]);
-            }
-            float wf[TNW][16];
-#pragma unroll
-            for (int j = 0; j < TNW; ++j) {
-                const float d = f16_bits_to_f32(sb[j]);
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    wf[j][e] = d * sbyte_to_float(q[j][e / 4], e % 4);
+                    xa[i][e] = raw.xv[i][e];
                 }
+            }
+            if (kb + 1u < kb_end) {
+                mma_load_block<L, TMW, TNW, XA>(wv, x, cols, wrow, tok, kb + 1u, half, raw);
             }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
@@ -134,7 +200,7 @@ __global__ __launch_bounds__(256) void gemm_mma_kernel(const uint8_t *__restrict
                 for (int i = 0; i < TMW; ++i) {
 #pragma unroll
                     for (int j = 0; j < TNW; ++j) {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[i][e], wf[j][e],
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i][e], wf[j][e],
                                                                          acc[i][j], 0, 0, 0);
                     }
                 }
@@ -198,62 +264,78 @@ struct MmaConfig {
     int tmw, tnw, s;
 };
 
-// Pick the tile and K split that leave the fewest idle SIMD-rounds: the
-// chip has 1024 SIMDs and one wave's MFMA stream occupies one of them.
-inline MmaConfig pick_mma_config(uint32_t rows, uint32_t cols, uint32_t batch) {
-    static const MmaConfig candidates[] = {
-        {2, 2, 1}, {2, 1, 1}, {1, 1, 1}, {2, 2, 2}, {2, 1, 2}, {1, 1, 2}, {2, 1, 4}, {1, 1, 4},
-    };
-    const uint32_t blocks = cols / 32u;
-    MmaConfig best = candidates[2];
-    double best_cost = 1e300;
-    for (const MmaConfig &c : candidates) {
-        if ((uint32_t)c.s > blocks) {
-            continue;
-        }
-        const uint64_t tiles = (uint64_t)((batch + 32u * c.tmw - 1) / (32u * c.tmw)) *
-                               ((rows + 32u * c.tnw - 1) / (32u * c.tnw));
-        const uint64_t waves = tiles * c.s;
-        const uint64_t rounds = (waves + 1023u) / 1024u;
-        // MFMA issues per wave, plus a charge for operand loads per issue
-        // (small tiles reload more) and for the split-K reduction.
-        const double mfma = (double)c.tmw * c.tnw * 16.0 * ((blocks + c.s - 1) / c.s);
-        const double load_penalty = 1.0 + 0.10 * (1.0 / c.tmw + 1.0 / c.tnw);
-        const double cost = rounds * (mfma * load_penalty) + (c.s > 1 ? 40.0 * c.tmw * c.tnw : 0.0);
-        if (cost < best_cost) {
-            best_cost = cost;
-            best = c;
-        }
+struct MmaProduct {
+    const uint8_t *w;
+    const float *x;
+    float *y;
+    uint32_t rows, cols, batch;
+};
+
+inline uint64_t mma_tiles(const MmaProduct &p, const MmaConfig &c) {
+    return (uint64_t)((p.batch + 32u * c.tmw - 1) / (32u * c.tmw)) *
+           ((p.rows + 32u * c.tnw - 1) / (32u * c.tnw));
+}
+
+// Tile and K split. Measured on MI355X at M = 512 over the Qwen3-0.6B
+// projection shapes, alone and as one list launch: a 64-token x 32-row wave
+// tile with K split over the 4 waves of a workgroup is best or tied
+// everywhere (f32 MFMA is slow enough that filling all 1024 SIMDs with short
+// MFMA streams matters more than operand reuse). Narrow batches use a
+// 32-token tile; K is split no finer than one Q8_0 block per wave.
+inline MmaConfig pick_mma_config(const MmaProduct *prods, int n) {
+    uint32_t max_batch = 0, min_blocks = 0xffffffffu;
+    for (int i = 0; i < n; ++i) {
+        max_batch = prods[i].batch > max_batch ? prods[i].batch : max_batch;
+        const uint32_t blocks = prods[i].cols / 32u;
+        min_blocks = blocks < min_blocks ? blocks : min_blocks;
     }
-    return best;
+    MmaConfig c;
+    c.tmw = max_batch > 32u ? 2 : 1;
+    c.tnw = 1;
+    c.s = min_blocks >= 4u ? 4 : (min_blocks >= 2u ? 2 : 1);
+    return c;
 }
 
 template <int L, int TMW, int TNW, int S, bool XA>
-inline hipError_t launch_mma_cfg(hipStream_t stream, const uint8_t *w, const float *x, float *y,
-                                 uint32_t rows, uint32_t cols, uint32_t batch) {
+inline hipError_t launch_mma_cfg(hipStream_t stream, const MmaProduct *prods, int n) {
     constexpr int P = 4 / S;
-    const uint32_t tiles_t = (batch + 32u * TMW - 1) / (32u * TMW);
-    const uint32_t tiles_n = (rows + 32u * TNW - 1) / (32u * TNW);
-    const uint64_t tiles = (uint64_t)tiles_t * tiles_n;
+    MmaArgs args;
+    args.n = (uint32_t)n;
+    uint64_t tiles = 0;
+    const MmaConfig c{TMW, TNW, S};
+    for (int i = 0; i < n; ++i) {
+        MmaDesc &d = args.d[i];
+        d.w = prods[i].w;
+        d.x = prods[i].x;
+        d.y = prods[i].y;
+        d.rows = prods[i].rows;
+        d.cols = prods[i].cols;
+        d.batch = prods[i].batch;
+        d.tile_begin = (uint32_t)tiles;
+        d.tiles_t = (prods[i].batch + 32u * TMW - 1) / (32u * TMW);
+        d.pad = 0;
+        tiles += mma_tiles(prods[i], c);
+    }
+    args.total_tiles = (uint32_t)tiles;
+    args.chunk_wgs = args.d[0].tiles_t >= (uint32_t)P ? args.d[0].tiles_t / P : 1u;
+    args.pad = 0;
     const uint32_t groups = (uint32_t)((tiles + P - 1) / P);
     const size_t lds = S > 1 ? (size_t)P * (S - 1) * TMW * TNW * 16 * WAVE * sizeof(float) : 0;
     hipLaunchKernelGGL((gemm_mma_kernel<L, TMW, TNW, S, XA>), dim3(groups), dim3(256), lds, stream,
-                       w, x, y, rows, cols, batch, tiles_t, tiles_n);
+                       args);
     return hipGetLastError();
 }
 
 template <int L, bool XA>
-inline hipError_t launch_mma_layout(hipStream_t stream, const uint8_t *w, const float *x, float *y,
-                                    uint32_t rows, uint32_t cols, uint32_t batch) {
-    const MmaConfig c = pick_mma_config(rows, cols, batch);
-#define TM_MMA_CASE(A, B, C)                                                           \
-    if (c.tmw == A && c.tnw == B && c.s == C) {                                        \
-        return launch_mma_cfg<L, A, B, C, XA>(stream, w, x, y, rows, cols, batch);     \
+inline hipError_t launch_mma_layout(hipStream_t stream, const MmaProduct *prods, int n,
+                                    const MmaConfig *forced) {
+    const MmaConfig c = forced != nullptr ? *forced : pick_mma_config(prods, n);
+#define TM_MMA_CASE(A, B, C)                                                  \
+    if (c.tmw == A && c.tnw == B && c.s == C) {                               \
+        return launch_mma_cfg<L, A, B, C, XA>(stream, prods, n);              \
     }
-    TM_MMA_CASE(2, 2, 1)
     TM_MMA_CASE(2, 1, 1)
     TM_MMA_CASE(1, 1, 1)
-    TM_MMA_CASE(2, 2, 2)
     TM_MMA_CASE(2, 1, 2)
     TM_MMA_CASE(1, 1, 2)
     TM_MMA_CASE(2, 1, 4)
@@ -262,15 +344,26 @@ inline hipError_t launch_mma_layout(hipStream_t stream, const uint8_t *w, const 
     return hipErrorInvalidValue;
 }
 
+// All products of one call share the weight layout and the 16-byte alignment
+// class of their activations (the caller groups them so).
+inline hipError_t launch_gemm_mma_list(hipStream_t stream, bool packed, bool xaligned,
+                                       const MmaProduct *prods, int n,
+                                       const MmaConfig *forced = nullptr) {
+    if (n <= 0 || n > MMA_MAX_DESCS) {
+        return hipErrorInvalidValue;
+    }
+    if (packed) {
+        return xaligned ? launch_mma_layout<PACKED, true>(stream, prods, n, forced)
+                        : launch_mma_layout<PACKED, false>(stream, prods, n, forced);
+    }
+    return xaligned ? launch_mma_layout<RAW, true>(stream, prods, n, forced)
+                    : launch_mma_layout<RAW, false>(stream, prods, n, forced);
+}
+
 inline hipError_t launch_gemm_mma(hipStream_t stream, bool packed, const uint8_t *w, const float *x,
                                   float *y, uint32_t rows, uint32_t cols, uint32_t batch) {
-    const bool xa = ((uintptr_t)x % 16u) == 0;
-    if (packed) {
-        return xa ? launch_mma_layout<PACKED, true>(stream, w, x, y, rows, cols, batch)
-                  : launch_mma_layout<PACKED, false>(stream, w, x, y, rows, cols, batch);
-    }
-    return xa ? launch_mma_layout<RAW, true>(stream, w, x, y, rows, cols, batch)
-              : launch_mma_layout<RAW, false>(stream, w, x, y, rows, cols, batch);
+    const MmaProduct p{w, x, y, rows, cols, batch};
+    return launch_gemm_mma_list(stream, packed, ((uintptr_t)x % 16u) == 0, &p, 1);
 }
 
 } // namespace q8

@@ -104,6 +104,49 @@ __device__ __forceinline__ void chunk(const WView<L> &wv, const float *x, uint32
     }
 }
 
+// Sums R per-lane partials over the wave and stores row r0 + r (token `t`).
+// For R == 8 the xor-butterfly halves the number of live values at each of
+// its first three steps (lanes with bit 5/4/3 set carry rows +4/+2/+1), so 10
+// shuffles serve 8 rows; every addition has the same two operands as in
+// q8::wave_sum, hence the same bits.
+template <int R>
+__device__ __forceinline__ void reduce_store(const float (&acc)[R], float *y, uint32_t r0,
+                                             uint32_t row_end, uint32_t lane, bool token_ok) {
+    if constexpr (R == 8) {
+        float a4[4], a2[2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float keep = (lane & 32u) ? acc[i + 4] : acc[i];
+            const float send = (lane & 32u) ? acc[i] : acc[i + 4];
+            a4[i] = keep + __shfl_xor(send, 32, WAVE);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const float keep = (lane & 16u) ? a4[i + 2] : a4[i];
+            const float send = (lane & 16u) ? a4[i] : a4[i + 2];
+            a2[i] = keep + __shfl_xor(send, 16, WAVE);
+        }
+        const float keep = (lane & 8u) ? a2[1] : a2[0];
+        const float send = (lane & 8u) ? a2[0] : a2[1];
+        float a1 = keep + __shfl_xor(send, 8, WAVE);
+        a1 += __shfl_xor(a1, 4, WAVE);
+        a1 += __shfl_xor(a1, 2, WAVE);
+        a1 += __shfl_xor(a1, 1, WAVE);
+        const uint32_t r = ((lane >> 5) & 1u) * 4u + ((lane >> 4) & 1u) * 2u + ((lane >> 3) & 1u);
+        if ((lane & 7u) == 0u && r0 + r < row_end && token_ok) {
+            y[r0 + r] = a1;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float total = wave_sum(acc[r]);
+            if (lane == 0u && r0 + r < row_end && token_ok) {
+                y[r0 + r] = total;
+            }
+        }
+    }
+}
+
 template <int L, int R, int TB, bool XA>
 __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
     const uint32_t lane = threadIdx.x & 63u;
@@ -134,6 +177,32 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
     }
     const uint32_t full = cols >> 10;
     const uint32_t tail0 = full << 10;
+
+    if constexpr (TB == 1) {
+        if (cols == 1024u) {
+            // The commonest decode shape: one chunk, so this lane's 16
+            // activations stay in registers for every row of the tile. Same
+            // arithmetic as the general path below (one chunk, acc from 0).
+            float xv[16];
+            load_x<16, XA>(x + lane * 16u, xv);
+            for (uint32_t r0 = row_first; r0 < row_end; r0 += R) {
+                uint32_t q[R][4], sb[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+                    wv.template load_quants<16>(row, lane * 16u, q[r]);
+                    sb[r] = wv.scale_bits(row, lane >> 1);
+                }
+                float acc[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    acc[r] = __builtin_fmaf(f16_bits_to_f32(sb[r]), piece_dot<16>(q[r], xv), 0.0f);
+                }
+                reduce_store<R>(acc, y, r0, row_end, lane, true);
+            }
+            return;
+        }
+    }
 
     for (uint32_t t0 = 0; t0 < batch; t0 += TB) {
         uint32_t tok[TB];
@@ -179,14 +248,14 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
                 chunk<L, R, TB, 1, XA>(wv, x, cols, row, tok, col0, lane, lane < 32u, acc);
             }
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
+            for (int t = 0; t < TB; ++t) {
+                float col_acc[R];
 #pragma unroll
-                for (int t = 0; t < TB; ++t) {
-                    const float total = wave_sum(acc[r][t]);
-                    if (lane == 0u && r0 + r < row_end && t0 + t < batch) {
-                        y[(size_t)(t0 + t) * rows + (r0 + r)] = total;
-                    }
+                for (int r = 0; r < R; ++r) {
+                    col_acc[r] = acc[r][t];
                 }
+                reduce_store<R>(col_acc, y + (size_t)(t0 + t) * rows, r0, row_end, lane,
+                                t0 + t < batch);
             }
         }
     }

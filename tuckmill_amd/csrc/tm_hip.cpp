@@ -58,9 +58,14 @@ struct Op {
     char label[kProfileName] = {0};
 };
 
+// `start` is either an event recorded just before the commit's work or, when
+// the stream was still busy with the previous commit, that commit's stop
+// event (the new work starts when the old one ends; one event fewer on the
+// stream per commit). A lent stop event is recycled by its borrower.
 struct Commit {
     uint64_t seq = 0;
     hipEvent_t start = nullptr, stop = nullptr;
+    bool stop_lent = false;
     std::vector<Alloc *> keep;
     uint64_t leased = 0;
     char label[kProfileName] = {0};
@@ -200,7 +205,9 @@ void settle(tm_hip_ctx *ctx) {
             account_profile(ctx, c.label, nanos);
             ctx->leased.fetch_sub(c.leased, std::memory_order_relaxed);
             ctx->event_pool.push_back(c.start);
-            ctx->event_pool.push_back(c.stop);
+            if (!c.stop_lent) {
+                ctx->event_pool.push_back(c.stop);
+            }
             release.insert(release.end(), c.keep.begin(), c.keep.end());
             ctx->pending.pop_front();
             ctx->completed.fetch_add(1, std::memory_order_release);
@@ -236,34 +243,47 @@ void add_unique(std::vector<Alloc *> &keep, Alloc *a) {
     keep.push_back(a);
 }
 
+// Products that may share a launch agree on this key.
 struct GemvKey {
+    bool mma;     // MFMA list kernel instead of the GEMV list kernel
     bool packed;
-    int tb;       // tokens per pass: 1 or 4
+    int tb;       // GEMV list kernel: tokens per pass (1 or 4); MFMA: tile/split code
     bool xalign;
     bool operator==(const GemvKey &o) const {
-        return packed == o.packed && tb == o.tb && xalign == o.xalign;
+        return mma == o.mma && packed == o.packed && tb == o.tb && xalign == o.xalign;
     }
 };
 
 GemvKey gemv_key(const Op &op) {
     GemvKey k;
+    k.mma = op.kind == OP_MMA;
     k.packed = op.packed;
-    k.tb = op.batch == 1 ? 1 : 4;
+    if (k.mma) {
+        // The tile shape and K split are chosen per product, so a product's
+        // result does not depend on what else shares its launch.
+        const q8::MmaProduct p{nullptr, nullptr, nullptr, op.rows, op.cols, op.batch};
+        const q8::MmaConfig c = q8::pick_mma_config(&p, 1);
+        k.tb = c.tmw * 16 + c.tnw * 8 + c.s;
+    } else {
+        k.tb = op.batch == 1 ? 1 : 4;
+    }
     const uintptr_t xp = (uintptr_t)op.a[1]->ptr + (uintptr_t)op.x_off * 4u;
-    k.xalign = (xp % 16u == 0) && (op.batch == 1 || op.cols % 4u == 0);
+    k.xalign = (xp % 16u == 0);
     return k;
 }
 
 uint32_t pick_rows_per_tile(uint32_t rows, uint32_t cols, uint32_t batch, int R) {
-    // Aim for about 16 KiB of weights per wave, at least one pass of R rows;
-    // small matrices get smaller tiles so that they still spread over CUs.
+    // About 16 KiB of weights per wave (measured best for streaming: 8-16 KiB;
+    // larger tiles lose bandwidth), at least one pass of R rows; a matrix
+    // that would give fewer than 256 tiles gets smaller ones so that a lone
+    // product still spreads over the CUs.
     (void)batch;
     uint32_t rpt = (16384u / cols);
     if (rpt < (uint32_t)R) {
         rpt = (uint32_t)R;
     }
     rpt = (rpt / (uint32_t)R) * (uint32_t)R;
-    while (rpt > (uint32_t)R && (rows + rpt - 1) / rpt < 2048u) {
+    while (rpt > (uint32_t)R && (rows + rpt - 1) / rpt < 256u) {
         rpt -= (uint32_t)R;
     }
     return rpt;
@@ -278,10 +298,27 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, const q8::GemvArgs &args) {
     return hipGetLastError();
 }
 
-constexpr int kGemvR1 = 4; // rows per pass at one token per pass
+constexpr int kGemvR1 = 8; // rows per pass at one token per pass
 constexpr int kGemvR4 = 2; // rows per pass at four tokens per pass
 
+hipError_t launch_mma_list(tm_hip_ctx *ctx, const std::vector<const Op *> &ops, GemvKey key) {
+    q8::MmaProduct prods[q8::MMA_MAX_DESCS];
+    int n = 0;
+    for (const Op *op : ops) {
+        prods[n++] = q8::MmaProduct{(const uint8_t *)op->a[0]->ptr,
+                                    (const float *)op->a[1]->ptr + op->x_off,
+                                    (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
+                                    op->batch};
+    }
+    ctx->launches.fetch_add(1, std::memory_order_relaxed);
+    const q8::MmaConfig c{key.tb / 16, (key.tb / 8) % 2, key.tb % 8};
+    return q8::launch_gemm_mma_list(ctx->stream, key.packed, key.xalign, prods, n, &c);
+}
+
 hipError_t launch_gemv_list(tm_hip_ctx *ctx, const std::vector<const Op *> &ops, GemvKey key) {
+    if (key.mma) {
+        return launch_mma_list(ctx, ops, key);
+    }
     q8::GemvArgs args;
     memset(&args, 0, sizeof args);
     const int R = key.tb == 1 ? kGemvR1 : kGemvR4;
@@ -356,12 +393,6 @@ hipError_t launch_single(tm_hip_ctx *ctx, const Op &op) {
                            ctx->stream, w, (uint8_t *)op.a[1]->ptr, op.rows, op.cols);
         break;
     }
-    case OP_MMA: {
-        ctx->launches.fetch_add(1, std::memory_order_relaxed);
-        return q8::launch_gemm_mma(ctx->stream, op.packed, w,
-                                   (const float *)op.a[1]->ptr + op.x_off,
-                                   (float *)op.a[2]->ptr + op.y_off, op.rows, op.cols, op.batch);
-    }
     case OP_QUANT: {
         ctx->launches.fetch_add(1, std::memory_order_relaxed);
         return q8::launch_quantize_act(ctx->stream, (const float *)op.a[0]->ptr + op.x_off,
@@ -395,8 +426,9 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
         return e;
     };
     for (const Op &op : ops) {
-        if (op.kind == OP_GEMV_LIST) {
+        if (op.kind == OP_GEMV_LIST || op.kind == OP_MMA) {
             const GemvKey key = gemv_key(op);
+            const int cap = key.mma ? q8::MMA_MAX_DESCS : q8::GEMV_MAX_DESCS;
             bool conflict = false;
             for (const Op *b : batch) {
                 // a[0] = w (read), a[1] = x (read), a[2] = y (written)
@@ -407,7 +439,7 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 }
             }
             if (!batch.empty() &&
-                (conflict || !(key == batch_key) || (int)batch.size() == q8::GEMV_MAX_DESCS)) {
+                (conflict || !(key == batch_key) || (int)batch.size() == cap)) {
                 hipError_t e = flush();
                 if (e != hipSuccess) {
                     return e;
@@ -433,9 +465,17 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
 int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, char *err,
                size_t cap) {
     Commit c;
+    bool fresh_start = true;
     {
         std::lock_guard<std::mutex> g(ctx->q_mu);
-        c.start = take_event(ctx);
+        if (!ctx->pending.empty() && !ctx->pending.back().stop_lent &&
+            hipEventQuery(ctx->pending.back().stop) == hipErrorNotReady) {
+            c.start = ctx->pending.back().stop;
+            ctx->pending.back().stop_lent = true;
+            fresh_start = false;
+        } else {
+            c.start = take_event(ctx);
+        }
         c.stop = take_event(ctx);
     }
     if (c.start == nullptr || c.stop == nullptr) {
@@ -455,7 +495,7 @@ int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, c
     if (ctx->profiling.load(std::memory_order_relaxed)) {
         snprintf(c.label, sizeof c.label, "%s", label);
     }
-    hipError_t e = hipEventRecord(c.start, ctx->stream);
+    hipError_t e = fresh_start ? hipEventRecord(c.start, ctx->stream) : hipSuccess;
     if (e == hipSuccess) {
         e = issue_ops(ctx, ops);
     }
@@ -635,7 +675,9 @@ void tm_hip_destroy(tm_hip_ctx *ctx) {
                 alloc_release(a);
             }
             (void)hipEventDestroy(c.start);
-            (void)hipEventDestroy(c.stop);
+            if (!c.stop_lent) {
+                (void)hipEventDestroy(c.stop);
+            }
         }
         ctx->pending.clear();
         for (hipEvent_t e : ctx->event_pool) {
