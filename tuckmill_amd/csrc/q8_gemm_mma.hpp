@@ -297,7 +297,8 @@ inline MmaConfig pick_mma_config(const MmaProduct *prods, int n) {
 }
 
 template <int L, int TMW, int TNW, int S, bool XA>
-inline hipError_t launch_mma_cfg(hipStream_t stream, const MmaProduct *prods, int n) {
+inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods,
+                                 int n) {
     constexpr int P = 4 / S;
     MmaArgs args;
     args.n = (uint32_t)n;
@@ -321,18 +322,18 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, const MmaProduct *prods, in
     args.pad = 0;
     const uint32_t groups = (uint32_t)((tiles + P - 1) / P);
     const size_t lds = S > 1 ? (size_t)P * (S - 1) * TMW * TNW * 16 * WAVE * sizeof(float) : 0;
-    hipLaunchKernelGGL((gemm_mma_kernel<L, TMW, TNW, S, XA>), dim3(groups), dim3(256), lds, stream,
-                       args);
+    Q8_LAUNCH((gemm_mma_kernel<L, TMW, TNW, S, XA>), dim3(groups), dim3(256), lds, stream, stop,
+              args);
     return hipGetLastError();
 }
 
 template <int L, bool XA>
-inline hipError_t launch_mma_layout(hipStream_t stream, const MmaProduct *prods, int n,
-                                    const MmaConfig *forced) {
+inline hipError_t launch_mma_layout(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods,
+                                    int n, const MmaConfig *forced) {
     const MmaConfig c = forced != nullptr ? *forced : pick_mma_config(prods, n);
 #define TM_MMA_CASE(A, B, C)                                                  \
     if (c.tmw == A && c.tnw == B && c.s == C) {                               \
-        return launch_mma_cfg<L, A, B, C, XA>(stream, prods, n);              \
+        return launch_mma_cfg<L, A, B, C, XA>(stream, stop, prods, n);              \
     }
     TM_MMA_CASE(2, 1, 1)
     TM_MMA_CASE(1, 1, 1)
@@ -346,24 +347,18 @@ inline hipError_t launch_mma_layout(hipStream_t stream, const MmaProduct *prods,
 
 // All products of one call share the weight layout and the 16-byte alignment
 // class of their activations (the caller groups them so).
-inline hipError_t launch_gemm_mma_list(hipStream_t stream, bool packed, bool xaligned,
-                                       const MmaProduct *prods, int n,
+inline hipError_t launch_gemm_mma_list(hipStream_t stream, hipEvent_t stop, bool packed,
+                                       bool xaligned, const MmaProduct *prods, int n,
                                        const MmaConfig *forced = nullptr) {
     if (n <= 0 || n > MMA_MAX_DESCS) {
         return hipErrorInvalidValue;
     }
     if (packed) {
-        return xaligned ? launch_mma_layout<PACKED, true>(stream, prods, n, forced)
-                        : launch_mma_layout<PACKED, false>(stream, prods, n, forced);
+        return xaligned ? launch_mma_layout<PACKED, true>(stream, stop, prods, n, forced)
+                        : launch_mma_layout<PACKED, false>(stream, stop, prods, n, forced);
     }
-    return xaligned ? launch_mma_layout<RAW, true>(stream, prods, n, forced)
-                    : launch_mma_layout<RAW, false>(stream, prods, n, forced);
-}
-
-inline hipError_t launch_gemm_mma(hipStream_t stream, bool packed, const uint8_t *w, const float *x,
-                                  float *y, uint32_t rows, uint32_t cols, uint32_t batch) {
-    const MmaProduct p{w, x, y, rows, cols, batch};
-    return launch_gemm_mma_list(stream, packed, ((uintptr_t)x % 16u) == 0, &p, 1);
+    return xaligned ? launch_mma_layout<RAW, true>(stream, stop, prods, n, forced)
+                    : launch_mma_layout<RAW, false>(stream, stop, prods, n, forced);
 }
 
 } // namespace q8

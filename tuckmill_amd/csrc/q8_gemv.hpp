@@ -77,7 +77,7 @@ __device__ __forceinline__ float piece_dot(const uint32_t *q, const float *x) {
 // One chunk of 64*NB columns starting at `col0`, for R rows and TB tokens.
 // `active` is false only for the upper half-wave of a trailing 32-column
 // chunk; inactive lanes still execute (on clamped addresses) and add 0.
-template <int L, int R, int TB, int NB, bool XA>
+template <int L, int R, int TB, int NB, bool XA, bool NT>
 __device__ __forceinline__ void chunk(const WView<L> &wv, const float *x, uint32_t cols,
                                       const uint32_t (&row)[R], const uint32_t (&tok)[TB],
                                       uint32_t col0, uint32_t lane, bool active,
@@ -88,7 +88,7 @@ __device__ __forceinline__ void chunk(const WView<L> &wv, const float *x, uint32
     uint32_t sb[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        wv.template load_quants<NB>(row[r], col, q[r]);
+        wv.template load_quants<NB, NT>(row[r], col, q[r]);
         sb[r] = wv.scale_bits(row[r], col >> 5);
     }
 #pragma unroll
@@ -177,28 +177,76 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
     }
     const uint32_t full = cols >> 10;
     const uint32_t tail0 = full << 10;
+    // With one pass over the tokens every quant is read once: stream it. (The
+    // f16 scales stay on plain loads: neighbouring rows share their cache
+    // lines.) The multi-token form re-reads the tile per token group: keep it
+    // cached.
+    constexpr bool NT = TB == 1;
 
-    if constexpr (TB == 1) {
-        if (cols == 1024u) {
-            // The commonest decode shape: one chunk, so this lane's 16
-            // activations stay in registers for every row of the tile. Same
-            // arithmetic as the general path below (one chunk, acc from 0).
+    if constexpr (TB == 1 && L == PACKED) {
+        if ((cols & 1023u) == 0u) {
+            // Whole 1024-column chunks only (every Qwen3 projection): the
+            // (row pass, chunk) steps form one software-pipelined sequence in
+            // which the 8 weight loads of step s+1 are in flight while step s
+            // is multiplied. With a single chunk this lane's 16 activations
+            // stay in registers for the whole tile. Same per-row arithmetic
+            // as the general path below: chunks in order, acc from 0.
+            const uint32_t nchunk = cols >> 10;
+            const uint32_t nsteps = ((row_end - row_first + R - 1) / R) * nchunk;
             float xv[16];
-            load_x<16, XA>(x + lane * 16u, xv);
-            for (uint32_t r0 = row_first; r0 < row_end; r0 += R) {
-                uint32_t q[R][4], sb[R];
+            if (nchunk == 1u) {
+                load_x<16, XA>(x + lane * 16u, xv);
+            }
+            uint32_t q[R][4], sb[R];
+            auto load_step = [&](uint32_t r0, uint32_t c, uint32_t (&qq)[R][4], uint32_t (&ss)[R]) {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
-                    wv.template load_quants<16>(row, lane * 16u, q[r]);
-                    sb[r] = wv.scale_bits(row, lane >> 1);
+                    wv.template load_quants<16, true>(row, (c << 10) + lane * 16u, qq[r]);
+                    ss[r] = wv.scale_bits(row, (c << 5) + (lane >> 1));
                 }
-                float acc[R];
+            };
+            uint32_t r0 = row_first, c = 0;
+            load_step(r0, c, q, sb);
+            float acc[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                acc[r] = 0.0f;
+            }
+            for (uint32_t step = 0; step < nsteps; ++step) {
+                if (nchunk > 1u) {
+                    load_x<16, XA>(x + (c << 10) + lane * 16u, xv);
+                }
+                uint32_t cn = c + 1u, rn = r0;
+                if (cn == nchunk) {
+                    cn = 0;
+                    rn = r0 + R;
+                }
+                uint32_t qn[R][4], sn[R];
+                if (step + 1u < nsteps) {
+                    load_step(rn, cn, qn, sn);
+                }
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    acc[r] = __builtin_fmaf(f16_bits_to_f32(sb[r]), piece_dot<16>(q[r], xv), 0.0f);
+                    acc[r] = __builtin_fmaf(f16_bits_to_f32(sb[r]), piece_dot<16>(q[r], xv), acc[r]);
                 }
-                reduce_store<R>(acc, y, r0, row_end, lane, true);
+                if (cn == 0u) {
+                    reduce_store<R>(acc, y, r0, row_end, lane, true);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        acc[r] = 0.0f;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        q[r][i] = qn[r][i];
+                    }
+                    sb[r] = sn[r];
+                }
+                c = cn;
+                r0 = rn;
             }
             return;
         }
@@ -225,27 +273,27 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
                 }
             }
             for (uint32_t c = 0; c < full; ++c) {
-                chunk<L, R, TB, 16, XA>(wv, x, cols, row, tok, c << 10, lane, true, acc);
+                chunk<L, R, TB, 16, XA, NT>(wv, x, cols, row, tok, c << 10, lane, true, acc);
             }
             uint32_t col0 = tail0;
             if (cols & 512u) {
-                chunk<L, R, TB, 8, XA>(wv, x, cols, row, tok, col0, lane, true, acc);
+                chunk<L, R, TB, 8, XA, NT>(wv, x, cols, row, tok, col0, lane, true, acc);
                 col0 += 512u;
             }
             if (cols & 256u) {
-                chunk<L, R, TB, 4, XA>(wv, x, cols, row, tok, col0, lane, true, acc);
+                chunk<L, R, TB, 4, XA, NT>(wv, x, cols, row, tok, col0, lane, true, acc);
                 col0 += 256u;
             }
             if (cols & 128u) {
-                chunk<L, R, TB, 2, XA>(wv, x, cols, row, tok, col0, lane, true, acc);
+                chunk<L, R, TB, 2, XA, NT>(wv, x, cols, row, tok, col0, lane, true, acc);
                 col0 += 128u;
             }
             if (cols & 64u) {
-                chunk<L, R, TB, 1, XA>(wv, x, cols, row, tok, col0, lane, true, acc);
+                chunk<L, R, TB, 1, XA, NT>(wv, x, cols, row, tok, col0, lane, true, acc);
                 col0 += 64u;
             }
             if (cols & 32u) {
-                chunk<L, R, TB, 1, XA>(wv, x, cols, row, tok, col0, lane, lane < 32u, acc);
+                chunk<L, R, TB, 1, XA, NT>(wv, x, cols, row, tok, col0, lane, lane < 32u, acc);
             }
 #pragma unroll
             for (int t = 0; t < TB; ++t) {

@@ -37,6 +37,9 @@ struct Alloc {
     std::atomic<int> refs{1};
     bool packed = false;
     uint32_t prows = 0, pcols = 0;
+    // Launch planning (under the caller's serialization): the planning epoch
+    // in which this allocation was last read / written by a listed product.
+    uint64_t read_epoch = 0, write_epoch = 0, keep_epoch = 0;
 };
 
 void alloc_release(Alloc *a) {
@@ -55,7 +58,8 @@ struct Op {
     unsigned writes_mask = 0; // bit i: a[i] is written
     uint32_t rows = 0, cols = 0, batch = 0, x_off = 0, y_off = 0, extra = 0;
     bool packed = false;
-    char label[kProfileName] = {0};
+    bool shape_label = false;  // profile label carries "<rows>x<cols>"
+    const char *what = "";     // static operator name
 };
 
 // `start` is either an event recorded just before the commit's work or, when
@@ -93,6 +97,7 @@ struct tm_hip_ctx {
     std::atomic<int> profiling{0};
     bool group_active = false;
     std::vector<Op> group_ops;
+    uint64_t plan_epoch = 0;
     std::mutex q_mu; // pending commits, event pool, profile table
     std::mutex copy_mu;
     std::deque<Commit> pending;
@@ -234,15 +239,6 @@ int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
 
 // ------------------------------------------------------------ launches ---
 
-void add_unique(std::vector<Alloc *> &keep, Alloc *a) {
-    for (Alloc *k : keep) {
-        if (k == a) {
-            return;
-        }
-    }
-    keep.push_back(a);
-}
-
 // Products that may share a launch agree on this key.
 struct GemvKey {
     bool mma;     // MFMA list kernel instead of the GEMV list kernel
@@ -273,12 +269,12 @@ GemvKey gemv_key(const Op &op) {
 }
 
 uint32_t pick_rows_per_tile(uint32_t rows, uint32_t cols, uint32_t batch, int R) {
-    // About 16 KiB of weights per wave (measured best for streaming: 8-16 KiB;
-    // larger tiles lose bandwidth), at least one pass of R rows; a matrix
-    // that would give fewer than 256 tiles gets smaller ones so that a lone
+    // About 8 KiB of weights per wave (measured best for streaming; 32 KiB
+    // and more lose bandwidth), at least one pass of R rows; a matrix that
+    // would give fewer than 256 tiles gets smaller ones so that a lone
     // product still spreads over the CUs.
     (void)batch;
-    uint32_t rpt = (16384u / cols);
+    uint32_t rpt = (8192u / cols);
     if (rpt < (uint32_t)R) {
         rpt = (uint32_t)R;
     }
@@ -290,18 +286,18 @@ uint32_t pick_rows_per_tile(uint32_t rows, uint32_t cols, uint32_t batch, int R)
 }
 
 template <int L, int R, int TB, bool XA>
-hipError_t launch_gemv(tm_hip_ctx *ctx, const q8::GemvArgs &args) {
+hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args) {
     const uint32_t groups = (args.total_tiles + 3u) / 4u;
-    hipLaunchKernelGGL((q8::gemv_list_kernel<L, R, TB, XA>), dim3(groups), dim3(256), 0, ctx->stream,
-                       args);
-    ctx->launches.fetch_add(1, std::memory_order_relaxed);
+    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA>), dim3(groups), dim3(256), 0, ctx->stream, stop,
+              args);
     return hipGetLastError();
 }
 
 constexpr int kGemvR1 = 8; // rows per pass at one token per pass
 constexpr int kGemvR4 = 2; // rows per pass at four tokens per pass
 
-hipError_t launch_mma_list(tm_hip_ctx *ctx, const std::vector<const Op *> &ops, GemvKey key) {
+hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
+                           GemvKey key) {
     q8::MmaProduct prods[q8::MMA_MAX_DESCS];
     int n = 0;
     for (const Op *op : ops) {
@@ -310,17 +306,18 @@ hipError_t launch_mma_list(tm_hip_ctx *ctx, const std::vector<const Op *> &ops, 
                                     (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
                                     op->batch};
     }
-    ctx->launches.fetch_add(1, std::memory_order_relaxed);
     const q8::MmaConfig c{key.tb / 16, (key.tb / 8) % 2, key.tb % 8};
-    return q8::launch_gemm_mma_list(ctx->stream, key.packed, key.xalign, prods, n, &c);
+    return q8::launch_gemm_mma_list(ctx->stream, stop, key.packed, key.xalign, prods, n, &c);
 }
 
-hipError_t launch_gemv_list(tm_hip_ctx *ctx, const std::vector<const Op *> &ops, GemvKey key) {
+hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
+                            GemvKey key) {
     if (key.mma) {
-        return launch_mma_list(ctx, ops, key);
+        return launch_mma_list(ctx, stop, ops, key);
     }
-    q8::GemvArgs args;
-    memset(&args, 0, sizeof args);
+    q8::GemvArgs args; // only the used descriptors are written (the struct is 12 KB)
+    args.n = 0;
+    args.pad[0] = args.pad[1] = 0;
     const int R = key.tb == 1 ? kGemvR1 : kGemvR4;
     uint32_t tiles = 0;
     for (const Op *op : ops) {
@@ -333,12 +330,14 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, const std::vector<const Op *> &ops,
         d.batch = op->batch;
         d.tile_begin = tiles;
         d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, op->batch, R);
+        d.pad = 0;
         tiles += (op->rows + d.rows_per_tile - 1) / d.rows_per_tile;
     }
     args.total_tiles = tiles;
-#define TM_GEMV_CASE(P, T, A)                                                          \
-    if (key.packed == (P) && key.tb == (T) && key.xalign == (A)) {                     \
-        return launch_gemv<(P) ? q8::PACKED : q8::RAW, (T) == 1 ? kGemvR1 : kGemvR4, T, A>(ctx, args); \
+#define TM_GEMV_CASE(P, T, A)                                                                \
+    if (key.packed == (P) && key.tb == (T) && key.xalign == (A)) {                           \
+        return launch_gemv<(P) ? q8::PACKED : q8::RAW, (T) == 1 ? kGemvR1 : kGemvR4, T, A>(  \
+            ctx, stop, args);                                                                \
     }
     TM_GEMV_CASE(true, 1, true)
     TM_GEMV_CASE(true, 1, false)
@@ -352,18 +351,19 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, const std::vector<const Op *> &ops,
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_single(tm_hip_ctx *ctx, const Op &op) {
+hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
     const uint8_t *w = op.a[0] ? (const uint8_t *)op.a[0]->ptr : nullptr;
+    hipStream_t st = ctx->stream;
     switch (op.kind) {
     case OP_ROW: {
         float *out = (float *)op.a[1]->ptr;
         dim3 grid((op.cols + 255u) / 256u);
         if (op.packed) {
-            hipLaunchKernelGGL(q8::row_kernel<q8::PACKED>, grid, dim3(256), 0, ctx->stream, w, out,
-                               op.rows, op.cols, op.extra, op.y_off);
+            Q8_LAUNCH(q8::row_kernel<q8::PACKED>, grid, dim3(256), 0, st, stop, w, out, op.rows,
+                      op.cols, op.extra, op.y_off);
         } else {
-            hipLaunchKernelGGL(q8::row_kernel<q8::RAW>, grid, dim3(256), 0, ctx->stream, w, out,
-                               op.rows, op.cols, op.extra, op.y_off);
+            Q8_LAUNCH(q8::row_kernel<q8::RAW>, grid, dim3(256), 0, st, stop, w, out, op.rows, op.cols,
+                      op.extra, op.y_off);
         }
         break;
     }
@@ -372,98 +372,118 @@ hipError_t launch_single(tm_hip_ctx *ctx, const Op &op) {
         const uint32_t *ids = (const uint32_t *)op.a[2]->ptr;
         dim3 grid((op.cols + 255u) / 256u);
         if (op.packed) {
-            hipLaunchKernelGGL(q8::row_indirect_kernel<q8::PACKED>, grid, dim3(256), 0, ctx->stream,
-                               w, out, ids, op.extra, op.rows, op.cols);
+            Q8_LAUNCH(q8::row_indirect_kernel<q8::PACKED>, grid, dim3(256), 0, st, stop, w, out, ids,
+                      op.extra, op.rows, op.cols);
         } else {
-            hipLaunchKernelGGL(q8::row_indirect_kernel<q8::RAW>, grid, dim3(256), 0, ctx->stream, w,
-                               out, ids, op.extra, op.rows, op.cols);
+            Q8_LAUNCH(q8::row_indirect_kernel<q8::RAW>, grid, dim3(256), 0, st, stop, w, out, ids,
+                      op.extra, op.rows, op.cols);
         }
         break;
     }
     case OP_COPY: {
         const float *src = (const float *)op.a[0]->ptr + op.x_off;
         float *dst = (float *)op.a[1]->ptr + op.y_off;
-        hipLaunchKernelGGL(q8::copy_f32_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0,
-                           ctx->stream, src, dst, op.extra);
+        Q8_LAUNCH(q8::copy_f32_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop, src,
+                  dst, op.extra);
         break;
     }
     case OP_PACK: {
         const size_t nblocks = (size_t)op.rows * (op.cols / 32u);
-        hipLaunchKernelGGL(q8::pack_kernel, dim3((unsigned)((nblocks + 255u) / 256u)), dim3(256), 0,
-                           ctx->stream, w, (uint8_t *)op.a[1]->ptr, op.rows, op.cols);
+        Q8_LAUNCH(q8::pack_kernel, dim3((unsigned)((nblocks + 255u) / 256u)), dim3(256), 0, st, stop,
+                  w, (uint8_t *)op.a[1]->ptr, op.rows, op.cols);
         break;
     }
-    case OP_QUANT: {
-        ctx->launches.fetch_add(1, std::memory_order_relaxed);
-        return q8::launch_quantize_act(ctx->stream, (const float *)op.a[0]->ptr + op.x_off,
+    case OP_QUANT:
+        return q8::launch_quantize_act(st, stop, (const float *)op.a[0]->ptr + op.x_off,
                                        (uint8_t *)op.a[1]->ptr, op.cols, op.batch);
-    }
-    case OP_I8: {
-        ctx->launches.fetch_add(1, std::memory_order_relaxed);
-        return q8::launch_gemm_i8(ctx->stream, op.packed, w, (const uint8_t *)op.a[1]->ptr,
+    case OP_I8:
+        return q8::launch_gemm_i8(st, stop, op.packed, w, (const uint8_t *)op.a[1]->ptr,
                                   (float *)op.a[2]->ptr + op.y_off,
                                   op.a[3] ? (int32_t *)op.a[3]->ptr : nullptr, op.rows, op.cols,
                                   op.batch);
-    }
     default:
         return hipErrorInvalidValue;
     }
-    ctx->launches.fetch_add(1, std::memory_order_relaxed);
     return hipGetLastError();
 }
 
-// Issue a sequence of recorded operations. Consecutive list-kernel products
-// that neither read nor overwrite each other's outputs share one launch.
-hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
-    std::vector<const Op *> batch;
-    GemvKey batch_key{};
-    auto flush = [&]() -> hipError_t {
-        if (batch.empty()) {
-            return hipSuccess;
+// One kernel launch of a commit: a list of products, or a single operation.
+struct Launch {
+    std::vector<const Op *> list; // empty: `single`
+    GemvKey key{};
+    const Op *single = nullptr;
+};
+
+// Plan the launches of a sequence of recorded operations. Consecutive
+// list-kernel products that neither read nor overwrite each other's outputs
+// share one launch; everything else launches on its own, in order.
+std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
+    std::vector<Launch> plan;
+    Launch cur;
+    // Hazards are tracked per allocation with an epoch stamp, so planning a
+    // step of n products costs O(n), not O(n^2).
+    uint64_t epoch = ++ctx->plan_epoch;
+    auto flush = [&]() {
+        if (!cur.list.empty()) {
+            plan.push_back(std::move(cur));
+            cur = Launch();
+            epoch = ++ctx->plan_epoch;
         }
-        hipError_t e = launch_gemv_list(ctx, batch, batch_key);
-        batch.clear();
-        return e;
     };
     for (const Op &op : ops) {
         if (op.kind == OP_GEMV_LIST || op.kind == OP_MMA) {
             const GemvKey key = gemv_key(op);
             const int cap = key.mma ? q8::MMA_MAX_DESCS : q8::GEMV_MAX_DESCS;
-            bool conflict = false;
-            for (const Op *b : batch) {
-                // a[0] = w (read), a[1] = x (read), a[2] = y (written)
-                if (op.a[2] == b->a[2] || op.a[2] == b->a[1] || op.a[2] == b->a[0] ||
-                    op.a[1] == b->a[2] || op.a[0] == b->a[2]) {
-                    conflict = true;
-                    break;
-                }
+            // a[0] = w (read), a[1] = x (read), a[2] = y (written): the product
+            // joins the open launch unless its output was read or written
+            // there, or one of its inputs was written there.
+            const bool conflict = op.a[2]->read_epoch == epoch || op.a[2]->write_epoch == epoch ||
+                                  op.a[1]->write_epoch == epoch || op.a[0]->write_epoch == epoch;
+            if (!cur.list.empty() &&
+                (conflict || !(key == cur.key) || (int)cur.list.size() == cap)) {
+                flush();
             }
-            if (!batch.empty() &&
-                (conflict || !(key == batch_key) || (int)batch.size() == cap)) {
-                hipError_t e = flush();
-                if (e != hipSuccess) {
-                    return e;
-                }
-            }
-            batch_key = key;
-            batch.push_back(&op);
+            cur.key = key;
+            cur.list.push_back(&op);
+            op.a[0]->read_epoch = epoch;
+            op.a[1]->read_epoch = epoch;
+            op.a[2]->write_epoch = epoch;
         } else {
-            hipError_t e = flush();
-            if (e != hipSuccess) {
-                return e;
-            }
-            e = launch_single(ctx, op);
-            if (e != hipSuccess) {
-                return e;
-            }
+            flush();
+            Launch one;
+            one.single = &op;
+            plan.push_back(std::move(one));
         }
     }
-    return flush();
+    flush();
+    return plan;
+}
+
+// Issue the launches; the last one carries the commit's stop event.
+hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, hipEvent_t stop,
+                     bool *stop_attached) {
+    const std::vector<Launch> plan = plan_launches(ctx, ops);
+    *stop_attached = false;
+    for (size_t i = 0; i < plan.size(); ++i) {
+        const bool last = i + 1 == plan.size();
+        const hipEvent_t ev = last ? stop : nullptr;
+        const Launch &l = plan[i];
+        hipError_t e = l.single != nullptr ? launch_single(ctx, ev, *l.single)
+                                           : launch_gemv_list(ctx, ev, l.list, l.key);
+        if (e != hipSuccess) {
+            return e;
+        }
+        ctx->launches.fetch_add(1, std::memory_order_relaxed);
+        if (last) {
+            *stop_attached = true;
+        }
+    }
+    return hipSuccess;
 }
 
 // Submit `ops` as one commit: start event, launches, stop event, leases.
-int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, char *err,
-               size_t cap) {
+int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, const char *what,
+               char *err, size_t cap) {
     Commit c;
     bool fresh_start = true;
     {
@@ -479,12 +499,16 @@ int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, c
         c.stop = take_event(ctx);
     }
     if (c.start == nullptr || c.stop == nullptr) {
-        return fail(err, cap, TM_HIP_ERR_INTERNAL, "%s: event creation failed", label);
+        return fail(err, cap, TM_HIP_ERR_INTERNAL, "%s: event creation failed", what);
     }
+    const uint64_t keep_epoch = ++ctx->plan_epoch;
+    c.keep.reserve(ops.size() * 3);
     for (const Op &op : ops) {
         for (int i = 0; i < op.n_alloc; ++i) {
-            if (op.a[i] != nullptr) {
-                add_unique(c.keep, op.a[i]);
+            Alloc *a = op.a[i];
+            if (a != nullptr && a->keep_epoch != keep_epoch) {
+                a->keep_epoch = keep_epoch;
+                c.keep.push_back(a);
             }
         }
     }
@@ -496,12 +520,15 @@ int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, c
         snprintf(c.label, sizeof c.label, "%s", label);
     }
     hipError_t e = fresh_start ? hipEventRecord(c.start, ctx->stream) : hipSuccess;
+    bool stop_attached = false;
     if (e == hipSuccess) {
-        e = issue_ops(ctx, ops);
+        e = issue_ops(ctx, ops, c.stop, &stop_attached);
     }
-    hipError_t e2 = hipEventRecord(c.stop, ctx->stream);
-    if (e == hipSuccess) {
-        e = e2;
+    if (!stop_attached) { // an empty group, or a launch that failed
+        hipError_t e2 = hipEventRecord(c.stop, ctx->stream);
+        if (e == hipSuccess) {
+            e = e2;
+        }
     }
     c.seq = ctx->committed.fetch_add(1, std::memory_order_relaxed) + 1;
     ctx->leased.fetch_add(c.leased, std::memory_order_relaxed);
@@ -511,20 +538,30 @@ int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, c
     }
     settle(ctx);
     if (e != hipSuccess) {
-        return hip_fail(err, cap, label, e);
+        return hip_fail(err, cap, what, e);
     }
     return TM_HIP_OK;
 }
 
-// Either appends to the open group or commits on its own.
-int submit(tm_hip_ctx *ctx, Op &op, const char *label, char *err, size_t cap) {
-    snprintf(op.label, sizeof op.label, "%s", label);
+// Either appends to the open group or commits on its own. The profile label
+// is only formatted when profiling is on (it is off on the hot path).
+int submit(tm_hip_ctx *ctx, Op &op, const char *what, char *err, size_t cap) {
+    op.what = what;
     if (ctx->group_active) {
         ctx->group_ops.push_back(op);
         return TM_HIP_OK;
     }
+    char label[kProfileName];
+    label[0] = '\0';
+    if (ctx->profiling.load(std::memory_order_relaxed)) {
+        if (op.shape_label) {
+            snprintf(label, sizeof label, "%s:%ux%u", what, op.rows, op.cols);
+        } else {
+            snprintf(label, sizeof label, "%s", what);
+        }
+    }
     std::vector<Op> one(1, op);
-    return commit_ops(ctx, one, label, err, cap);
+    return commit_ops(ctx, one, label, what, err, cap);
 }
 
 struct DeviceProbe {
@@ -579,19 +616,16 @@ int check_product(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_bu
     const size_t w_need = (size_t)rows * ((size_t)cols / 32u) * 34u;
     const size_t x_need = ((size_t)x_off + (size_t)batch * cols) * 4u;
     const size_t y_need = ((size_t)y_off + (size_t)batch * rows) * 4u;
-    char name[64];
-    snprintf(name, sizeof name, "%s.weights", what);
-    int rc = check_buffer(ctx, w, w_need, err, cap, name);
-    if (rc != TM_HIP_OK) {
-        return rc == TM_HIP_ERR_BOUNDS ? TM_HIP_ERR_BOUNDS : rc;
-    }
-    snprintf(name, sizeof name, "%s.x", what);
-    if ((rc = check_buffer(ctx, x, x_need, err, cap, name)) != TM_HIP_OK) {
-        return rc;
-    }
-    snprintf(name, sizeof name, "%s.y", what);
-    if ((rc = check_buffer(ctx, y, y_need, err, cap, name)) != TM_HIP_OK) {
-        return rc;
+    tm_hip_buffer *bufs[3] = {w, x, y};
+    const size_t needs[3] = {w_need, x_need, y_need};
+    static const char *const suffix[3] = {"weights", "x", "y"};
+    for (int i = 0; i < 3; ++i) {
+        const tm_hip_buffer *b = bufs[i];
+        if (b == nullptr || b->owner != ctx || needs[i] == 0 || b->len < needs[i]) {
+            char name[64]; // only the refusal path formats the operand name
+            snprintf(name, sizeof name, "%s.%s", what, suffix[i]);
+            return check_buffer(ctx, bufs[i], needs[i], err, cap, name);
+        }
     }
     if (w->alloc->packed && (w->alloc->prows != rows || w->alloc->pcols != cols)) {
         return fail(err, cap, TM_HIP_ERR_UNSUPPORTED,
@@ -944,7 +978,7 @@ int tm_hip_end_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {
     std::vector<Op> ops;
     ops.swap(ctx->group_ops);
     // An empty group still commits once, like an empty command buffer.
-    return commit_ops(ctx, ops, "group", err, err_cap);
+    return commit_ops(ctx, ops, "group", "group", err, err_cap);
 }
 
 int tm_hip_abort_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {
@@ -988,13 +1022,8 @@ static int product_list(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_
     op.x_off = x_off;
     op.y_off = y_off;
     op.packed = w->alloc->packed;
-    char label[kProfileName];
-    if (ctx->profiling.load(std::memory_order_relaxed)) {
-        snprintf(label, sizeof label, "%s:%ux%u", what, rows, cols);
-    } else {
-        snprintf(label, sizeof label, "%s", what);
-    }
-    return submit(ctx, op, label, err, err_cap);
+    op.shape_label = true; // native/metal/tm_metal.m:1008-1015
+    return submit(ctx, op, what, err, err_cap);
 }
 
 int tm_hip_q8_0_gemv(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
@@ -1184,7 +1213,7 @@ int tm_hip_q8_0_pack(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t rows, uint32_t 
     op.rows = rows;
     op.cols = cols;
     std::vector<Op> one(1, op);
-    rc = commit_ops(ctx, one, "q8_0_pack", err, err_cap);
+    rc = commit_ops(ctx, one, "q8_0_pack", "q8_0_pack", err, err_cap);
     // The handle now names the sealed copy; the raw bytes stay leased by the
     // commit above until the pack kernel has read them.
     Alloc *old = w->alloc;

@@ -269,7 +269,8 @@ class HipContext {
     explicit HipContext(std::shared_ptr<ContextInner> inner) : inner_(std::move(inner)) {}
     template <class F> void operate(const char *what, F f) const {
         std::lock_guard<std::mutex> g(inner_->lock);
-        char err[ERR_CAP] = {0};
+        char err[ERR_CAP];
+        err[0] = '\0';
         int code = f(err);
         if (code != 0) {
             throw hip_error(code, err, what);

@@ -25,14 +25,20 @@ struct tmh_product {
 struct tmh_timing {
     double wall_ms;     // host clock around the timed steps, fence to fence
     double gpu_ms;      // sum of the commits' HIP-event times on the context's stream
+    double host_ms;     // host time spent issuing the timed steps (before the final fence)
     uint64_t launches;  // kernel launches issued by the timed steps
     uint64_t commits;
 };
 
-static void issue(const HipContext &gpu, const tmh_product *p, uint32_t n) {
+struct Bound {
+    HipBuffer w, x, y;
+};
+
+static void issue(const HipContext &gpu, const tmh_product *p, const std::vector<Bound> &b,
+                  uint32_t n) {
     for (uint32_t i = 0; i < n; ++i) {
         const tmh_product &q = p[i];
-        HipBuffer w = gpu.borrow_buffer(q.w), x = gpu.borrow_buffer(q.x), y = gpu.borrow_buffer(q.y);
+        const HipBuffer &w = b[i].w, &x = b[i].x, &y = b[i].y;
         switch (q.kind) {
         case TMH_GEMV: gpu.q8_0_gemv(w, x, y, q.rows, q.cols); break;
         case TMH_GEMM: gpu.q8_0_gemm(w, x, y, q.rows, q.cols, q.batch, 0, 0); break;
@@ -48,11 +54,17 @@ int tmh_run_steps(tm_hip_ctx *ctx, const tmh_product *products, uint32_t n, uint
                   uint32_t steps, int grouped, tmh_timing *out, char *err, size_t err_cap) {
     try {
         HipContext gpu = HipContext::borrow(ctx);
+        std::vector<Bound> bound;
+        bound.reserve(n);
+        for (uint32_t i = 0; i < n; ++i) {
+            bound.push_back(Bound{gpu.borrow_buffer(products[i].w), gpu.borrow_buffer(products[i].x),
+                                  gpu.borrow_buffer(products[i].y)});
+        }
         auto one_step = [&]() {
             if (grouped) {
-                gpu.grouped([&]() { issue(gpu, products, n); });
+                gpu.grouped([&]() { issue(gpu, products, bound, n); });
             } else {
-                issue(gpu, products, n);
+                issue(gpu, products, bound, n);
             }
         };
         for (uint32_t s = 0; s < warmup; ++s) {
@@ -66,10 +78,12 @@ int tmh_run_steps(tm_hip_ctx *ctx, const tmh_product *products, uint32_t n, uint
         for (uint32_t s = 0; s < steps; ++s) {
             one_step();
         }
+        const auto th = std::chrono::steady_clock::now();
         gpu.fence();
         const auto t1 = std::chrono::steady_clock::now();
         if (out != nullptr) {
             out->wall_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+            out->host_ms = std::chrono::duration<double, std::milli>(th - t0).count();
             out->gpu_ms = (double)(gpu.gpu_nanos_total() - nanos0) / 1e6;
             out->launches = gpu.kernel_launches() - launches0;
             out->commits = gpu.committed_dispatches() - commits0;
