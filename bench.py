@@ -182,6 +182,142 @@ def bench_gemm(host, ctx, steps, warmup):
     return out
 
 
+def _weights_pool(ctx, shapes, copies, seed_base):
+    """`copies` distinct sealed weight sets of `shapes` [(name, rows, cols)]."""
+    pool = []
+    for c in range(copies):
+        for name, rows, cols in shapes:
+            raw = S.make_weights(rows, cols, seed_base + 17 * c + len(pool))
+            pool.append((name, rows, cols, H.Matrix.load(ctx, raw, cols, rows)))
+    return pool
+
+
+def bench_gemma(host, ctx, steps, warmup):
+    """BASELINE config 3: Gemma-3-1B shapes (hidden 1152 = 36 blocks per row,
+    FFN 6912, lm_head 262144 x 1152). M = 1: a 26-layer FFN + lm_head step
+    (79 GEMVs, 981 MB of weights) in one group. M = 512: the three FFN shapes
+    in one group, and the lm_head on its own."""
+    out = {"workload": "Gemma-3-1B shapes (BASELINE config 3)"}
+    layers = 26
+    ffn = [s for s in S.GEMMA3_1B if s[0] != "lm_head"]
+    head = [s for s in S.GEMMA3_1B if s[0] == "lm_head"][0]
+    pool = _weights_pool(ctx, ffn, layers, 3000) + _weights_pool(ctx, [head], 1, 3999)
+    products, keep = [], []
+    for name, rows, cols, m in pool:
+        xb = ctx.buffer(cols * 4)
+        xb.upload(0, S.make_activations(cols, rows))
+        yb = ctx.buffer(rows * 4)
+        keep += [xb, yb]
+        products.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, 1, TMH_GEMV))
+    step_bytes = sum(S.gemv_bytes(p.rows, p.cols) for p in products)
+    t = run_steps(host, ctx, products, warmup, steps, grouped=True)
+    us = t.wall_ms / steps * 1e3
+    out["gemv_step"] = {"products": len(products), "algorithmic_bytes": step_bytes, "us": us,
+                        "gbs": step_bytes / us / 1e3, "pct_of_hbm_peak": step_bytes / us / 1e3 / 80.0,
+                        "launch_us": t.gpu_ms * 1e3 / t.launches}
+    head_p = products[-1]
+    t = run_steps(host, ctx, [head_p], warmup, steps, grouped=False)
+    us = t.gpu_ms / steps * 1e3
+    hb = S.gemv_bytes(head_p.rows, head_p.cols)
+    out["lm_head_gemv"] = {"rows": head_p.rows, "cols": head_p.cols, "algorithmic_bytes": hb,
+                           "us": us, "gbs": hb / us / 1e3, "pct_of_hbm_peak": hb / us / 1e3 / 80.0}
+    # M = 512
+    M = 512
+    gsteps, gwarm = max(5, steps // 20), max(2, warmup // 20)
+    gp = []
+    for name, rows, cols, m in pool[:3]:
+        xb = ctx.buffer(M * cols * 4)
+        xb.upload(0, S.make_activations(M * cols, rows + 1))
+        yb = ctx.buffer(M * rows * 4)
+        keep += [xb, yb]
+        gp.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA))
+    flops = sum(2.0 * M * p.rows * p.cols for p in gp)
+    t = run_steps(host, ctx, gp, gwarm, gsteps, grouped=True)
+    us = t.gpu_ms / gsteps * 1e3
+    out["ffn_gemm_m512"] = {"flops": flops, "us": us, "tflops": flops / us / 1e6,
+                            "frac_of_f32_mfma_peak": flops / us / 1e6 / MFMA_F32_PEAK_TFLOPS}
+    name, rows, cols, m = pool[-1]
+    xb = ctx.buffer(M * cols * 4)
+    xb.upload(0, S.make_activations(M * cols, 7))
+    yb = ctx.buffer(M * rows * 4)
+    keep += [xb, yb]
+    flops = 2.0 * M * rows * cols
+    t = run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA)],
+                  2, 5, grouped=False)
+    us = t.gpu_ms / 5 * 1e3
+    out["lm_head_gemm_m512"] = {"flops": flops, "us": us, "tflops": flops / us / 1e6,
+                                "frac_of_f32_mfma_peak": flops / us / 1e6 / MFMA_F32_PEAK_TFLOPS}
+    for b in keep:
+        b.free()
+    for _, _, _, m in pool:
+        m.buf.free()
+    return out
+
+
+def bench_sweep(host, ctx, steps, warmup):
+    """BASELINE config 4: 2B-class shapes (hidden 2048, FFN 6144), M in
+    {1, 8, 64, 512, 2048}, f32 activations and the int8-activation profile.
+    Each point runs over 20 distinct weight copies per shape (535 MB in all),
+    so small M is measured against HBM, not against the caches."""
+    copies = 20
+    pool = _weights_pool(ctx, list(S.SWEEP_2B), copies, 4000)
+    wbytes = sum(S.q8_0_bytes(r, c) for _, r, c, _ in pool)
+    out = {"workload": "2B-class sweep (BASELINE config 4)", "weight_copies": copies,
+           "weights_bytes": wbytes, "points": []}
+    maxM = 2048
+    maxc = max(c for _, _, c, _ in pool)
+    maxr = max(r for _, r, _, _ in pool)
+    xb = ctx.buffer(maxM * maxc * 4)
+    xb.upload(0, S.make_activations(maxM * maxc, 99))
+    widths = sorted({c for _, _, c, _ in pool})
+    xqs = {c: ctx.buffer(maxM * (c + c // 32 * 4)) for c in widths}
+    ys = [ctx.buffer(maxM * maxr * 4) for _ in pool]
+    for M in (1, 8, 64, 512, 2048):
+        n = max(3, steps // (40 if M < 64 else 200 if M < 512 else 1000))
+        w = max(2, n // 5)
+        flops = sum(2.0 * M * r * c for _, r, c, _ in pool)
+        abytes = sum(S.q8_0_bytes(r, c) + 4 * M * c + 4 * M * r for _, r, c, _ in pool)
+        paths = []
+        if M == 1:
+            paths.append(("f32 gemv", TMH_GEMV, M))
+        if 1 < M <= 32:
+            paths.append(("f32 gemm (gemv arithmetic)", TMH_GEMM, M))
+        if 2 <= M <= 512:
+            paths.append(("f32 mfma", TMH_GEMM_MMA, M))
+        if M > 512:
+            paths.append(("f32 mfma (slices of 512)", TMH_GEMM_MMA, 512))
+        paths.append(("i8 mfma", TMH_GEMM_I8, M))
+        for label, kind, mb in paths:
+            prods = []
+            slices = (M + mb - 1) // mb
+            quant_us = None
+            if kind == TMH_GEMM_I8:
+                # activations are quantized once per distinct width (timed apart)
+                qprods = [tmh_product(None, xb.raw, xqs[c].raw, 1, c, M, TMH_QUANT) for c in widths]
+                tq = run_steps(host, ctx, qprods, 1, 3, grouped=True)
+                quant_us = tq.gpu_ms / 3 * 1e3
+                for (name, r, c, m), yb in zip(pool, ys):
+                    prods.append(tmh_product(m.buf.raw, xqs[c].raw, yb.raw, r, c, M, kind))
+            else:
+                for (name, r, c, m), yb in zip(pool, ys):
+                    for _ in range(slices):
+                        prods.append(tmh_product(m.buf.raw, xb.raw, yb.raw, r, c, mb, kind))
+            t = run_steps(host, ctx, prods, w, n, grouped=True)
+            us = t.gpu_ms / n * 1e3
+            out["points"].append({
+                "M": M, "path": label, "us": us, "launches": t.launches / n,
+                "gbs": abytes / us / 1e3, "pct_of_hbm_peak": abytes / us / 1e3 / 80.0,
+                "tflops": flops / us / 1e6,
+                "frac_of_mfma_peak": flops / us / 1e6 / (MFMA_I8_PEAK_TOPS if kind == TMH_GEMM_I8
+                                                        else MFMA_F32_PEAK_TFLOPS),
+                "quantize_act_us": quant_us})
+    for b in [xb] + list(xqs.values()) + ys:
+        b.free()
+    for _, _, _, m in pool:
+        m.buf.free()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -192,6 +328,9 @@ def main():
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--ungrouped", action="store_true",
                     help="one commit per GEMV instead of one group per step")
+    ap.add_argument("--workload", choices=["decode", "gemma", "sweep"], default="decode",
+                    help="decode (default, the headline line); gemma / sweep print the "
+                         "BASELINE config 3 / 4 measurements as one JSON object")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one MI355X: this path runs on a single GPU "
@@ -201,6 +340,11 @@ def main():
         raise SystemExit(f"bench.py needs an MI355X: {p.info}")
     host = load_host()
     ctx = H.HipContext.open()
+    if args.workload != "decode":
+        fn = bench_gemma if args.workload == "gemma" else bench_sweep
+        print(json.dumps(fn(host, ctx, args.steps, args.warmup)), flush=True)
+        ctx.close()
+        return
 
     products, keep, host_side = build_decode_step(ctx, keep_host=args.cpu_seconds > 0)
     step_bytes = sum(S.gemv_bytes(pr.rows, pr.cols) for pr in products)

@@ -141,7 +141,8 @@ def test_in_flight_bytes_stay_visible_until_completion(ctx):
     assert ctx.allocated_bytes() == 0
     leased = ctx.in_flight_bytes()
     assert leased >= total, f"dropped-but-leased buffers must remain visible: {leased}"
-    assert ctx.live_gpu_bytes() >= leased
+    live = ctx.live_gpu_bytes()  # leases only shrink as commits complete
+    assert live >= ctx.in_flight_bytes()
     ctx.fence()
     assert ctx.in_flight_bytes() == 0, "leases release at completion"
 

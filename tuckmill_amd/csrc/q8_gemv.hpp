@@ -147,7 +147,150 @@ __device__ __forceinline__ void reduce_store(const float (&acc)[R], float *y, ui
     }
 }
 
-template <int L, int R, int TB, bool XA>
+// The decode path: one token, sealed weights, at least one whole 1024-column
+// chunk per row. TAILMASK = cols % 1024 selects the tail pieces at compile time
+// (bit 512/256/128/64/32 -> a piece of 8/4/2/1/1 quants per lane).
+//
+// Per pass of R rows the arithmetic is: acc = 0; tail pieces in descending
+// width; whole chunks in ascending order; reduce. The loads run one step ahead
+// of the multiplies: while chunk c is multiplied the R weight loads of chunk
+// c+1 are in flight, and during the last chunk of a pass the tail pieces and
+// the first chunk of the next pass are. Tail pieces come first in a pass so
+// that their registers are free again before the next prefetch is issued.
+// With a single chunk per row this lane's activations never leave registers.
+template <int R, bool XA, int TAILMASK>
+__device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const float *x, float *y,
+                                            uint32_t cols, uint32_t row_first, uint32_t row_end,
+                                            uint32_t lane) {
+    constexpr bool T8 = (TAILMASK & 512) != 0, T4 = (TAILMASK & 256) != 0;
+    constexpr bool T2 = (TAILMASK & 128) != 0, T1 = (TAILMASK & 64) != 0;
+    constexpr bool TH = (TAILMASK & 32) != 0;
+    const uint32_t full = cols >> 10;
+    const uint32_t c8 = full << 10;
+    const uint32_t c4 = c8 + (T8 ? 512u : 0u);
+    const uint32_t c2 = c4 + (T4 ? 256u : 0u);
+    const uint32_t c1 = c2 + (T2 ? 128u : 0u);
+    const uint32_t ch = c1 + (T1 ? 64u : 0u);
+    const bool low = lane < 32u;
+
+    // activations of the tail pieces: loop invariant, kept in registers
+    float x8[8], x4[4], x2[2], x1[1], xh[1];
+    if constexpr (T8) load_x<8, XA>(x + c8 + lane * 8u, x8);
+    if constexpr (T4) load_x<4, XA>(x + c4 + lane * 4u, x4);
+    if constexpr (T2) load_x<2, XA>(x + c2 + lane * 2u, x2);
+    if constexpr (T1) load_x<1, XA>(x + c1 + lane, x1);
+    if constexpr (TH) load_x<1, XA>(x + ch + (low ? lane : 0u), xh);
+    float xv[16];
+    if (full == 1u) {
+        load_x<16, XA>(x + lane * 16u, xv);
+    }
+
+    uint32_t q8[R][2], q4[R][1], q2[R][1], q1[R][1], qh[R][1];
+    uint32_t s8[R], s4[R], s2[R], s1[R], sh[R];
+    auto load_tails = [&](uint32_t r0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+            if constexpr (T8) {
+                wv.template load_quants<8, true>(row, c8 + lane * 8u, q8[r]);
+                s8[r] = wv.scale_bits(row, (c8 + lane * 8u) >> 5);
+            }
+            if constexpr (T4) {
+                wv.template load_quants<4, true>(row, c4 + lane * 4u, q4[r]);
+                s4[r] = wv.scale_bits(row, (c4 + lane * 4u) >> 5);
+            }
+            if constexpr (T2) {
+                wv.template load_quants<2, true>(row, c2 + lane * 2u, q2[r]);
+                s2[r] = wv.scale_bits(row, (c2 + lane * 2u) >> 5);
+            }
+            if constexpr (T1) {
+                wv.template load_quants<1, true>(row, c1 + lane, q1[r]);
+                s1[r] = wv.scale_bits(row, (c1 + lane) >> 5);
+            }
+            if constexpr (TH) {
+                wv.template load_quants<1, true>(row, ch + (low ? lane : 0u), qh[r]);
+                sh[r] = wv.scale_bits(row, ch >> 5);
+            }
+        }
+    };
+    uint32_t q[R][4], sb[R];
+    auto load_chunk = [&](uint32_t r0, uint32_t c, uint32_t (&qq)[R][4], uint32_t (&ss)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+            wv.template load_quants<16, true>(row, (c << 10) + lane * 16u, qq[r]);
+            ss[r] = wv.scale_bits(row, (c << 5) + (lane >> 1));
+        }
+    };
+
+    // One flat sequence of (pass, chunk) steps; the tail pieces of a pass
+    // travel with its first chunk.
+    const uint32_t nsteps = ((row_end - row_first + R - 1) / R) * full;
+    uint32_t r0 = row_first, c = 0;
+    if constexpr (TAILMASK != 0) {
+        load_tails(r0);
+    }
+    load_chunk(r0, 0, q, sb);
+    float acc[R];
+    for (uint32_t step = 0; step < nsteps; ++step) {
+        if (c == 0u) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float a = 0.0f;
+                if constexpr (T8) a = __builtin_fmaf(f16_bits_to_f32(s8[r]), piece_dot<8>(q8[r], x8), a);
+                if constexpr (T4) a = __builtin_fmaf(f16_bits_to_f32(s4[r]), piece_dot<4>(q4[r], x4), a);
+                if constexpr (T2) a = __builtin_fmaf(f16_bits_to_f32(s2[r]), piece_dot<2>(q2[r], x2), a);
+                if constexpr (T1) a = __builtin_fmaf(f16_bits_to_f32(s1[r]), piece_dot<1>(q1[r], x1), a);
+                if constexpr (TH) {
+                    const float d = low ? f16_bits_to_f32(sh[r]) : 0.0f;
+                    const float sd = low ? piece_dot<1>(qh[r], xh) : 0.0f;
+                    a = __builtin_fmaf(d, sd, a);
+                }
+                acc[r] = a;
+            }
+        }
+        if (full > 1u) {
+            load_x<16, XA>(x + (c << 10) + lane * 16u, xv);
+        }
+        uint32_t cn = c + 1u, rn = r0;
+        if (cn == full) {
+            cn = 0;
+            rn = r0 + R;
+        }
+        uint32_t qn[R][4], sn[R];
+        if (step + 1u < nsteps) {
+            if constexpr (TAILMASK != 0) {
+                if (cn == 0u) {
+                    load_tails(rn); // the current pass consumed its tail pieces at c == 0
+                }
+            }
+            load_chunk(rn, cn, qn, sn);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            acc[r] = __builtin_fmaf(f16_bits_to_f32(sb[r]), piece_dot<16>(q[r], xv), acc[r]);
+        }
+        if (cn == 0u) {
+            reduce_store<R>(acc, y, r0, row_end, lane, true);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                q[r][i] = qn[r][i];
+            }
+            sb[r] = sn[r];
+        }
+        c = cn;
+        r0 = rn;
+    }
+}
+
+// TAILS selects which column tails get the streaming decode path: 0 = none
+// (cols a multiple of 1024 only; fewest registers, the Qwen3 shapes), 1 = also
+// cols % 1024 == 128 and == 768 (the Gemma-3-1B shapes). The host picks the
+// smallest set that covers the products of a launch.
+template <int L, int R, int TB, bool XA, int TAILS = 0>
 __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -184,71 +327,25 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
     constexpr bool NT = TB == 1;
 
     if constexpr (TB == 1 && L == PACKED) {
-        if ((cols & 1023u) == 0u) {
-            // Whole 1024-column chunks only (every Qwen3 projection): the
-            // (row pass, chunk) steps form one software-pipelined sequence in
-            // which the 8 weight loads of step s+1 are in flight while step s
-            // is multiplied. With a single chunk this lane's 16 activations
-            // stay in registers for the whole tile. Same per-row arithmetic
-            // as the general path below: chunks in order, acc from 0.
-            const uint32_t nchunk = cols >> 10;
-            const uint32_t nsteps = ((row_end - row_first + R - 1) / R) * nchunk;
-            float xv[16];
-            if (nchunk == 1u) {
-                load_x<16, XA>(x + lane * 16u, xv);
+        // One token, sealed weights: the decode path, software-pipelined (see
+        // stream_rows). Column tails seen in practice are instantiated; other
+        // shapes take the general path below. Same arithmetic either way.
+        if (full >= 1u) {
+            const uint32_t tail = cols & 1023u;
+            if (tail == 0u) {
+                stream_rows<R, XA, 0>(wv, x, y, cols, row_first, row_end, lane);
+                return;
             }
-            uint32_t q[R][4], sb[R];
-            auto load_step = [&](uint32_t r0, uint32_t c, uint32_t (&qq)[R][4], uint32_t (&ss)[R]) {
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
-                    wv.template load_quants<16, true>(row, (c << 10) + lane * 16u, qq[r]);
-                    ss[r] = wv.scale_bits(row, (c << 5) + (lane >> 1));
+            if constexpr (TAILS >= 1) {
+                if (tail == 128u) { // hidden 1152 (Gemma-3-1B)
+                    stream_rows<R, XA, 128>(wv, x, y, cols, row_first, row_end, lane);
+                    return;
                 }
-            };
-            uint32_t r0 = row_first, c = 0;
-            load_step(r0, c, q, sb);
-            float acc[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                acc[r] = 0.0f;
+                if (tail == 768u) { // FFN 6912 (Gemma-3-1B); half the rows per pass
+                    stream_rows<R / 2, XA, 768>(wv, x, y, cols, row_first, row_end, lane);
+                    return;
+                }
             }
-            for (uint32_t step = 0; step < nsteps; ++step) {
-                if (nchunk > 1u) {
-                    load_x<16, XA>(x + (c << 10) + lane * 16u, xv);
-                }
-                uint32_t cn = c + 1u, rn = r0;
-                if (cn == nchunk) {
-                    cn = 0;
-                    rn = r0 + R;
-                }
-                uint32_t qn[R][4], sn[R];
-                if (step + 1u < nsteps) {
-                    load_step(rn, cn, qn, sn);
-                }
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    acc[r] = __builtin_fmaf(f16_bits_to_f32(sb[r]), piece_dot<16>(q[r], xv), acc[r]);
-                }
-                if (cn == 0u) {
-                    reduce_store<R>(acc, y, r0, row_end, lane, true);
-#pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        acc[r] = 0.0f;
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        q[r][i] = qn[r][i];
-                    }
-                    sb[r] = sn[r];
-                }
-                c = cn;
-                r0 = rn;
-            }
-            return;
         }
     }
 
@@ -272,9 +369,8 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
                     acc[r][t] = 0.0f;
                 }
             }
-            for (uint32_t c = 0; c < full; ++c) {
-                chunk<L, R, TB, 16, XA, NT>(wv, x, cols, row, tok, c << 10, lane, true, acc);
-            }
+            // Column order is part of the arithmetic: tail pieces first, then
+            // the whole 1024-column chunks in ascending order.
             uint32_t col0 = tail0;
             if (cols & 512u) {
                 chunk<L, R, TB, 8, XA, NT>(wv, x, cols, row, tok, col0, lane, true, acc);
@@ -294,6 +390,9 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
             }
             if (cols & 32u) {
                 chunk<L, R, TB, 1, XA, NT>(wv, x, cols, row, tok, col0, lane, lane < 32u, acc);
+            }
+            for (uint32_t c = 0; c < full; ++c) {
+                chunk<L, R, TB, 16, XA, NT>(wv, x, cols, row, tok, c << 10, lane, true, acc);
             }
 #pragma unroll
             for (int t = 0; t < TB; ++t) {

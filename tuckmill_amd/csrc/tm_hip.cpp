@@ -286,10 +286,17 @@ uint32_t pick_rows_per_tile(uint32_t rows, uint32_t cols, uint32_t batch, int R)
 }
 
 template <int L, int R, int TB, bool XA>
-hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args) {
+hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args, bool tails) {
     const uint32_t groups = (args.total_tiles + 3u) / 4u;
-    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA>), dim3(groups), dim3(256), 0, ctx->stream, stop,
-              args);
+    if constexpr (L == q8::PACKED && TB == 1) {
+        if (tails) {
+            Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1>), dim3(groups), dim3(256), 0,
+                      ctx->stream, stop, args);
+            return hipGetLastError();
+        }
+    }
+    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 0>), dim3(groups), dim3(256), 0, ctx->stream,
+              stop, args);
     return hipGetLastError();
 }
 
@@ -320,7 +327,10 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<
     args.pad[0] = args.pad[1] = 0;
     const int R = key.tb == 1 ? kGemvR1 : kGemvR4;
     uint32_t tiles = 0;
+    bool tails = false; // some product has a column tail with a streaming path of its own
     for (const Op *op : ops) {
+        const uint32_t tail = op->cols & 1023u;
+        tails = tails || (op->cols >= 1024u && (tail == 128u || tail == 768u));
         q8::GemvDesc &d = args.d[args.n++];
         d.w = (const uint8_t *)op->a[0]->ptr;
         d.x = (const float *)op->a[1]->ptr + op->x_off;
@@ -337,7 +347,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<
 #define TM_GEMV_CASE(P, T, A)                                                                \
     if (key.packed == (P) && key.tb == (T) && key.xalign == (A)) {                           \
         return launch_gemv<(P) ? q8::PACKED : q8::RAW, (T) == 1 ? kGemvR1 : kGemvR4, T, A>(  \
-            ctx, stop, args);                                                                \
+            ctx, stop, args, tails);                                                         \
     }
     TM_GEMV_CASE(true, 1, true)
     TM_GEMV_CASE(true, 1, false)
@@ -677,7 +687,7 @@ tm_hip_ctx *tm_hip_create(char *err, size_t err_cap) {
     }
     // Fail at creation, not at first use, when the device code is missing.
     hipFuncAttributes attr;
-    e = hipFuncGetAttributes(&attr, (const void *)q8::gemv_list_kernel<q8::PACKED, kGemvR1, 1, true>);
+    e = hipFuncGetAttributes(&attr, (const void *)q8::gemv_list_kernel<q8::PACKED, kGemvR1, 1, true, 0>);
     if (e != hipSuccess) {
         fail(err, err_cap, TM_HIP_ERR_SOURCE, "kernels for this device are missing: %s",
              hipGetErrorString(e));
