@@ -35,6 +35,10 @@ from tuckmill_amd import synth as S  # noqa: E402
 HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E bandwidth
 MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X published dense f32 matrix rate
 MFMA_I8_PEAK_TOPS = 5000.0
+# HBM bytes per launch of the decode step's GEMV list kernel, from the FETCH_SIZE and
+# WRITE_SIZE counter runs summarised in profiles/gemv_list_kernel__decode_step__pmc_traffic.txt
+# (fetch counter x 2.000 + write counter x 1.000, factors from a plain copy kernel).
+DECODE_STEP_TRAFFIC_BYTES = 644.69e6
 
 
 class tmh_product(ctypes.Structure):
@@ -318,6 +322,29 @@ def bench_sweep(host, ctx, steps, warmup):
     return out
 
 
+def run_traffic(host, ctx):
+    """A short, fixed sequence for hardware-counter runs (rocprofv3 --pmc):
+    a plain f32 copy of known size (the calibration kernel: 256 MiB read,
+    256 MiB written per dispatch), five decode steps and three M = 512 GEMM
+    groups. Prints the algorithmic bytes of each so that the counter values
+    per dispatch can be set beside them."""
+    n = 64 << 20  # f32 elements
+    src, dst = ctx.buffer(n * 4), ctx.buffer(n * 4)
+    for _ in range(3):
+        ctx.copy_f32(src, 0, dst, 0, n)
+    ctx.fence()
+    products, keep, _ = build_decode_step(ctx, keep_host=False)
+    step_bytes = sum(S.gemv_bytes(pr.rows, pr.cols) for pr in products)
+    run_steps(host, ctx, products, 0, 5, grouped=True)
+    g = bench_gemm(host, ctx, 3, 0)
+    print(json.dumps({"copy_f32_kernel": {"read_bytes": n * 4, "written_bytes": n * 4},
+                      "gemv_list_kernel": {"algorithmic_bytes_per_dispatch": step_bytes,
+                                           "weights_bytes": sum(S.q8_0_bytes(p.rows, p.cols)
+                                                                for p in products)},
+                      "gemm_mma_kernel": {"flops_per_group_dispatch": g["flops_per_step"]}}),
+          flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -328,7 +355,7 @@ def main():
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--ungrouped", action="store_true",
                     help="one commit per GEMV instead of one group per step")
-    ap.add_argument("--workload", choices=["decode", "gemma", "sweep"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "gemma", "sweep", "traffic"], default="decode",
                     help="decode (default, the headline line); gemma / sweep print the "
                          "BASELINE config 3 / 4 measurements as one JSON object")
     args = ap.parse_args()
@@ -340,6 +367,10 @@ def main():
         raise SystemExit(f"bench.py needs an MI355X: {p.info}")
     host = load_host()
     ctx = H.HipContext.open()
+    if args.workload == "traffic":
+        run_traffic(host, ctx)
+        ctx.close()
+        return
     if args.workload != "decode":
         fn = bench_gemma if args.workload == "gemma" else bench_sweep
         print(json.dumps(fn(host, ctx, args.steps, args.warmup)), flush=True)
@@ -372,7 +403,8 @@ def main():
         },
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": DECODE_STEP_TRAFFIC_BYTES if launches_per_step == 1.0 else None,
             "kernel": "q8::gemv_list_kernel",
             "launches_per_step": launches_per_step,
             "avg_launch_us": launch_us,
