@@ -274,7 +274,7 @@ def bench_sweep(host, ctx, steps, warmup):
     xb = ctx.buffer(maxM * maxc * 4)
     xb.upload(0, S.make_activations(maxM * maxc, 99))
     widths = sorted({c for _, _, c, _ in pool})
-    xqs = {c: ctx.buffer(maxM * (c + c // 32 * 4)) for c in widths}
+    xqs = {c: ctx.buffer(H.xq_bytes(c, maxM)) for c in widths}
     ys = [ctx.buffer(maxM * maxr * 4) for _ in pool]
     for M in (1, 8, 64, 512, 2048):
         n = max(3, steps // (40 if M < 64 else 200 if M < 512 else 1000))

@@ -179,11 +179,12 @@ int tm_hip_q8_0_pack(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t rows, uint32_t 
 
 /* Quantize `batch` rows of `cols` f32 activations (at element offset x_off
  * of `x`) to Q8_0 with the rule of crates/tuckcore/src/tensor.rs:184-206.
- * `xq` receives batch*cols int8 quants (token-major) followed by
- * batch*(cols/32) f32 scales (token-major; each the f32 value of the
- * f16-rounded scale): batch * (cols + cols/32*4) bytes in all.
- * Device form of the `llama-cpu` numerical profile's first step
- * (crates/tuckcore/src/forward.rs:783-793). */
+ * `xq` receives batch*cols int8 quants (token-major) followed by the f32
+ * scales (each the f32 value of the f16-rounded scale) stored block-major as
+ * [cols/32][bpad], bpad = batch rounded up to a multiple of 4; entries of
+ * the padding tokens are not written. Bytes needed:
+ * batch*cols + (cols/32)*bpad*4. Device form of the `llama-cpu` numerical
+ * profile's first step (crates/tuckcore/src/forward.rs:783-793). */
 int tm_hip_q8_0_quantize_act(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *xq, uint32_t cols,
                              uint32_t batch, uint32_t x_off, char *err, size_t err_cap);
 

@@ -61,15 +61,16 @@ def test_hip_path_reproduces_the_golden_products(i, packed):
         ctx.fence()
         got = yb.download_f32(0, batch * rows).reshape(batch, rows)
         assert np.max(np.abs(got - want)) / scale <= 1e-5
-    blocks = cols // 32
-    xq = ctx.buffer(batch * (cols + blocks * 4))
+    from tuckmill_amd import hip as H
+
+    xq = ctx.buffer(H.xq_bytes(cols, batch))
     yb = ctx.buffer(batch * rows * 4)
     ctx.q8_0_quantize_act(xb, xq, cols, batch)
     ctx.q8_0_gemm_i8(wb, xq, yb, rows, cols, batch)
     ctx.fence()
-    raw = xq.download(0, batch * (cols + blocks * 4))
-    assert np.array_equal(raw[:batch * cols].view(np.int8).reshape(-1, 32), G[f"case{i}_xq"])
-    assert np.array_equal(raw[batch * cols:].view(np.uint32), G[f"case{i}_xd"].view(np.uint32))
+    qs, ds = H.xq_split(xq.download(0, H.xq_bytes(cols, batch)), cols, batch)
+    assert np.array_equal(qs.reshape(-1, 32), G[f"case{i}_xq"])
+    assert np.array_equal(ds.reshape(-1).view(np.uint32), G[f"case{i}_xd"].view(np.uint32))
     got = yb.download_f32(0, batch * rows).reshape(batch, rows)
     assert np.array_equal(got.view(np.uint32), G[f"case{i}_y_q8"].view(np.uint32))
     ctx.close()

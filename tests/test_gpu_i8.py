@@ -30,13 +30,10 @@ def quantize_on_gpu(ctx, x, cols, batch, x_off=0):
     xs = np.zeros(x_off + batch * cols, np.float32)
     xs[x_off:] = x
     xb = upload_new(ctx, xs)
-    blocks = cols // 32
-    xq = ctx.buffer(batch * (cols + blocks * 4))
+    xq = ctx.buffer(H.xq_bytes(cols, batch))
     ctx.q8_0_quantize_act(xb, xq, cols, batch, x_off)
     ctx.fence()
-    raw = xq.download(0, batch * (cols + blocks * 4))
-    qs = raw[:batch * cols].view(np.int8).reshape(batch, blocks, 32)
-    ds = raw[batch * cols:].view(np.float32).reshape(batch, blocks)
+    qs, ds = H.xq_split(xq.download(0, H.xq_bytes(cols, batch)), cols, batch)
     return xq, qs, ds
 
 
@@ -64,7 +61,8 @@ def test_activation_quantizer_is_bit_exact(ctx, cols, batch, scale):
 
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("rows,cols,batch", [(16, 32, 1), (40, 64, 3), (100, 96, 77),
-                                             (1024, 1024, 16), (333, 1152, 40), (2048, 2048, 8)])
+                                             (1024, 1024, 16), (333, 1152, 40), (2048, 2048, 8),
+                                             (70, 1024, 17), (48, 160, 33), (65, 2048, 130)])
 def test_gemm_i8_block_dots_and_result_are_bit_exact(ctx, rows, cols, batch, packed):
     blocks = cols // 32
     w = S.make_weights(rows, cols, rows + cols)
@@ -119,3 +117,25 @@ def test_i8_argument_refusals(ctx):
     with pytest.raises(H.TuckmillError) as e:
         ctx.q8_0_gemm_i8(b, b, b, 4, 32, 1, 0, ctx.buffer(8))
     assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS
+
+
+def test_independent_i8_products_in_a_group_share_one_launch(ctx):
+    cols, batch = 1024, 48
+    x = S.make_activations(batch * cols, 3)
+    xb = upload_new(ctx, x)
+    xq = ctx.buffer(H.xq_bytes(cols, batch))
+    mats = []
+    for i, rows in enumerate((512, 256, 256)):
+        w = S.make_weights(rows, cols, 70 + i)
+        mats.append((w, rows, weights_buffer(ctx, w, rows, cols, True), ctx.buffer(batch * rows * 4)))
+    launches = ctx.kernel_launches()
+    ctx.begin_group()
+    ctx.q8_0_quantize_act(xb, xq, cols, batch)
+    for w, rows, wb, yb in mats:
+        ctx.q8_0_gemm_i8(wb, xq, yb, rows, cols, batch)
+    ctx.end_group()
+    assert ctx.kernel_launches() == launches + 2  # the quantizer, then one list launch
+    ctx.fence()
+    for w, rows, wb, yb in mats:
+        want = O.gemm_q8_0_q8_0(w, rows, cols, x, batch, threads=4)
+        assert np.array_equal(bits(yb.download_f32(0, batch * rows)), bits(want.reshape(-1)))

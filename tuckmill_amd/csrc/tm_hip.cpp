@@ -241,20 +241,25 @@ int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
 
 // Products that may share a launch agree on this key.
 struct GemvKey {
-    bool mma;     // MFMA list kernel instead of the GEMV list kernel
+    OpKind kind;  // OP_GEMV_LIST, OP_MMA or OP_I8: which list kernel
     bool packed;
-    int tb;       // GEMV list kernel: tokens per pass (1 or 4); MFMA: tile/split code
-    bool xalign;
+    int tb;       // GEMV: tokens per pass (1 or 4); MFMA f32: tile/split code; int8: tile code
+    bool xalign;  // GEMV / MFMA f32: activations 16-byte aligned; int8: block dots are written out
     bool operator==(const GemvKey &o) const {
-        return mma == o.mma && packed == o.packed && tb == o.tb && xalign == o.xalign;
+        return kind == o.kind && packed == o.packed && tb == o.tb && xalign == o.xalign;
     }
 };
 
 GemvKey gemv_key(const Op &op) {
     GemvKey k;
-    k.mma = op.kind == OP_MMA;
+    k.kind = op.kind;
     k.packed = op.packed;
-    if (k.mma) {
+    if (op.kind == OP_I8) {
+        k.tb = q8::pick_i8_config(op.batch);
+        k.xalign = op.a[3] != nullptr;
+        return k;
+    }
+    if (op.kind == OP_MMA) {
         // The tile shape and K split are chosen per product, so a product's
         // result does not depend on what else shares its launch.
         const q8::MmaProduct p{nullptr, nullptr, nullptr, op.rows, op.cols, op.batch};
@@ -317,10 +322,26 @@ hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<c
     return q8::launch_gemm_mma_list(ctx->stream, stop, key.packed, key.xalign, prods, n, &c);
 }
 
+hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
+                          GemvKey key) {
+    q8::I8Product prods[q8::I8_MAX_DESCS];
+    int n = 0;
+    for (const Op *op : ops) {
+        prods[n++] = q8::I8Product{(const uint8_t *)op->a[0]->ptr, (const uint8_t *)op->a[1]->ptr,
+                                   (float *)op->a[2]->ptr + op->y_off,
+                                   op->a[3] != nullptr ? (int32_t *)op->a[3]->ptr : nullptr,
+                                   op->rows, op->cols, op->batch};
+    }
+    return q8::launch_gemm_i8_list(ctx->stream, stop, key.packed, key.xalign, key.tb, prods, n);
+}
+
 hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
                             GemvKey key) {
-    if (key.mma) {
+    if (key.kind == OP_MMA) {
         return launch_mma_list(ctx, stop, ops, key);
+    }
+    if (key.kind == OP_I8) {
+        return launch_i8_list(ctx, stop, ops, key);
     }
     q8::GemvArgs args; // only the used descriptors are written (the struct is 12 KB)
     args.n = 0;
@@ -406,11 +427,6 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
     case OP_QUANT:
         return q8::launch_quantize_act(st, stop, (const float *)op.a[0]->ptr + op.x_off,
                                        (uint8_t *)op.a[1]->ptr, op.cols, op.batch);
-    case OP_I8:
-        return q8::launch_gemm_i8(st, stop, op.packed, w, (const uint8_t *)op.a[1]->ptr,
-                                  (float *)op.a[2]->ptr + op.y_off,
-                                  op.a[3] ? (int32_t *)op.a[3]->ptr : nullptr, op.rows, op.cols,
-                                  op.batch);
     default:
         return hipErrorInvalidValue;
     }
@@ -441,14 +457,20 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
         }
     };
     for (const Op &op : ops) {
-        if (op.kind == OP_GEMV_LIST || op.kind == OP_MMA) {
+        if (op.kind == OP_GEMV_LIST || op.kind == OP_MMA || op.kind == OP_I8) {
             const GemvKey key = gemv_key(op);
-            const int cap = key.mma ? q8::MMA_MAX_DESCS : q8::GEMV_MAX_DESCS;
-            // a[0] = w (read), a[1] = x (read), a[2] = y (written): the product
-            // joins the open launch unless its output was read or written
-            // there, or one of its inputs was written there.
-            const bool conflict = op.a[2]->read_epoch == epoch || op.a[2]->write_epoch == epoch ||
-                                  op.a[1]->write_epoch == epoch || op.a[0]->write_epoch == epoch;
+            const int cap = key.kind == OP_MMA  ? q8::MMA_MAX_DESCS
+                            : key.kind == OP_I8 ? q8::I8_MAX_DESCS
+                                                : q8::GEMV_MAX_DESCS;
+            // a[0] = w (read), a[1] = x (read), a[2] = y (written), a[3] =
+            // optional second output: the product joins the open launch
+            // unless an output of it was read or written there, or one of
+            // its inputs was written there.
+            bool conflict = op.a[2]->read_epoch == epoch || op.a[2]->write_epoch == epoch ||
+                            op.a[1]->write_epoch == epoch || op.a[0]->write_epoch == epoch;
+            if (op.a[3] != nullptr) {
+                conflict = conflict || op.a[3]->read_epoch == epoch || op.a[3]->write_epoch == epoch;
+            }
             if (!cur.list.empty() &&
                 (conflict || !(key == cur.key) || (int)cur.list.size() == cap)) {
                 flush();
@@ -458,6 +480,9 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             op.a[0]->read_epoch = epoch;
             op.a[1]->read_epoch = epoch;
             op.a[2]->write_epoch = epoch;
+            if (op.a[3] != nullptr) {
+                op.a[3]->write_epoch = epoch;
+            }
         } else {
             flush();
             Launch one;
@@ -1243,7 +1268,7 @@ int tm_hip_q8_0_quantize_act(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *x
                     batch, TM_HIP_GEMM_I8_MAX_BATCH);
     }
     const size_t x_need = ((size_t)x_off + (size_t)batch * cols) * 4u;
-    const size_t q_need = (size_t)batch * ((size_t)cols + (size_t)(cols / 32u) * 4u);
+    const size_t q_need = q8::xq_bytes(cols, batch);
     int rc;
     if ((rc = check_buffer(ctx, x, x_need, err, err_cap, "q8_0_quantize_act.x")) != TM_HIP_OK ||
         (rc = check_buffer(ctx, xq, q_need, err, err_cap, "q8_0_quantize_act.xq")) != TM_HIP_OK) {
@@ -1278,7 +1303,7 @@ int tm_hip_q8_0_gemm_i8(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm
     }
     const size_t blocks = cols / 32u;
     const size_t w_need = (size_t)rows * blocks * 34u;
-    const size_t q_need = (size_t)batch * ((size_t)cols + blocks * 4u);
+    const size_t q_need = q8::xq_bytes(cols, batch);
     const size_t y_need = ((size_t)y_off + (size_t)batch * rows) * 4u;
     int rc;
     if ((rc = check_buffer(ctx, w, w_need, err, err_cap, "q8_0_gemm_i8.weights")) != TM_HIP_OK ||

@@ -401,6 +401,22 @@ def q8_0_bytes(rows: int, cols: int) -> int:
     return rows * (cols // 32) * 34
 
 
+def xq_bytes(cols: int, batch: int) -> int:
+    """Size of a quantized-activation buffer (see tm_hip_q8_0_quantize_act)."""
+    bpad = (batch + 3) & ~3
+    return batch * cols + (cols // 32) * bpad * 4
+
+
+def xq_split(raw: np.ndarray, cols: int, batch: int):
+    """(quants int8 [batch, cols/32, 32], scales f32 [batch, cols/32]) of a
+    downloaded quantized-activation buffer."""
+    blocks = cols // 32
+    bpad = (batch + 3) & ~3
+    qs = raw[:batch * cols].view(np.int8).reshape(batch, blocks, 32)
+    ds = raw[batch * cols:batch * cols + blocks * bpad * 4].view(np.float32).reshape(blocks, bpad)
+    return qs, np.ascontiguousarray(ds[:, :batch].T)
+
+
 class Matrix:
     """A device projection matrix: the HIP form of the reference's ``Matrix``
     (crates/tuckcore/src/engine/metal.rs:106-226) for Q8_0 weights."""
