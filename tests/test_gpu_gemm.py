@@ -70,15 +70,21 @@ def test_batch_one_gemm_is_bit_identical_to_gemv(ctx):
         assert np.array_equal(bits(single), bits(batch))
 
 
+@pytest.mark.parametrize("x_off", [0, 3])
 @pytest.mark.parametrize("rows,cols,batch", [(64, 1024, 32), (100, 1152, 7), (33, 96, 5),
-                                             (513, 2048, 13), (40, 6912, 3)])
-def test_every_token_of_the_small_gemm_equals_its_own_gemv(ctx, rows, cols, batch):
+                                             (513, 2048, 13), (40, 6912, 3), (520, 2048, 8),
+                                             (100, 3072, 2), (33, 1024, 4), (4099, 6144, 16),
+                                             (41, 6912, 9), (64, 1056, 3), (50, 2016, 5),
+                                             (8, 1024, 17), (9, 4096, 31)])
+def test_every_token_of_the_small_gemm_equals_its_own_gemv(ctx, rows, cols, batch, x_off):
     # Stronger than the reference's batch = 1 identity: the exact (speculative
-    # verify) path must reproduce decode for every token.
+    # verify) path must reproduce decode for every token. Covers every
+    # waves x tokens-per-wave split of the small-batch kernel, column tails,
+    # row tails and activations that are not 16-byte aligned.
     w = S.make_weights(rows, cols, 31 + rows)
     x = S.make_activations(cols * batch, 77)
     wb = weights_buffer(ctx, w, rows, cols, True)
-    got = run_gemm(ctx, ctx.q8_0_gemm, wb, x, rows, cols, batch).reshape(batch, rows)
+    got = run_gemm(ctx, ctx.q8_0_gemm, wb, x, rows, cols, batch, x_off, 5)[5:].reshape(batch, rows)
     want = O.gemm_q8_0_f32(w, rows, cols, x, batch)
     assert norm_err(got, want) <= 1e-5
     for b in range(batch):

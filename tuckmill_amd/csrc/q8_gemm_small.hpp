@@ -1,0 +1,226 @@
+// Small-batch Q8_0 product with the GEMV's arithmetic (2 <= batch <= 32,
+// sealed weights, cols >= 1024): the exact / speculative-verify
+// path (contract: native/metal/tm_metal.h:161-164,
+// crates/tuckcore/src/engine/metal.rs:81-83).
+//
+// At these batch sizes the product is bound by f32 vector multiply-adds and by
+// registers, not by HBM: a lane needs batch x 16 activations per weight piece.
+// So the NW waves of a workgroup share one tile of rows and split the TOKENS:
+// wave w owns tokens w*TW .. w*TW+TW-1. The weights of a step (8 rows x 1024
+// columns) are fetched once per workgroup straight into LDS (buffer_load ...
+// lds, 16 bytes per lane: no registers are held while the data is in flight),
+// double-buffered, and every wave reads its lane's 16 quants of each row back
+// with one ds_read_b128. A wave then keeps only 8 x TW accumulators and TW x 16
+// activations in registers, and a weight byte is converted once per wave.
+//
+// Per-(row, token) arithmetic is exactly the decode kernel's (q8_gemv.hpp):
+// the lane -> column mapping, the left-to-right fused multiply-adds over a
+// lane's 16 quants, one fused multiply-add per block scale with chunks in
+// ascending order, and the same butterfly; every token is bit-identical to its
+// own GEMV.
+#pragma once
+
+#include "q8_gemv.hpp"
+
+namespace q8 {
+
+constexpr int SMALL_R = 8; // rows per step
+
+// TAIL: some product of the launch has cols % 1024 != 0 (kept out of the
+// common instantiation: the tail code costs registers even when it never runs).
+template <int NW, int TW, bool XA, bool TAIL>
+__global__ __launch_bounds__(NW * 64) void gemm_split_list_kernel(const GemvArgs args) {
+    constexpr int R = SMALL_R;
+    // Two separate objects (not one array indexed by parity): the compiler then
+    // sees that reads of one buffer cannot alias the fetch into the other and
+    // does not wait for the prefetch before reading.
+    __shared__ __attribute__((aligned(16))) uint8_t stage_a[R * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t stage_b[R * 1024];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t tile = blockIdx.x; // one tile per workgroup; the grid is exactly total_tiles
+    uint32_t lo = 0, hi = args.n;
+    while (hi - lo > 1u) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (args.d[mid].tile_begin <= tile) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    const GemvDesc &d = args.d[lo];
+    const uint32_t rows = d.rows, cols = d.cols, batch = d.batch;
+    const WView<PACKED> wv(d.w, rows, cols);
+    const float *x = d.x;
+    float *y = d.y;
+    const uint32_t row_first = (tile - d.tile_begin) * d.rows_per_tile;
+    uint32_t row_end = row_first + d.rows_per_tile;
+    if (row_end > rows) {
+        row_end = rows;
+    }
+    const uint32_t full = cols >> 10;
+    const uint32_t nsteps = ((row_end - row_first + R - 1) / R) * full;
+
+    uint32_t xoff[TW], tok[TW];
+    bool tok_ok[TW];
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+        const uint32_t tk = wave * TW + t;
+        tok_ok[t] = tk < batch;
+        tok[t] = tok_ok[t] ? tk : batch - 1u;
+        xoff[t] = tok[t] * cols + lane * 16u;
+    }
+    const bool has_tokens = wave * TW < batch; // wave-uniform
+
+    // Wave w fetches rows 2w and 2w+1 of a step; lane l's 16 bytes land at
+    // row * 1024 + l * 16 of the stage buffer. The fetch is a buffer load (not
+    // a global one): the compiler's wait-count bookkeeping treats a global
+    // load into LDS as a flat access and would make every later wait drain
+    // the prefetch too. The descriptor covers the tile's quants only.
+    const uint8_t *tile_q = wv.q + (size_t)row_first * cols;
+    const size_t tile_len = (size_t)(row_end - row_first) * cols;
+    const __amdgpu_buffer_rsrc_t tile_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)tile_q, 0, tile_len > 0xffffffffull ? 0xffffffffu : (uint32_t)tile_len, 0x00020000);
+    auto fetch = [&](uint32_t r0, uint32_t c, uint8_t *stage) {
+#pragma unroll
+        for (int i = 0; i < R / NW; ++i) {
+            const uint32_t r = wave * (R / NW) + i;
+            const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+            const uint32_t base = __builtin_amdgcn_readfirstlane((row - row_first) * cols + (c << 10));
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                tile_rs, (__attribute__((address_space(3))) void *)(stage + r * 1024), 16,
+                lane * 16u, base, 0, 0);
+        }
+    };
+    auto load_scales = [&](uint32_t r0, uint32_t c, uint32_t (&ss)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+            ss[r] = wv.scale_bits(row, (c << 5) + (lane >> 1));
+        }
+    };
+
+    uint32_t sb[R], sn[R];
+    fetch(row_first, 0, stage_a);
+    load_scales(row_first, 0, sb);
+    uint32_t r0 = row_first, c = 0;
+    float acc[R][TW];
+    auto do_step = [&](uint32_t step, uint8_t *cur, uint8_t *nxt) {
+        // The fetch of this step has landed (each wave waits for its own part,
+        // then all meet), and every wave has finished reading the other buffer.
+        __syncthreads();
+        uint32_t cn = c + 1u, rn = r0;
+        if (cn == full) {
+            cn = 0;
+            rn = r0 + R;
+        }
+        // This step's activations are requested before the next step's
+        // weights: the memory counter retires in order, and the multiplies
+        // below must not wait for the prefetch.
+        // This step's activations are requested before the next step's
+        // weights: the memory counter retires in order, and the multiplies
+        // below must not wait for the prefetch. (Requesting them a whole step
+        // ahead was measured slower: the registers cost more than the wait.)
+        float xv[TW][16];
+#pragma unroll
+        for (int t = 0; t < TW; ++t) {
+            load_x<16, XA>(x + xoff[t] + (c << 10), xv[t]);
+        }
+        __builtin_amdgcn_sched_barrier(0); // keep the instruction scheduler from swapping the two
+        // The prefetch is unconditional (the last step fetches its own data
+        // again, into the buffer nobody reads any more): with a branch here the
+        // wait for the activations above would have to cover both paths and
+        // would drain the prefetch too.
+        const bool last = step + 1u == nsteps;
+        fetch(last ? r0 : rn, last ? c : cn, nxt);
+        load_scales(last ? r0 : rn, last ? c : cn, sn);
+        if (has_tokens) {
+            if (c == 0u) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+#pragma unroll
+                    for (int t = 0; t < TW; ++t) {
+                        acc[r][t] = 0.0f;
+                    }
+                }
+                // Column tail first, as in the decode kernel; these few pieces
+                // come straight from global memory.
+                if (TAIL && (cols & 1023u)) {
+                    uint32_t row[R];
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        row[r] = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+                    }
+                    uint32_t col0 = full << 10;
+                    if (cols & 512u) {
+                        chunk<PACKED, R, TW, 8, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
+                        col0 += 512u;
+                    }
+                    if (cols & 256u) {
+                        chunk<PACKED, R, TW, 4, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
+                        col0 += 256u;
+                    }
+                    if (cols & 128u) {
+                        chunk<PACKED, R, TW, 2, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
+                        col0 += 128u;
+                    }
+                    if (cols & 64u) {
+                        chunk<PACKED, R, TW, 1, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
+                        col0 += 64u;
+                    }
+                    if (cols & 32u) {
+                        chunk<PACKED, R, TW, 1, XA, false>(wv, x, cols, row, tok, col0, lane,
+                                                           lane < 32u, acc);
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const uint4 qv = *(const uint4 *)(cur + r * 1024 + lane * 16u);
+                const uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
+                float qf[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    qf[i] = sbyte_to_float(q[i / 4], i % 4);
+                }
+                const float dsc = f16_bits_to_f32(sb[r]);
+#pragma unroll
+                for (int t = 0; t < TW; ++t) {
+                    float s = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        s = __builtin_fmaf(qf[i], xv[t][i], s);
+                    }
+                    acc[r][t] = __builtin_fmaf(dsc, s, acc[r][t]);
+                }
+            }
+            if (cn == 0u) {
+#pragma unroll
+                for (int t = 0; t < TW; ++t) {
+                    float col_acc[R];
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        col_acc[r] = acc[r][t];
+                    }
+                    reduce_store<R>(col_acc, y + (size_t)(wave * TW + t) * rows, r0, row_end, lane,
+                                    tok_ok[t]);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            sb[r] = sn[r];
+        }
+        c = cn;
+        r0 = rn;
+    };
+    for (uint32_t step = 0; step < nsteps; step += 2u) {
+        do_step(step, stage_a, stage_b);
+        if (step + 1u < nsteps) {
+            do_step(step + 1u, stage_b, stage_a);
+        }
+    }
+    __syncthreads(); // no fetch may still be in flight when the workgroup gives up its LDS
+}
+
+} // namespace q8

@@ -24,6 +24,7 @@
 #include "q8_gemm_i8.hpp"
 #include "q8_gemm_mma.hpp"
 #include "q8_gemv.hpp"
+#include "q8_gemm_small.hpp"
 #include "q8_misc.hpp"
 
 namespace {
@@ -243,7 +244,9 @@ int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
 struct GemvKey {
     OpKind kind;  // OP_GEMV_LIST, OP_MMA or OP_I8: which list kernel
     bool packed;
-    int tb;       // GEMV: tokens per pass (1 or 4); MFMA f32: tile/split code; int8: tile code
+    int tb;       // GEMV: tokens per pass (1 or 4), or 200 + 10 * waves + tokens per wave
+                  // for the token-split small-batch kernel;
+                  // MFMA f32: tile/split code; int8: tile code
     bool xalign;  // GEMV / MFMA f32: activations 16-byte aligned; int8: block dots are written out
     bool operator==(const GemvKey &o) const {
         return kind == o.kind && packed == o.packed && tb == o.tb && xalign == o.xalign;
@@ -267,19 +270,27 @@ GemvKey gemv_key(const Op &op) {
         k.tb = c.tmw * 16 + c.tnw * 8 + c.s;
     } else {
         k.tb = op.batch == 1 ? 1 : 4;
+        if (op.batch > 1 && op.packed && op.cols >= 1024u) {
+            // token-split kernel: 200 + 10 * waves + tokens per wave (measured
+            // on 2B-class shapes; the alternatives were within 5 %)
+            k.tb = 200 + (op.batch <= 2 ? 12 : op.batch <= 4 ? 14 : op.batch <= 8 ? 24
+                          : op.batch <= 16 ? 44 : 48);
+            if (op.cols & 1023u) {
+                k.tb += 100; // the instantiation that also handles a column tail
+            }
+        }
     }
     const uintptr_t xp = (uintptr_t)op.a[1]->ptr + (uintptr_t)op.x_off * 4u;
     k.xalign = (xp % 16u == 0);
     return k;
 }
 
-uint32_t pick_rows_per_tile(uint32_t rows, uint32_t cols, uint32_t batch, int R) {
+uint32_t pick_rows_per_tile(uint32_t rows, uint32_t cols, uint32_t tile_bytes, int R) {
     // About 8 KiB of weights per wave (measured best for streaming; 32 KiB
     // and more lose bandwidth), at least one pass of R rows; a matrix that
     // would give fewer than 256 tiles gets smaller ones so that a lone
     // product still spreads over the CUs.
-    (void)batch;
-    uint32_t rpt = (8192u / cols);
+    uint32_t rpt = (tile_bytes / cols);
     if (rpt < (uint32_t)R) {
         rpt = (uint32_t)R;
     }
@@ -346,7 +357,9 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<
     q8::GemvArgs args; // only the used descriptors are written (the struct is 12 KB)
     args.n = 0;
     args.pad[0] = args.pad[1] = 0;
-    const int R = key.tb == 1 ? kGemvR1 : kGemvR4;
+    const int R = (key.tb == 1 || key.tb >= 200) ? kGemvR1 : kGemvR4;
+    // a workgroup's tile in the token-split kernel, a wave's tile otherwise
+    const uint32_t tile_bytes = key.tb >= 200 ? 32768u : 8192u;
     uint32_t tiles = 0;
     bool tails = false; // some product has a column tail with a streaming path of its own
     for (const Op *op : ops) {
@@ -360,11 +373,29 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<
         d.cols = op->cols;
         d.batch = op->batch;
         d.tile_begin = tiles;
-        d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, op->batch, R);
+        d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
         d.pad = 0;
         tiles += (op->rows + d.rows_per_tile - 1) / d.rows_per_tile;
     }
     args.total_tiles = tiles;
+#define TM_SPLIT_CASE(W, T, A, TL)                                                           \
+    if (key.tb == ((TL) ? 300 : 200) + (W) * 10 + (T) && key.xalign == (A)) {                \
+        Q8_LAUNCH((q8::gemm_split_list_kernel<W, T, A, TL>), dim3(tiles), dim3((W) * 64), 0, \
+                  ctx->stream, stop, args);                                                  \
+        return hipGetLastError();                                                            \
+    }
+#define TM_SPLIT_ALL(W, T)                                                                   \
+    TM_SPLIT_CASE(W, T, true, false)                                                         \
+    TM_SPLIT_CASE(W, T, false, false)                                                        \
+    TM_SPLIT_CASE(W, T, true, true)                                                          \
+    TM_SPLIT_CASE(W, T, false, true)
+    TM_SPLIT_ALL(1, 2)
+    TM_SPLIT_ALL(1, 4)
+    TM_SPLIT_ALL(2, 4)
+    TM_SPLIT_ALL(4, 4)
+    TM_SPLIT_ALL(4, 8)
+#undef TM_SPLIT_ALL
+#undef TM_SPLIT_CASE
 #define TM_GEMV_CASE(P, T, A)                                                                \
     if (key.packed == (P) && key.tb == (T) && key.xalign == (A)) {                           \
         return launch_gemv<(P) ? q8::PACKED : q8::RAW, (T) == 1 ? kGemvR1 : kGemvR4, T, A>(  \
