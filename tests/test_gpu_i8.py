@@ -62,7 +62,11 @@ def test_activation_quantizer_is_bit_exact(ctx, cols, batch, scale):
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("rows,cols,batch", [(16, 32, 1), (40, 64, 3), (100, 96, 77),
                                              (1024, 1024, 16), (333, 1152, 40), (2048, 2048, 8),
-                                             (70, 1024, 17), (48, 160, 33), (65, 2048, 130)])
+                                             (70, 1024, 17), (48, 160, 33), (65, 2048, 130),
+                                             # decode-sized batches: the streaming kernel
+                                             (4099, 2048, 1), (33, 6144, 2), (520, 1152, 4),
+                                             (41, 6912, 5), (1000, 3072, 8), (9, 2016, 7),
+                                             (64, 1056, 6), (17000, 1024, 2)])
 def test_gemm_i8_block_dots_and_result_are_bit_exact(ctx, rows, cols, batch, packed):
     blocks = cols // 32
     w = S.make_weights(rows, cols, rows + cols)

@@ -22,6 +22,7 @@
 #include <vector>
 
 #include "q8_gemm_i8.hpp"
+#include "q8_gemv_i8.hpp"
 #include "q8_gemm_mma.hpp"
 #include "q8_gemv.hpp"
 #include "q8_gemm_small.hpp"
@@ -259,6 +260,9 @@ GemvKey gemv_key(const Op &op) {
     k.packed = op.packed;
     if (op.kind == OP_I8) {
         k.tb = q8::pick_i8_config(op.batch);
+        if (op.packed && op.batch <= q8::GEMV_I8_MAX_BATCH) {
+            k.tb = 10 + q8::gemv_i8_tokens(op.batch); // the streaming kernel
+        }
         k.xalign = op.a[3] != nullptr;
         return k;
     }
@@ -342,6 +346,9 @@ hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<co
                                    (float *)op->a[2]->ptr + op->y_off,
                                    op->a[3] != nullptr ? (int32_t *)op->a[3]->ptr : nullptr,
                                    op->rows, op->cols, op->batch};
+    }
+    if (key.tb >= 10) {
+        return q8::launch_gemv_i8_list(ctx->stream, stop, key.xalign, key.tb - 10, prods, n);
     }
     return q8::launch_gemm_i8_list(ctx->stream, stop, key.packed, key.xalign, key.tb, prods, n);
 }
