@@ -260,7 +260,8 @@ def bench_gemma(host, ctx, steps, warmup):
 
 def bench_sweep(host, ctx, steps, warmup):
     """BASELINE config 4: 2B-class shapes (hidden 2048, FFN 6144), M in
-    {1, 8, 64, 512, 2048}, f32 activations and the int8-activation profile.
+    {1, 8, 64, 512, 2048} plus the small batches in between, f32 activations
+    and the int8-activation profile.
     Each point runs over 20 distinct weight copies per shape (535 MB in all),
     so small M is measured against HBM, not against the caches."""
     copies = 20
@@ -276,8 +277,8 @@ def bench_sweep(host, ctx, steps, warmup):
     widths = sorted({c for _, _, c, _ in pool})
     xqs = {c: ctx.buffer(H.xq_bytes(c, maxM)) for c in widths}
     ys = [ctx.buffer(maxM * maxr * 4) for _ in pool]
-    for M in (1, 8, 64, 512, 2048):
-        n = max(3, steps // (40 if M < 64 else 200 if M < 512 else 1000))
+    for M in (1, 2, 4, 8, 16, 32, 64, 512, 2048):
+        n = max(3, steps // (10 if M < 64 else 200 if M < 512 else 1000))
         w = max(2, n // 5)
         flops = sum(2.0 * M * r * c for _, r, c, _ in pool)
         abytes = sum(S.q8_0_bytes(r, c) + 4 * M * c + 4 * M * r for _, r, c, _ in pool)
@@ -290,7 +291,7 @@ def bench_sweep(host, ctx, steps, warmup):
             paths.append(("f32 mfma", TMH_GEMM_MMA, M))
         if M > 512:
             paths.append(("f32 mfma (slices of 512)", TMH_GEMM_MMA, 512))
-        paths.append(("i8 mfma", TMH_GEMM_I8, M))
+        paths.append(("i8 streaming dot4" if M <= 16 else "i8 mfma", TMH_GEMM_I8, M))
         for label, kind, mb in paths:
             prods = []
             slices = (M + mb - 1) // mb

@@ -349,19 +349,21 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
         }
     }
 
-    // Row passes outermost: the R rows of a pass are re-read for every group
-    // of TB tokens, but back to back, so only the first read goes to HBM.
-    for (uint32_t r0 = row_first; r0 < row_end; r0 += R) {
-        uint32_t row[R];
+    // The general form (raw layout, narrow matrices, other column tails).
+    // Token groups outermost: with the row passes outermost this path, which
+    // the decode shapes never take, doubled the kernel's register count and
+    // halved the occupancy of the streaming path above.
+    for (uint32_t t0 = 0; t0 < batch; t0 += TB) {
+        uint32_t tok[TB];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            row[r] = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+        for (int t = 0; t < TB; ++t) {
+            tok[t] = (t0 + t < batch) ? t0 + t : batch - 1u;
         }
-        for (uint32_t t0 = 0; t0 < batch; t0 += TB) {
-            uint32_t tok[TB];
+        for (uint32_t r0 = row_first; r0 < row_end; r0 += R) {
+            uint32_t row[R];
 #pragma unroll
-            for (int t = 0; t < TB; ++t) {
-                tok[t] = (t0 + t < batch) ? t0 + t : batch - 1u;
+            for (int r = 0; r < R; ++r) {
+                row[r] = (r0 + r < row_end) ? r0 + r : row_end - 1u;
             }
             float acc[R][TB];
 #pragma unroll

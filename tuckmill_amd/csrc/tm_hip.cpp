@@ -1128,7 +1128,11 @@ int tm_hip_q8_0_gemm_mma(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm
         return rc;
     }
     Op op;
-    op.kind = OP_MMA;
+    // Below this batch a 32-token MFMA tile is mostly padding and the vector
+    // kernels (GEMV arithmetic, which is within any tolerance of itself) are
+    // faster: 1 token -> the decode kernel, 2..16 -> the token-split kernel.
+    const bool small = w->alloc->packed && (batch == 1 || (batch <= 16 && cols >= 1024u));
+    op.kind = small ? OP_GEMV_LIST : OP_MMA;
     op.a[0] = w->alloc;
     op.a[1] = x->alloc;
     op.a[2] = y->alloc;
