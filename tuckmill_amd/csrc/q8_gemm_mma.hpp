@@ -260,6 +260,189 @@ __global__ __launch_bounds__(256) void gemm_mma_kernel(const MmaArgs args) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Persistent form of the kernel above for the common configuration (one slot
+// per workgroup, K split over its 4 waves, TNW = 1, sealed or raw weights).
+//
+// Measured on the M = 512 projection set: a wave of the one-tile-per-workgroup
+// kernel spends about as long before its first MFMA (first operands: 11 k
+// cycles median) and after its last (barrier, reduction by one wave, stores:
+// 7 k median) as it needs to issue its MFMAs (16 k), and vector instructions
+// do not overlap with f32 MFMAs on this part (each costs the matrix pipe about
+// five cycles). So here
+//   * a workgroup walks a strided list of tiles and requests the first block
+//     of the next tile before it finishes the current one;
+//   * the two operand sets are used in turn with no register copies: per
+//     block only the dequantisation d*q remains beside the MFMAs;
+//   * every wave writes its partial tile to LDS and reduces and stores one
+//     quarter of it (sum order wave 0, 1, 2, 3 as before).
+struct MmaTileCtx {
+    const uint8_t *w;
+    const float *x;
+    float *y;
+    uint32_t rows, cols, batch, t0, n0, kb_begin, kb_end;
+};
+
+template <int L, int TMW, bool XA>
+__global__ __launch_bounds__(256) void gemm_mma_persistent_kernel(const MmaArgs args) {
+    constexpr int S = 4;
+    constexpr int NV = TMW * 16;          // accumulator values per lane
+    constexpr int QV = NV / S;            // values a wave reduces and stores
+    __shared__ float red[S][NV][WAVE];
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t s = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t idx = lane & 31u, half = lane >> 5;
+    const uint32_t nwg = gridDim.x;
+
+    // Same workgroup -> XCD dealing as gemm_mma_kernel (gridDim.x is a multiple
+    // of 8, so workgroup b keeps its XCD for every tile of its list).
+    auto tile_of = [&](uint32_t g) -> uint32_t {
+        const uint32_t cw = args.chunk_wgs;
+        const uint32_t span = 8u * cw;
+        const uint32_t g_full = (args.total_tiles / span) * span;
+        if (g < g_full) {
+            const uint32_t xcd = g & 7u, j = g >> 3;
+            g = ((j / cw) * 8u + xcd) * cw + (j % cw);
+        }
+        return g;
+    };
+    auto decode = [&](uint32_t g, MmaTileCtx &c) {
+        const uint32_t tile = tile_of(g);
+        uint32_t lo = 0, hi = args.n;
+        while (hi - lo > 1u) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (args.d[mid].tile_begin <= tile) {
+                lo = mid;
+            } else {
+                hi = mid;
+            }
+        }
+        const MmaDesc &d = args.d[lo];
+        c.w = d.w; c.x = d.x; c.y = d.y;
+        c.rows = d.rows; c.cols = d.cols; c.batch = d.batch;
+        const uint32_t local = tile - d.tile_begin;
+        c.t0 = (local % d.tiles_t) * (32u * TMW);
+        c.n0 = (local / d.tiles_t) * 32u;
+        const uint32_t blocks = d.cols >> 5;
+        c.kb_begin = (uint32_t)(((uint64_t)blocks * s) / S);
+        c.kb_end = (uint32_t)(((uint64_t)blocks * (s + 1u)) / S);
+    };
+    auto load = [&](const MmaTileCtx &c, uint32_t kb, MmaRaw<TMW, 1> &raw) {
+        const WView<L> wv(c.w, c.rows, c.cols);
+        const uint32_t r = c.n0 + idx;
+        const uint32_t wrow[1] = {r < c.rows ? r : c.rows - 1u};
+        uint32_t tok[TMW];
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+            const uint32_t t = c.t0 + 32u * i + idx;
+            tok[i] = t < c.batch ? t : c.batch - 1u;
+        }
+        mma_load_block<L, TMW, 1, XA>(wv, c.x, c.cols, wrow, tok, kb, half, raw);
+    };
+
+    floatx16 acc[TMW];
+    auto block = [&](const MmaRaw<TMW, 1> &cur) {
+        float wf[16];
+        const float dsc = f16_bits_to_f32(cur.sb[0]);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            wf[e] = dsc * sbyte_to_float(cur.q[0][e / 4], e % 4);
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+#pragma unroll
+            for (int i = 0; i < TMW; ++i) {
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(cur.xv[i][e], wf[e], acc[i], 0, 0, 0);
+            }
+        }
+    };
+
+    uint32_t g = blockIdx.x;
+    if (g >= args.total_tiles) {
+        return;
+    }
+    MmaTileCtx cur;
+    decode(g, cur);
+    MmaRaw<TMW, 1> ra, rb;
+    load(cur, cur.kb_begin, ra); // invariant: `ra` holds the first block of the tile about to run
+    while (true) {
+        const uint32_t gn = g + nwg;
+        const bool more = gn < args.total_tiles; // uniform over the workgroup
+        MmaTileCtx nxt = cur;
+        if (more) {
+            decode(gn, nxt);
+        }
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                acc[i][v] = 0.0f;
+            }
+        }
+        // The wave's blocks, two per trip; every step requests the operands
+        // of the following step first (the next tile's first block at the
+        // end: without a next tile the last block is requested once more).
+        uint32_t kb = cur.kb_begin;
+        const uint32_t ke = cur.kb_end;
+        for (; kb + 2u < ke; kb += 2u) {
+            load(cur, kb + 1u, rb);
+            __builtin_amdgcn_sched_barrier(0);
+            block(ra);
+            load(cur, kb + 2u, ra);
+            __builtin_amdgcn_sched_barrier(0);
+            block(rb);
+        }
+        if (kb + 2u == ke) { // two blocks left
+            load(cur, kb + 1u, rb);
+            __builtin_amdgcn_sched_barrier(0);
+            block(ra);
+            load(nxt, more ? nxt.kb_begin : kb + 1u, ra);
+            __builtin_amdgcn_sched_barrier(0);
+            block(rb);
+        } else if (kb + 1u == ke) { // one block left
+            load(nxt, more ? nxt.kb_begin : kb, rb);
+            __builtin_amdgcn_sched_barrier(0);
+            block(ra);
+            ra = rb;
+        } else if (more) { // a wave without blocks (fewer blocks than waves)
+            load(nxt, nxt.kb_begin, ra);
+        }
+
+        // Reduction over the 4 k-slices: everybody parks its partial tile,
+        // then wave s adds values s*QV .. s*QV+QV-1 in slice order and stores.
+        __syncthreads(); // the previous tile's partials have been read
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                red[s][i * 16 + v][lane] = acc[i][v];
+            }
+        }
+        __syncthreads();
+        const uint32_t n = cur.n0 + idx;
+#pragma unroll
+        for (int k = 0; k < QV; ++k) {
+            const uint32_t q = s * QV + k;
+            float sum = red[0][q][lane];
+#pragma unroll
+            for (int o = 1; o < S; ++o) {
+                sum += red[o][q][lane];
+            }
+            const uint32_t i = q >> 4, v = q & 15u;
+            const uint32_t t = cur.t0 + 32u * i + 8u * (v >> 2) + 4u * half + (v & 3u);
+            if (t < cur.batch && n < cur.rows) {
+                cur.y[(size_t)t * cur.rows + n] = sum;
+            }
+        }
+        if (!more) {
+            break;
+        }
+        g = gn;
+        cur = nxt;
+    }
+}
+
 struct MmaConfig {
     int tmw, tnw, s;
 };
@@ -321,6 +504,28 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
     args.chunk_wgs = args.d[0].tiles_t >= (uint32_t)P ? args.d[0].tiles_t / P : 1u;
     args.pad = 0;
     const uint32_t groups = (uint32_t)((tiles + P - 1) / P);
+    if constexpr (S == 4 && TNW == 1) {
+        // Persistent form: as many workgroups as stay resident (a multiple of
+        // 8), each walking a strided list of tiles.
+        static const uint32_t resident = [] {
+            int per_cu = 0, dev = 0, cus = 0;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &per_cu, (const void *)gemm_mma_persistent_kernel<L, TMW, XA>, 256, 0) != hipSuccess ||
+                hipGetDevice(&dev) != hipSuccess ||
+                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+                per_cu <= 0 || cus <= 0) {
+                (void)hipGetLastError();
+                return 512u;
+            }
+            return ((uint32_t)per_cu * (uint32_t)cus) & ~7u;
+        }();
+        const uint32_t wgs = groups < resident ? groups : resident;
+        if (wgs == groups || wgs % 8u == 0u) {
+            Q8_LAUNCH((gemm_mma_persistent_kernel<L, TMW, XA>), dim3(wgs), dim3(256), 0, stream, stop,
+                      args);
+            return hipGetLastError();
+        }
+    }
     const size_t lds = S > 1 ? (size_t)P * (S - 1) * TMW * TNW * 16 * WAVE * sizeof(float) : 0;
     Q8_LAUNCH((gemm_mma_kernel<L, TMW, TNW, S, XA>), dim3(groups), dim3(256), lds, stream, stop,
               args);
