@@ -116,6 +116,46 @@ int tm_hip_download_after(tm_hip_ctx *ctx, tm_hip_buffer *src, size_t off, void 
 int tm_hip_copy_f32(tm_hip_ctx *ctx, tm_hip_buffer *src, uint32_t src_off, tm_hip_buffer *dst,
                     uint32_t dst_off, uint32_t n, char *err, size_t err_cap);
 
+/* ---- the small f32 operators either side of a product ----------------------
+ * All are usable inside a dispatch group; a zero length is refused with
+ * TM_HIP_ERR_BOUNDS (rmsnorm: a zero shape with TM_HIP_ERR_UNSUPPORTED), as in
+ * the reference host code (native/metal/tm_metal.m:770-810, :1096-1177). */
+
+/* y[i] = x[i] * factor, i < n (native/metal/tm_metal.h:88-90). */
+int tm_hip_f32_scale(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *y, float factor, uint32_t n,
+                     char *err, size_t err_cap);
+
+/* y[i] = y[i] + alpha * a[i], i < n: multiply, then add, unfused
+ * (native/metal/tm_metal.h:115-116). */
+int tm_hip_f32_axpy(tm_hip_ctx *ctx, tm_hip_buffer *a, tm_hip_buffer *y, float alpha, uint32_t n,
+                    char *err, size_t err_cap);
+
+/* y[row] = x[row] / sqrt(mean(x[row]^2) + eps) * weight for `rows` rows of
+ * `cols`; in place (x == y) is allowed (native/metal/tm_metal.h:147-149,
+ * crates/tuckcore/src/forward.rs:911-927). */
+int tm_hip_rmsnorm_f32(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *weight, tm_hip_buffer *y,
+                       uint32_t rows, uint32_t cols, float eps, char *err, size_t err_cap);
+
+/* out[i] = silu(gate[i]) * up[i], silu(g) = g / (1 + exp(-g))
+ * (native/metal/tm_metal.h:189-191, crates/tuckcore/src/forward.rs:906-908). */
+int tm_hip_silu_mul_f32(tm_hip_ctx *ctx, tm_hip_buffer *gate, tm_hip_buffer *up, tm_hip_buffer *out,
+                        uint32_t n, char *err, size_t err_cap);
+
+/* out[i] = gelu_tanh(gate[i]) * up[i], ggml's tanh form
+ * (native/metal/tm_metal.h:193-195, native/metal/kernels.metal:382-396). */
+int tm_hip_gelu_tanh_mul_f32(tm_hip_ctx *ctx, tm_hip_buffer *gate, tm_hip_buffer *up,
+                             tm_hip_buffer *out, uint32_t n, char *err, size_t err_cap);
+
+/* Greedy argmax of x[0..n) into out[out_index] (u32), the CPU rule: NaN
+ * skipped, largest value wins, ties to the lowest index, 0xFFFFFFFF when every
+ * entry is NaN. `partial` is TM_HIP_ARGMAX_PARTIAL_BYTES of scratch
+ * (native/metal/tm_metal.h:92-98, crates/backend/src/sampling.rs:66-83). The
+ * result can feed tm_hip_row_indirect_f32 inside the same group. */
+#define TM_HIP_ARGMAX_NONE 0xFFFFFFFFu
+#define TM_HIP_ARGMAX_PARTIAL_BYTES 512
+int tm_hip_argmax_f32(tm_hip_ctx *ctx, tm_hip_buffer *x, uint32_t n, tm_hip_buffer *partial,
+                      tm_hip_buffer *out, uint32_t out_index, char *err, size_t err_cap);
+
 /* Grouped encoding: operations between begin and end are submitted as ONE
  * commit at end_group; abort_group discards them unsubmitted. Copies and
  * fence require no open group (native/metal/tm_metal.h:125-135). Inside a

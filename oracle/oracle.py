@@ -22,7 +22,8 @@ __all__ = [
     "quantize_row_q8_0", "dot_q8_0_x_f32", "dot_q8_0_q8_0", "gemv_q8_0_f32",
     "gemv_q8_0_q8_0", "gemm_q8_0_f32", "gemm_q8_0_q8_0", "gemv_q8_0_f32_dequant_first",
     "gemv_q8_0_f64", "Rng", "boundary_weights", "boundary_input", "KRng",
-    "random_q8_0_row", "block_sumi",
+    "random_q8_0_row", "block_sumi", "rmsnorm", "silu_mul", "gelu_tanh_mul", "axpy", "scale",
+    "argmax", "ARGMAX_NONE",
 ]
 
 
@@ -78,6 +79,13 @@ def lib() -> ctypes.CDLL:
         L.q8o_krng_next_f32.restype = c.c_float
         L.q8o_krng_next_f32.argtypes = [c.POINTER(c.c_uint64), c.c_float]
         L.q8o_random_q8_0_row.argtypes = [c.POINTER(c.c_uint64), c.c_size_t, u8p]
+        L.q8o_rmsnorm.argtypes = [f32p, f32p, c.c_size_t, c.c_float, f32p]
+        L.q8o_silu_mul.argtypes = [f32p, f32p, c.c_size_t, f32p]
+        L.q8o_gelu_tanh_mul.argtypes = [f32p, f32p, c.c_size_t, f32p]
+        L.q8o_axpy.argtypes = [f32p, c.c_float, c.c_size_t, f32p]
+        L.q8o_scale.argtypes = [f32p, c.c_float, c.c_size_t, f32p]
+        L.q8o_argmax.restype = c.c_uint32
+        L.q8o_argmax.argtypes = [f32p, c.c_size_t]
         _lib = L
     return _lib
 
@@ -236,6 +244,55 @@ def gemv_q8_0_f64(w, rows, cols, x) -> np.ndarray:
     y = np.empty(rows, dtype=np.float64)
     lib().q8o_gemv_q8_0_f64(_ptr(w), rows, cols, _ptr(x), _ptr(y))
     return y
+
+
+# ------------------------------------------ operators around the products --
+
+def rmsnorm(x, w, eps) -> np.ndarray:
+    """One row (crates/tuckcore/src/forward.rs:911-927)."""
+    x, w = _f32(x).ravel(), _f32(w).ravel()
+    if x.size == 0 or x.size != w.size:
+        raise OracleError("Internal", "rmsnorm: x and weight lengths differ or are zero")
+    y = np.empty_like(x)
+    lib().q8o_rmsnorm(_ptr(x), _ptr(w), x.size, float(eps), _ptr(y))
+    return y
+
+
+def silu_mul(gate, up) -> np.ndarray:
+    gate, up = _f32(gate).ravel(), _f32(up).ravel()
+    out = np.empty_like(gate)
+    lib().q8o_silu_mul(_ptr(gate), _ptr(up), gate.size, _ptr(out))
+    return out
+
+
+def gelu_tanh_mul(gate, up) -> np.ndarray:
+    gate, up = _f32(gate).ravel(), _f32(up).ravel()
+    out = np.empty_like(gate)
+    lib().q8o_gelu_tanh_mul(_ptr(gate), _ptr(up), gate.size, _ptr(out))
+    return out
+
+
+def axpy(a, alpha, y) -> np.ndarray:
+    a = _f32(a).ravel()
+    out = _f32(y).ravel().copy()
+    lib().q8o_axpy(_ptr(a), float(alpha), a.size, _ptr(out))
+    return out
+
+
+def scale(x, factor) -> np.ndarray:
+    x = _f32(x).ravel()
+    out = np.empty_like(x)
+    lib().q8o_scale(_ptr(x), float(factor), x.size, _ptr(out))
+    return out
+
+
+ARGMAX_NONE = 0xFFFFFFFF
+
+
+def argmax(x) -> int:
+    """Greedy rule of crates/backend/src/sampling.rs:69-83; ARGMAX_NONE when all NaN."""
+    x = _f32(x).ravel()
+    return int(lib().q8o_argmax(_ptr(x), x.size))
 
 
 # ------------------------------------------------------------- generators --

@@ -364,3 +364,73 @@ void q8o_random_q8_0_row(uint64_t *state, size_t blocks, uint8_t *out) {
         }
     }
 }
+
+/* ---- the small f32 operators either side of a product -------------------- */
+
+/* crates/tuckcore/src/forward.rs:917-927: sequential f32 sum of squares,
+ * inv = 1 / sqrt(ss / n + eps), y = (x * inv) * w. */
+void q8o_rmsnorm(const float *x, const float *w, size_t n, float eps, float *y) {
+    float ss = 0.0f;
+    for (size_t i = 0; i < n; ++i) {
+        ss += x[i] * x[i];
+    }
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+    for (size_t i = 0; i < n; ++i) {
+        y[i] = x[i] * inv * w[i];
+    }
+}
+
+/* crates/tuckcore/src/forward.rs:906-908 and the gate of
+ * crates/metal/src/tests.rs:648: (g / (1 + exp(-g))) * up. */
+void q8o_silu_mul(const float *gate, const float *up, size_t n, float *out) {
+    for (size_t i = 0; i < n; ++i) {
+        const float g = gate[i];
+        out[i] = (g / (1.0f + expf(-g))) * up[i];
+    }
+}
+
+/* native/metal/kernels.metal:382-396 (no CPU twin in the reference): ggml's
+ * tanh GELU, 0.5 x (1 + tanh(sqrt(2/pi) x (1 + 0.044715 x^2))) * up. */
+void q8o_gelu_tanh_mul(const float *gate, const float *up, size_t n, float *out) {
+    for (size_t i = 0; i < n; ++i) {
+        const float x = gate[i];
+        const float inner = 0.7978845608028654f * x * (1.0f + 0.044715f * x * x);
+        out[i] = 0.5f * x * (1.0f + tanhf(inner)) * up[i];
+    }
+}
+
+/* native/metal/kernels.metal:26-36: y += alpha * a (multiply, then add). */
+void q8o_axpy(const float *a, float alpha, size_t n, float *y) {
+    for (size_t i = 0; i < n; ++i) {
+        const float p = alpha * a[i];
+        y[i] = y[i] + p;
+    }
+}
+
+/* native/metal/kernels.metal:14-24 */
+void q8o_scale(const float *x, float factor, size_t n, float *y) {
+    for (size_t i = 0; i < n; ++i) {
+        y[i] = x[i] * factor;
+    }
+}
+
+/* crates/backend/src/sampling.rs:69-83: NaN skipped, strict >, so ties go to
+ * the lowest index; 0xFFFFFFFF when every entry is NaN
+ * (crates/metal/src/tests.rs:1257-1270). */
+uint32_t q8o_argmax(const float *x, size_t n) {
+    int have = 0;
+    size_t bi = 0;
+    float bv = 0.0f;
+    for (size_t i = 0; i < n; ++i) {
+        const float v = x[i];
+        if (v != v) {
+            continue;
+        }
+        if (!have || v > bv) {
+            have = 1;
+            bi = i;
+            bv = v;
+        }
+    }
+    return have ? (uint32_t)bi : 0xFFFFFFFFu;
+}

@@ -89,6 +89,18 @@ float q8o_krng_next_f32(uint64_t *state, float scale);
 /* crates/tuckcore/src/kernels.rs:445-456 (random_q8_0_row). */
 void q8o_random_q8_0_row(uint64_t *state, size_t blocks, uint8_t *out);
 
+
+/* ---- the small f32 operators either side of a product --------------------
+ * rmsnorm: crates/tuckcore/src/forward.rs:917-927; silu_mul: forward.rs:906-908;
+ * gelu_tanh_mul: native/metal/kernels.metal:382-396; axpy / scale:
+ * kernels.metal:14-36; argmax: crates/backend/src/sampling.rs:69-83. */
+void q8o_rmsnorm(const float *x, const float *w, size_t n, float eps, float *y);
+void q8o_silu_mul(const float *gate, const float *up, size_t n, float *out);
+void q8o_gelu_tanh_mul(const float *gate, const float *up, size_t n, float *out);
+void q8o_axpy(const float *a, float alpha, size_t n, float *y);
+void q8o_scale(const float *x, float factor, size_t n, float *y);
+uint32_t q8o_argmax(const float *x, size_t n);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,169 @@
+"""GPU parity of the small f32 operators either side of a product.
+
+Follows crates/metal/src/tests.rs:585-654 (rmsnorm, silu_mul; the reference's
+1e-5 * max(|want|, 1) tolerance) and :1250-1350 (argmax: exact, and the
+indirect embedding lookup fed by it).
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from tuckmill_amd import hip as H
+from tuckmill_amd import synth as S
+
+from q8util import bits, require_gpu, upload_new, weights_buffer
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = require_gpu()
+    yield c
+    c.close()
+
+
+def grid_values(rng, n):
+    # the value grid of crates/metal/src/tests.rs:591-593
+    return np.array([((rng.next() % 20_001) - 10_000.0) / 1000.0 for _ in range(n)], np.float32)
+
+
+def close(got, want):
+    return np.all(np.abs(got - want) <= 1e-5 * np.maximum(np.abs(want), 1.0))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1024), (16, 128), (8, 128), (1, 7), (3, 1152), (2, 6912)])
+def test_rmsnorm_matches_the_scalar_reference(ctx, rows, cols):
+    rng = O.Rng(11 + rows + cols)
+    x = grid_values(rng, rows * cols)
+    w = np.array([0.5 + (rng.next() % 1000) / 1000.0 for _ in range(cols)], np.float32)
+    eps = 1e-6
+    xb, wb = upload_new(ctx, x), upload_new(ctx, w)
+    yb = ctx.buffer(rows * cols * 4)
+    ctx.rmsnorm(xb, wb, yb, rows, cols, eps)
+    ctx.fence()
+    got = yb.download_f32(0, rows * cols).reshape(rows, cols)
+    for r in range(rows):
+        assert close(got[r], O.rmsnorm(x[r * cols:(r + 1) * cols], w, eps)), f"row {r}"
+    # in place
+    ctx.rmsnorm(xb, wb, xb, rows, cols, eps)
+    ctx.fence()
+    assert np.array_equal(bits(xb.download_f32(0, rows * cols)), bits(got.reshape(-1)))
+
+
+@pytest.mark.parametrize("n", [3072, 3071, 1, 6912 * 3 + 5])
+def test_gated_activations_match_the_scalar_reference(ctx, n):
+    rng = O.Rng(19 + n)
+    gate, up = grid_values(rng, n), grid_values(rng, n)
+    gb, ub = upload_new(ctx, gate), upload_new(ctx, up)
+    ob = ctx.buffer(n * 4)
+    ctx.silu_mul(gb, ub, ob, n)
+    ctx.fence()
+    assert close(ob.download_f32(0, n), O.silu_mul(gate, up))
+    ctx.gelu_tanh_mul(gb, ub, ob, n)
+    ctx.fence()
+    assert close(ob.download_f32(0, n), O.gelu_tanh_mul(gate, up))
+    # the engine's use: the result overwrites the gate (engine/metal.rs:492)
+    ctx.gelu_tanh_mul(gb, ub, gb, n)
+    ctx.fence()
+    assert close(gb.download_f32(0, n), O.gelu_tanh_mul(gate, up))
+
+
+@pytest.mark.parametrize("n", [1, 255, 1024, 100_003])
+def test_axpy_and_scale_are_bit_exact(ctx, n):
+    a = S.make_activations(n, 5)
+    y = S.make_activations(n, 6)
+    ab, yb = upload_new(ctx, a), upload_new(ctx, y)
+    ctx.f32_axpy(ab, yb, 0.37, n)
+    ctx.fence()
+    assert np.array_equal(bits(yb.download_f32(0, n)), bits(O.axpy(a, 0.37, y)))
+    sb = ctx.buffer(n * 4)
+    ctx.f32_scale(ab, sb, -1.25e-3, n)
+    ctx.fence()
+    assert np.array_equal(bits(sb.download_f32(0, n)), bits(O.scale(a, -1.25e-3)))
+
+
+def test_argmax_matches_the_cpu_greedy_rule_exactly(ctx):
+    # crates/metal/src/tests.rs:1250-1320
+    nan, inf = np.nan, np.inf
+    cases = [np.array(c, np.float32) for c in (
+        [1.0, 3.0, 2.0], [3.0, 3.0], [nan, 1.0], [nan, inf], [nan, nan, nan], [-inf, -inf],
+        [-0.0, 0.0], [0.0, -0.0], [7.5])]
+    rng = O.Rng(0xA11CE)
+    n = 248_320
+    big = np.array([((rng.next() >> 40) / float(1 << 24)) * 20.0 - 10.0 for _ in range(n)],
+                   np.float32)
+    for k in (200_000, 77_777, 131_071, 77_776):
+        big[k] = 42.0
+    big[5] = nan
+    cases.append(big)
+    for ln in (255, 256, 16_384, 16_385, 70_001):
+        v = np.ones(ln, np.float32)
+        v[ln - 1] = 2.0
+        v[ln // 2] = 2.0
+        cases.append(v)
+    partial = ctx.buffer(H.ARGMAX_PARTIAL_BYTES)
+    out = ctx.buffer(8)
+    for c, x in enumerate(cases):
+        xb = upload_new(ctx, x)
+        ctx.argmax_f32(xb, x.size, partial, out, 1)
+        ctx.fence()
+        got = int(out.download(4, 4).view(np.uint32)[0])
+        assert got == O.argmax(x), f"case {c} (len {x.size})"
+        xb.free()
+    empty = ctx.buffer(4)
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.argmax_f32(empty, 0, partial, out, 0)
+    assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS
+    with pytest.raises(H.TuckmillError):
+        ctx.argmax_f32(empty, 1, partial, out, 2)  # out_index past the buffer
+    with pytest.raises(H.TuckmillError):
+        ctx.argmax_f32(empty, 1, ctx.buffer(256), out, 0)  # partial too small
+
+
+def test_a_decode_tail_runs_in_one_group(ctx):
+    # norm -> lm_head GEMV -> argmax -> embedding row of the chosen token, one
+    # commit (the shape of crates/tuckcore/src/engine/metal.rs decode tail).
+    rows, cols = 4096, 1024
+    w = S.make_weights(rows, cols, 77)
+    x = S.make_activations(cols, 78)
+    g = (0.5 + np.abs(S.make_activations(cols, 79))).astype(np.float32)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    xb, gb = upload_new(ctx, x), upload_new(ctx, g)
+    hb, yb = ctx.buffer(cols * 4), ctx.buffer(rows * 4)
+    partial, ids, emb = ctx.buffer(H.ARGMAX_PARTIAL_BYTES), ctx.buffer(8), ctx.buffer(cols * 4)
+    commits = ctx.committed_dispatches()
+    ctx.begin_group()
+    ctx.rmsnorm(xb, gb, hb, 1, cols, 1e-6)
+    ctx.q8_0_gemv(wb, hb, yb, rows, cols)
+    ctx.argmax_f32(yb, rows, partial, ids, 0)
+    ctx.row_indirect_f32(wb, 8, rows, cols, ids, 0, emb)
+    ctx.end_group()
+    assert ctx.committed_dispatches() == commits + 1
+    ctx.fence()
+    h = hb.download_f32(0, cols)
+    assert close(h, O.rmsnorm(x, g, 1e-6))
+    logits = yb.download_f32(0, rows)
+    want_logits = O.gemv_q8_0_f32(w, rows, cols, h)
+    assert np.max(np.abs(logits - want_logits)) <= 1e-5 * np.max(np.abs(want_logits))
+    token = int(ids.download(0, 4).view(np.uint32)[0])
+    assert token == O.argmax(logits)
+    row_bytes = (cols // 32) * 34
+    want_row = O.dequant_q8_0(w[token * row_bytes:(token + 1) * row_bytes])
+    assert np.array_equal(bits(emb.download_f32(0, cols)), bits(want_row))
+
+
+def test_neighbor_argument_refusals(ctx):
+    b = ctx.buffer(64)
+    small = ctx.buffer(8)
+    for call in (lambda: ctx.silu_mul(b, b, b, 0), lambda: ctx.f32_axpy(b, b, 1.0, 0),
+                 lambda: ctx.gelu_tanh_mul(b, small, b, 16), lambda: ctx.f32_scale(b, small, 1.0, 16)):
+        with pytest.raises(H.TuckmillError) as e:
+            call()
+        assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.rmsnorm(b, b, b, 0, 16, 1e-6)
+    assert e.value.abi_code == H.TM_HIP_ERR_UNSUPPORTED
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.rmsnorm(b, small, b, 1, 16, 1e-6)  # weight shorter than cols
+    assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS

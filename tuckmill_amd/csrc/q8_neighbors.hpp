@@ -1,0 +1,167 @@
+// The small f32 operators either side of a Q8_0 product in a decode or prefill
+// step: RMSNorm before the projections, the gated activations and the residual
+// update after them, greedy argmax after the vocabulary projection.
+// Reference kernels: native/metal/kernels.metal:14-36 (scale, axpy), :142-226
+// (argmax), :341-362 (rmsnorm), :382-406 (gelu_tanh_mul, silu_mul); CPU
+// definitions: crates/tuckcore/src/forward.rs:906-927,
+// crates/backend/src/sampling.rs:69-83.
+//
+// All of them move a few KB to a few hundred KB: on this part they are bound by
+// launch latency, not by HBM, so each is one plain kernel (argmax: two) meant to
+// be recorded inside a dispatch group.
+#pragma once
+
+#include "q8_common.hpp"
+
+namespace q8 {
+
+// y[i] = x[i] * factor
+__global__ __launch_bounds__(256) void scale_kernel(const float *x, float *y, float factor,
+                                                    uint32_t n) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) {
+        y[i] = x[i] * factor;
+    }
+}
+
+// y[i] = y[i] + alpha * a[i]   (multiply, then add: no contraction)
+__global__ __launch_bounds__(256) void axpy_kernel(const float *a, float *y, float alpha,
+                                                   uint32_t n) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) {
+        const float p = __fmul_rn(alpha, a[i]);
+        y[i] = __fadd_rn(y[i], p);
+    }
+}
+
+// out[i] = silu(gate[i]) * up[i],  silu(g) = g / (1 + exp(-g))
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float *gate, const float *up,
+                                                       float *out, uint32_t n) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) {
+        const float g = gate[i];
+        const float s = g / (1.0f + expf(-g));
+        out[i] = s * up[i];
+    }
+}
+
+// out[i] = gelu_tanh(gate[i]) * up[i], ggml's tanh form
+// 0.5 x (1 + tanh(sqrt(2/pi) x (1 + 0.044715 x^2))), evaluated in the order of
+// kernels.metal:391-395.
+__global__ __launch_bounds__(256) void gelu_tanh_mul_kernel(const float *gate, const float *up,
+                                                            float *out, uint32_t n) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) {
+        const float x = gate[i];
+        const float inner = 0.7978845608028654f * x * (1.0f + 0.044715f * x * x);
+        out[i] = 0.5f * x * (1.0f + tanhf(inner)) * up[i];
+    }
+}
+
+// One workgroup of 256 threads per row: y = x * (1 / sqrt(mean(x^2) + eps)) * w.
+// The sum of squares is taken per thread over a strided slice, then over the
+// wave by the fixed butterfly and over the four waves in order (deterministic;
+// not the CPU's sequential order, hence tolerance-qualified like the
+// reference's own GPU kernel). In place (x == y) is safe: a thread rereads only
+// the elements it writes, after the barrier.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float *x, const float *weight, float *y,
+                                                      uint32_t cols, float eps) {
+    __shared__ float part[4];
+    const float *xr = x + (size_t)blockIdx.x * cols;
+    float *yr = y + (size_t)blockIdx.x * cols;
+    float acc = 0.0f;
+    for (uint32_t i = threadIdx.x; i < cols; i += 256u) {
+        const float v = xr[i];
+        acc += v * v;
+    }
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63u) == 0u) {
+        part[threadIdx.x >> 6] = acc;
+    }
+    __syncthreads();
+    const float sumsq = ((part[0] + part[1]) + part[2]) + part[3];
+    const float inv = 1.0f / sqrtf(sumsq / (float)cols + eps);
+    for (uint32_t i = threadIdx.x; i < cols; i += 256u) {
+        yr[i] = xr[i] * inv * weight[i];
+    }
+}
+
+// Greedy argmax, the CPU rule: NaN entries are skipped, the largest value
+// wins, ties go to the lowest index; ARGMAX_NONE when every entry is NaN.
+// "a is better than b" is a strict total order on (value, index) pairs, so any
+// reduction tree returns the sequential scan's answer.
+constexpr uint32_t ARGMAX_NONE = 0xffffffffu;
+constexpr uint32_t ARGMAX_GROUPS = 64;   // partial results: 64 f32 values, then 64 u32 indices
+constexpr uint32_t ARGMAX_PARTIAL_BYTES = ARGMAX_GROUPS * 8u;
+
+__device__ __forceinline__ bool argmax_better(float av, uint32_t ai, float bv, uint32_t bi) {
+    if (ai == ARGMAX_NONE) {
+        return false;
+    }
+    if (bi == ARGMAX_NONE) {
+        return true;
+    }
+    return av > bv || (av == bv && ai < bi);
+}
+
+__device__ __forceinline__ void argmax_workgroup(float &v, uint32_t &i, float *tv, uint32_t *ti) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(v, off, WAVE);
+        const uint32_t oi = (uint32_t)__shfl_xor((int)i, off, WAVE);
+        if (argmax_better(ov, oi, v, i)) {
+            v = ov;
+            i = oi;
+        }
+    }
+    const uint32_t wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63u) == 0u) {
+        tv[wave] = v;
+        ti[wave] = i;
+    }
+    __syncthreads();
+    v = tv[0];
+    i = ti[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+        if (argmax_better(tv[w], ti[w], v, i)) {
+            v = tv[w];
+            i = ti[w];
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float *x, float *part_v,
+                                                             uint32_t *part_i, uint32_t n) {
+    __shared__ float tv[4];
+    __shared__ uint32_t ti[4];
+    float v = -__builtin_inff();
+    uint32_t i = ARGMAX_NONE;
+    for (uint32_t k = blockIdx.x * 256u + threadIdx.x; k < n; k += ARGMAX_GROUPS * 256u) {
+        const float xv = x[k];
+        if (xv == xv && argmax_better(xv, k, v, i)) {
+            v = xv;
+            i = k;
+        }
+    }
+    argmax_workgroup(v, i, tv, ti);
+    if (threadIdx.x == 0u) {
+        part_v[blockIdx.x] = v;
+        part_i[blockIdx.x] = i;
+    }
+}
+
+__global__ __launch_bounds__(256) void argmax_final_kernel(const float *part_v,
+                                                           const uint32_t *part_i, uint32_t *out,
+                                                           uint32_t out_index) {
+    __shared__ float tv[4];
+    __shared__ uint32_t ti[4];
+    float v = threadIdx.x < ARGMAX_GROUPS ? part_v[threadIdx.x] : -__builtin_inff();
+    uint32_t i = threadIdx.x < ARGMAX_GROUPS ? part_i[threadIdx.x] : ARGMAX_NONE;
+    argmax_workgroup(v, i, tv, ti);
+    if (threadIdx.x == 0u) {
+        out[out_index] = i;
+    }
+}
+
+} // namespace q8

@@ -27,6 +27,7 @@
 #include "q8_gemv.hpp"
 #include "q8_gemm_small.hpp"
 #include "q8_misc.hpp"
+#include "q8_neighbors.hpp"
 
 namespace {
 
@@ -51,7 +52,10 @@ void alloc_release(Alloc *a) {
     }
 }
 
-enum OpKind { OP_GEMV_LIST, OP_MMA, OP_ROW, OP_ROW_INDIRECT, OP_COPY, OP_PACK, OP_QUANT, OP_I8 };
+enum OpKind {
+    OP_GEMV_LIST, OP_MMA, OP_ROW, OP_ROW_INDIRECT, OP_COPY, OP_PACK, OP_QUANT, OP_I8,
+    OP_SCALE, OP_AXPY, OP_SILU_MUL, OP_GELU_MUL, OP_RMSNORM, OP_ARGMAX
+};
 
 struct Op {
     OpKind kind;
@@ -59,6 +63,7 @@ struct Op {
     int n_alloc = 0;
     unsigned writes_mask = 0; // bit i: a[i] is written
     uint32_t rows = 0, cols = 0, batch = 0, x_off = 0, y_off = 0, extra = 0;
+    float scalar = 0.0f;       // factor / alpha / eps of the small f32 operators
     bool packed = false;
     bool shape_label = false;  // profile label carries "<rows>x<cols>"
     const char *what = "";     // static operator name
@@ -454,6 +459,42 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
         float *dst = (float *)op.a[1]->ptr + op.y_off;
         Q8_LAUNCH(q8::copy_f32_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop, src,
                   dst, op.extra);
+        break;
+    }
+    case OP_SCALE:
+        Q8_LAUNCH(q8::scale_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
+                  (const float *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.scalar, op.extra);
+        break;
+    case OP_AXPY:
+        Q8_LAUNCH(q8::axpy_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
+                  (const float *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.scalar, op.extra);
+        break;
+    case OP_SILU_MUL:
+        Q8_LAUNCH(q8::silu_mul_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
+                  (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
+                  op.extra);
+        break;
+    case OP_GELU_MUL:
+        Q8_LAUNCH(q8::gelu_tanh_mul_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
+                  (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
+                  op.extra);
+        break;
+    case OP_RMSNORM:
+        Q8_LAUNCH(q8::rmsnorm_kernel, dim3(op.rows), dim3(256), 0, st, stop,
+                  (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
+                  op.cols, op.scalar);
+        break;
+    case OP_ARGMAX: {
+        float *part_v = (float *)op.a[1]->ptr;
+        uint32_t *part_i = (uint32_t *)((uint8_t *)op.a[1]->ptr + q8::ARGMAX_GROUPS * 4u);
+        hipLaunchKernelGGL(q8::argmax_partial_kernel, dim3(q8::ARGMAX_GROUPS), dim3(256), 0, st,
+                           (const float *)op.a[0]->ptr, part_v, part_i, op.extra);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            return e;
+        }
+        Q8_LAUNCH(q8::argmax_final_kernel, dim3(1), dim3(256), 0, st, stop, (const float *)part_v,
+                  (const uint32_t *)part_i, (uint32_t *)op.a[2]->ptr, op.y_off);
         break;
     }
     case OP_PACK: {
@@ -1025,6 +1066,156 @@ int tm_hip_copy_f32(tm_hip_ctx *ctx, tm_hip_buffer *src, uint32_t src_off, tm_hi
     op.y_off = dst_off;
     op.extra = n;
     return submit(ctx, op, "copy_f32", err, err_cap);
+}
+
+// ---- the small f32 operators either side of a product ----------------------
+
+namespace {
+
+// x -> y over n f32 elements with one scalar (native/metal/tm_metal.m:770-810).
+int submit_1d(tm_hip_ctx *ctx, OpKind kind, tm_hip_buffer *a, tm_hip_buffer *b, float scalar,
+              uint32_t n, char *err, size_t cap, const char *what) {
+    if (check_ctx(ctx, err, cap, what) != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (n == 0) {
+        return fail(err, cap, TM_HIP_ERR_BOUNDS, "%s: zero length", what);
+    }
+    int rc;
+    if ((rc = check_buffer(ctx, a, (size_t)n * 4u, err, cap, what)) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, b, (size_t)n * 4u, err, cap, what)) != TM_HIP_OK) {
+        return rc;
+    }
+    if (a->alloc->packed || b->alloc->packed) {
+        return fail(err, cap, TM_HIP_ERR_UNSUPPORTED, "%s: sealed weight buffer", what);
+    }
+    Op op;
+    op.kind = kind;
+    op.a[0] = a->alloc;
+    op.a[1] = b->alloc;
+    op.n_alloc = 2;
+    op.writes_mask = 2;
+    op.extra = n;
+    op.scalar = scalar;
+    return submit(ctx, op, what, err, cap);
+}
+
+// out[i] = f(gate[i]) * up[i] (native/metal/tm_metal.m:1143-1177).
+int submit_glu(tm_hip_ctx *ctx, OpKind kind, tm_hip_buffer *gate, tm_hip_buffer *up,
+               tm_hip_buffer *out, uint32_t n, char *err, size_t cap, const char *what) {
+    if (check_ctx(ctx, err, cap, what) != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (n == 0) {
+        return fail(err, cap, TM_HIP_ERR_BOUNDS, "%s: zero length", what);
+    }
+    tm_hip_buffer *bufs[3] = {gate, up, out};
+    static const char *const names[3] = {"gate", "up", "out"};
+    for (int i = 0; i < 3; ++i) {
+        char name[64];
+        snprintf(name, sizeof name, "%s.%s", what, names[i]);
+        const int rc = check_buffer(ctx, bufs[i], (size_t)n * 4u, err, cap, name);
+        if (rc != TM_HIP_OK) {
+            return rc;
+        }
+        if (bufs[i]->alloc->packed) {
+            return fail(err, cap, TM_HIP_ERR_UNSUPPORTED, "%s: sealed weight buffer", name);
+        }
+    }
+    Op op;
+    op.kind = kind;
+    op.a[0] = gate->alloc;
+    op.a[1] = up->alloc;
+    op.a[2] = out->alloc;
+    op.n_alloc = 3;
+    op.writes_mask = 4;
+    op.extra = n;
+    return submit(ctx, op, what, err, cap);
+}
+
+} // namespace
+
+int tm_hip_f32_scale(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *y, float factor, uint32_t n,
+                     char *err, size_t err_cap) {
+    return submit_1d(ctx, OP_SCALE, x, y, factor, n, err, err_cap, "f32_scale");
+}
+
+int tm_hip_f32_axpy(tm_hip_ctx *ctx, tm_hip_buffer *a, tm_hip_buffer *y, float alpha, uint32_t n,
+                    char *err, size_t err_cap) {
+    return submit_1d(ctx, OP_AXPY, a, y, alpha, n, err, err_cap, "f32_axpy");
+}
+
+int tm_hip_silu_mul_f32(tm_hip_ctx *ctx, tm_hip_buffer *gate, tm_hip_buffer *up, tm_hip_buffer *out,
+                        uint32_t n, char *err, size_t err_cap) {
+    return submit_glu(ctx, OP_SILU_MUL, gate, up, out, n, err, err_cap, "silu_mul");
+}
+
+int tm_hip_gelu_tanh_mul_f32(tm_hip_ctx *ctx, tm_hip_buffer *gate, tm_hip_buffer *up,
+                             tm_hip_buffer *out, uint32_t n, char *err, size_t err_cap) {
+    return submit_glu(ctx, OP_GELU_MUL, gate, up, out, n, err, err_cap, "gelu_tanh_mul");
+}
+
+int tm_hip_rmsnorm_f32(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *weight, tm_hip_buffer *y,
+                       uint32_t rows, uint32_t cols, float eps, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "rmsnorm") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (rows == 0 || cols == 0) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "rmsnorm: zero shape");
+    }
+    const size_t x_need = (size_t)rows * cols * 4u;
+    int rc;
+    if ((rc = check_buffer(ctx, x, x_need, err, err_cap, "rmsnorm.x")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, weight, (size_t)cols * 4u, err, err_cap, "rmsnorm.weight")) !=
+            TM_HIP_OK ||
+        (rc = check_buffer(ctx, y, x_need, err, err_cap, "rmsnorm.y")) != TM_HIP_OK) {
+        return rc;
+    }
+    if (x->alloc->packed || weight->alloc->packed || y->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "rmsnorm: sealed weight buffer");
+    }
+    Op op;
+    op.kind = OP_RMSNORM;
+    op.a[0] = x->alloc;
+    op.a[1] = weight->alloc;
+    op.a[2] = y->alloc;
+    op.n_alloc = 3;
+    op.writes_mask = 4;
+    op.rows = rows;
+    op.cols = cols;
+    op.scalar = eps;
+    return submit(ctx, op, "rmsnorm", err, err_cap);
+}
+
+int tm_hip_argmax_f32(tm_hip_ctx *ctx, tm_hip_buffer *x, uint32_t n, tm_hip_buffer *partial,
+                      tm_hip_buffer *out, uint32_t out_index, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "argmax_f32") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (n == 0) {
+        return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "argmax_f32: empty input");
+    }
+    int rc;
+    if ((rc = check_buffer(ctx, x, (size_t)n * 4u, err, err_cap, "argmax_f32.x")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, partial, q8::ARGMAX_PARTIAL_BYTES, err, err_cap,
+                           "argmax_f32.partial")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, out, ((size_t)out_index + 1u) * 4u, err, err_cap,
+                           "argmax_f32.out")) != TM_HIP_OK) {
+        return rc;
+    }
+    if (x->alloc->packed || partial->alloc->packed || out->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "argmax_f32: sealed weight buffer");
+    }
+    Op op;
+    op.kind = OP_ARGMAX;
+    op.a[0] = x->alloc;
+    op.a[1] = partial->alloc;
+    op.a[2] = out->alloc;
+    op.n_alloc = 3;
+    op.writes_mask = 6;
+    op.extra = n;
+    op.y_off = out_index;
+    return submit(ctx, op, "argmax_f32", err, err_cap);
 }
 
 int tm_hip_begin_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {

@@ -25,6 +25,8 @@ ERR_CAP = 512  # crates/metal/src/lib.rs:32
 GEMM_MAX_BATCH = 32  # crates/metal/src/lib.rs:28-30
 GEMM_MMA_MAX_BATCH = 512
 GEMM_I8_MAX_BATCH = 2048
+ARGMAX_NONE = 0xFFFFFFFF  # crates/metal/src/lib.rs (ARGMAX_NONE), native/metal/kernels.metal:143
+ARGMAX_PARTIAL_BYTES = 512
 STAGING_CHUNK_BYTES = 4 << 20  # crates/tuckcore/src/qwen35_gpu.rs:1176
 
 TM_HIP_ERR_NO_DEVICE = -1
@@ -80,6 +82,24 @@ _SIGS = {
     "tm_hip_download_after": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
                                              ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
                                              ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_f32_scale": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                         ctypes.c_float, ctypes.c_uint32, ctypes.c_char_p,
+                                         ctypes.c_size_t]),
+    "tm_hip_f32_axpy": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                        ctypes.c_float, ctypes.c_uint32, ctypes.c_char_p,
+                                        ctypes.c_size_t]),
+    "tm_hip_rmsnorm_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                           ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32,
+                                           ctypes.c_float, ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_silu_mul_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                            ctypes.c_void_p, ctypes.c_uint32, ctypes.c_char_p,
+                                            ctypes.c_size_t]),
+    "tm_hip_gelu_tanh_mul_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                 ctypes.c_void_p, ctypes.c_uint32, ctypes.c_char_p,
+                                                 ctypes.c_size_t]),
+    "tm_hip_argmax_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
+                                          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
+                                          ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_copy_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
                                        ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32,
                                        ctypes.c_char_p, ctypes.c_size_t]),
@@ -266,6 +286,29 @@ class HipContext:
         self._check_owned(w, ids, out)
         self._operate("row_indirect", self._lib.tm_hip_row_indirect_f32, w.raw, type_id, rows, cols,
                       ids.raw, slot, out.raw)
+
+    # -- the small f32 operators either side of a product (crates/metal/src/lib.rs:1027-1060,
+    #    :2244-2319) --
+    def f32_scale(self, x, y, factor, n):
+        self._operate("f32_scale", self._lib.tm_hip_f32_scale, x.raw, y.raw, float(factor), n)
+
+    def f32_axpy(self, a, y, alpha, n):
+        self._operate("f32_axpy", self._lib.tm_hip_f32_axpy, a.raw, y.raw, float(alpha), n)
+
+    def rmsnorm(self, x, weight, y, rows, cols, eps):
+        self._operate("rmsnorm", self._lib.tm_hip_rmsnorm_f32, x.raw, weight.raw, y.raw, rows, cols,
+                      float(eps))
+
+    def silu_mul(self, gate, up, out, n):
+        self._operate("silu_mul", self._lib.tm_hip_silu_mul_f32, gate.raw, up.raw, out.raw, n)
+
+    def gelu_tanh_mul(self, gate, up, out, n):
+        self._operate("gelu_tanh_mul", self._lib.tm_hip_gelu_tanh_mul_f32, gate.raw, up.raw,
+                      out.raw, n)
+
+    def argmax_f32(self, x, n, partial, out, out_index):
+        self._operate("argmax_f32", self._lib.tm_hip_argmax_f32, x.raw, n, partial.raw, out.raw,
+                      out_index)
 
     def copy_f32(self, src, src_off, dst, dst_off, n):
         self._check_owned(src, dst)

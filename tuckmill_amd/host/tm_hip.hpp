@@ -236,6 +236,44 @@ class HipContext {
                                            out.raw(), e, ERR_CAP);
         });
     }
+    // The small f32 operators either side of a product
+    // (crates/metal/src/lib.rs:1027-1060, :2244-2319).
+    void f32_scale(const HipBuffer &x, const HipBuffer &y, float factor, uint32_t n) const {
+        operate("f32_scale", [&](char *e) {
+            return tm_hip_f32_scale(raw(), x.raw(), y.raw(), factor, n, e, ERR_CAP);
+        });
+    }
+    void f32_axpy(const HipBuffer &a, const HipBuffer &y, float alpha, uint32_t n) const {
+        operate("f32_axpy", [&](char *e) {
+            return tm_hip_f32_axpy(raw(), a.raw(), y.raw(), alpha, n, e, ERR_CAP);
+        });
+    }
+    void rmsnorm(const HipBuffer &x, const HipBuffer &weight, const HipBuffer &y, uint32_t rows,
+                 uint32_t cols, float eps) const {
+        operate("rmsnorm", [&](char *e) {
+            return tm_hip_rmsnorm_f32(raw(), x.raw(), weight.raw(), y.raw(), rows, cols, eps, e,
+                                      ERR_CAP);
+        });
+    }
+    void silu_mul(const HipBuffer &gate, const HipBuffer &up, const HipBuffer &out,
+                  uint32_t n) const {
+        operate("silu_mul", [&](char *e) {
+            return tm_hip_silu_mul_f32(raw(), gate.raw(), up.raw(), out.raw(), n, e, ERR_CAP);
+        });
+    }
+    void gelu_tanh_mul(const HipBuffer &gate, const HipBuffer &up, const HipBuffer &out,
+                       uint32_t n) const {
+        operate("gelu_tanh_mul", [&](char *e) {
+            return tm_hip_gelu_tanh_mul_f32(raw(), gate.raw(), up.raw(), out.raw(), n, e, ERR_CAP);
+        });
+    }
+    void argmax_f32(const HipBuffer &x, uint32_t n, const HipBuffer &partial, const HipBuffer &out,
+                    uint32_t out_index) const {
+        operate("argmax_f32", [&](char *e) {
+            return tm_hip_argmax_f32(raw(), x.raw(), n, partial.raw(), out.raw(), out_index, e,
+                                     ERR_CAP);
+        });
+    }
     void q8_0_pack(const HipBuffer &w, uint32_t rows, uint32_t cols) const {
         operate("q8_0_pack",
                 [&](char *e) { return tm_hip_q8_0_pack(raw(), w.raw(), rows, cols, e, ERR_CAP); });
