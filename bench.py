@@ -54,6 +54,7 @@ class tmh_timing(ctypes.Structure):
 
 
 TMH_GEMV, TMH_GEMM, TMH_GEMM_MMA, TMH_GEMM_I8, TMH_QUANT = range(5)
+TMH_RMSNORM, TMH_SILU_MUL, TMH_AXPY, TMH_ARGMAX = range(5, 9)
 
 
 def load_host():
@@ -323,6 +324,78 @@ def bench_sweep(host, ctx, steps, warmup):
     return out
 
 
+def bench_chain(host, ctx, steps, warmup):
+    """The decode step with its data dependencies: per layer rmsnorm -> q,k,v -> o ->
+    residual -> rmsnorm -> gate,up -> silu_mul -> down -> residual, then final norm,
+    lm_head and greedy argmax, Qwen3-0.6B shapes, one dispatch group per token
+    (attention, RoPE and the KV cache are not part of this path: o reads a stand-in
+    buffer). Products that do not depend on each other still share a launch (q,k,v and
+    gate,up), everything else is ordered, so the step is bound by launch latency, not by
+    HBM: this is the figure a graph replay or wider fusion would have to beat."""
+    hidden, qdim, kvdim, ffn, vocab = 1024, 2048, 1024, 3072, 151_936
+    layers = S.QWEN3_0_6B_LAYERS
+    keep, prods = [], []
+
+    def fbuf(n, seed=None):
+        b = ctx.buffer(n * 4)
+        if seed is not None:
+            b.upload(0, S.make_activations(n, seed))
+        keep.append(b)
+        return b
+
+    def mat(rows, cols, seed):
+        m = H.Matrix.load(ctx, S.make_weights(rows, cols, seed), cols, rows)
+        keep.append(m)
+        return m
+
+    h, n, t = fbuf(hidden, 1), fbuf(hidden), fbuf(hidden)
+    q, k, v, attn = fbuf(qdim), fbuf(kvdim), fbuf(kvdim), fbuf(qdim, 2)
+    gate, up = fbuf(ffn), fbuf(ffn)
+    logits, partial, token = fbuf(vocab), ctx.buffer(H.ARGMAX_PARTIAL_BYTES), ctx.buffer(8)
+    keep += [partial, token]
+    wbytes = 0
+
+    def product(m, x, y, rows, cols):
+        nonlocal wbytes
+        wbytes += S.gemv_bytes(rows, cols)
+        prods.append(tmh_product(m.buf.raw, x.raw, y.raw, rows, cols, 1, TMH_GEMV))
+
+    for layer in range(layers):
+        g1, g2 = fbuf(hidden, 100 + layer), fbuf(hidden, 200 + layer)
+        prods.append(tmh_product(g1.raw, h.raw, n.raw, 1, hidden, 1, TMH_RMSNORM))
+        product(mat(qdim, hidden, 5000 + 7 * layer), n, q, qdim, hidden)
+        product(mat(kvdim, hidden, 5001 + 7 * layer), n, k, kvdim, hidden)
+        product(mat(kvdim, hidden, 5002 + 7 * layer), n, v, kvdim, hidden)
+        product(mat(hidden, qdim, 5003 + 7 * layer), attn, t, hidden, qdim)
+        prods.append(tmh_product(h.raw, t.raw, h.raw, 1, hidden, 1, TMH_AXPY))
+        prods.append(tmh_product(g2.raw, h.raw, n.raw, 1, hidden, 1, TMH_RMSNORM))
+        product(mat(ffn, hidden, 5004 + 7 * layer), n, gate, ffn, hidden)
+        product(mat(ffn, hidden, 5005 + 7 * layer), n, up, ffn, hidden)
+        prods.append(tmh_product(gate.raw, up.raw, gate.raw, 1, ffn, 1, TMH_SILU_MUL))
+        product(mat(hidden, ffn, 5006 + 7 * layer), gate, t, hidden, ffn)
+        prods.append(tmh_product(h.raw, t.raw, h.raw, 1, hidden, 1, TMH_AXPY))
+    gf = fbuf(hidden, 999)
+    prods.append(tmh_product(gf.raw, h.raw, n.raw, 1, hidden, 1, TMH_RMSNORM))
+    product(mat(vocab, hidden, 6000), n, logits, vocab, hidden)
+    prods.append(tmh_product(partial.raw, logits.raw, token.raw, 1, vocab, 1, TMH_ARGMAX))
+    ctx.fence()
+    tg = run_steps(host, ctx, prods, warmup, steps, grouped=True)
+    out = {"workload": "Qwen3-0.6B decode step with data dependencies (no attention)",
+           "operators_per_step": len(prods), "algorithmic_bytes": wbytes,
+           "grouped": {"us": tg.wall_ms / steps * 1e3, "gpu_us": tg.gpu_ms / steps * 1e3,
+                       "launches_per_step": tg.launches / steps,
+                       "gbs": wbytes / (tg.wall_ms / steps * 1e-3) / 1e9,
+                       "host_issue_us": tg.host_ms / steps * 1e3}}
+    n_un = max(10, steps // 10)
+    tu = run_steps(host, ctx, prods, 3, n_un, grouped=False)
+    out["one_commit_per_operator"] = {"us": tu.wall_ms / n_un * 1e3,
+                                      "launches_per_step": tu.launches / n_un,
+                                      "gbs": wbytes / (tu.wall_ms / n_un * 1e-3) / 1e9}
+    for obj in keep:
+        (obj.buf if isinstance(obj, H.Matrix) else obj).free()
+    return out
+
+
 def run_traffic(host, ctx):
     """A short, fixed sequence for hardware-counter runs (rocprofv3 --pmc):
     a plain f32 copy of known size (the calibration kernel: 256 MiB read,
@@ -356,7 +429,7 @@ def main():
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--ungrouped", action="store_true",
                     help="one commit per GEMV instead of one group per step")
-    ap.add_argument("--workload", choices=["decode", "gemma", "sweep", "traffic"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "gemma", "sweep", "chain", "traffic"], default="decode",
                     help="decode (default, the headline line); gemma / sweep print the "
                          "BASELINE config 3 / 4 measurements as one JSON object")
     args = ap.parse_args()
@@ -373,7 +446,7 @@ def main():
         ctx.close()
         return
     if args.workload != "decode":
-        fn = bench_gemma if args.workload == "gemma" else bench_sweep
+        fn = {"gemma": bench_gemma, "sweep": bench_sweep, "chain": bench_chain}[args.workload]
         print(json.dumps(fn(host, ctx, args.steps, args.warmup)), flush=True)
         ctx.close()
         return

@@ -167,3 +167,54 @@ def test_neighbor_argument_refusals(ctx):
     with pytest.raises(H.TuckmillError) as e:
         ctx.rmsnorm(b, small, b, 1, 16, 1e-6)  # weight shorter than cols
     assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS
+
+
+@pytest.mark.parametrize("packed", [True, False])
+def test_residual_update_behind_its_product_shares_the_launch(ctx, packed):
+    # o-projection followed by h += t, as in every layer of a decode step: inside
+    # a group the update rides in the product's epilogue (one launch instead of
+    # two) and must give the bits of the two separate operators.
+    rows, cols = 1024, 2048
+    w = S.make_weights(rows, cols, 91)
+    x = S.make_activations(cols, 92)
+    h0 = S.make_activations(rows, 93)
+    wb = weights_buffer(ctx, w, rows, cols, packed)
+    xb = upload_new(ctx, x)
+    results = []
+    for grouped in (False, True):
+        hb, tb = upload_new(ctx, h0), ctx.buffer(rows * 4)
+        launches = ctx.kernel_launches()
+        if grouped:
+            ctx.begin_group()
+        ctx.q8_0_gemv(wb, xb, tb, rows, cols)
+        ctx.f32_axpy(tb, hb, 0.5, rows)
+        if grouped:
+            ctx.end_group()
+        ctx.fence()
+        assert ctx.kernel_launches() - launches == (1 if grouped else 2)
+        results.append((tb.download_f32(0, rows).copy(), hb.download_f32(0, rows).copy()))
+    assert np.array_equal(bits(results[0][0]), bits(results[1][0]))
+    assert np.array_equal(bits(results[0][1]), bits(results[1][1]))
+    t = O.gemv_q8_0_f32(w, rows, cols, x)
+    assert np.max(np.abs(results[1][0] - t)) <= 1e-5 * np.max(np.abs(t))
+    assert np.array_equal(bits(results[1][1]), bits(O.axpy(results[1][0], 0.5, h0)))
+
+
+def test_residual_update_is_not_fused_when_it_would_reorder_accesses(ctx):
+    # h is also the product's input: the update must wait for the whole product.
+    rows = cols = 1024
+    w = S.make_weights(rows, cols, 94)
+    h0 = S.make_activations(cols, 95)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    hb, tb = upload_new(ctx, h0), ctx.buffer(rows * 4)
+    launches = ctx.kernel_launches()
+    ctx.begin_group()
+    ctx.q8_0_gemv(wb, hb, tb, rows, cols)
+    ctx.f32_axpy(tb, hb, 1.0, rows)
+    ctx.end_group()
+    ctx.fence()
+    assert ctx.kernel_launches() - launches == 2
+    t = tb.download_f32(0, rows)
+    want_t = O.gemv_q8_0_f32(w, rows, cols, h0)
+    assert np.max(np.abs(t - want_t)) <= 1e-5 * np.max(np.abs(want_t))
+    assert np.array_equal(bits(hb.download_f32(0, rows)), bits(O.axpy(t, 1.0, h0)))

@@ -14,7 +14,8 @@ import pytest
 
 from tuckmill_amd import build as B
 
-DECODE_KERNEL = "_ZN2q816gemv_list_kernelILi1ELi8ELi1ELb1ELi0EEEvNS_8GemvArgsE"
+# gemv_list_kernel<PACKED, 8 rows, 1 token, aligned x, no tail set, any list capacity>
+DECODE_KERNEL = re.compile(r"Function Name: _ZN2q816gemv_list_kernelILi1ELi8ELi1ELb1ELi0ELi\d+EEE")
 
 
 def test_decode_kernel_keeps_four_waves_per_simd(tmp_path):
@@ -28,11 +29,12 @@ def test_decode_kernel_keeps_four_waves_per_simd(tmp_path):
     res = subprocess.run(cmd, capture_output=True, text=True)
     assert res.returncode == 0, res.stderr[-2000:]
     lines = res.stderr.splitlines()
-    start = [i for i, l in enumerate(lines) if "Function Name: " + DECODE_KERNEL in l]
+    start = [i for i, l in enumerate(lines) if DECODE_KERNEL.search(l)]
     assert start, "decode kernel not found in the resource remarks"
-    block = "\n".join(lines[start[0]:start[0] + 14])
-    vgprs = int(re.search(r" VGPRs: (\d+)", block).group(1))
-    spill = int(re.search(r"VGPRs Spill: (\d+)", block).group(1))
-    occupancy = int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", block).group(1))
-    assert spill == 0
-    assert vgprs <= 128 and occupancy >= 4, f"{vgprs} VGPRs, {occupancy} waves/SIMD"
+    for at in start:  # the long- and the short-list instantiation
+        block = "\n".join(lines[at:at + 14])
+        vgprs = int(re.search(r" VGPRs: (\d+)", block).group(1))
+        spill = int(re.search(r"VGPRs Spill: (\d+)", block).group(1))
+        occupancy = int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", block).group(1))
+        assert spill == 0
+        assert vgprs <= 128 and occupancy >= 4, f"{vgprs} VGPRs, {occupancy} waves/SIMD"

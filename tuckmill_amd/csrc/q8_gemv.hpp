@@ -31,19 +31,30 @@ struct GemvDesc {
     uint32_t tile_begin;   // index of this product's first tile in the launch
     uint32_t rows_per_tile;
     uint32_t pad;
+    // Optional fused residual update (one token only): res[r] += alpha * y[r],
+    // multiply then add, exactly what a separate axpy over y would compute.
+    float *res;
+    float alpha;
+    uint32_t pad2;
 };
 
 // The list travels in the kernel-argument segment (read through the scalar
-// cache): 256 * 48 + 16 = 12304 bytes, enough for a whole decode step of a
+// cache): 224 * 64 + 16 = 14352 bytes, enough for a whole decode step of a
 // 28-layer model (197 products) in one launch.
-constexpr int GEMV_MAX_DESCS = 256;
+constexpr int GEMV_MAX_DESCS = 224;
 
-struct GemvArgs {
+template <int ND> struct GemvArgsT {
     uint32_t n;
     uint32_t total_tiles;
     uint32_t pad[2];
-    GemvDesc d[GEMV_MAX_DESCS];
+    GemvDesc d[ND];
 };
+using GemvArgs = GemvArgsT<GEMV_MAX_DESCS>;
+
+// Most launches of a real step carry one to three products (q/k/v, gate/up, a
+// lone projection between two dependent operators): they use a short argument
+// block instead of the 12 KB one, which is copied and fetched per launch.
+constexpr int GEMV_FEW_DESCS = 4;
 
 template <int NB, bool XA>
 __device__ __forceinline__ void load_x(const float *p, float *out) {
@@ -111,7 +122,8 @@ __device__ __forceinline__ void chunk(const WView<L> &wv, const float *x, uint32
 // q8::wave_sum, hence the same bits.
 template <int R>
 __device__ __forceinline__ void reduce_store(const float (&acc)[R], float *y, uint32_t r0,
-                                             uint32_t row_end, uint32_t lane, bool token_ok) {
+                                             uint32_t row_end, uint32_t lane, bool token_ok,
+                                             float *res = nullptr, float alpha = 0.0f) {
     if constexpr (R == 8) {
         float a4[4], a2[2];
 #pragma unroll
@@ -135,6 +147,9 @@ __device__ __forceinline__ void reduce_store(const float (&acc)[R], float *y, ui
         const uint32_t r = ((lane >> 5) & 1u) * 4u + ((lane >> 4) & 1u) * 2u + ((lane >> 3) & 1u);
         if ((lane & 7u) == 0u && r0 + r < row_end && token_ok) {
             y[r0 + r] = a1;
+            if (res != nullptr) {
+                res[r0 + r] = __fadd_rn(res[r0 + r], __fmul_rn(alpha, a1));
+            }
         }
     } else {
 #pragma unroll
@@ -142,6 +157,9 @@ __device__ __forceinline__ void reduce_store(const float (&acc)[R], float *y, ui
             const float total = wave_sum(acc[r]);
             if (lane == 0u && r0 + r < row_end && token_ok) {
                 y[r0 + r] = total;
+                if (res != nullptr) {
+                    res[r0 + r] = __fadd_rn(res[r0 + r], __fmul_rn(alpha, total));
+                }
             }
         }
     }
@@ -161,7 +179,7 @@ __device__ __forceinline__ void reduce_store(const float (&acc)[R], float *y, ui
 template <int R, bool XA, int TAILMASK>
 __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const float *x, float *y,
                                             uint32_t cols, uint32_t row_first, uint32_t row_end,
-                                            uint32_t lane) {
+                                            uint32_t lane, float *res, float alpha) {
     constexpr bool T8 = (TAILMASK & 512) != 0, T4 = (TAILMASK & 256) != 0;
     constexpr bool T2 = (TAILMASK & 128) != 0, T1 = (TAILMASK & 64) != 0;
     constexpr bool TH = (TAILMASK & 32) != 0;
@@ -271,7 +289,7 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const float
             acc[r] = __builtin_fmaf(f16_bits_to_f32(sb[r]), piece_dot<16>(q[r], xv), acc[r]);
         }
         if (cn == 0u) {
-            reduce_store<R>(acc, y, r0, row_end, lane, true);
+            reduce_store<R>(acc, y, r0, row_end, lane, true, res, alpha);
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -290,8 +308,8 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const float
 // (cols a multiple of 1024 only; fewest registers, the Qwen3 shapes), 1 = also
 // cols % 1024 == 128 and == 768 (the Gemma-3-1B shapes). The host picks the
 // smallest set that covers the products of a launch.
-template <int L, int R, int TB, bool XA, int TAILS = 0>
-__global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
+template <int L, int R, int TB, bool XA, int TAILS = 0, int ND = GEMV_MAX_DESCS>
+__global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t tile = blockIdx.x * 4u + wave;
@@ -333,16 +351,16 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
         if (full >= 1u) {
             const uint32_t tail = cols & 1023u;
             if (tail == 0u) {
-                stream_rows<R, XA, 0>(wv, x, y, cols, row_first, row_end, lane);
+                stream_rows<R, XA, 0>(wv, x, y, cols, row_first, row_end, lane, d.res, d.alpha);
                 return;
             }
             if constexpr (TAILS >= 1) {
                 if (tail == 128u) { // hidden 1152 (Gemma-3-1B)
-                    stream_rows<R, XA, 128>(wv, x, y, cols, row_first, row_end, lane);
+                    stream_rows<R, XA, 128>(wv, x, y, cols, row_first, row_end, lane, d.res, d.alpha);
                     return;
                 }
                 if (tail == 768u) { // FFN 6912 (Gemma-3-1B); half the rows per pass
-                    stream_rows<R / 2, XA, 768>(wv, x, y, cols, row_first, row_end, lane);
+                    stream_rows<R / 2, XA, 768>(wv, x, y, cols, row_first, row_end, lane, d.res, d.alpha);
                     return;
                 }
             }
@@ -406,7 +424,7 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgs args) {
                     col_acc[r] = acc[r][t];
                 }
                 reduce_store<R>(col_acc, y + (size_t)(t0 + t) * rows, r0, row_end, lane,
-                                t0 + t < batch);
+                                t0 + t < batch, d.res, d.alpha); // res is only set for one token
             }
         }
     }

@@ -314,6 +314,23 @@ template <int L, int R, int TB, bool XA>
 hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args, bool tails) {
     const uint32_t groups = (args.total_tiles + 3u) / 4u;
     if constexpr (L == q8::PACKED && TB == 1) {
+        if (args.n <= (uint32_t)q8::GEMV_FEW_DESCS) { // short argument block
+            q8::GemvArgsT<q8::GEMV_FEW_DESCS> few;
+            few.n = args.n;
+            few.total_tiles = args.total_tiles;
+            few.pad[0] = few.pad[1] = 0;
+            for (uint32_t i = 0; i < args.n; ++i) {
+                few.d[i] = args.d[i];
+            }
+            if (tails) {
+                Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1, q8::GEMV_FEW_DESCS>), dim3(groups),
+                          dim3(256), 0, ctx->stream, stop, few);
+            } else {
+                Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 0, q8::GEMV_FEW_DESCS>), dim3(groups),
+                          dim3(256), 0, ctx->stream, stop, few);
+            }
+            return hipGetLastError();
+        }
         if (tails) {
             Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1>), dim3(groups), dim3(256), 0,
                       ctx->stream, stop, args);
@@ -359,7 +376,7 @@ hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<co
 }
 
 hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
-                            GemvKey key) {
+                            const std::vector<const Op *> &residual, GemvKey key) {
     if (key.kind == OP_MMA) {
         return launch_mma_list(ctx, stop, ops, key);
     }
@@ -387,6 +404,10 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<
         d.tile_begin = tiles;
         d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
         d.pad = 0;
+        const Op *fused = residual[args.n - 1];
+        d.res = fused != nullptr ? (float *)fused->a[1]->ptr : nullptr;
+        d.alpha = fused != nullptr ? fused->scalar : 0.0f;
+        d.pad2 = 0;
         tiles += (op->rows + d.rows_per_tile - 1) / d.rows_per_tile;
     }
     args.total_tiles = tiles;
@@ -515,6 +536,7 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
 // One kernel launch of a commit: a list of products, or a single operation.
 struct Launch {
     std::vector<const Op *> list; // empty: `single`
+    std::vector<const Op *> residual; // per list entry: an axpy fused into it, or null
     GemvKey key{};
     const Op *single = nullptr;
 };
@@ -556,6 +578,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             }
             cur.key = key;
             cur.list.push_back(&op);
+            cur.residual.push_back(nullptr);
             op.a[0]->read_epoch = epoch;
             op.a[1]->read_epoch = epoch;
             op.a[2]->write_epoch = epoch;
@@ -563,6 +586,22 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 op.a[3]->write_epoch = epoch;
             }
         } else {
+            // A residual update  h += alpha * t  right behind the one-token
+            // product that wrote t rides in that product's epilogue (same
+            // multiply-then-add per element), which saves a dependent launch:
+            // t = a[0] must be exactly the product's whole output, and h must
+            // be untouched by everything else in the open launch.
+            if (op.kind == OP_AXPY && !cur.list.empty() && cur.key.kind == OP_GEMV_LIST) {
+                const Op *prod = cur.list.back();
+                Alloc *h = op.a[1];
+                if (cur.residual.back() == nullptr && prod->batch == 1 && prod->a[2] == op.a[0] &&
+                    prod->y_off == 0 && prod->rows == op.extra && h != op.a[0] &&
+                    h->read_epoch != epoch && h->write_epoch != epoch) {
+                    cur.residual.back() = &op;
+                    h->write_epoch = epoch;
+                    continue;
+                }
+            }
             flush();
             Launch one;
             one.single = &op;
@@ -583,7 +622,7 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, hipEvent_t sto
         const hipEvent_t ev = last ? stop : nullptr;
         const Launch &l = plan[i];
         hipError_t e = l.single != nullptr ? launch_single(ctx, ev, *l.single)
-                                           : launch_gemv_list(ctx, ev, l.list, l.key);
+                                           : launch_gemv_list(ctx, ev, l.list, l.residual, l.key);
         if (e != hipSuccess) {
             return e;
         }

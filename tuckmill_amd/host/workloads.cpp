@@ -15,7 +15,14 @@ using namespace tuckmill_hip;
 
 extern "C" {
 
-enum { TMH_GEMV = 0, TMH_GEMM = 1, TMH_GEMM_MMA = 2, TMH_GEMM_I8 = 3, TMH_QUANT = 4 };
+enum {
+    TMH_GEMV = 0, TMH_GEMM = 1, TMH_GEMM_MMA = 2, TMH_GEMM_I8 = 3, TMH_QUANT = 4,
+    // the operators either side of a product; `cols` is the element count:
+    TMH_RMSNORM = 5,  // w = weight, x -> y, `rows` rows of `cols`
+    TMH_SILU_MUL = 6, // w = gate, x = up -> y
+    TMH_AXPY = 7,     // y += x (alpha = 1), w unused (pass y)
+    TMH_ARGMAX = 8    // x -> y[0], w = 512 bytes of scratch
+};
 
 struct tmh_product {
     tm_hip_buffer *w, *x, *y; // for TMH_GEMM_I8, x is the quantized activation buffer
@@ -45,6 +52,10 @@ static void issue(const HipContext &gpu, const tmh_product *p, const std::vector
         case TMH_GEMM_MMA: gpu.q8_0_gemm_mma(w, x, y, q.rows, q.cols, q.batch, 0, 0); break;
         case TMH_GEMM_I8: gpu.q8_0_gemm_i8(w, x, y, q.rows, q.cols, q.batch, 0); break;
         case TMH_QUANT: gpu.q8_0_quantize_act(x, y, q.cols, q.batch, 0); break;
+        case TMH_RMSNORM: gpu.rmsnorm(x, w, y, q.rows, q.cols, 1e-6f); break;
+        case TMH_SILU_MUL: gpu.silu_mul(w, x, y, q.cols); break;
+        case TMH_AXPY: gpu.f32_axpy(x, y, 1.0f, q.cols); break;
+        case TMH_ARGMAX: gpu.argmax_f32(x, q.cols, w, y, 0); break;
         default: throw TuckmillError(ErrorCode::InvalidRequest, "unknown product kind");
         }
     }
