@@ -218,3 +218,72 @@ def test_residual_update_is_not_fused_when_it_would_reorder_accesses(ctx):
     want_t = O.gemv_q8_0_f32(w, rows, cols, h0)
     assert np.max(np.abs(t - want_t)) <= 1e-5 * np.max(np.abs(want_t))
     assert np.array_equal(bits(hb.download_f32(0, rows)), bits(O.axpy(t, 1.0, h0)))
+
+
+def test_rmsnorm_in_front_of_its_products_is_fused_into_their_launch(ctx):
+    # norm -> q, k, v (one launch) -> o with its residual update -> norm -> gate, up:
+    # grouped, the norms ride in the launches of the products that read them and the
+    # update in the epilogue of o; every buffer must hold the bits of the separate run.
+    hidden, qdim, kvdim, ffn = 1024, 2048, 1024, 3072
+    mats = {}
+    for i, (name, rows, cols) in enumerate([("q", qdim, hidden), ("k", kvdim, hidden),
+                                            ("v", kvdim, hidden), ("o", hidden, qdim),
+                                            ("gate", ffn, hidden), ("up", ffn, hidden)]):
+        w = S.make_weights(rows, cols, 300 + i)
+        mats[name] = (w, rows, cols, weights_buffer(ctx, w, rows, cols, True))
+    h0 = S.make_activations(hidden, 310)
+    g1 = (0.5 + np.abs(S.make_activations(hidden, 311))).astype(np.float32)
+    g2 = (0.5 + np.abs(S.make_activations(hidden, 312))).astype(np.float32)
+    attn = S.make_activations(qdim, 313)
+    g1b, g2b, attnb = upload_new(ctx, g1), upload_new(ctx, g2), upload_new(ctx, attn)
+    runs = []
+    for grouped in (False, True):
+        hb = upload_new(ctx, h0)
+        nb, n2b, tb = ctx.buffer(hidden * 4), ctx.buffer(hidden * 4), ctx.buffer(hidden * 4)
+        out = {k: ctx.buffer(mats[k][1] * 4) for k in ("q", "k", "v", "gate", "up")}
+        launches = ctx.kernel_launches()
+        if grouped:
+            ctx.begin_group()
+        ctx.rmsnorm(hb, g1b, nb, 1, hidden, 1e-6)
+        for k in ("q", "k", "v"):
+            ctx.q8_0_gemv(mats[k][3], nb, out[k], mats[k][1], hidden)
+        ctx.q8_0_gemv(mats["o"][3], attnb, tb, hidden, qdim)
+        ctx.f32_axpy(tb, hb, 1.0, hidden)
+        ctx.rmsnorm(hb, g2b, n2b, 1, hidden, 1e-6)
+        for k in ("gate", "up"):
+            ctx.q8_0_gemv(mats[k][3], n2b, out[k], mats[k][1], hidden)
+        if grouped:
+            ctx.end_group()
+        ctx.fence()
+        used = ctx.kernel_launches() - launches
+        # grouped: {norm, q, k, v} + {o with its update} + {norm, gate, up}
+        assert used == (3 if grouped else 9), used
+        got = {k: out[k].download_f32(0, mats[k][1]).copy() for k in out}
+        got.update(n=nb.download_f32(0, hidden).copy(), n2=n2b.download_f32(0, hidden).copy(),
+                   h=hb.download_f32(0, hidden).copy(), t=tb.download_f32(0, hidden).copy())
+        runs.append(got)
+    for k in runs[0]:
+        assert np.array_equal(bits(runs[0][k]), bits(runs[1][k])), k
+    n = O.rmsnorm(h0, g1, 1e-6)
+    assert close(runs[1]["n"], n)
+    q = O.gemv_q8_0_f32(mats["q"][0], qdim, hidden, runs[1]["n"])
+    assert np.max(np.abs(runs[1]["q"] - q)) <= 1e-5 * np.max(np.abs(q))
+    assert np.array_equal(bits(runs[1]["h"]), bits(O.axpy(runs[1]["t"], 1.0, h0)))
+    assert close(runs[1]["n2"], O.rmsnorm(runs[1]["h"], g2, 1e-6))
+
+
+def test_a_norm_nobody_reads_still_runs(ctx):
+    hidden = 2048
+    h = S.make_activations(hidden, 320)
+    g = np.ones(hidden, np.float32)
+    w = S.make_weights(64, hidden, 321)
+    wb = weights_buffer(ctx, w, 64, hidden, True)
+    hb, gb, nb, yb = upload_new(ctx, h), upload_new(ctx, g), ctx.buffer(hidden * 4), ctx.buffer(256)
+    ctx.begin_group()
+    ctx.rmsnorm(hb, gb, nb, 1, hidden, 1e-5)
+    ctx.q8_0_gemv(wb, hb, yb, 64, hidden)  # reads h, not the norm's output
+    ctx.end_group()
+    ctx.fence()
+    assert close(nb.download_f32(0, hidden), O.rmsnorm(h, g, 1e-5))
+    want = O.gemv_q8_0_f32(w, 64, hidden, h)
+    assert np.max(np.abs(yb.download_f32(0, 64) - want)) <= 1e-5 * np.max(np.abs(want))

@@ -14,8 +14,8 @@ import pytest
 
 from tuckmill_amd import build as B
 
-# gemv_list_kernel<PACKED, 8 rows, 1 token, aligned x, no tail set, any list capacity>
-DECODE_KERNEL = re.compile(r"Function Name: _ZN2q816gemv_list_kernelILi1ELi8ELi1ELb1ELi0ELi\d+EEE")
+# gemv_list_kernel<PACKED, 8 rows, 1 token, aligned x, no tail set, any list capacity, no fused norm>
+DECODE_KERNEL = re.compile(r"Function Name: _ZN2q816gemv_list_kernelILi1ELi8ELi1ELb1ELi0ELi\d+ELb0EEE")
 
 
 def test_decode_kernel_keeps_four_waves_per_simd(tmp_path):

@@ -39,14 +39,26 @@ struct GemvDesc {
 };
 
 // The list travels in the kernel-argument segment (read through the scalar
-// cache): 224 * 64 + 16 = 14352 bytes, enough for a whole decode step of a
+// cache): 224 * 64 + 40 = 14376 bytes, enough for a whole decode step of a
 // 28-layer model (197 products) in one launch.
 constexpr int GEMV_MAX_DESCS = 224;
+
+// Descriptor flag bits (GemvDesc::pad): the product's activations are the
+// launch's fused RMSNorm output, and this product's first tile writes it out.
+constexpr uint32_t GEMV_X_NORMED = 1u, GEMV_WRITES_NORM = 2u;
 
 template <int ND> struct GemvArgsT {
     uint32_t n;
     uint32_t total_tiles;
-    uint32_t pad[2];
+    // At most one fused RMSNorm per launch (norm_w == nullptr: none):
+    // n = h / sqrt(mean(h^2) + eps) * w over norm_cols elements, a multiple of
+    // 1024; products flagged GEMV_X_NORMED read n without it going through
+    // memory, one of them also stores it to norm_out.
+    float norm_eps;
+    uint32_t pad;
+    const float *norm_h;
+    const float *norm_w;
+    float *norm_out;
     GemvDesc d[ND];
 };
 using GemvArgs = GemvArgsT<GEMV_MAX_DESCS>;
@@ -165,6 +177,52 @@ __device__ __forceinline__ void reduce_store(const float (&acc)[R], float *y, ui
     }
 }
 
+// Where a lane's 16 activations of a chunk come from: memory, or the fused
+// RMSNorm of the launch, (h * inv) * w with the operations of rmsnorm_kernel.
+struct PlainX {
+    const float *x;
+    template <bool XA>
+    __device__ __forceinline__ void load16(uint32_t col, float (&out)[16]) const {
+        load_x<16, XA>(x + col, out);
+    }
+};
+struct NormedX {
+    const float *h, *w;
+    float inv;
+    template <bool XA>
+    __device__ __forceinline__ void load16(uint32_t col, float (&out)[16]) const {
+        float hv[16], wv[16];
+        load_x<16, true>(h + col, hv);
+        load_x<16, true>(w + col, wv);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            out[i] = hv[i] * inv * wv[i];
+        }
+    }
+};
+
+// Sum of squares of a row in the order every kernel that must agree uses: lane
+// l adds its elements 1024*c + 16*l + i sequentially (c, then i, ascending;
+// multiply, then add), the 64 partials go through q8::wave_sum.
+__device__ __forceinline__ float row_sumsq(const float *h, uint32_t cols, uint32_t lane) {
+    float acc = 0.0f;
+    for (uint32_t e0 = lane * 16u; e0 < cols; e0 += 1024u) {
+        if (e0 + 16u <= cols) {
+            float hv[16];
+            load_x<16, false>(h + e0, hv);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                acc += hv[i] * hv[i];
+            }
+        } else {
+            for (uint32_t e = e0; e < cols; ++e) {
+                acc += h[e] * h[e];
+            }
+        }
+    }
+    return wave_sum(acc);
+}
+
 // The decode path: one token, sealed weights, at least one whole 1024-column
 // chunk per row. TAILMASK = cols % 1024 selects the tail pieces at compile time
 // (bit 512/256/128/64/32 -> a piece of 8/4/2/1/1 quants per lane).
@@ -176,10 +234,15 @@ __device__ __forceinline__ void reduce_store(const float (&acc)[R], float *y, ui
 // the first chunk of the next pass are. Tail pieces come first in a pass so
 // that their registers are free again before the next prefetch is issued.
 // With a single chunk per row this lane's activations never leave registers.
-template <int R, bool XA, int TAILMASK>
-__device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const float *x, float *y,
+template <int R, bool XA, int TAILMASK, class XS = PlainX>
+__device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs, float *y,
                                             uint32_t cols, uint32_t row_first, uint32_t row_end,
                                             uint32_t lane, float *res, float alpha) {
+    static_assert(TAILMASK == 0 || sizeof(XS) == sizeof(PlainX), "tails read plain activations");
+    const float *x = nullptr;
+    if constexpr (TAILMASK != 0) {
+        x = xs.x;
+    }
     constexpr bool T8 = (TAILMASK & 512) != 0, T4 = (TAILMASK & 256) != 0;
     constexpr bool T2 = (TAILMASK & 128) != 0, T1 = (TAILMASK & 64) != 0;
     constexpr bool TH = (TAILMASK & 32) != 0;
@@ -200,7 +263,7 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const float
     if constexpr (TH) load_x<1, XA>(x + ch + (low ? lane : 0u), xh);
     float xv[16];
     if (full == 1u) {
-        load_x<16, XA>(x + lane * 16u, xv);
+        xs.template load16<XA>(lane * 16u, xv);
     }
 
     uint32_t q8[R][2], q4[R][1], q2[R][1], q1[R][1], qh[R][1];
@@ -268,7 +331,7 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const float
             }
         }
         if (full > 1u) {
-            load_x<16, XA>(x + (c << 10) + lane * 16u, xv);
+            xs.template load16<XA>((c << 10) + lane * 16u, xv);
         }
         uint32_t cn = c + 1u, rn = r0;
         if (cn == full) {
@@ -308,7 +371,9 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const float
 // (cols a multiple of 1024 only; fewest registers, the Qwen3 shapes), 1 = also
 // cols % 1024 == 128 and == 768 (the Gemma-3-1B shapes). The host picks the
 // smallest set that covers the products of a launch.
-template <int L, int R, int TB, bool XA, int TAILS = 0, int ND = GEMV_MAX_DESCS>
+// NORM: the launch carries a fused RMSNorm (a separate instantiation, so that
+// the plain decode kernel keeps its register budget).
+template <int L, int R, int TB, bool XA, int TAILS = 0, int ND = GEMV_MAX_DESCS, bool NORM = false>
 __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -344,6 +409,29 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
     // cached.
     constexpr bool NT = TB == 1;
 
+    if constexpr (NORM && TB == 1 && L == PACKED) {
+        if (d.pad & GEMV_X_NORMED) {
+            // Every wave recomputes the row's scale (a few hundred operations)
+            // instead of waiting for a separate kernel to publish it.
+            const float sumsq = row_sumsq(args.norm_h, cols, lane);
+            const float inv = 1.0f / sqrtf(sumsq / (float)cols + args.norm_eps);
+            const NormedX xs{args.norm_h, args.norm_w, inv};
+            if ((d.pad & GEMV_WRITES_NORM) && tile == d.tile_begin) {
+                for (uint32_t c = 0; c < full; ++c) {
+                    float o[16];
+                    xs.template load16<true>((c << 10) + lane * 16u, o);
+                    float4 *dst = (float4 *)(args.norm_out + (c << 10) + lane * 16u);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        dst[i] = make_float4(o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]);
+                    }
+                }
+            }
+            stream_rows<R, true, 0, NormedX>(wv, xs, y, cols, row_first, row_end, lane, d.res,
+                                             d.alpha);
+            return;
+        }
+    }
     if constexpr (TB == 1 && L == PACKED) {
         // One token, sealed weights: the decode path, software-pipelined (see
         // stream_rows). Column tails seen in practice are instantiated; other
@@ -351,16 +439,16 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
         if (full >= 1u) {
             const uint32_t tail = cols & 1023u;
             if (tail == 0u) {
-                stream_rows<R, XA, 0>(wv, x, y, cols, row_first, row_end, lane, d.res, d.alpha);
+                stream_rows<R, XA, 0>(wv, PlainX{x}, y, cols, row_first, row_end, lane, d.res, d.alpha);
                 return;
             }
             if constexpr (TAILS >= 1) {
                 if (tail == 128u) { // hidden 1152 (Gemma-3-1B)
-                    stream_rows<R, XA, 128>(wv, x, y, cols, row_first, row_end, lane, d.res, d.alpha);
+                    stream_rows<R, XA, 128>(wv, PlainX{x}, y, cols, row_first, row_end, lane, d.res, d.alpha);
                     return;
                 }
                 if (tail == 768u) { // FFN 6912 (Gemma-3-1B); half the rows per pass
-                    stream_rows<R / 2, XA, 768>(wv, x, y, cols, row_first, row_end, lane, d.res, d.alpha);
+                    stream_rows<R / 2, XA, 768>(wv, PlainX{x}, y, cols, row_first, row_end, lane, d.res, d.alpha);
                     return;
                 }
             }

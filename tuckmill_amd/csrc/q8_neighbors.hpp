@@ -11,7 +11,7 @@
 // be recorded inside a dispatch group.
 #pragma once
 
-#include "q8_common.hpp"
+#include "q8_gemv.hpp"
 
 namespace q8 {
 
@@ -58,31 +58,27 @@ __global__ __launch_bounds__(256) void gelu_tanh_mul_kernel(const float *gate, c
     }
 }
 
-// One workgroup of 256 threads per row: y = x * (1 / sqrt(mean(x^2) + eps)) * w.
-// The sum of squares is taken per thread over a strided slice, then over the
-// wave by the fixed butterfly and over the four waves in order (deterministic;
-// not the CPU's sequential order, hence tolerance-qualified like the
-// reference's own GPU kernel). In place (x == y) is safe: a thread rereads only
-// the elements it writes, after the barrier.
+// One wave per row (four rows per workgroup): y = (x * inv) * w with
+// inv = 1 / sqrt(mean(x^2) + eps). The sum of squares is q8::row_sumsq's: fixed
+// order, not the CPU's sequential one, hence tolerance-qualified like the
+// reference's own GPU kernel; the GEMV kernel's fused form computes the same
+// bits. In place (x == y) is safe: a lane rereads only what it writes itself.
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float *x, const float *weight, float *y,
-                                                      uint32_t cols, float eps) {
-    __shared__ float part[4];
-    const float *xr = x + (size_t)blockIdx.x * cols;
-    float *yr = y + (size_t)blockIdx.x * cols;
-    float acc = 0.0f;
-    for (uint32_t i = threadIdx.x; i < cols; i += 256u) {
-        const float v = xr[i];
-        acc += v * v;
+                                                      uint32_t rows, uint32_t cols, float eps) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= rows) {
+        return;
     }
-    acc = wave_sum(acc);
-    if ((threadIdx.x & 63u) == 0u) {
-        part[threadIdx.x >> 6] = acc;
-    }
-    __syncthreads();
-    const float sumsq = ((part[0] + part[1]) + part[2]) + part[3];
+    const float *xr = x + (size_t)row * cols;
+    float *yr = y + (size_t)row * cols;
+    const float sumsq = row_sumsq(xr, cols, lane);
     const float inv = 1.0f / sqrtf(sumsq / (float)cols + eps);
-    for (uint32_t i = threadIdx.x; i < cols; i += 256u) {
-        yr[i] = xr[i] * inv * weight[i];
+    for (uint32_t e0 = lane * 16u; e0 < cols; e0 += 1024u) {
+        const uint32_t e1 = e0 + 16u < cols ? e0 + 16u : cols;
+        for (uint32_t e = e0; e < e1; ++e) {
+            yr[e] = xr[e] * inv * weight[e];
+        }
     }
 }
 

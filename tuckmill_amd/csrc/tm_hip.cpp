@@ -314,13 +314,26 @@ template <int L, int R, int TB, bool XA>
 hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args, bool tails) {
     const uint32_t groups = (args.total_tiles + 3u) / 4u;
     if constexpr (L == q8::PACKED && TB == 1) {
+        const bool norm = args.norm_w != nullptr; // the planner only fuses into aligned, tail-free launches
         if (args.n <= (uint32_t)q8::GEMV_FEW_DESCS) { // short argument block
             q8::GemvArgsT<q8::GEMV_FEW_DESCS> few;
             few.n = args.n;
             few.total_tiles = args.total_tiles;
-            few.pad[0] = few.pad[1] = 0;
+            few.norm_eps = args.norm_eps;
+            few.pad = 0;
+            few.norm_h = args.norm_h;
+            few.norm_w = args.norm_w;
+            few.norm_out = args.norm_out;
             for (uint32_t i = 0; i < args.n; ++i) {
                 few.d[i] = args.d[i];
+            }
+            if (norm) {
+                if constexpr (XA) {
+                    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, true, 0, q8::GEMV_FEW_DESCS, true>),
+                              dim3(groups), dim3(256), 0, ctx->stream, stop, few);
+                    return hipGetLastError();
+                }
+                return hipErrorInvalidValue;
             }
             if (tails) {
                 Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1, q8::GEMV_FEW_DESCS>), dim3(groups),
@@ -330,6 +343,14 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &arg
                           dim3(256), 0, ctx->stream, stop, few);
             }
             return hipGetLastError();
+        }
+        if (norm) {
+            if constexpr (XA) {
+                Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, true, 0, q8::GEMV_MAX_DESCS, true>),
+                          dim3(groups), dim3(256), 0, ctx->stream, stop, args);
+                return hipGetLastError();
+            }
+            return hipErrorInvalidValue;
         }
         if (tails) {
             Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1>), dim3(groups), dim3(256), 0,
@@ -344,6 +365,16 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &arg
 
 constexpr int kGemvR1 = 8; // rows per pass at one token per pass
 constexpr int kGemvR4 = 2; // rows per pass at four tokens per pass
+
+// One kernel launch of a commit: a list of products, or a single operation.
+struct Launch {
+    std::vector<const Op *> list; // empty: `single`
+    std::vector<const Op *> residual; // per list entry: an axpy fused into it, or null
+    std::vector<bool> normed;         // per list entry: reads the fused RMSNorm's output
+    const Op *norm = nullptr;         // an RMSNorm fused in front of the flagged entries
+    GemvKey key{};
+    const Op *single = nullptr;
+};
 
 hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
                            GemvKey key) {
@@ -375,8 +406,10 @@ hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<co
     return q8::launch_gemm_i8_list(ctx->stream, stop, key.packed, key.xalign, key.tb, prods, n);
 }
 
-hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
-                            const std::vector<const Op *> &residual, GemvKey key) {
+hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch) {
+    const std::vector<const Op *> &ops = launch.list;
+    const std::vector<const Op *> &residual = launch.residual;
+    const GemvKey key = launch.key;
     if (key.kind == OP_MMA) {
         return launch_mma_list(ctx, stop, ops, key);
     }
@@ -385,7 +418,12 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<
     }
     q8::GemvArgs args; // only the used descriptors are written (the struct is 12 KB)
     args.n = 0;
-    args.pad[0] = args.pad[1] = 0;
+    args.pad = 0;
+    args.norm_eps = launch.norm != nullptr ? launch.norm->scalar : 0.0f;
+    args.norm_h = launch.norm != nullptr ? (const float *)launch.norm->a[0]->ptr : nullptr;
+    args.norm_w = launch.norm != nullptr ? (const float *)launch.norm->a[1]->ptr : nullptr;
+    args.norm_out = launch.norm != nullptr ? (float *)launch.norm->a[2]->ptr : nullptr;
+    bool norm_written = false;
     const int R = (key.tb == 1 || key.tb >= 200) ? kGemvR1 : kGemvR4;
     // a workgroup's tile in the token-split kernel, a wave's tile otherwise
     const uint32_t tile_bytes = key.tb >= 200 ? 32768u : 8192u;
@@ -404,6 +442,11 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<
         d.tile_begin = tiles;
         d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
         d.pad = 0;
+        if (launch.norm != nullptr && launch.normed[args.n - 1]) {
+            d.x = args.norm_h; // not read through: the kernel normalises norm_h itself
+            d.pad = q8::GEMV_X_NORMED | (norm_written ? 0u : q8::GEMV_WRITES_NORM);
+            norm_written = true;
+        }
         const Op *fused = residual[args.n - 1];
         d.res = fused != nullptr ? (float *)fused->a[1]->ptr : nullptr;
         d.alpha = fused != nullptr ? fused->scalar : 0.0f;
@@ -501,9 +544,9 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
                   op.extra);
         break;
     case OP_RMSNORM:
-        Q8_LAUNCH(q8::rmsnorm_kernel, dim3(op.rows), dim3(256), 0, st, stop,
+        Q8_LAUNCH(q8::rmsnorm_kernel, dim3((op.rows + 3u) / 4u), dim3(256), 0, st, stop,
                   (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
-                  op.cols, op.scalar);
+                  op.rows, op.cols, op.scalar);
         break;
     case OP_ARGMAX: {
         float *part_v = (float *)op.a[1]->ptr;
@@ -533,14 +576,6 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
     return hipGetLastError();
 }
 
-// One kernel launch of a commit: a list of products, or a single operation.
-struct Launch {
-    std::vector<const Op *> list; // empty: `single`
-    std::vector<const Op *> residual; // per list entry: an axpy fused into it, or null
-    GemvKey key{};
-    const Op *single = nullptr;
-};
-
 // Plan the launches of a sequence of recorded operations. Consecutive
 // list-kernel products that neither read nor overwrite each other's outputs
 // share one launch; everything else launches on its own, in order.
@@ -551,11 +586,23 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
     // step of n products costs O(n), not O(n^2).
     uint64_t epoch = ++ctx->plan_epoch;
     auto flush = [&]() {
+        if (cur.norm != nullptr) {
+            bool used = false;
+            for (bool b : cur.normed) {
+                used = used || b;
+            }
+            if (!used) { // nothing took the norm in: it launches on its own, first
+                Launch one;
+                one.single = cur.norm;
+                plan.push_back(std::move(one));
+                cur.norm = nullptr;
+            }
+        }
         if (!cur.list.empty()) {
             plan.push_back(std::move(cur));
-            cur = Launch();
-            epoch = ++ctx->plan_epoch;
         }
+        cur = Launch();
+        epoch = ++ctx->plan_epoch;
     };
     for (const Op &op : ops) {
         if (op.kind == OP_GEMV_LIST || op.kind == OP_MMA || op.kind == OP_I8) {
@@ -563,28 +610,53 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             const int cap = key.kind == OP_MMA  ? q8::MMA_MAX_DESCS
                             : key.kind == OP_I8 ? q8::I8_MAX_DESCS
                                                 : q8::GEMV_MAX_DESCS;
+            // While a fused RMSNorm is pending only the decode kernel's
+            // products may join its launch; the ones that read the norm's
+            // whole output as their activations take it in without it going
+            // through memory.
+            const bool decode_kind =
+                key.kind == OP_GEMV_LIST && key.tb == 1 && key.packed && key.xalign;
+            const bool normed = cur.norm != nullptr && decode_kind && op.a[1] == cur.norm->a[2] &&
+                                op.x_off == 0 && op.cols == cur.norm->cols;
+            if (cur.norm != nullptr && !decode_kind) {
+                flush();
+            }
             // a[0] = w (read), a[1] = x (read), a[2] = y (written), a[3] =
             // optional second output: the product joins the open launch
             // unless an output of it was read or written there, or one of
             // its inputs was written there.
             bool conflict = op.a[2]->read_epoch == epoch || op.a[2]->write_epoch == epoch ||
-                            op.a[1]->write_epoch == epoch || op.a[0]->write_epoch == epoch;
+                            (!normed && op.a[1]->write_epoch == epoch) ||
+                            op.a[0]->write_epoch == epoch;
             if (op.a[3] != nullptr) {
                 conflict = conflict || op.a[3]->read_epoch == epoch || op.a[3]->write_epoch == epoch;
             }
-            if (!cur.list.empty() &&
-                (conflict || !(key == cur.key) || (int)cur.list.size() == cap)) {
+            const bool open = !cur.list.empty() || cur.norm != nullptr;
+            if (open && (conflict || (!cur.list.empty() && !(key == cur.key)) ||
+                         (int)cur.list.size() == cap)) {
                 flush();
             }
+            const bool takes_norm = normed && cur.norm != nullptr; // still pending after a flush?
             cur.key = key;
             cur.list.push_back(&op);
             cur.residual.push_back(nullptr);
+            cur.normed.push_back(takes_norm);
             op.a[0]->read_epoch = epoch;
             op.a[1]->read_epoch = epoch;
             op.a[2]->write_epoch = epoch;
             if (op.a[3] != nullptr) {
                 op.a[3]->write_epoch = epoch;
             }
+        } else if (op.kind == OP_RMSNORM && op.rows == 1 && op.cols >= 1024u &&
+                   (op.cols & 1023u) == 0u && op.a[0] != op.a[2]) {
+            // One row in front of its consumers (the norm before q/k/v, before
+            // gate/up, before the vocabulary projection): held back and fused
+            // into the launch of the products that read it, if any follow.
+            flush();
+            cur.norm = &op;
+            op.a[0]->read_epoch = epoch;
+            op.a[1]->read_epoch = epoch;
+            op.a[2]->write_epoch = epoch;
         } else {
             // A residual update  h += alpha * t  right behind the one-token
             // product that wrote t rides in that product's epilogue (same
@@ -622,7 +694,7 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, hipEvent_t sto
         const hipEvent_t ev = last ? stop : nullptr;
         const Launch &l = plan[i];
         hipError_t e = l.single != nullptr ? launch_single(ctx, ev, *l.single)
-                                           : launch_gemv_list(ctx, ev, l.list, l.residual, l.key);
+                                           : launch_gemv_list(ctx, ev, l);
         if (e != hipSuccess) {
             return e;
         }
