@@ -143,3 +143,23 @@ def test_independent_i8_products_in_a_group_share_one_launch(ctx):
     for w, rows, wb, yb in mats:
         want = O.gemm_q8_0_q8_0(w, rows, cols, x, batch, threads=4)
         assert np.array_equal(bits(yb.download_f32(0, batch * rows)), bits(want.reshape(-1)))
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(128, 1024, 64), (129, 2048, 65), (300, 1152, 200),
+                                             (64, 96, 77), (1000, 64, 512), (257, 6144, 129),
+                                             (70, 32, 64), (513, 3072, 300)])
+def test_lds_staged_i8_gemm_is_bit_exact(ctx, rows, cols, batch):
+    # Prefill-sized batches over sealed weights without the verification output
+    # take the LDS-staged kernel: partial token and row tiles, K stages that end
+    # inside the last stage, both workgroup shapes.
+    w = S.make_weights(rows, cols, 3 * rows + cols)
+    x = S.make_activations(cols * batch, batch + 1)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    xq, qs, ds = quantize_on_gpu(ctx, x, cols, batch)
+    yb = ctx.buffer((5 + batch * rows) * 4)
+    ctx.q8_0_gemm_i8(wb, xq, yb, rows, cols, batch, 5)
+    ctx.fence()
+    out = yb.download_f32(0, 5 + batch * rows)
+    assert not out[:5].any()
+    want = O.gemm_q8_0_q8_0(w, rows, cols, x, batch, threads=8)
+    assert np.array_equal(bits(out[5:]), bits(want.reshape(-1)))

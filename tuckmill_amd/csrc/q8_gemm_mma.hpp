@@ -504,7 +504,15 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
     args.chunk_wgs = args.d[0].tiles_t >= (uint32_t)P ? args.d[0].tiles_t / P : 1u;
     args.pad = 0;
     const uint32_t groups = (uint32_t)((tiles + P - 1) / P);
-    if constexpr (S == 4 && TNW == 1) {
+    uint32_t min_batch = 0xffffffffu;
+    for (int i = 0; i < n; ++i) {
+        min_batch = prods[i].batch < min_batch ? prods[i].batch : min_batch;
+    }
+    // Measured on the 2B-class shapes: the persistent form wins from 256 tokens
+    // up (several token tiles per weight row tile); below that its static tile
+    // lists balance worse than the hardware's workgroup dispatch (M = 64: 1.8x
+    // slower), so smaller batches keep one tile per workgroup.
+    if constexpr (S == 4 && TNW == 1) if (min_batch >= 256u) {
         // Persistent form: as many workgroups as stay resident (a multiple of
         // 8), each walking a strided list of tiles.
         static const uint32_t resident = [] {

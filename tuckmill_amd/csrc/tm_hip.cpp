@@ -23,6 +23,7 @@
 
 #include "q8_gemm_i8.hpp"
 #include "q8_gemv_i8.hpp"
+#include "q8_gemm_i8_lds.hpp"
 #include "q8_gemm_mma.hpp"
 #include "q8_gemv.hpp"
 #include "q8_gemm_small.hpp"
@@ -267,6 +268,10 @@ GemvKey gemv_key(const Op &op) {
         k.tb = q8::pick_i8_config(op.batch);
         if (op.packed && op.batch <= q8::GEMV_I8_MAX_BATCH) {
             k.tb = 10 + q8::gemv_i8_tokens(op.batch); // the streaming kernel
+        } else if (op.packed && op.a[3] == nullptr && op.batch >= q8::GEMM_I8_LDS_MIN_BATCH &&
+                   (uint64_t)op.rows * op.cols < (1ull << 32) &&
+                   (uint64_t)op.batch * op.cols < (1ull << 32)) {
+            k.tb = op.batch <= 64u ? 20 : 21; // the LDS-staged kernel, by workgroup shape
         }
         k.xalign = op.a[3] != nullptr;
         return k;
@@ -399,6 +404,9 @@ hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<co
                                    (float *)op->a[2]->ptr + op->y_off,
                                    op->a[3] != nullptr ? (int32_t *)op->a[3]->ptr : nullptr,
                                    op->rows, op->cols, op->batch};
+    }
+    if (key.tb >= 20) {
+        return q8::launch_gemm_i8_lds_list(ctx->stream, stop, prods, n);
     }
     if (key.tb >= 10) {
         return q8::launch_gemv_i8_list(ctx->stream, stop, key.xalign, key.tb - 10, prods, n);
