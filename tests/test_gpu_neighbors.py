@@ -287,3 +287,72 @@ def test_a_norm_nobody_reads_still_runs(ctx):
     assert close(nb.download_f32(0, hidden), O.rmsnorm(h, g, 1e-5))
     want = O.gemv_q8_0_f32(w, 64, hidden, h)
     assert np.max(np.abs(yb.download_f32(0, 64) - want)) <= 1e-5 * np.max(np.abs(want))
+
+
+@pytest.mark.parametrize("act,in_place,with_norm", [("silu", True, True), ("silu", False, False),
+                                                    ("gelu", True, False), ("gelu", False, True)])
+def test_gated_activation_behind_gate_and_up_is_fused(ctx, act, in_place, with_norm):
+    # [norm ->] gate, up -> act(gate) * up -> down with its residual update: grouped,
+    # one wave computes a row of gate and of up and applies the activation itself.
+    # Every buffer must hold the bits of the separate operators.
+    hidden, ffn = 1024, 3072 + 8  # a row count that leaves a partial last tile
+    wg, wu = S.make_weights(ffn, hidden, 401), S.make_weights(ffn, hidden, 402)
+    wd = S.make_weights(hidden, 1024 * 3, 403)
+    wgb, wub = weights_buffer(ctx, wg, ffn, hidden, True), weights_buffer(ctx, wu, ffn, hidden, True)
+    h0 = S.make_activations(hidden, 404)
+    gw = (0.5 + np.abs(S.make_activations(hidden, 405))).astype(np.float32)
+    gwb = upload_new(ctx, gw)
+    runs = []
+    for grouped in (False, True):
+        hb, nb = upload_new(ctx, h0), ctx.buffer(hidden * 4)
+        gb, ub = ctx.buffer(ffn * 4), ctx.buffer(ffn * 4)
+        ob = gb if in_place else ctx.buffer(ffn * 4)
+        launches = ctx.kernel_launches()
+        if grouped:
+            ctx.begin_group()
+        xin = hb
+        if with_norm:
+            ctx.rmsnorm(hb, gwb, nb, 1, hidden, 1e-6)
+            xin = nb
+        ctx.q8_0_gemv(wgb, xin, gb, ffn, hidden)
+        ctx.q8_0_gemv(wub, xin, ub, ffn, hidden)
+        (ctx.silu_mul if act == "silu" else ctx.gelu_tanh_mul)(gb, ub, ob, ffn)
+        if grouped:
+            ctx.end_group()
+        ctx.fence()
+        used = ctx.kernel_launches() - launches
+        assert used == (1 if grouped else 3 + int(with_norm)), used
+        runs.append({"gate": gb.download_f32(0, ffn).copy(), "up": ub.download_f32(0, ffn).copy(),
+                     "out": ob.download_f32(0, ffn).copy(), "n": nb.download_f32(0, hidden).copy()})
+    for k in runs[0]:
+        assert np.array_equal(bits(runs[0][k]), bits(runs[1][k])), k
+    x = O.rmsnorm(h0, gw, 1e-6) if with_norm else h0
+    if with_norm:
+        assert close(runs[1]["n"], x)
+        x = runs[1]["n"]
+    g, u = O.gemv_q8_0_f32(wg, ffn, hidden, x), O.gemv_q8_0_f32(wu, ffn, hidden, x)
+    assert np.max(np.abs(runs[1]["up"] - u)) <= 1e-5 * np.max(np.abs(u))
+    if not in_place:
+        assert np.max(np.abs(runs[1]["gate"] - g)) <= 1e-5 * np.max(np.abs(g))
+    want = (O.silu_mul if act == "silu" else O.gelu_tanh_mul)(g, u)
+    assert np.all(np.abs(runs[1]["out"] - want) <= 2e-5 * np.maximum(np.abs(want), 1.0))
+    del wd
+
+
+def test_gated_activation_is_not_fused_when_out_is_the_up_buffer(ctx):
+    hidden, ffn = 1024, 256
+    wg, wu = S.make_weights(ffn, hidden, 411), S.make_weights(ffn, hidden, 412)
+    wgb, wub = weights_buffer(ctx, wg, ffn, hidden, True), weights_buffer(ctx, wu, ffn, hidden, True)
+    x = S.make_activations(hidden, 413)
+    xb, gb, ub = upload_new(ctx, x), ctx.buffer(ffn * 4), ctx.buffer(ffn * 4)
+    launches = ctx.kernel_launches()
+    ctx.begin_group()
+    ctx.q8_0_gemv(wgb, xb, gb, ffn, hidden)
+    ctx.q8_0_gemv(wub, xb, ub, ffn, hidden)
+    ctx.silu_mul(gb, ub, ub, ffn)
+    ctx.end_group()
+    ctx.fence()
+    assert ctx.kernel_launches() - launches == 2
+    g, u = O.gemv_q8_0_f32(wg, ffn, hidden, x), O.gemv_q8_0_f32(wu, ffn, hidden, x)
+    want = O.silu_mul(g, u)
+    assert np.all(np.abs(ub.download_f32(0, ffn) - want) <= 2e-5 * np.maximum(np.abs(want), 1.0))

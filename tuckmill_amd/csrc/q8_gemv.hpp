@@ -46,6 +46,9 @@ constexpr int GEMV_MAX_DESCS = 224;
 // Descriptor flag bits (GemvDesc::pad): the product's activations are the
 // launch's fused RMSNorm output, and this product's first tile writes it out.
 constexpr uint32_t GEMV_X_NORMED = 1u, GEMV_WRITES_NORM = 2u;
+// This product and the next descriptor are the gate and up projections of a
+// fused gated activation (see stream_rows_glu).
+constexpr uint32_t GEMV_PAIR = 4u;
 
 template <int ND> struct GemvArgsT {
     uint32_t n;
@@ -223,6 +226,35 @@ __device__ __forceinline__ float row_sumsq(const float *h, uint32_t cols, uint32
     return wave_sum(acc);
 }
 
+// Which weight rows a pass of R accumulators covers: R consecutive rows of one
+// matrix, or R/2 rows of a gate matrix followed by the same R/2 rows of an up
+// matrix (the fused gated-activation form: both results of a row end up in one
+// wave).
+struct SingleRows {
+    WView<PACKED> wv;
+    static constexpr bool pair = false;
+    template <int R>
+    __device__ __forceinline__ void chunk(int r, uint32_t r0, uint32_t row_end, uint32_t c,
+                                          uint32_t lane, uint32_t (&q)[4], uint32_t &sb) const {
+        const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+        wv.template load_quants<16, true>(row, (c << 10) + lane * 16u, q);
+        sb = wv.scale_bits(row, (c << 5) + (lane >> 1));
+    }
+};
+struct PairRows {
+    WView<PACKED> gate, up;
+    static constexpr bool pair = true;
+    template <int R>
+    __device__ __forceinline__ void chunk(int r, uint32_t r0, uint32_t row_end, uint32_t c,
+                                          uint32_t lane, uint32_t (&q)[4], uint32_t &sb) const {
+        const uint32_t j = (uint32_t)(r % (R / 2));
+        const uint32_t row = (r0 + j < row_end) ? r0 + j : row_end - 1u;
+        const WView<PACKED> &wv = r < R / 2 ? gate : up;
+        wv.template load_quants<16, true>(row, (c << 10) + lane * 16u, q);
+        sb = wv.scale_bits(row, (c << 5) + (lane >> 1));
+    }
+};
+
 // The decode path: one token, sealed weights, at least one whole 1024-column
 // chunk per row. TAILMASK = cols % 1024 selects the tail pieces at compile time
 // (bit 512/256/128/64/32 -> a piece of 8/4/2/1/1 quants per lane).
@@ -234,11 +266,21 @@ __device__ __forceinline__ float row_sumsq(const float *h, uint32_t cols, uint32
 // the first chunk of the next pass are. Tail pieces come first in a pass so
 // that their registers are free again before the next prefetch is issued.
 // With a single chunk per row this lane's activations never leave registers.
-template <int R, bool XA, int TAILMASK, class XS = PlainX>
-__device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs, float *y,
-                                            uint32_t cols, uint32_t row_first, uint32_t row_end,
-                                            uint32_t lane, float *res, float alpha) {
+// `sink(acc, r0)` receives the R per-lane partial sums of a finished pass.
+template <int R, bool XA, int TAILMASK, class XS, class ROWS, class SINK>
+__device__ __forceinline__ void stream_rows_to(const ROWS rows_src, const XS xs, uint32_t cols,
+                                               uint32_t row_first, uint32_t row_end, uint32_t lane,
+                                               SINK sink) {
     static_assert(TAILMASK == 0 || sizeof(XS) == sizeof(PlainX), "tails read plain activations");
+    static_assert(TAILMASK == 0 || !ROWS::pair, "the paired form has no tail pieces");
+    constexpr uint32_t ADV = ROWS::pair ? R / 2 : R; // rows a pass advances by
+    const WView<PACKED> &wv = [&]() -> const WView<PACKED> & {
+        if constexpr (ROWS::pair) {
+            return rows_src.gate;
+        } else {
+            return rows_src.wv;
+        }
+    }();
     const float *x = nullptr;
     if constexpr (TAILMASK != 0) {
         x = xs.x;
@@ -298,15 +340,13 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs
     auto load_chunk = [&](uint32_t r0, uint32_t c, uint32_t (&qq)[R][4], uint32_t (&ss)[R]) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
-            wv.template load_quants<16, true>(row, (c << 10) + lane * 16u, qq[r]);
-            ss[r] = wv.scale_bits(row, (c << 5) + (lane >> 1));
+            rows_src.template chunk<R>(r, r0, row_end, c, lane, qq[r], ss[r]);
         }
     };
 
     // One flat sequence of (pass, chunk) steps; the tail pieces of a pass
     // travel with its first chunk.
-    const uint32_t nsteps = ((row_end - row_first + R - 1) / R) * full;
+    const uint32_t nsteps = ((row_end - row_first + ADV - 1) / ADV) * full;
     uint32_t r0 = row_first, c = 0;
     if constexpr (TAILMASK != 0) {
         load_tails(r0);
@@ -336,7 +376,7 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs
         uint32_t cn = c + 1u, rn = r0;
         if (cn == full) {
             cn = 0;
-            rn = r0 + R;
+            rn = r0 + ADV;
         }
         uint32_t qn[R][4], sn[R];
         if (step + 1u < nsteps) {
@@ -352,7 +392,7 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs
             acc[r] = __builtin_fmaf(f16_bits_to_f32(sb[r]), piece_dot<16>(q[r], xv), acc[r]);
         }
         if (cn == 0u) {
-            reduce_store<R>(acc, y, r0, row_end, lane, true, res, alpha);
+            sink(acc, r0);
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -367,11 +407,86 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs
     }
 }
 
+// One matrix: reduce each pass over the wave and store (plus the optional
+// fused residual update).
+template <int R, bool XA, int TAILMASK, class XS = PlainX>
+__device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs, float *y,
+                                            uint32_t cols, uint32_t row_first, uint32_t row_end,
+                                            uint32_t lane, float *res, float alpha) {
+    stream_rows_to<R, XA, TAILMASK>(SingleRows{wv}, xs, cols, row_first, row_end, lane,
+                                    [&](const float (&acc)[R], uint32_t r0) {
+                                        reduce_store<R>(acc, y, r0, row_end, lane, true, res, alpha);
+                                    });
+}
+
+// Gate and up projection of the same activations with the gated activation on
+// top: out[r] = act(gate[r]) * up[r], act = silu (kind 0) or ggml's tanh GELU
+// (kind 1), the expressions of silu_mul_kernel / gelu_tanh_mul_kernel. After
+// the butterfly of reduce_store<8>, lanes 0, 8, 16, 24 hold the gate rows
+// r0..r0+3 and lanes 32, 40, 48, 56 the up rows; one exchange pairs them. The
+// raw projections are stored as well (the gate's only when `out` is another
+// buffer: in place, the activation replaces it as the separate operator would).
+__device__ __forceinline__ float glu_act(float g, float u, uint32_t kind) {
+    if (kind == 0u) {
+        const float s = g / (1.0f + expf(-g));
+        return s * u;
+    }
+    const float inner = 0.7978845608028654f * g * (1.0f + 0.044715f * g * g);
+    return 0.5f * g * (1.0f + tanhf(inner)) * u;
+}
+
+template <bool XA, class XS>
+__device__ __forceinline__ void stream_rows_glu(const WView<PACKED> &wg, const WView<PACKED> &wu,
+                                                const XS xs, float *gate_out, float *up_out,
+                                                float *out, uint32_t kind, uint32_t cols,
+                                                uint32_t row_first, uint32_t row_end,
+                                                uint32_t lane) {
+    constexpr int R = 8;
+    stream_rows_to<R, XA, 0>(
+        PairRows{wg, wu}, xs, cols, row_first, row_end, lane,
+        [&](const float (&acc)[R], uint32_t r0) {
+            // the butterfly of reduce_store<8>: same operands per addition
+            float a4[4], a2[2];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float keep = (lane & 32u) ? acc[i + 4] : acc[i];
+                const float send = (lane & 32u) ? acc[i] : acc[i + 4];
+                a4[i] = keep + __shfl_xor(send, 32, WAVE);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const float keep = (lane & 16u) ? a4[i + 2] : a4[i];
+                const float send = (lane & 16u) ? a4[i] : a4[i + 2];
+                a2[i] = keep + __shfl_xor(send, 16, WAVE);
+            }
+            const float keep = (lane & 8u) ? a2[1] : a2[0];
+            const float send = (lane & 8u) ? a2[0] : a2[1];
+            float a1 = keep + __shfl_xor(send, 8, WAVE);
+            a1 += __shfl_xor(a1, 4, WAVE);
+            a1 += __shfl_xor(a1, 2, WAVE);
+            a1 += __shfl_xor(a1, 1, WAVE);
+            const float other = __shfl_xor(a1, 32, WAVE);
+            const uint32_t row = r0 + ((lane >> 4) & 1u) * 2u + ((lane >> 3) & 1u);
+            if ((lane & 7u) == 0u && row < row_end) {
+                if (lane & 32u) {
+                    up_out[row] = a1;
+                } else {
+                    const float act = glu_act(a1, other, kind);
+                    if (out != gate_out) {
+                        gate_out[row] = a1;
+                    }
+                    out[row] = act;
+                }
+            }
+        });
+}
+
 // TAILS selects which column tails get the streaming decode path: 0 = none
 // (cols a multiple of 1024 only; fewest registers, the Qwen3 shapes), 1 = also
 // cols % 1024 == 128 and == 768 (the Gemma-3-1B shapes). The host picks the
 // smallest set that covers the products of a launch.
-// NORM: the launch carries a fused RMSNorm (a separate instantiation, so that
+// NORM: the launch carries fused forms, an RMSNorm in front of its products
+// and/or gate-up pairs with their activation (a separate instantiation, so that
 // the plain decode kernel keeps its register budget).
 template <int L, int R, int TB, bool XA, int TAILS = 0, int ND = GEMV_MAX_DESCS, bool NORM = false>
 __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args) {
@@ -410,16 +525,19 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
     constexpr bool NT = TB == 1;
 
     if constexpr (NORM && TB == 1 && L == PACKED) {
-        if (d.pad & GEMV_X_NORMED) {
+        if (d.pad & (GEMV_X_NORMED | GEMV_PAIR)) {
             // Every wave recomputes the row's scale (a few hundred operations)
             // instead of waiting for a separate kernel to publish it.
-            const float sumsq = row_sumsq(args.norm_h, cols, lane);
-            const float inv = 1.0f / sqrtf(sumsq / (float)cols + args.norm_eps);
-            const NormedX xs{args.norm_h, args.norm_w, inv};
+            float inv = 0.0f;
+            if (d.pad & GEMV_X_NORMED) {
+                const float sumsq = row_sumsq(args.norm_h, cols, lane);
+                inv = 1.0f / sqrtf(sumsq / (float)cols + args.norm_eps);
+            }
+            const NormedX xn{args.norm_h, args.norm_w, inv};
             if ((d.pad & GEMV_WRITES_NORM) && tile == d.tile_begin) {
                 for (uint32_t c = 0; c < full; ++c) {
                     float o[16];
-                    xs.template load16<true>((c << 10) + lane * 16u, o);
+                    xn.template load16<true>((c << 10) + lane * 16u, o);
                     float4 *dst = (float4 *)(args.norm_out + (c << 10) + lane * 16u);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
@@ -427,8 +545,23 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
                     }
                 }
             }
-            stream_rows<R, true, 0, NormedX>(wv, xs, y, cols, row_first, row_end, lane, d.res,
-                                             d.alpha);
+            if (d.pad & GEMV_PAIR) {
+                // gate (this descriptor) and up (the next one, which owns no
+                // tiles; its `res` is the activation's output, its `alpha` the kind)
+                const GemvDesc &d2 = args.d[lo + 1];
+                const WView<PACKED> wu(d2.w, rows, cols);
+                const uint32_t kind = (uint32_t)d2.alpha;
+                if (d.pad & GEMV_X_NORMED) {
+                    stream_rows_glu<true>(wv, wu, xn, y, d2.y, d2.res, kind, cols, row_first,
+                                          row_end, lane);
+                } else {
+                    stream_rows_glu<true>(wv, wu, PlainX{x}, y, d2.y, d2.res, kind, cols, row_first,
+                                          row_end, lane);
+                }
+            } else {
+                stream_rows<R, true, 0, NormedX>(wv, xn, y, cols, row_first, row_end, lane, d.res,
+                                                 d.alpha);
+            }
             return;
         }
     }

@@ -316,10 +316,11 @@ uint32_t pick_rows_per_tile(uint32_t rows, uint32_t cols, uint32_t tile_bytes, i
 }
 
 template <int L, int R, int TB, bool XA>
-hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args, bool tails) {
+hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args, bool tails,
+                       bool fused) {
     const uint32_t groups = (args.total_tiles + 3u) / 4u;
     if constexpr (L == q8::PACKED && TB == 1) {
-        const bool norm = args.norm_w != nullptr; // the planner only fuses into aligned, tail-free launches
+        const bool norm = fused; // the planner only fuses into aligned launches of the decode kernel
         if (args.n <= (uint32_t)q8::GEMV_FEW_DESCS) { // short argument block
             q8::GemvArgsT<q8::GEMV_FEW_DESCS> few;
             few.n = args.n;
@@ -375,6 +376,8 @@ constexpr int kGemvR4 = 2; // rows per pass at four tokens per pass
 struct Launch {
     std::vector<const Op *> list; // empty: `single`
     std::vector<const Op *> residual; // per list entry: an axpy fused into it, or null
+    std::vector<const Op *> glu;      // per list entry: this product and the next are the gate
+                                      // and up projections of this fused gated activation
     std::vector<bool> normed;         // per list entry: reads the fused RMSNorm's output
     const Op *norm = nullptr;         // an RMSNorm fused in front of the flagged entries
     GemvKey key{};
@@ -432,6 +435,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     args.norm_w = launch.norm != nullptr ? (const float *)launch.norm->a[1]->ptr : nullptr;
     args.norm_out = launch.norm != nullptr ? (float *)launch.norm->a[2]->ptr : nullptr;
     bool norm_written = false;
+    bool fused = launch.norm != nullptr; // the launch needs the kernel variant with fused forms
     const int R = (key.tb == 1 || key.tb >= 200) ? kGemvR1 : kGemvR4;
     // a workgroup's tile in the token-split kernel, a wave's tile otherwise
     const uint32_t tile_bytes = key.tb >= 200 ? 32768u : 8192u;
@@ -450,16 +454,30 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         d.tile_begin = tiles;
         d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
         d.pad = 0;
+        const size_t at = args.n - 1;
+        const bool pair_first = launch.glu[at] != nullptr;
+        const bool pair_second = at > 0 && launch.glu[at - 1] != nullptr;
+        if (pair_first) { // a tile covers the same rows of both matrices: half the rows each
+            d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes / 2u, 4);
+            d.pad |= q8::GEMV_PAIR;
+            fused = true;
+        }
         if (launch.norm != nullptr && launch.normed[args.n - 1]) {
             d.x = args.norm_h; // not read through: the kernel normalises norm_h itself
-            d.pad = q8::GEMV_X_NORMED | (norm_written ? 0u : q8::GEMV_WRITES_NORM);
+            d.pad |= q8::GEMV_X_NORMED | (norm_written ? 0u : q8::GEMV_WRITES_NORM);
             norm_written = true;
         }
-        const Op *fused = residual[args.n - 1];
-        d.res = fused != nullptr ? (float *)fused->a[1]->ptr : nullptr;
-        d.alpha = fused != nullptr ? fused->scalar : 0.0f;
+        const Op *update = residual[args.n - 1];
+        d.res = update != nullptr ? (float *)update->a[1]->ptr : nullptr;
+        d.alpha = update != nullptr ? update->scalar : 0.0f;
         d.pad2 = 0;
-        tiles += (op->rows + d.rows_per_tile - 1) / d.rows_per_tile;
+        if (pair_second) { // owns no tiles; carries the activation's output and kind
+            const Op *act = launch.glu[at - 1];
+            d.res = (float *)act->a[2]->ptr;
+            d.alpha = act->kind == OP_GELU_MUL ? 1.0f : 0.0f;
+        } else {
+            tiles += (op->rows + d.rows_per_tile - 1) / d.rows_per_tile;
+        }
     }
     args.total_tiles = tiles;
 #define TM_SPLIT_CASE(W, T, A, TL)                                                           \
@@ -483,7 +501,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
 #define TM_GEMV_CASE(P, T, A)                                                                \
     if (key.packed == (P) && key.tb == (T) && key.xalign == (A)) {                           \
         return launch_gemv<(P) ? q8::PACKED : q8::RAW, (T) == 1 ? kGemvR1 : kGemvR4, T, A>(  \
-            ctx, stop, args, tails);                                                         \
+            ctx, stop, args, tails, fused);                                                         \
     }
     TM_GEMV_CASE(true, 1, true)
     TM_GEMV_CASE(true, 1, false)
@@ -648,6 +666,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             cur.key = key;
             cur.list.push_back(&op);
             cur.residual.push_back(nullptr);
+            cur.glu.push_back(nullptr);
             cur.normed.push_back(takes_norm);
             op.a[0]->read_epoch = epoch;
             op.a[1]->read_epoch = epoch;
@@ -671,10 +690,43 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             // multiply-then-add per element), which saves a dependent launch:
             // t = a[0] must be exactly the product's whole output, and h must
             // be untouched by everything else in the open launch.
+            // A gated activation right behind the gate and up projections it
+            // consumes (same activations, same shape, decode kernel): both
+            // rows of a pair are computed by one wave, which applies the
+            // activation itself. `out` may be the gate buffer (in place).
+            if ((op.kind == OP_SILU_MUL || op.kind == OP_GELU_MUL) && cur.list.size() >= 2 &&
+                cur.key.kind == OP_GEMV_LIST && cur.key.tb == 1 && cur.key.packed &&
+                cur.key.xalign) {
+                const size_t n = cur.list.size();
+                const Op *pg = cur.list[n - 2], *pu = cur.list[n - 1];
+                Alloc *out = op.a[2];
+                const bool shapes = pg->batch == 1 && pu->batch == 1 && pg->a[1] == pu->a[1] &&
+                                    pg->x_off == pu->x_off && pg->rows == pu->rows &&
+                                    pg->cols == pu->cols && pg->cols >= 1024u &&
+                                    (pg->cols & 1023u) == 0u && pg->y_off == 0 && pu->y_off == 0 &&
+                                    op.extra == pg->rows;
+                const bool wiring = pg->a[2] == op.a[0] && pu->a[2] == op.a[1] &&
+                                    pg->a[2] != pu->a[2] && out != pu->a[2];
+                const bool free_entries = cur.residual[n - 2] == nullptr &&
+                                          cur.residual[n - 1] == nullptr &&
+                                          cur.glu[n - 2] == nullptr && cur.glu[n - 1] == nullptr &&
+                                          (n < 3 || cur.glu[n - 3] == nullptr) &&
+                                          cur.normed[n - 2] == cur.normed[n - 1];
+                const bool out_free = out == pg->a[2] ||
+                                      (out->read_epoch != epoch && out->write_epoch != epoch);
+                if (shapes && wiring && free_entries && out_free) {
+                    cur.glu[n - 2] = &op;
+                    out->write_epoch = epoch;
+                    continue;
+                }
+            }
             if (op.kind == OP_AXPY && !cur.list.empty() && cur.key.kind == OP_GEMV_LIST) {
                 const Op *prod = cur.list.back();
                 Alloc *h = op.a[1];
-                if (cur.residual.back() == nullptr && prod->batch == 1 && prod->a[2] == op.a[0] &&
+                const size_t n = cur.list.size();
+                const bool in_pair = cur.glu[n - 1] != nullptr || (n >= 2 && cur.glu[n - 2] != nullptr);
+                if (!in_pair && cur.residual.back() == nullptr && prod->batch == 1 &&
+                    prod->a[2] == op.a[0] &&
                     prod->y_off == 0 && prod->rows == op.extra && h != op.a[0] &&
                     h->read_epoch != epoch && h->write_epoch != epoch) {
                     cur.residual.back() = &op;
