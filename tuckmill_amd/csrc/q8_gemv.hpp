@@ -68,7 +68,7 @@ using GemvArgs = GemvArgsT<GEMV_MAX_DESCS>;
 
 // Most launches of a real step carry one to three products (q/k/v, gate/up, a
 // lone projection between two dependent operators): they use a short argument
-// block instead of the 12 KB one, which is copied and fetched per launch.
+// block instead of the 14 KB one, which is copied and fetched per launch.
 constexpr int GEMV_FEW_DESCS = 4;
 
 template <int NB, bool XA>

@@ -247,17 +247,30 @@ int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
 
 // ------------------------------------------------------------ launches ---
 
-// Products that may share a launch agree on this key.
+// Which kernel family and instantiation a recorded product launches with.
+// Products that may share a launch agree on the whole key.
+enum Variant : uint8_t {
+    V_DECODE,     // gemv_list_kernel, one token per pass (the streaming decode kernel)
+    V_GENERAL,    // gemv_list_kernel, four tokens per pass (raw layout / narrow small batches)
+    V_SPLIT,      // gemm_split_list_kernel: p0 = waves, p1 = tokens per wave, p2 = column tail
+    V_MMA,        // f32 MFMA GEMM: p0 = tmw, p1 = tnw, p2 = K split
+    V_I8_TILE,    // register-fed int8 MFMA GEMM: p0 = tile configuration
+    V_I8_STREAM,  // int8 streaming kernel: p0 = tokens per pass
+    V_I8_LDS      // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (0: 1x4 waves, 1: 2x2)
+};
+
 struct GemvKey {
-    OpKind kind;  // OP_GEMV_LIST, OP_MMA or OP_I8: which list kernel
-    bool packed;
-    int tb;       // GEMV: tokens per pass (1 or 4), or 200 + 10 * waves + tokens per wave
-                  // for the token-split small-batch kernel;
-                  // MFMA f32: tile/split code; int8: tile code
-    bool xalign;  // GEMV / MFMA f32: activations 16-byte aligned; int8: block dots are written out
+    OpKind kind = OP_GEMV_LIST; // OP_GEMV_LIST, OP_MMA or OP_I8
+    Variant variant = V_DECODE;
+    uint8_t p0 = 0, p1 = 0, p2 = 0;
+    bool packed = false;
+    bool flag = false; // GEMV / MFMA f32: activations 16-byte aligned; int8: block dots are written out
     bool operator==(const GemvKey &o) const {
-        return kind == o.kind && packed == o.packed && tb == o.tb && xalign == o.xalign;
+        return kind == o.kind && variant == o.variant && p0 == o.p0 && p1 == o.p1 && p2 == o.p2 &&
+               packed == o.packed && flag == o.flag;
     }
+    // one token, sealed weights, aligned activations: the kernel the planner's fusions target
+    bool decode() const { return kind == OP_GEMV_LIST && variant == V_DECODE && packed && flag; }
 };
 
 GemvKey gemv_key(const Op &op) {
@@ -265,37 +278,44 @@ GemvKey gemv_key(const Op &op) {
     k.kind = op.kind;
     k.packed = op.packed;
     if (op.kind == OP_I8) {
-        k.tb = q8::pick_i8_config(op.batch);
+        k.flag = op.a[3] != nullptr;
         if (op.packed && op.batch <= q8::GEMV_I8_MAX_BATCH) {
-            k.tb = 10 + q8::gemv_i8_tokens(op.batch); // the streaming kernel
+            k.variant = V_I8_STREAM;
+            k.p0 = (uint8_t)q8::gemv_i8_tokens(op.batch);
         } else if (op.packed && op.a[3] == nullptr && op.batch >= q8::GEMM_I8_LDS_MIN_BATCH &&
                    (uint64_t)op.rows * op.cols < (1ull << 32) &&
                    (uint64_t)op.batch * op.cols < (1ull << 32)) {
-            k.tb = op.batch <= 64u ? 20 : 21; // the LDS-staged kernel, by workgroup shape
+            k.variant = V_I8_LDS;
+            k.p0 = op.batch <= 64u ? 0 : 1;
+        } else {
+            k.variant = V_I8_TILE;
+            k.p0 = (uint8_t)q8::pick_i8_config(op.batch);
         }
-        k.xalign = op.a[3] != nullptr;
         return k;
     }
+    const uintptr_t xp = (uintptr_t)op.a[1]->ptr + (uintptr_t)op.x_off * 4u;
+    k.flag = (xp % 16u == 0);
     if (op.kind == OP_MMA) {
         // The tile shape and K split are chosen per product, so a product's
         // result does not depend on what else shares its launch.
         const q8::MmaProduct p{nullptr, nullptr, nullptr, op.rows, op.cols, op.batch};
         const q8::MmaConfig c = q8::pick_mma_config(&p, 1);
-        k.tb = c.tmw * 16 + c.tnw * 8 + c.s;
+        k.variant = V_MMA;
+        k.p0 = (uint8_t)c.tmw;
+        k.p1 = (uint8_t)c.tnw;
+        k.p2 = (uint8_t)c.s;
+    } else if (op.batch == 1) {
+        k.variant = V_DECODE;
+    } else if (op.packed && op.cols >= 1024u) {
+        // waves x tokens per wave, measured on 2B-class shapes (the
+        // alternatives were within 5 %)
+        k.variant = V_SPLIT;
+        k.p0 = op.batch <= 4 ? 1 : op.batch <= 8 ? 2 : 4;
+        k.p1 = op.batch <= 2 ? 2 : op.batch <= 16 ? 4 : 8;
+        k.p2 = (op.cols & 1023u) != 0u; // the instantiation that also handles a column tail
     } else {
-        k.tb = op.batch == 1 ? 1 : 4;
-        if (op.batch > 1 && op.packed && op.cols >= 1024u) {
-            // token-split kernel: 200 + 10 * waves + tokens per wave (measured
-            // on 2B-class shapes; the alternatives were within 5 %)
-            k.tb = 200 + (op.batch <= 2 ? 12 : op.batch <= 4 ? 14 : op.batch <= 8 ? 24
-                          : op.batch <= 16 ? 44 : 48);
-            if (op.cols & 1023u) {
-                k.tb += 100; // the instantiation that also handles a column tail
-            }
-        }
+        k.variant = V_GENERAL;
     }
-    const uintptr_t xp = (uintptr_t)op.a[1]->ptr + (uintptr_t)op.x_off * 4u;
-    k.xalign = (xp % 16u == 0);
     return k;
 }
 
@@ -394,8 +414,8 @@ hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<c
                                     (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
                                     op->batch};
     }
-    const q8::MmaConfig c{key.tb / 16, (key.tb / 8) % 2, key.tb % 8};
-    return q8::launch_gemm_mma_list(ctx->stream, stop, key.packed, key.xalign, prods, n, &c);
+    const q8::MmaConfig c{key.p0, key.p1, key.p2};
+    return q8::launch_gemm_mma_list(ctx->stream, stop, key.packed, key.flag, prods, n, &c);
 }
 
 hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
@@ -408,13 +428,13 @@ hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<co
                                    op->a[3] != nullptr ? (int32_t *)op->a[3]->ptr : nullptr,
                                    op->rows, op->cols, op->batch};
     }
-    if (key.tb >= 20) {
+    if (key.variant == V_I8_LDS) {
         return q8::launch_gemm_i8_lds_list(ctx->stream, stop, prods, n);
     }
-    if (key.tb >= 10) {
-        return q8::launch_gemv_i8_list(ctx->stream, stop, key.xalign, key.tb - 10, prods, n);
+    if (key.variant == V_I8_STREAM) {
+        return q8::launch_gemv_i8_list(ctx->stream, stop, key.flag, key.p0, prods, n);
     }
-    return q8::launch_gemm_i8_list(ctx->stream, stop, key.packed, key.xalign, key.tb, prods, n);
+    return q8::launch_gemm_i8_list(ctx->stream, stop, key.packed, key.flag, key.p0, prods, n);
 }
 
 hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch) {
@@ -427,7 +447,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     if (key.kind == OP_I8) {
         return launch_i8_list(ctx, stop, ops, key);
     }
-    q8::GemvArgs args; // only the used descriptors are written (the struct is 12 KB)
+    q8::GemvArgs args; // only the used descriptors are written (the struct is 14 KB)
     args.n = 0;
     args.pad = 0;
     args.norm_eps = launch.norm != nullptr ? launch.norm->scalar : 0.0f;
@@ -436,9 +456,9 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     args.norm_out = launch.norm != nullptr ? (float *)launch.norm->a[2]->ptr : nullptr;
     bool norm_written = false;
     bool fused = launch.norm != nullptr; // the launch needs the kernel variant with fused forms
-    const int R = (key.tb == 1 || key.tb >= 200) ? kGemvR1 : kGemvR4;
+    const int R = key.variant == V_GENERAL ? kGemvR4 : kGemvR1;
     // a workgroup's tile in the token-split kernel, a wave's tile otherwise
-    const uint32_t tile_bytes = key.tb >= 200 ? 32768u : 8192u;
+    const uint32_t tile_bytes = key.variant == V_SPLIT ? 32768u : 8192u;
     uint32_t tiles = 0;
     bool tails = false; // some product has a column tail with a streaming path of its own
     for (const Op *op : ops) {
@@ -481,7 +501,8 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     }
     args.total_tiles = tiles;
 #define TM_SPLIT_CASE(W, T, A, TL)                                                           \
-    if (key.tb == ((TL) ? 300 : 200) + (W) * 10 + (T) && key.xalign == (A)) {                \
+    if (key.variant == V_SPLIT && key.p0 == (W) && key.p1 == (T) && key.p2 == ((TL) ? 1 : 0) && \
+        key.flag == (A)) {                                                                   \
         Q8_LAUNCH((q8::gemm_split_list_kernel<W, T, A, TL>), dim3(tiles), dim3((W) * 64), 0, \
                   ctx->stream, stop, args);                                                  \
         return hipGetLastError();                                                            \
@@ -499,7 +520,8 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
 #undef TM_SPLIT_ALL
 #undef TM_SPLIT_CASE
 #define TM_GEMV_CASE(P, T, A)                                                                \
-    if (key.packed == (P) && key.tb == (T) && key.xalign == (A)) {                           \
+    if (key.packed == (P) && key.variant == ((T) == 1 ? V_DECODE : V_GENERAL) &&             \
+        key.flag == (A)) {                                                                   \
         return launch_gemv<(P) ? q8::PACKED : q8::RAW, (T) == 1 ? kGemvR1 : kGemvR4, T, A>(  \
             ctx, stop, args, tails, fused);                                                         \
     }
@@ -640,8 +662,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             // products may join its launch; the ones that read the norm's
             // whole output as their activations take it in without it going
             // through memory.
-            const bool decode_kind =
-                key.kind == OP_GEMV_LIST && key.tb == 1 && key.packed && key.xalign;
+            const bool decode_kind = key.decode();
             const bool normed = cur.norm != nullptr && decode_kind && op.a[1] == cur.norm->a[2] &&
                                 op.x_off == 0 && op.cols == cur.norm->cols;
             if (cur.norm != nullptr && !decode_kind) {
@@ -695,8 +716,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             // rows of a pair are computed by one wave, which applies the
             // activation itself. `out` may be the gate buffer (in place).
             if ((op.kind == OP_SILU_MUL || op.kind == OP_GELU_MUL) && cur.list.size() >= 2 &&
-                cur.key.kind == OP_GEMV_LIST && cur.key.tb == 1 && cur.key.packed &&
-                cur.key.xalign) {
+                cur.key.decode()) {
                 const size_t n = cur.list.size();
                 const Op *pg = cur.list[n - 2], *pu = cur.list[n - 1];
                 Alloc *out = op.a[2];
