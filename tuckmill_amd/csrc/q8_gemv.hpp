@@ -572,7 +572,16 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
         if (full >= 1u) {
             const uint32_t tail = cols & 1023u;
             if (tail == 0u) {
-                stream_rows<R, XA, 0>(wv, PlainX{x}, y, cols, row_first, row_end, lane, d.res, d.alpha);
+                if (d.rows_per_tile % (R / 2) != 0u) { // a small product cut into shorter tiles
+                    stream_rows<R / 4, XA, 0>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
+                                              d.res, d.alpha);
+                } else if (d.rows_per_tile % R != 0u) {
+                    stream_rows<R / 2, XA, 0>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
+                                              d.res, d.alpha);
+                } else {
+                    stream_rows<R, XA, 0>(wv, PlainX{x}, y, cols, row_first, row_end, lane, d.res,
+                                          d.alpha);
+                }
                 return;
             }
             if constexpr (TAILS >= 1) {

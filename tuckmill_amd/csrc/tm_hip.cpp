@@ -460,6 +460,11 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     // a workgroup's tile in the token-split kernel, a wave's tile otherwise
     const uint32_t tile_bytes = key.variant == V_SPLIT ? 32768u : 8192u;
     uint32_t tiles = 0;
+    uint64_t launch_bytes = 0;
+    for (const Op *op : ops) {
+        launch_bytes += (uint64_t)op->rows * (op->cols / 32u) * 34u;
+    }
+    const bool small_launch = launch_bytes < (16u << 20);
     bool tails = false; // some product has a column tail with a streaming path of its own
     for (const Op *op : ops) {
         const uint32_t tail = op->cols & 1023u;
@@ -473,6 +478,17 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         d.batch = op->batch;
         d.tile_begin = tiles;
         d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
+        if (small_launch && key.decode() && d.rows_per_tile == (uint32_t)R &&
+            (op->cols & 1023u) == 0u && (op->rows + R - 1) / R < 256u) {
+            // Fewer than 256 tiles even at one pass per wave, in a launch that
+            // is all latency (a projection of a few MB between two dependent
+            // operators): half-height tiles put twice as many waves on it.
+            // Inside a large launch full-height tiles stream better.
+            d.rows_per_tile = (uint32_t)R / 2u;
+            if ((op->rows + R / 2 - 1) / (R / 2) < 512u) {
+                d.rows_per_tile = (uint32_t)R / 4u;
+            }
+        }
         d.pad = 0;
         const size_t at = args.n - 1;
         const bool pair_first = launch.glu[at] != nullptr;
