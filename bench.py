@@ -74,8 +74,9 @@ def run_steps(host, ctx, products, warmup, steps, grouped=True) -> tmh_timing:
     arr = (tmh_product * len(products))(*products)
     t = tmh_timing()
     err = ctypes.create_string_buffer(H.ERR_CAP)
-    rc = host.tmh_run_steps(ctx.raw, arr, len(products), warmup, steps, 1 if grouped else 0,
-                            ctypes.byref(t), err, H.ERR_CAP)
+    mode = 2 if grouped == "recorded" else (1 if grouped else 0)
+    rc = host.tmh_run_steps(ctx.raw, arr, len(products), warmup, steps, mode, ctypes.byref(t), err,
+                            H.ERR_CAP)
     if rc != 0:
         raise SystemExit(f"step runner failed ({rc}): {err.value.decode()}")
     return t
@@ -386,6 +387,16 @@ def bench_chain(host, ctx, steps, warmup):
                        "launches_per_step": tg.launches / steps,
                        "gbs": wbytes / (tg.wall_ms / steps * 1e-3) / 1e9,
                        "host_issue_us": tg.host_ms / steps * 1e3}}
+    tr = run_steps(host, ctx, prods, warmup, steps, grouped="recorded")
+    out["recorded_step_replayed"] = {"us": tr.wall_ms / steps * 1e3, "gpu_us": tr.gpu_ms / steps * 1e3,
+                                     "launches_per_step": tr.launches / steps,
+                                     "gbs": wbytes / (tr.wall_ms / steps * 1e-3) / 1e9,
+                                     "host_issue_us": tr.host_ms / steps * 1e3}
+    # Over many steps the host is throttled by the depth of the hardware queue,
+    # so its own cost per token is measured on a run short enough to fit.
+    for name, mode in (("grouped", True), ("recorded_step_replayed", "recorded")):
+        ts = run_steps(host, ctx, prods, 2, 6, grouped=mode)
+        out[name]["host_issue_us_short_run"] = ts.host_ms / 6 * 1e3
     n_un = max(10, steps // 10)
     tu = run_steps(host, ctx, prods, 3, n_un, grouped=False)
     out["one_commit_per_operator"] = {"us": tu.wall_ms / n_un * 1e3,

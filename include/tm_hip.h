@@ -165,6 +165,25 @@ int tm_hip_begin_group(tm_hip_ctx *ctx, char *err, size_t err_cap);
 int tm_hip_end_group(tm_hip_ctx *ctx, char *err, size_t err_cap);
 int tm_hip_abort_group(tm_hip_ctx *ctx, char *err, size_t err_cap);
 
+/* A recorded group. The reference encodes the same operators on the same
+ * buffers again for every generated token (one command buffer per token:
+ * crates/tuckcore/src/qwen35_gpu.rs:71-77 around the per-layer calls of
+ * crates/tuckcore/src/engine/metal.rs:496-511, :1125-1131); Metal command
+ * buffers cannot be resubmitted, HIP graphs can. end_group_recorded closes the
+ * open group like end_group but, instead of committing it, keeps its planned
+ * launches as a replayable step (nothing runs yet); every step_run is one
+ * commit that executes them again on the current contents of the same buffers,
+ * with the results end_group would give. The step holds a reference on every
+ * buffer it touches until step_free (freeing a buffer handle earlier is
+ * allowed; the memory lives on), and on the weight bytes as they were laid out
+ * when it was recorded: seal weights before recording. A group that holds no
+ * operation cannot be recorded. step_free waits for queued replays. */
+typedef struct tm_hip_step tm_hip_step;
+int tm_hip_end_group_recorded(tm_hip_ctx *ctx, tm_hip_step **out, char *err, size_t err_cap);
+int tm_hip_step_run(tm_hip_ctx *ctx, tm_hip_step *step, char *err, size_t err_cap);
+uint32_t tm_hip_step_launches(const tm_hip_ctx *ctx, const tm_hip_step *step);
+void tm_hip_step_free(tm_hip_ctx *ctx, tm_hip_step *step);
+
 /* Block until every commit has completed; refused while a group is open
  * (native/metal/tm_metal.h:289-291). */
 int tm_hip_fence(tm_hip_ctx *ctx, char *err, size_t err_cap);

@@ -14,8 +14,16 @@
 // Launch with an optional stop event attached to the dispatch itself: the
 // event completes with the kernel and costs no extra packet on the stream
 // (a separate hipEventRecord after each launch measured +3 us per launch).
-#define Q8_LAUNCH(kernel, grid, block, lds, stream, stop_event, ...) \
-    hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, nullptr, stop_event, 0, __VA_ARGS__)
+// Without an event it is the plain launch, the form stream capture records.
+#define Q8_LAUNCH(kernel, grid, block, lds, stream, stop_event, ...)                              \
+    do {                                                                                          \
+        if ((stop_event) == nullptr) {                                                            \
+            hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                    \
+        } else {                                                                                  \
+            hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, nullptr, stop_event, 0,       \
+                                  __VA_ARGS__);                                                   \
+        }                                                                                         \
+    } while (0)
 
 namespace q8 {
 

@@ -105,6 +105,7 @@ struct tm_hip_ctx {
     std::atomic<int> profiling{0};
     bool group_active = false;
     std::vector<Op> group_ops;
+    std::vector<struct tm_hip_step *> steps; // recorded steps not yet freed
     uint64_t plan_epoch = 0;
     std::mutex q_mu; // pending commits, event pool, profile table
     std::mutex copy_mu;
@@ -119,6 +120,18 @@ struct tm_hip_buffer {
     Alloc *alloc;
     size_t len;
     int shared;
+};
+
+// A recorded dispatch group: its planned launches as an instantiated HIP graph
+// (kernel nodes only) and a reference on every allocation they touch, held
+// until the step is freed.
+struct tm_hip_step {
+    tm_hip_ctx *owner = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::vector<Alloc *> keep;
+    uint32_t launches = 0;
+    uint32_t operators = 0;
 };
 
 namespace {
@@ -802,9 +815,12 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, hipEvent_t sto
     return hipSuccess;
 }
 
-// Submit `ops` as one commit: start event, launches, stop event, leases.
-int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, const char *what,
-               char *err, size_t cap) {
+// Submit one commit: start event, the work `issue` puts on the stream, stop
+// event, leases on `keep` until the stop event has been reached. `issue`
+// receives the stop event and reports whether its last launch carries it.
+template <typename Issue>
+int commit_work(tm_hip_ctx *ctx, std::vector<Alloc *> keep, const char *label, const char *what,
+                Issue issue, char *err, size_t cap) {
     Commit c;
     bool fresh_start = true;
     {
@@ -822,17 +838,7 @@ int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, c
     if (c.start == nullptr || c.stop == nullptr) {
         return fail(err, cap, TM_HIP_ERR_INTERNAL, "%s: event creation failed", what);
     }
-    const uint64_t keep_epoch = ++ctx->plan_epoch;
-    c.keep.reserve(ops.size() * 3);
-    for (const Op &op : ops) {
-        for (int i = 0; i < op.n_alloc; ++i) {
-            Alloc *a = op.a[i];
-            if (a != nullptr && a->keep_epoch != keep_epoch) {
-                a->keep_epoch = keep_epoch;
-                c.keep.push_back(a);
-            }
-        }
-    }
+    c.keep = std::move(keep);
     for (Alloc *a : c.keep) {
         a->refs.fetch_add(1, std::memory_order_relaxed);
         c.leased += a->len;
@@ -843,9 +849,9 @@ int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, c
     hipError_t e = fresh_start ? hipEventRecord(c.start, ctx->stream) : hipSuccess;
     bool stop_attached = false;
     if (e == hipSuccess) {
-        e = issue_ops(ctx, ops, c.stop, &stop_attached);
+        e = issue(c.stop, &stop_attached);
     }
-    if (!stop_attached) { // an empty group, or a launch that failed
+    if (!stop_attached) { // an empty group, a replayed step, or a launch that failed
         hipError_t e2 = hipEventRecord(c.stop, ctx->stream);
         if (e == hipSuccess) {
             e = e2;
@@ -862,6 +868,33 @@ int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, c
         return hip_fail(err, cap, what, e);
     }
     return TM_HIP_OK;
+}
+
+// Every allocation the operations touch, once each.
+std::vector<Alloc *> allocs_of(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
+    std::vector<Alloc *> keep;
+    const uint64_t keep_epoch = ++ctx->plan_epoch;
+    keep.reserve(ops.size() * 3);
+    for (const Op &op : ops) {
+        for (int i = 0; i < op.n_alloc; ++i) {
+            Alloc *a = op.a[i];
+            if (a != nullptr && a->keep_epoch != keep_epoch) {
+                a->keep_epoch = keep_epoch;
+                keep.push_back(a);
+            }
+        }
+    }
+    return keep;
+}
+
+int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, const char *what,
+               char *err, size_t cap) {
+    return commit_work(
+        ctx, allocs_of(ctx, ops), label, what,
+        [&](hipEvent_t stop, bool *stop_attached) {
+            return issue_ops(ctx, ops, stop, stop_attached);
+        },
+        err, cap);
 }
 
 // Either appends to the open group or commits on its own. The profile label
@@ -960,6 +993,17 @@ int check_product(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_bu
     return TM_HIP_OK;
 }
 
+// The stream must be idle with respect to the step's replays.
+void step_dispose(tm_hip_step *step) {
+    (void)hipGraphExecDestroy(step->exec);
+    (void)hipGraphDestroy(step->graph);
+    for (Alloc *a : step->keep) {
+        alloc_release(a);
+    }
+    step->owner = nullptr;
+    delete step;
+}
+
 } // namespace
 
 // ================================================================ ABI =====
@@ -1023,6 +1067,10 @@ void tm_hip_destroy(tm_hip_ctx *ctx) {
         (void)hipStreamSynchronize(ctx->stream);
     }
     settle(ctx);
+    for (tm_hip_step *step : ctx->steps) { // recorded steps the caller never freed
+        step_dispose(step);
+    }
+    ctx->steps.clear();
     {
         std::lock_guard<std::mutex> g(ctx->q_mu);
         for (Commit &c : ctx->pending) { // only after a device error
@@ -1450,6 +1498,125 @@ int tm_hip_end_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {
     ops.swap(ctx->group_ops);
     // An empty group still commits once, like an empty command buffer.
     return commit_ops(ctx, ops, "group", "group", err, err_cap);
+}
+
+int tm_hip_end_group_recorded(tm_hip_ctx *ctx, tm_hip_step **out, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "end_group_recorded") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (out == nullptr) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "end_group_recorded: null result pointer");
+    }
+    *out = nullptr;
+    if (!ctx->group_active) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "end_group_recorded: no dispatch group is open");
+    }
+    ctx->group_active = false;
+    std::vector<Op> ops;
+    ops.swap(ctx->group_ops);
+    if (ops.empty()) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "end_group_recorded: the group holds no operation");
+    }
+    tm_hip_step *step = new (std::nothrow) tm_hip_step();
+    if (step == nullptr) {
+        return fail(err, err_cap, TM_HIP_ERR_ALLOC, "end_group_recorded: handle allocation failed");
+    }
+    step->owner = ctx;
+    step->operators = (uint32_t)ops.size();
+    const std::vector<Launch> plan = plan_launches(ctx, ops);
+    // Relaxed mode: the launchers may query occupancy while the stream records.
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed);
+    if (e != hipSuccess) {
+        delete step;
+        return hip_fail(err, err_cap, "end_group_recorded: begin capture", e);
+    }
+    hipError_t launch_err = hipSuccess;
+    for (const Launch &l : plan) {
+        launch_err = l.single != nullptr ? launch_single(ctx, nullptr, *l.single)
+                                         : launch_gemv_list(ctx, nullptr, l);
+        if (launch_err != hipSuccess) {
+            break;
+        }
+    }
+    e = hipStreamEndCapture(ctx->stream, &step->graph);
+    if (launch_err != hipSuccess || e != hipSuccess || step->graph == nullptr) {
+        (void)hipGetLastError();
+        if (step->graph != nullptr) {
+            (void)hipGraphDestroy(step->graph);
+        }
+        delete step;
+        return hip_fail(err, err_cap, "end_group_recorded: recording the launches",
+                        launch_err != hipSuccess ? launch_err : e);
+    }
+    e = hipGraphInstantiate(&step->exec, step->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipGraphDestroy(step->graph);
+        delete step;
+        return hip_fail(err, err_cap, "end_group_recorded: graph instantiation", e);
+    }
+    step->launches = (uint32_t)plan.size();
+    step->keep = allocs_of(ctx, ops);
+    for (Alloc *a : step->keep) {
+        a->refs.fetch_add(1, std::memory_order_relaxed);
+    }
+    ctx->steps.push_back(step);
+    *out = step;
+    return TM_HIP_OK;
+}
+
+int tm_hip_step_run(tm_hip_ctx *ctx, tm_hip_step *step, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "step_run") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (step == nullptr || step->owner != ctx) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "step_run: step does not belong to this context (different context or null)");
+    }
+    if (ctx->group_active) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "step_run: a dispatch group is open; end or abort it first");
+    }
+    const int rc = commit_work(
+        ctx, step->keep, "step", "step_run",
+        [&](hipEvent_t, bool *stop_attached) {
+            *stop_attached = false;
+            return hipGraphLaunch(step->exec, ctx->stream);
+        },
+        err, err_cap);
+    if (rc == TM_HIP_OK) {
+        ctx->launches.fetch_add(step->launches, std::memory_order_relaxed);
+    }
+    return rc;
+}
+
+uint32_t tm_hip_step_launches(const tm_hip_ctx *ctx, const tm_hip_step *step) {
+    if (ctx == nullptr || step == nullptr || step->owner != ctx) {
+        return 0;
+    }
+    return step->launches;
+}
+
+void tm_hip_step_free(tm_hip_ctx *ctx, tm_hip_step *step) {
+    if (ctx == nullptr || step == nullptr) {
+        return;
+    }
+    if (step->owner != ctx) {
+        fprintf(stderr, "tm_hip: step_free from a different context refused\n");
+        return;
+    }
+    // Replays still queued read the graph's kernel arguments and the buffers.
+    (void)hipStreamSynchronize(ctx->stream);
+    settle(ctx);
+    for (size_t i = 0; i < ctx->steps.size(); ++i) {
+        if (ctx->steps[i] == step) {
+            ctx->steps.erase(ctx->steps.begin() + (long)i);
+            break;
+        }
+    }
+    step_dispose(step);
 }
 
 int tm_hip_abort_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {

@@ -106,6 +106,12 @@ _SIGS = {
     "tm_hip_begin_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_end_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_abort_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_end_group_recorded": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p),
+                                                 ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_step_run": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_char_p,
+                                       ctypes.c_size_t]),
+    "tm_hip_step_launches": (ctypes.c_uint32, [ctypes.c_void_p, ctypes.c_void_p]),
+    "tm_hip_step_free": (None, [ctypes.c_void_p, ctypes.c_void_p]),
     "tm_hip_fence": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_q8_0_gemv": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_uint32] * 2 +
                          [ctypes.c_char_p, ctypes.c_size_t]),
@@ -259,6 +265,12 @@ class HipContext:
 
     def abort_group(self):
         self._operate("abort_group", self._lib.tm_hip_abort_group)
+
+    def end_group_recorded(self) -> "HipStep":
+        """Closes the open group as a replayable step instead of committing it."""
+        raw = ctypes.c_void_p()
+        self._operate("end_group_recorded", self._lib.tm_hip_end_group_recorded, ctypes.byref(raw))
+        return HipStep(self._inner, self._lib, raw)
 
     def fence(self):
         self._operate("fence", self._lib.tm_hip_fence)
@@ -438,6 +450,40 @@ class HipBuffer:
         if code != 0:
             raise hip_error(code, err.value.decode(), "download_after")
         return out
+
+
+class HipStep:
+    """A recorded dispatch group (``HipContext.end_group_recorded``): ``run()``
+    replays its launches as one commit; ``free()`` (or garbage collection)
+    releases the graph and the buffer references it holds."""
+
+    def __init__(self, ctx: _Inner, lib, raw):
+        self._ctx = ctx
+        self._lib = lib
+        self.raw = raw
+
+    def run(self):
+        with self._ctx.lock:
+            err = ctypes.create_string_buffer(ERR_CAP)
+            code = self._lib.tm_hip_step_run(self._ctx.raw, self.raw, err, ERR_CAP)
+        if code != 0:
+            raise hip_error(code, err.value.decode(), "step_run")
+
+    @property
+    def launches(self) -> int:
+        return int(self._lib.tm_hip_step_launches(self._ctx.raw, self.raw))
+
+    def free(self):
+        if self.raw and self._ctx.raw:
+            with self._ctx.lock:
+                self._lib.tm_hip_step_free(self._ctx.raw, self.raw)
+        self.raw = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
 
 
 def q8_0_bytes(rows: int, cols: int) -> int:

@@ -146,6 +146,36 @@ class HipBuffer {
     bool owned_ = true;
 };
 
+// A recorded dispatch group (tm_hip_end_group_recorded): replayed with run(),
+// released with the last copy of the handle.
+class RecordedStep {
+  public:
+    RecordedStep() = default;
+    void run() const {
+        std::lock_guard<std::mutex> g(state_->ctx->lock);
+        char err[ERR_CAP] = {0};
+        int code = tm_hip_step_run(state_->ctx->raw, state_->raw, err, ERR_CAP);
+        if (code != 0) {
+            throw hip_error(code, err, "step_run");
+        }
+    }
+    uint32_t launches() const { return tm_hip_step_launches(state_->ctx->raw, state_->raw); }
+
+  private:
+    friend class HipContext;
+    struct State {
+        std::shared_ptr<ContextInner> ctx;
+        tm_hip_step *raw = nullptr;
+        ~State() {
+            if (raw != nullptr && ctx && ctx->raw != nullptr) {
+                std::lock_guard<std::mutex> g(ctx->lock);
+                tm_hip_step_free(ctx->raw, raw);
+            }
+        }
+    };
+    std::shared_ptr<State> state_;
+};
+
 class HipContext {
   public:
     static HipContext open() {
@@ -201,6 +231,28 @@ class HipContext {
             throw;
         }
         end_group();
+    }
+
+    // Record `encode` as a replayable step instead of committing it.
+    template <class F> RecordedStep recorded(F encode) const {
+        begin_group();
+        try {
+            encode();
+        } catch (...) {
+            try {
+                abort_group();
+            } catch (...) {
+            }
+            throw;
+        }
+        tm_hip_step *raw_step = nullptr;
+        operate("end_group_recorded",
+                [&](char *e) { return tm_hip_end_group_recorded(raw(), &raw_step, e, ERR_CAP); });
+        RecordedStep step;
+        step.state_ = std::make_shared<RecordedStep::State>();
+        step.state_->ctx = inner_;
+        step.state_->raw = raw_step;
+        return step;
     }
 
     void q8_0_gemv(const HipBuffer &w, const HipBuffer &x, const HipBuffer &y, uint32_t rows,

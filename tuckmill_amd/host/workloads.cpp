@@ -3,8 +3,9 @@
 // A "step" is one pass of the hot path: a list of Q8_0 products issued the
 // way the reference's engine issues a token step — one dispatch group per
 // step (crates/tuckcore/src/engine/metal.rs:2462, qwen35_gpu.rs:66-85) — or
-// one commit per product when `grouped` is 0. The loop lives in native code
-// so that the measured time is the library's, not an interpreter's.
+// one commit per product when `grouped` is 0; `grouped` 2 records the group
+// once and replays it every step. The loop lives in native code so that the
+// measured time is the library's, not an interpreter's.
 #include <chrono>
 #include <cstdio>
 #include <cstring>
@@ -71,8 +72,14 @@ int tmh_run_steps(tm_hip_ctx *ctx, const tmh_product *products, uint32_t n, uint
             bound.push_back(Bound{gpu.borrow_buffer(products[i].w), gpu.borrow_buffer(products[i].x),
                                   gpu.borrow_buffer(products[i].y)});
         }
+        RecordedStep recorded;
+        if (grouped == 2) {
+            recorded = gpu.recorded([&]() { issue(gpu, products, bound, n); });
+        }
         auto one_step = [&]() {
-            if (grouped) {
+            if (grouped == 2) {
+                recorded.run();
+            } else if (grouped) {
                 gpu.grouped([&]() { issue(gpu, products, bound, n); });
             } else {
                 issue(gpu, products, bound, n);
