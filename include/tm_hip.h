@@ -218,10 +218,30 @@ int tm_hip_q8_0_row_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *out, u
                         uint32_t cols, uint32_t out_off, char *err, size_t err_cap);
 
 /* out[i] = row ids[slot] of `w` dequantized to f32; an id >= rows writes
- * zeros. Only type_id 8 (Q8_0) is built (native/metal/tm_metal.h:100-106). */
+ * zeros. type_id 8 is Q8_0 (cols a multiple of 32), type_id 1 is F16
+ * (native/metal/tm_metal.h:100-106, native/metal/tm_metal.m:874-885). */
 int tm_hip_row_indirect_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t type_id, uint32_t rows,
                             uint32_t cols, tm_hip_buffer *ids, uint32_t slot, tm_hip_buffer *out,
                             char *err, size_t err_cap);
+
+/* ---- F16 weight twins of the products ---- */
+
+/* y[r] = dot(f32(w_row_r), x); `w` holds rows*cols f16 values, any cols > 0
+ * (native/metal/tm_metal.h:141-144). */
+int tm_hip_f16_gemv(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                    uint32_t rows, uint32_t cols, char *err, size_t err_cap);
+
+/* The contract of tm_hip_q8_0_gemm on F16 weights: batch 1..=32, offsets in
+ * f32 elements, token b bit-identical to the GEMV on x[b]
+ * (native/metal/tm_metal.h:179-181, native/metal/kernels.metal:638-668). */
+int tm_hip_f16_gemm(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                    uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off, uint32_t y_off,
+                    char *err, size_t err_cap);
+
+/* out[out_off + i] = f32(w[row][i]), i < cols; exact
+ * (native/metal/tm_metal.h:155-157). */
+int tm_hip_f16_row_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *out, uint32_t row,
+                       uint32_t cols, uint32_t out_off, char *err, size_t err_cap);
 
 /* ---- additions with no Metal counterpart ---- */
 

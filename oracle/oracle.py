@@ -23,7 +23,7 @@ __all__ = [
     "gemv_q8_0_q8_0", "gemm_q8_0_f32", "gemm_q8_0_q8_0", "gemv_q8_0_f32_dequant_first",
     "gemv_q8_0_f64", "Rng", "boundary_weights", "boundary_input", "KRng",
     "random_q8_0_row", "block_sumi", "rmsnorm", "silu_mul", "gelu_tanh_mul", "axpy", "scale",
-    "argmax", "ARGMAX_NONE",
+    "argmax", "ARGMAX_NONE", "dot_f16_x_f32", "gemm_f16_f32", "f16_bytes",
 ]
 
 
@@ -70,6 +70,10 @@ def lib() -> ctypes.CDLL:
         for name in ("q8o_gemm_q8_0_f32", "q8o_gemm_q8_0_q8_0"):
             getattr(L, name).argtypes = [u8p, c.c_size_t, c.c_size_t, f32p, c.c_size_t,
                                          f32p, c.c_int]
+        L.q8o_validate_f16_row.argtypes = [c.c_size_t, c.c_size_t]
+        L.q8o_dot_f16_x_f32.restype = c.c_float
+        L.q8o_dot_f16_x_f32.argtypes = [u8p, c.c_size_t, f32p]
+        L.q8o_gemm_f16_f32.argtypes = [u8p, c.c_size_t, c.c_size_t, f32p, c.c_size_t, f32p]
         L.q8o_gemv_q8_0_f32_dequant_first.argtypes = [u8p, c.c_size_t, c.c_size_t, f32p, f32p]
         L.q8o_gemv_q8_0_f64.argtypes = [u8p, c.c_size_t, c.c_size_t, f32p, c.c_void_p]
         L.q8o_rng_next.restype = c.c_uint64
@@ -150,6 +154,43 @@ def dot_q8_0_x_f32(row, x) -> np.float32:
         raise OracleError("Internal", f"Q8_0 x f32 dot expects {row.size // 34 * 32} "
                           f"activation elements, got {x.size}")
     return np.float32(lib().q8o_dot_q8_0_x_f32(_ptr(row), row.size // 34, _ptr(x)))
+
+
+def dot_f16_x_f32(row, x) -> np.float32:
+    """kernels.rs:402-410 over scalar::dot_f16_x_f32, with its checked boundary."""
+    row = _u8(row)
+    x = _f32(x).ravel()
+    rc = lib().q8o_validate_f16_row(row.size, x.size)
+    if rc == -1:
+        raise OracleError("InvalidArtifact", f"packed F16 row length {row.size} is not a "
+                          "positive multiple of 2 bytes")
+    if rc == -2:
+        raise OracleError("Internal", f"F16 x f32 dot expects {row.size // 2} activation "
+                          f"elements, got {x.size}")
+    return np.float32(lib().q8o_dot_f16_x_f32(_ptr(row), row.size // 2, _ptr(x)))
+
+
+def gemm_f16_f32(w, rows, cols, x, batch=1) -> np.ndarray:
+    """y[b, r] = dot_f16_x_f32(row r of w, x[b]); w holds rows*cols f16 values."""
+    w = _u8(w)
+    x = _f32(x).ravel()
+    if rows <= 0 or cols <= 0 or w.size != rows * cols * 2:
+        raise OracleError("InvalidArtifact", f"weight bytes {w.size} != {rows}x{cols} F16")
+    if x.size != batch * cols:
+        raise OracleError("Internal", f"expects {batch * cols} activation elements, got {x.size}")
+    y = np.empty(batch * rows, dtype=np.float32)
+    lib().q8o_gemm_f16_f32(_ptr(w), rows, cols, _ptr(x), batch, _ptr(y))
+    return y.reshape(batch, rows) if batch > 1 else y
+
+
+def f16_bytes(values) -> np.ndarray:
+    """f32 values -> little-endian f16 bytes through f32_to_f16_bits (the
+    fixture construction of crates/metal/src/tests.rs:688-695)."""
+    v = _f32(values).ravel()
+    out = np.empty(v.size, dtype="<u2")
+    for i, f in enumerate(v):
+        out[i] = f32_to_f16_bits(f)
+    return out.view(np.uint8)
 
 
 def dot_q8_0_q8_0(row, x_qs, x_d) -> np.float32:

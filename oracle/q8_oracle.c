@@ -8,7 +8,7 @@
  * Pinning status (which known answers fix each function is listed next to
  * it; the tests that apply them live in tests/test_oracle_*.py):
  *   f16_to_f32, f32_to_f16_bits, dequant, quantize_row_q8_0,
- *   dot_q8_0_x_f32, dot_q8_0_q8_0, the generators: pinned.
+ *   dot_q8_0_x_f32, dot_q8_0_q8_0, dot_f16_x_f32, the generators: pinned.
  *   No function here is "parity unpinned".
  */
 #include "q8_oracle.h"
@@ -138,6 +138,41 @@ int q8o_validate_q8_0_row(size_t row_bytes, size_t x_len) {
         return -2;
     }
     return 0;
+}
+
+/* crates/tuckcore/src/kernels.rs:167-178 */
+int q8o_validate_f16_row(size_t row_bytes, size_t x_len) {
+    if (row_bytes == 0 || row_bytes % 2 != 0) {
+        return -1;
+    }
+    if (x_len != row_bytes / 2) {
+        return -2;
+    }
+    return 0;
+}
+
+/* crates/tuckcore/src/kernels.rs:223-232. Pinned by the zero row
+ * (kernels.rs:596-598), the error cases (kernels.rs:583-586), exact integer
+ * cases (small integers are exact in f16 and their products and sums in f32),
+ * an order-sensitive case that only the sequential sum from 0.0 satisfies,
+ * and a float64 evaluation within the rounding bound. */
+float q8o_dot_f16_x_f32(const uint8_t *row, size_t elems, const float *x) {
+    float acc = 0.0f;
+    for (size_t i = 0; i < elems; ++i) {
+        float w = q8o_f16_to_f32(read_u16_le(row + 2 * i));
+        float p = w * x[i];
+        acc += p;
+    }
+    return acc;
+}
+
+void q8o_gemm_f16_f32(const uint8_t *w, size_t rows, size_t cols, const float *x, size_t batch,
+                      float *y) {
+    for (size_t b = 0; b < batch; ++b) {
+        for (size_t r = 0; r < rows; ++r) {
+            y[b * rows + r] = q8o_dot_f16_x_f32(w + r * cols * 2, cols, x + b * cols);
+        }
+    }
 }
 
 /* crates/tuckcore/src/kernels.rs:153-165 */

@@ -51,6 +51,19 @@ float q8o_dot_q8_0_x_f32(const uint8_t *row, size_t blocks, const float *x);
 float q8o_dot_q8_0_q8_0(const uint8_t *row, size_t blocks, const int8_t *x_qs,
                         const float *x_d, int32_t *sumi_out);
 
+/* F16 weight rows (the reference's F16 twins of the Q8_0 products).
+ * crates/tuckcore/src/kernels.rs:167-178: 0 when the row is a positive even
+ * number of bytes and x_len == row_bytes / 2; -1 malformed row, -2 length. */
+int q8o_validate_f16_row(size_t row_bytes, size_t x_len);
+/* crates/tuckcore/src/kernels.rs:223-232 (scalar::dot_f16_x_f32):
+ * acc += f16_to_f32(w[i]) * x[i], sequential from 0.0, unfused. */
+float q8o_dot_f16_x_f32(const uint8_t *row, size_t elems, const float *x);
+/* y[b*rows + r] = dot_f16_x_f32(row r, x[b]) (the row loop of
+ * forward.rs:703-735 over F16 rows; native/metal/kernels.metal:296-315,
+ * :638-668 state the same contract for the device). */
+void q8o_gemm_f16_f32(const uint8_t *w, size_t rows, size_t cols, const float *x, size_t batch,
+                      float *y);
+
 /* Row loop of crates/tuckcore/src/forward.rs:703-735 (matvec_fused):
  * y[r] = dot_q8_0_x_f32(row r, x). `threads` > 1 partitions rows (rows are
  * independent, so the output is bit-identical for every thread count). */

@@ -29,6 +29,7 @@
 #include "q8_gemm_small.hpp"
 #include "q8_misc.hpp"
 #include "q8_neighbors.hpp"
+#include "f16_gemv.hpp"
 
 namespace {
 
@@ -55,7 +56,8 @@ void alloc_release(Alloc *a) {
 
 enum OpKind {
     OP_GEMV_LIST, OP_MMA, OP_ROW, OP_ROW_INDIRECT, OP_COPY, OP_PACK, OP_QUANT, OP_I8,
-    OP_SCALE, OP_AXPY, OP_SILU_MUL, OP_GELU_MUL, OP_RMSNORM, OP_ARGMAX
+    OP_SCALE, OP_AXPY, OP_SILU_MUL, OP_GELU_MUL, OP_RMSNORM, OP_ARGMAX,
+    OP_F16_GEMM, OP_F16_ROW, OP_F16_ROW_INDIRECT
 };
 
 struct Op {
@@ -638,6 +640,20 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
                   (const uint32_t *)part_i, (uint32_t *)op.a[2]->ptr, op.y_off);
         break;
     }
+    case OP_F16_GEMM:
+        return q8::launch_f16_gemm(st, stop, (const uint16_t *)op.a[0]->ptr,
+                                   (const float *)op.a[1]->ptr + op.x_off,
+                                   (float *)op.a[2]->ptr + op.y_off, op.rows, op.cols, op.batch);
+    case OP_F16_ROW:
+        Q8_LAUNCH(q8::f16_row_kernel, dim3((op.cols + 255u) / 256u), dim3(256), 0, st, stop,
+                  (const uint16_t *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.cols, op.extra,
+                  op.y_off);
+        break;
+    case OP_F16_ROW_INDIRECT:
+        Q8_LAUNCH(q8::f16_row_indirect_kernel, dim3((op.cols + 255u) / 256u), dim3(256), 0, st, stop,
+                  (const uint16_t *)op.a[0]->ptr, (float *)op.a[1]->ptr,
+                  (const uint32_t *)op.a[2]->ptr, op.extra, op.rows, op.cols);
+        break;
     case OP_PACK: {
         const size_t nblocks = (size_t)op.rows * (op.cols / 32u);
         Q8_LAUNCH(q8::pack_kernel, dim3((unsigned)((nblocks + 255u) / 256u)), dim3(256), 0, st, stop,
@@ -1756,13 +1772,16 @@ int tm_hip_row_indirect_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t type_id,
     if (check_ctx(ctx, err, err_cap, "row_indirect") != TM_HIP_OK) {
         return TM_HIP_ERR_UNSUPPORTED;
     }
-    if (!(type_id == 8u && cols > 0 && (cols % 32u) == 0u)) {
+    // native/metal/tm_metal.m:874-885: Q8_0 (type 8) or F16 (type 1)
+    const bool f16 = type_id == 1u && cols > 0;
+    if (!f16 && !(type_id == 8u && cols > 0 && (cols % 32u) == 0u)) {
         return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
-                    "row_indirect: type %u with cols %u is unsupported (only Q8_0, type 8, with "
-                    "cols a positive multiple of 32)",
+                    "row_indirect: type %u with cols %u is unsupported (Q8_0, type 8, with cols a "
+                    "positive multiple of 32, or F16, type 1)",
                     type_id, cols);
     }
-    const size_t w_need = (size_t)rows * ((size_t)cols / 32u) * 34u;
+    const size_t w_need = f16 ? (size_t)rows * (size_t)cols * 2u
+                              : (size_t)rows * ((size_t)cols / 32u) * 34u;
     if (rows == 0) {
         return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "row_indirect: zero rows");
     }
@@ -1774,6 +1793,10 @@ int tm_hip_row_indirect_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t type_id,
             TM_HIP_OK) {
         return rc;
     }
+    if (f16 && w->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "row_indirect: type 1 (F16) names a sealed Q8_0 weight buffer");
+    }
     if (w->alloc->packed && (w->alloc->prows != rows || w->alloc->pcols != cols)) {
         return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
                     "row_indirect: weights were sealed as %ux%u but the call names %ux%u",
@@ -1783,7 +1806,7 @@ int tm_hip_row_indirect_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t type_id,
         return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "row_indirect: sealed weight buffer");
     }
     Op op;
-    op.kind = OP_ROW_INDIRECT;
+    op.kind = f16 ? OP_F16_ROW_INDIRECT : OP_ROW_INDIRECT;
     op.a[0] = w->alloc;
     op.a[1] = out->alloc;
     op.a[2] = ids->alloc;
@@ -1794,6 +1817,93 @@ int tm_hip_row_indirect_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t type_id,
     op.extra = slot;
     op.packed = w->alloc->packed;
     return submit(ctx, op, "row_indirect", err, err_cap);
+}
+
+// ------------------------------------------------- F16 weight twins ------
+
+// native/metal/tm_metal.m:1279-1290 (shape, then bounds) with w_need of :1349.
+static int f16_product(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                       uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off,
+                       uint32_t y_off, const char *what, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, what) != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (rows == 0 || cols == 0 || batch == 0 || batch > q8::F16_GEMM_MAX_BATCH) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "%s: rows %u, cols %u, batch %u (1..=%u)",
+                    what, rows, cols, batch, q8::F16_GEMM_MAX_BATCH);
+    }
+    const size_t needs[3] = {(size_t)rows * (size_t)cols * 2u,
+                             ((size_t)x_off + (size_t)batch * cols) * 4u,
+                             ((size_t)y_off + (size_t)batch * rows) * 4u};
+    tm_hip_buffer *bufs[3] = {w, x, y};
+    static const char *const suffix[3] = {"weights", "x", "y"};
+    for (int i = 0; i < 3; ++i) {
+        char name[64];
+        snprintf(name, sizeof name, "%s.%s", what, suffix[i]);
+        const int rc = check_buffer(ctx, bufs[i], needs[i], err, err_cap, name);
+        if (rc != TM_HIP_OK) {
+            return rc;
+        }
+        if (bufs[i]->alloc->packed) {
+            return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "%s is a sealed Q8_0 weight buffer",
+                        name);
+        }
+    }
+    Op op;
+    op.kind = OP_F16_GEMM;
+    op.a[0] = w->alloc;
+    op.a[1] = x->alloc;
+    op.a[2] = y->alloc;
+    op.n_alloc = 3;
+    op.writes_mask = 4;
+    op.rows = rows;
+    op.cols = cols;
+    op.batch = batch;
+    op.x_off = x_off;
+    op.y_off = y_off;
+    op.shape_label = true;
+    return submit(ctx, op, what, err, err_cap);
+}
+
+int tm_hip_f16_gemv(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                    uint32_t rows, uint32_t cols, char *err, size_t err_cap) {
+    return f16_product(ctx, w, x, y, rows, cols, 1, 0, 0, "f16_gemv", err, err_cap);
+}
+
+int tm_hip_f16_gemm(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
+                    uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off, uint32_t y_off,
+                    char *err, size_t err_cap) {
+    return f16_product(ctx, w, x, y, rows, cols, batch, x_off, y_off, "f16_gemm", err, err_cap);
+}
+
+int tm_hip_f16_row_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *out, uint32_t row,
+                       uint32_t cols, uint32_t out_off, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "f16_row") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (cols == 0) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "f16_row: zero cols");
+    }
+    int rc;
+    if ((rc = check_buffer(ctx, w, ((size_t)row + 1u) * (size_t)cols * 2u, err, err_cap,
+                           "f16_row.weights")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, out, ((size_t)out_off + cols) * 4u, err, err_cap, "f16_row.out")) !=
+            TM_HIP_OK) {
+        return rc;
+    }
+    if (w->alloc->packed || out->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "f16_row: sealed Q8_0 weight buffer");
+    }
+    Op op;
+    op.kind = OP_F16_ROW;
+    op.a[0] = w->alloc;
+    op.a[1] = out->alloc;
+    op.n_alloc = 2;
+    op.writes_mask = 2;
+    op.cols = cols;
+    op.extra = row;
+    op.y_off = out_off;
+    return submit(ctx, op, "f16_row", err, err_cap);
 }
 
 // ---------------------------------------------------------- additions ----

@@ -121,6 +121,12 @@ _SIGS = {
                              [ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_q8_0_row_f32": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_uint32] * 3 +
                             [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_f16_gemv": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_uint32] * 2 +
+                        [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_f16_gemm": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_uint32] * 5 +
+                        [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_f16_row_f32": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_uint32] * 3 +
+                           [ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_row_indirect_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
                                                ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
                                                ctypes.c_uint32, ctypes.c_void_p, ctypes.c_char_p,
@@ -293,6 +299,20 @@ class HipContext:
     def q8_0_row(self, w, out, row: int, cols: int, out_off: int = 0):
         self._check_owned(w, out)
         self._operate("q8_0_row", self._lib.tm_hip_q8_0_row_f32, w.raw, out.raw, row, cols, out_off)
+
+    # -- F16 weight twins ----------------------------------------------------
+    def f16_gemv(self, w, x, y, rows: int, cols: int):
+        self._check_owned(w, x, y)
+        self._operate("f16_gemv", self._lib.tm_hip_f16_gemv, w.raw, x.raw, y.raw, rows, cols)
+
+    def f16_gemm(self, w, x, y, rows, cols, batch, x_off=0, y_off=0):
+        self._check_owned(w, x, y)
+        self._operate("f16_gemm", self._lib.tm_hip_f16_gemm, w.raw, x.raw, y.raw, rows, cols,
+                      batch, x_off, y_off)
+
+    def f16_row(self, w, out, row: int, cols: int, out_off: int = 0):
+        self._check_owned(w, out)
+        self._operate("f16_row", self._lib.tm_hip_f16_row_f32, w.raw, out.raw, row, cols, out_off)
 
     def row_indirect_f32(self, w, type_id, rows, cols, ids, slot, out):
         self._check_owned(w, ids, out)
@@ -508,7 +528,8 @@ def xq_split(raw: np.ndarray, cols: int, batch: int):
 
 class Matrix:
     """A device projection matrix: the HIP form of the reference's ``Matrix``
-    (crates/tuckcore/src/engine/metal.rs:106-226) for Q8_0 weights."""
+    (crates/tuckcore/src/engine/metal.rs:106-226): Q8_0 blocks (type 8) or
+    F16 halves (type 1), uploaded raw."""
 
     def __init__(self, buf: HipBuffer, type_id: int, in_dim: int, out_dim: int):
         self.buf = buf
@@ -517,8 +538,8 @@ class Matrix:
         self.out_dim = out_dim
 
     @staticmethod
-    def plan(in_dim: int, out_dim: int) -> int:
-        return q8_0_bytes(out_dim, in_dim)
+    def plan(in_dim: int, out_dim: int, type_id: int = 8) -> int:
+        return out_dim * in_dim * 2 if type_id == 1 else q8_0_bytes(out_dim, in_dim)
 
     @staticmethod
     def load(ctx: HipContext, raw, in_dim: int, out_dim: int, type_id: int = 8,
@@ -527,12 +548,12 @@ class Matrix:
         the seal step that re-lays the weights out for the device."""
         if out_dim <= 1:
             raise TuckmillError("Internal", "1-D tensors use the f32 path")
-        if type_id != 8:
+        if type_id not in (1, 8):
             raise TuckmillError("UnsupportedQuantization",
-                                f"engine matrices on this path must be Q8_0; got type {type_id}")
+                                f"engine matrices must be F16 or Q8_0; got type {type_id}")
         raw = np.ascontiguousarray(np.frombuffer(raw, dtype=np.uint8) if not
                                    isinstance(raw, np.ndarray) else raw).view(np.uint8).ravel()
-        total = Matrix.plan(in_dim, out_dim)
+        total = Matrix.plan(in_dim, out_dim, type_id)
         if raw.size != total:
             raise TuckmillError("InvalidArtifact", f"tensor holds {raw.size} bytes, "
                                 f"expected {total}")
@@ -542,26 +563,33 @@ class Matrix:
             n = min(STAGING_CHUNK_BYTES, total - off)
             buf.upload(off, raw[off:off + n])
             off += n
-        if seal:
+        if seal and type_id == 8:
             ctx.q8_0_pack(buf, out_dim, in_dim)
         return Matrix(buf, type_id, in_dim, out_dim)
 
     def gemv(self, ctx: HipContext, x: HipBuffer, y: HipBuffer):
-        ctx.q8_0_gemv(self.buf, x, y, self.out_dim, self.in_dim)
+        if self.type_id == 1:
+            ctx.f16_gemv(self.buf, x, y, self.out_dim, self.in_dim)
+        else:
+            ctx.q8_0_gemv(self.buf, x, y, self.out_dim, self.in_dim)
 
     def gemm(self, ctx: HipContext, x: HipBuffer, y: HipBuffer, batch: int, exact: bool):
         rows, cols = self.out_dim, self.in_dim
-        if not exact and 2 <= batch <= GEMM_MMA_MAX_BATCH:
+        if not exact and self.type_id == 8 and 2 <= batch <= GEMM_MMA_MAX_BATCH:
             ctx.q8_0_gemm_mma(self.buf, x, y, rows, cols, batch, 0, 0)
             return
+        product = ctx.f16_gemm if self.type_id == 1 else ctx.q8_0_gemm
         t0 = 0
         while t0 < batch:
             n = min(batch - t0, GEMM_MAX_BATCH)
-            ctx.q8_0_gemm(self.buf, x, y, rows, cols, n, t0 * cols, t0 * rows)
+            product(self.buf, x, y, rows, cols, n, t0 * cols, t0 * rows)
             t0 += n
 
     def row_indirect(self, ctx: HipContext, ids: HipBuffer, slot: int, out: HipBuffer):
         ctx.row_indirect_f32(self.buf, self.type_id, self.out_dim, self.in_dim, ids, slot, out)
 
     def row_into(self, ctx: HipContext, row: int, out: HipBuffer, out_off: int):
-        ctx.q8_0_row(self.buf, out, row, self.in_dim, out_off)
+        if self.type_id == 1:
+            ctx.f16_row(self.buf, out, row, self.in_dim, out_off)
+        else:
+            ctx.q8_0_row(self.buf, out, row, self.in_dim, out_off)

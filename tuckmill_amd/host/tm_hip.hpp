@@ -281,6 +281,25 @@ class HipContext {
             return tm_hip_q8_0_row_f32(raw(), w.raw(), out.raw(), row, cols, out_off, e, ERR_CAP);
         });
     }
+    void f16_gemv(const HipBuffer &w, const HipBuffer &x, const HipBuffer &y, uint32_t rows,
+                  uint32_t cols) const {
+        operate("f16_gemv", [&](char *e) {
+            return tm_hip_f16_gemv(raw(), w.raw(), x.raw(), y.raw(), rows, cols, e, ERR_CAP);
+        });
+    }
+    void f16_gemm(const HipBuffer &w, const HipBuffer &x, const HipBuffer &y, uint32_t rows,
+                  uint32_t cols, uint32_t batch, uint32_t x_off, uint32_t y_off) const {
+        operate("f16_gemm", [&](char *e) {
+            return tm_hip_f16_gemm(raw(), w.raw(), x.raw(), y.raw(), rows, cols, batch, x_off, y_off,
+                                   e, ERR_CAP);
+        });
+    }
+    void f16_row(const HipBuffer &w, const HipBuffer &out, uint32_t row, uint32_t cols,
+                 uint32_t out_off) const {
+        operate("f16_row", [&](char *e) {
+            return tm_hip_f16_row_f32(raw(), w.raw(), out.raw(), row, cols, out_off, e, ERR_CAP);
+        });
+    }
     void row_indirect_f32(const HipBuffer &w, uint32_t type_id, uint32_t rows, uint32_t cols,
                           const HipBuffer &ids, uint32_t slot, const HipBuffer &out) const {
         operate("row_indirect", [&](char *e) {
@@ -373,7 +392,9 @@ class HipContext {
 // (crates/tuckcore/src/engine/metal.rs:106-226).
 class Matrix {
   public:
-    static uint64_t plan(uint64_t in_dim, uint64_t out_dim) { return out_dim * (in_dim / 32u) * 34u; }
+    static uint64_t plan(uint64_t in_dim, uint64_t out_dim, uint32_t type_id = 8) {
+        return type_id == 1 ? out_dim * in_dim * 2u : out_dim * (in_dim / 32u) * 34u;
+    }
 
     // Staged raw upload in 4 MiB slices (engine/metal.rs:138-147), then the
     // seal step that re-lays the weights out for coalesced device loads.
@@ -382,11 +403,11 @@ class Matrix {
         if (out_dim <= 1) {
             throw TuckmillError(ErrorCode::Internal, "1-D tensors use the f32 path");
         }
-        if (type_id != 8) {
+        if (type_id != 1 && type_id != 8) {
             throw TuckmillError(ErrorCode::UnsupportedQuantization,
-                                "engine matrices on this path must be Q8_0");
+                                "engine matrices must be F16 or Q8_0");
         }
-        const size_t total = (size_t)plan(in_dim, out_dim);
+        const size_t total = (size_t)plan(in_dim, out_dim, type_id);
         Matrix m;
         m.buf = gpu.buffer(total, true);
         for (size_t off = 0; off < total;) {
@@ -394,7 +415,7 @@ class Matrix {
             m.buf.upload(off, raw + off, n);
             off += n;
         }
-        if (seal) {
+        if (seal && type_id == 8) {
             gpu.q8_0_pack(m.buf, (uint32_t)out_dim, (uint32_t)in_dim);
         }
         m.type_id = type_id;
@@ -404,7 +425,11 @@ class Matrix {
     }
 
     void gemv(const HipContext &gpu, const HipBuffer &x, const HipBuffer &y) const {
-        gpu.q8_0_gemv(buf, x, y, (uint32_t)out_dim, (uint32_t)in_dim);
+        if (type_id == 1) {
+            gpu.f16_gemv(buf, x, y, (uint32_t)out_dim, (uint32_t)in_dim);
+        } else {
+            gpu.q8_0_gemv(buf, x, y, (uint32_t)out_dim, (uint32_t)in_dim);
+        }
     }
 
     // engine/metal.rs:171-196: batch 1 and `exact` keep the GEMV's per-row
@@ -412,13 +437,17 @@ class Matrix {
     void gemm(const HipContext &gpu, const HipBuffer &x, const HipBuffer &y, uint32_t batch,
               bool exact) const {
         const uint32_t rows = (uint32_t)out_dim, cols = (uint32_t)in_dim;
-        if (!exact && batch >= 2 && batch <= GEMM_MMA_MAX_BATCH) {
+        if (!exact && type_id == 8 && batch >= 2 && batch <= GEMM_MMA_MAX_BATCH) {
             gpu.q8_0_gemm_mma(buf, x, y, rows, cols, batch, 0, 0);
             return;
         }
         for (uint32_t t0 = 0; t0 < batch;) {
             const uint32_t n = std::min(batch - t0, GEMM_MAX_BATCH);
-            gpu.q8_0_gemm(buf, x, y, rows, cols, n, t0 * cols, t0 * rows);
+            if (type_id == 1) {
+                gpu.f16_gemm(buf, x, y, rows, cols, n, t0 * cols, t0 * rows);
+            } else {
+                gpu.q8_0_gemm(buf, x, y, rows, cols, n, t0 * cols, t0 * rows);
+            }
             t0 += n;
         }
     }
@@ -429,7 +458,11 @@ class Matrix {
     }
 
     void row_into(const HipContext &gpu, uint32_t row, const HipBuffer &out, uint32_t out_off) const {
-        gpu.q8_0_row(buf, out, row, (uint32_t)in_dim, out_off);
+        if (type_id == 1) {
+            gpu.f16_row(buf, out, row, (uint32_t)in_dim, out_off);
+        } else {
+            gpu.q8_0_row(buf, out, row, (uint32_t)in_dim, out_off);
+        }
     }
 
     HipBuffer buf;
