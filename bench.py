@@ -54,7 +54,7 @@ class tmh_timing(ctypes.Structure):
 
 
 TMH_GEMV, TMH_GEMM, TMH_GEMM_MMA, TMH_GEMM_I8, TMH_QUANT = range(5)
-TMH_RMSNORM, TMH_SILU_MUL, TMH_AXPY, TMH_ARGMAX = range(5, 9)
+TMH_RMSNORM, TMH_SILU_MUL, TMH_AXPY, TMH_ARGMAX, TMH_F16_GEMM = range(5, 10)
 
 
 def load_host():
@@ -325,6 +325,39 @@ def bench_sweep(host, ctx, steps, warmup):
     return out
 
 
+def bench_f16(host, ctx, steps, warmup):
+    """The F16 twins on the 2B-class projection shapes: 20 copies of each matrix as
+    F16 (1.0 GB per pass), batch 1, 2, 4, 8 and 32, one commit per pass."""
+    copies = 20
+    rng = np.random.default_rng(7)
+    mats = []
+    for name, r, c in S.SWEEP_2B:
+        h = (rng.standard_normal(r * c, dtype=np.float32) * np.float32(0.02)).astype(np.float16)
+        for _ in range(copies):
+            b = ctx.buffer(r * c * 2)
+            b.upload(0, h.view(np.uint8))
+            mats.append((r, c, b))
+    wbytes = sum(r * c * 2 for r, c, _ in mats)
+    maxc = max(c for _, c, _ in mats)
+    maxr = max(r for r, _, _ in mats)
+    xb = ctx.buffer(32 * maxc * 4)
+    xb.upload(0, S.make_activations(32 * maxc, 98))
+    ys = [ctx.buffer(32 * maxr * 4) for _ in mats]
+    out = {"workload": "F16 twins, 2B-class shapes", "weights_bytes": wbytes, "points": []}
+    for M in (1, 2, 4, 8, 32):
+        n = max(3, steps // 10)
+        prods = [tmh_product(b.raw, xb.raw, yb.raw, r, c, M, TMH_F16_GEMM)
+                 for (r, c, b), yb in zip(mats, ys)]
+        t = run_steps(host, ctx, prods, max(2, n // 5), n, grouped=True)
+        us = t.gpu_ms / n * 1e3
+        abytes = wbytes + sum(4 * M * (r + c) for r, c, _ in mats)
+        out["points"].append({"M": M, "us": us, "launches": t.launches / n, "gbs": abytes / us / 1e3,
+                              "pct_of_hbm_peak": abytes / us / 1e3 / 80.0})
+    for b in [xb] + ys + [m[2] for m in mats]:
+        b.free()
+    return out
+
+
 def bench_chain(host, ctx, steps, warmup):
     """The decode step with its data dependencies: per layer rmsnorm -> q,k,v -> o ->
     residual -> rmsnorm -> gate,up -> silu_mul -> down -> residual, then final norm,
@@ -440,7 +473,7 @@ def main():
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--ungrouped", action="store_true",
                     help="one commit per GEMV instead of one group per step")
-    ap.add_argument("--workload", choices=["decode", "gemma", "sweep", "chain", "traffic"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "gemma", "sweep", "chain", "f16", "traffic"], default="decode",
                     help="decode (default, the headline line); gemma / sweep print the "
                          "BASELINE config 3 / 4 measurements as one JSON object")
     args = ap.parse_args()
@@ -457,7 +490,8 @@ def main():
         ctx.close()
         return
     if args.workload != "decode":
-        fn = {"gemma": bench_gemma, "sweep": bench_sweep, "chain": bench_chain}[args.workload]
+        fn = {"gemma": bench_gemma, "sweep": bench_sweep, "chain": bench_chain,
+              "f16": bench_f16}[args.workload]
         print(json.dumps(fn(host, ctx, args.steps, args.warmup)), flush=True)
         ctx.close()
         return

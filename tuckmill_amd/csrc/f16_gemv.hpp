@@ -26,26 +26,37 @@ constexpr uint32_t F16_GEMM_MAX_BATCH = 32; // native/metal/tm_metal.m:1279-1283
 __device__ __forceinline__ float f16_lo(uint32_t v) { return f16_bits_to_f32(v & 0xffffu); }
 __device__ __forceinline__ float f16_hi(uint32_t v) { return f16_bits_to_f32(v >> 16); }
 
-// VEC: cols % 8 == 0 (16-byte loads of 8 halves per lane). A wave owns
-// `rows_per_tile` rows (a multiple of 8), 8 rows per pass, TB tokens per sweep
-// over its rows; the weights of the next (pass, chunk) step are requested
-// before the current one is used.
+// VEC: cols % 8 == 0 for every product of the launch (16-byte loads of 8
+// halves per lane). Like the Q8_0 kernels it is a list kernel: independent
+// products of a dispatch group share one launch, a wave finds its product by
+// its tile number. A wave owns `rows_per_tile` rows (a multiple of 8), 8 rows
+// per pass, TB tokens per sweep over its rows; the weights of the next
+// (pass, chunk) step are requested before the current one is used.
 template <int TB, bool VEC>
-__global__ __launch_bounds__(256) void f16_gemm_kernel(const uint16_t *__restrict__ w,
-                                                       const float *__restrict__ x,
-                                                       float *__restrict__ y, uint32_t rows,
-                                                       uint32_t cols, uint32_t batch,
-                                                       uint32_t rows_per_tile) {
+__global__ __launch_bounds__(256) void f16_gemm_list_kernel(const GemvArgs args) {
     constexpr int R = 8;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t tile = blockIdx.x * 4u + wave;
-    const uint64_t first64 = (uint64_t)tile * rows_per_tile;
-    if (first64 >= rows) {
+    if (tile >= args.total_tiles) {
         return;
     }
-    const uint32_t row_first = (uint32_t)first64;
-    const uint32_t row_end = rows - row_first < rows_per_tile ? rows : row_first + rows_per_tile;
+    uint32_t lo = 0, hi = args.n;
+    while (hi - lo > 1u) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (args.d[mid].tile_begin <= tile) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    const GemvDesc &d = args.d[lo];
+    const uint16_t *__restrict__ w = (const uint16_t *)d.w;
+    const float *__restrict__ x = d.x;
+    float *__restrict__ y = d.y;
+    const uint32_t rows = d.rows, cols = d.cols, batch = d.batch;
+    const uint32_t row_first = (tile - d.tile_begin) * d.rows_per_tile;
+    const uint32_t row_end = rows - row_first < d.rows_per_tile ? rows : row_first + d.rows_per_tile;
     const uint32_t nchunks = (cols + 511u) >> 9;
     const uint32_t passes = (row_end - row_first + R - 1) / R;
     const uint32_t nsteps = passes * nchunks;
@@ -209,33 +220,73 @@ inline uint32_t f16_rows_per_tile(uint32_t rows, uint32_t cols) {
     return rpt;
 }
 
-template <int TB>
-inline hipError_t launch_f16_gemm_tb(hipStream_t stream, hipEvent_t stop, const uint16_t *w,
-                                     const float *x, float *y, uint32_t rows, uint32_t cols,
-                                     uint32_t batch) {
-    const uint32_t rpt = f16_rows_per_tile(rows, cols);
-    const uint32_t tiles = (rows + rpt - 1u) / rpt;
-    const dim3 grid((tiles + 3u) / 4u);
-    if ((cols & 7u) == 0u) {
-        Q8_LAUNCH((f16_gemm_kernel<TB, true>), grid, dim3(256), 0, stream, stop, w, x, y, rows, cols,
-                  batch, rpt);
-    } else {
-        Q8_LAUNCH((f16_gemm_kernel<TB, false>), grid, dim3(256), 0, stream, stop, w, x, y, rows, cols,
-                  batch, rpt);
+struct F16Product {
+    const uint16_t *w;
+    const float *x;
+    float *y;
+    uint32_t rows, cols, batch;
+};
+
+template <int TB, bool VEC>
+inline hipError_t launch_f16_list_cfg(hipStream_t stream, hipEvent_t stop, const F16Product *prods,
+                                      int n) {
+    GemvArgs args; // only the used descriptors are written
+    args.n = (uint32_t)n;
+    args.pad = 0;
+    args.norm_eps = 0.0f;
+    args.norm_h = nullptr;
+    args.norm_w = nullptr;
+    args.norm_out = nullptr;
+    uint64_t tiles = 0;
+    for (int i = 0; i < n; ++i) {
+        GemvDesc &d = args.d[i];
+        d.w = (const uint8_t *)prods[i].w;
+        d.x = prods[i].x;
+        d.y = prods[i].y;
+        d.rows = prods[i].rows;
+        d.cols = prods[i].cols;
+        d.batch = prods[i].batch;
+        d.tile_begin = (uint32_t)tiles;
+        d.rows_per_tile = f16_rows_per_tile(prods[i].rows, prods[i].cols);
+        d.pad = 0;
+        d.res = nullptr;
+        d.alpha = 0.0f;
+        d.pad2 = 0;
+        tiles += (prods[i].rows + d.rows_per_tile - 1u) / d.rows_per_tile;
     }
+    if (tiles == 0 || tiles > 0xffffffffull) {
+        return hipErrorInvalidValue;
+    }
+    args.total_tiles = (uint32_t)tiles;
+    Q8_LAUNCH((f16_gemm_list_kernel<TB, VEC>), dim3((unsigned)((tiles + 3u) / 4u)), dim3(256), 0,
+              stream, stop, args);
     return hipGetLastError();
 }
 
-inline hipError_t launch_f16_gemm(hipStream_t stream, hipEvent_t stop, const uint16_t *w,
-                                  const float *x, float *y, uint32_t rows, uint32_t cols,
-                                  uint32_t batch) {
-    if (rows == 0 || cols == 0 || batch == 0 || batch > F16_GEMM_MAX_BATCH) {
+// Every product of the list has f16_tokens(batch) == tb; vec: all cols % 8 == 0.
+inline hipError_t launch_f16_list(hipStream_t stream, hipEvent_t stop, int tb, bool vec,
+                                  const F16Product *prods, int n) {
+    if (n <= 0 || n > GEMV_MAX_DESCS) {
         return hipErrorInvalidValue;
     }
-    switch (f16_tokens(batch)) {
-    case 1: return launch_f16_gemm_tb<1>(stream, stop, w, x, y, rows, cols, batch);
-    case 2: return launch_f16_gemm_tb<2>(stream, stop, w, x, y, rows, cols, batch);
-    default: return launch_f16_gemm_tb<4>(stream, stop, w, x, y, rows, cols, batch);
+    for (int i = 0; i < n; ++i) {
+        if (prods[i].rows == 0 || prods[i].cols == 0 || prods[i].batch == 0 ||
+            prods[i].batch > F16_GEMM_MAX_BATCH || (vec && (prods[i].cols & 7u) != 0u)) {
+            return hipErrorInvalidValue;
+        }
+    }
+    switch (tb) {
+    case 1:
+        return vec ? launch_f16_list_cfg<1, true>(stream, stop, prods, n)
+                   : launch_f16_list_cfg<1, false>(stream, stop, prods, n);
+    case 2:
+        return vec ? launch_f16_list_cfg<2, true>(stream, stop, prods, n)
+                   : launch_f16_list_cfg<2, false>(stream, stop, prods, n);
+    case 4:
+        return vec ? launch_f16_list_cfg<4, true>(stream, stop, prods, n)
+                   : launch_f16_list_cfg<4, false>(stream, stop, prods, n);
+    default:
+        return hipErrorInvalidValue;
     }
 }
 

@@ -271,11 +271,12 @@ enum Variant : uint8_t {
     V_MMA,        // f32 MFMA GEMM: p0 = tmw, p1 = tnw, p2 = K split
     V_I8_TILE,    // register-fed int8 MFMA GEMM: p0 = tile configuration
     V_I8_STREAM,  // int8 streaming kernel: p0 = tokens per pass
-    V_I8_LDS      // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (0: 1x4 waves, 1: 2x2)
+    V_I8_LDS,     // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (0: 1x4 waves, 1: 2x2)
+    V_F16         // F16-weight list kernel: p0 = tokens per sweep, flag = every row 16-byte aligned
 };
 
 struct GemvKey {
-    OpKind kind = OP_GEMV_LIST; // OP_GEMV_LIST, OP_MMA or OP_I8
+    OpKind kind = OP_GEMV_LIST; // OP_GEMV_LIST, OP_MMA, OP_I8 or OP_F16_GEMM
     Variant variant = V_DECODE;
     uint8_t p0 = 0, p1 = 0, p2 = 0;
     bool packed = false;
@@ -306,6 +307,12 @@ GemvKey gemv_key(const Op &op) {
             k.variant = V_I8_TILE;
             k.p0 = (uint8_t)q8::pick_i8_config(op.batch);
         }
+        return k;
+    }
+    if (op.kind == OP_F16_GEMM) {
+        k.variant = V_F16;
+        k.p0 = (uint8_t)q8::f16_tokens(op.batch);
+        k.flag = (op.cols & 7u) == 0u;
         return k;
     }
     const uintptr_t xp = (uintptr_t)op.a[1]->ptr + (uintptr_t)op.x_off * 4u;
@@ -461,6 +468,18 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     }
     if (key.kind == OP_I8) {
         return launch_i8_list(ctx, stop, ops, key);
+    }
+    if (key.kind == OP_F16_GEMM) {
+        std::vector<q8::F16Product> prods;
+        prods.reserve(ops.size());
+        for (const Op *op : ops) {
+            prods.push_back(q8::F16Product{(const uint16_t *)op->a[0]->ptr,
+                                           (const float *)op->a[1]->ptr + op->x_off,
+                                           (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
+                                           op->batch});
+        }
+        return q8::launch_f16_list(ctx->stream, stop, key.p0, key.flag, prods.data(),
+                                   (int)prods.size());
     }
     q8::GemvArgs args; // only the used descriptors are written (the struct is 14 KB)
     args.n = 0;
@@ -640,10 +659,6 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
                   (const uint32_t *)part_i, (uint32_t *)op.a[2]->ptr, op.y_off);
         break;
     }
-    case OP_F16_GEMM:
-        return q8::launch_f16_gemm(st, stop, (const uint16_t *)op.a[0]->ptr,
-                                   (const float *)op.a[1]->ptr + op.x_off,
-                                   (float *)op.a[2]->ptr + op.y_off, op.rows, op.cols, op.batch);
     case OP_F16_ROW:
         Q8_LAUNCH(q8::f16_row_kernel, dim3((op.cols + 255u) / 256u), dim3(256), 0, st, stop,
                   (const uint16_t *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.cols, op.extra,
@@ -698,7 +713,8 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
         epoch = ++ctx->plan_epoch;
     };
     for (const Op &op : ops) {
-        if (op.kind == OP_GEMV_LIST || op.kind == OP_MMA || op.kind == OP_I8) {
+        if (op.kind == OP_GEMV_LIST || op.kind == OP_MMA || op.kind == OP_I8 ||
+            op.kind == OP_F16_GEMM) {
             const GemvKey key = gemv_key(op);
             const int cap = key.kind == OP_MMA  ? q8::MMA_MAX_DESCS
                             : key.kind == OP_I8 ? q8::I8_MAX_DESCS
