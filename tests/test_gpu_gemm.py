@@ -182,3 +182,39 @@ def test_independent_mma_products_in_a_group_share_one_launch(ctx):
         assert np.array_equal(bits(grouped), bits(alone))
         want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
         assert norm_err(grouped.reshape(batch, rows), want) <= 1e-5
+
+
+@pytest.mark.parametrize("packed", [True, False])
+def test_a_large_mma_group_has_the_bits_of_its_products_alone(ctx, packed):
+    # Enough wave tiles in one launch for the work-queue kernel (a wave owns a
+    # tile over the whole of K and takes tiles from a device-side counter);
+    # each product alone has too few and runs the K-split kernels. Same bits,
+    # for K of 32, 33, 64 and 96 blocks, ragged rows and a ragged last token tile.
+    shapes = [(4100, 1024, 500), (2048, 2048, 512), (1024, 3072, 512), (3000, 1056, 450),
+              (4096, 1024, 512), (1024, 3072, 200)]
+    mats = []
+    for i, (rows, cols, batch) in enumerate(shapes):
+        w = S.make_weights(rows, cols, 900 + i)
+        x = S.make_activations(batch * cols, 950 + i)
+        mats.append((w, x, rows, cols, batch, weights_buffer(ctx, w, rows, cols, packed),
+                     upload_new(ctx, x), ctx.buffer(batch * rows * 4)))
+    launches = ctx.kernel_launches()
+    for _ in range(2):   # twice: the second launch finds the counters as the first left them
+        for m in mats:
+            m[7].zero(0, m[4] * m[2] * 4)
+        ctx.begin_group()
+        for w, x, rows, cols, batch, wb, xb, yb in mats:
+            ctx.q8_0_gemm_mma(wb, xb, yb, rows, cols, batch, 0, 0)
+        ctx.end_group()
+        ctx.fence()
+    assert ctx.kernel_launches() == launches + 2
+    for i, (w, x, rows, cols, batch, wb, xb, yb) in enumerate(mats):
+        grouped = yb.download_f32(0, batch * rows).copy()
+        alone = run_gemm(ctx, ctx.q8_0_gemm_mma, wb, x, rows, cols, batch)
+        assert np.array_equal(bits(grouped), bits(alone)), f"product {i}"
+        if i in (0, 3):
+            want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+            assert norm_err(grouped.reshape(batch, rows), want) <= 1e-5
+    for m in mats:
+        for b in m[5:]:
+            b.free()

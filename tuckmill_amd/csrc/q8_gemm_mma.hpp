@@ -443,6 +443,188 @@ __global__ __launch_bounds__(256) void gemm_mma_persistent_kernel(const MmaArgs 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Work-queue form for launches with more wave tiles than the chip holds waves.
+//
+// A wave owns a 32*TMW-token x 32-row tile over the WHOLE of K and takes its
+// next tile from a counter in device memory, so nothing synchronises: no
+// workgroup barrier, no partial tiles through LDS, and tiles of different
+// length (products with different K share a launch, longest first) balance
+// themselves. The result has the bits of the K-split kernels above: the wave
+// runs the four K quarters one after the other, each as its own MFMA chain
+// from zero, and adds the four partial tiles in slice order.
+//
+// queue[0] hands out tiles beyond the first one per wave, queue[1] counts
+// finished waves; the last wave to finish sets both back to zero, so a launch
+// needs them zero on entry and leaves them zero (launches that share the
+// counters must not overlap: one stream per context). Every wave ends after
+// exactly one grab past the end of the list.
+template <int L, int TMW, bool XA>
+__global__ __launch_bounds__(256, 2) void gemm_mma_queue_kernel(const MmaArgs args, uint32_t *queue) {
+    constexpr int S = 4;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t idx = lane & 31u, half = lane >> 5;
+    const uint32_t nwaves = gridDim.x * 4u; // <= total_tiles (the launcher sees to it)
+    const uint32_t total = args.total_tiles;
+
+    auto decode = [&](uint32_t tile, MmaTileCtx &c) {
+        uint32_t lo = 0, hi = args.n;
+        while (hi - lo > 1u) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (args.d[mid].tile_begin <= tile) {
+                lo = mid;
+            } else {
+                hi = mid;
+            }
+        }
+        const MmaDesc &d = args.d[lo];
+        c.w = d.w; c.x = d.x; c.y = d.y;
+        c.rows = d.rows; c.cols = d.cols; c.batch = d.batch;
+        const uint32_t local = tile - d.tile_begin;
+        c.t0 = (local % d.tiles_t) * (32u * TMW);
+        c.n0 = (local / d.tiles_t) * 32u;
+        c.kb_begin = 0;
+        c.kb_end = d.cols >> 5;
+    };
+    auto load = [&](const MmaTileCtx &c, uint32_t kb, MmaRaw<TMW, 1> &raw) {
+        const WView<L> wv(c.w, c.rows, c.cols);
+        const uint32_t r = c.n0 + idx;
+        const uint32_t wrow[1] = {r < c.rows ? r : c.rows - 1u};
+        uint32_t tok[TMW];
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+            const uint32_t t = c.t0 + 32u * i + idx;
+            tok[i] = t < c.batch ? t : c.batch - 1u;
+        }
+        mma_load_block<L, TMW, 1, XA>(wv, c.x, c.cols, wrow, tok, kb, half, raw);
+    };
+
+    floatx16 acc[TMW];
+    auto block = [&](const MmaRaw<TMW, 1> &cur) {
+        float wf[16];
+        const float dsc = f16_bits_to_f32(cur.sb[0]);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            wf[e] = dsc * sbyte_to_float(cur.q[0][e / 4], e % 4);
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+#pragma unroll
+            for (int i = 0; i < TMW; ++i) {
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(cur.xv[i][e], wf[e], acc[i], 0, 0, 0);
+            }
+        }
+    };
+
+    MmaRaw<TMW, 1> ra, rb;
+    // Blocks [kb0, kb1) of `c` (at least one), `ra` holding block kb0 on entry
+    // and block `nkb` of `nc` on exit: every step requests the operands of the
+    // following step before it issues its own MFMAs.
+    auto quarter = [&](const MmaTileCtx &c, uint32_t kb0, uint32_t kb1, const MmaTileCtx &nc,
+                       uint32_t nkb) {
+        uint32_t kb = kb0;
+        for (; kb + 2u < kb1; kb += 2u) {
+            load(c, kb + 1u, rb);
+            __builtin_amdgcn_sched_barrier(0);
+            block(ra);
+            load(c, kb + 2u, ra);
+            __builtin_amdgcn_sched_barrier(0);
+            block(rb);
+        }
+        if (kb + 2u == kb1) {
+            load(c, kb + 1u, rb);
+            __builtin_amdgcn_sched_barrier(0);
+            block(ra);
+            load(nc, nkb, ra);
+            __builtin_amdgcn_sched_barrier(0);
+            block(rb);
+        } else {
+            load(nc, nkb, rb);
+            __builtin_amdgcn_sched_barrier(0);
+            block(ra);
+            ra = rb;
+        }
+    };
+
+    uint32_t tile = blockIdx.x * 4u + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    MmaTileCtx cur;
+    decode(tile, cur);
+    load(cur, 0, ra);
+    while (true) {
+        // Ask for the next tile now; the answer is looked at before the last quarter.
+        uint32_t ticket = 0;
+        if (lane == 0u) {
+            ticket = atomicAdd(&queue[0], 1u);
+        }
+        const uint32_t blocks = cur.kb_end;
+        floatx16 sum[TMW];
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                sum[i][v] = 0.0f;
+            }
+        }
+        auto fold = [&]() {
+#pragma unroll
+            for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    sum[i][v] += acc[i][v];
+                    acc[i][v] = 0.0f;
+                }
+            }
+        };
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                acc[i][v] = 0.0f;
+            }
+        }
+        for (uint32_t s = 0; s + 1u < (uint32_t)S; ++s) {
+            const uint32_t kb0 = (uint32_t)(((uint64_t)blocks * s) / S);
+            const uint32_t kb1 = (uint32_t)(((uint64_t)blocks * (s + 1u)) / S);
+            quarter(cur, kb0, kb1, cur, kb1);
+            fold();
+        }
+        const uint32_t next = nwaves + __builtin_amdgcn_readfirstlane(ticket);
+        const bool more = next < total;
+        MmaTileCtx nxt = cur;
+        if (more) {
+            decode(next, nxt);
+        }
+        const uint32_t kb3 = (uint32_t)(((uint64_t)blocks * 3u) / S);
+        quarter(cur, kb3, blocks, nxt, more ? 0u : blocks - 1u);
+        fold();
+
+        // sum[i][v] is (token 8*(v/4) + 4*half + v%4, row idx) of token tile i
+        const uint32_t n = cur.n0 + idx;
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t t = cur.t0 + 32u * i + 8u * (v / 4) + 4u * half + (v % 4);
+                if (t < cur.batch && n < cur.rows) {
+                    cur.y[(size_t)t * cur.rows + n] = sum[i][v];
+                }
+            }
+        }
+        if (!more) {
+            break;
+        }
+        tile = next;
+        cur = nxt;
+    }
+    if (lane == 0u) {
+        const uint32_t done = atomicAdd(&queue[1], 1u);
+        if (done == nwaves - 1u) { // every other wave has made its last grab
+            atomicExch(&queue[0], 0u);
+            atomicExch(&queue[1], 0u);
+        }
+    }
+}
+
 struct MmaConfig {
     int tmw, tnw, s;
 };
@@ -479,14 +661,43 @@ inline MmaConfig pick_mma_config(const MmaProduct *prods, int n) {
     return c;
 }
 
+// Resident workgroups of a 256-thread kernel on the current device (a multiple of 8).
+template <class K> inline uint32_t mma_resident_wgs(K kernel) {
+    int per_cu = 0, dev = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)kernel, 256, 0) !=
+            hipSuccess ||
+        hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        per_cu <= 0 || cus <= 0) {
+        (void)hipGetLastError();
+        return 512u;
+    }
+    return ((uint32_t)per_cu * (uint32_t)cus) & ~7u;
+}
+
+// Launches with at least this many wave tiles per resident wave use the work-queue kernel.
+constexpr uint32_t MMA_QUEUE_MIN_TILES_PER_WAVE = 8;
+
 template <int L, int TMW, int TNW, int S, bool XA>
-inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods,
-                                 int n) {
+inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods_in,
+                                 int n, uint32_t *queue) {
     constexpr int P = 4 / S;
     MmaArgs args;
     args.n = (uint32_t)n;
     uint64_t tiles = 0;
     const MmaConfig c{TMW, TNW, S};
+    // Longest K first: the work-queue kernel hands tiles out in list order, and
+    // the long ones must not be the last to start. (The order of the list does
+    // not change any product's result.)
+    MmaProduct prods[MMA_MAX_DESCS];
+    for (int i = 0; i < n; ++i) {
+        int at = i;
+        while (at > 0 && prods[at - 1].cols < prods_in[i].cols) {
+            prods[at] = prods[at - 1];
+            --at;
+        }
+        prods[at] = prods_in[i];
+    }
     for (int i = 0; i < n; ++i) {
         MmaDesc &d = args.d[i];
         d.w = prods[i].w;
@@ -512,21 +723,20 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
     // up (several token tiles per weight row tile); below that its static tile
     // lists balance worse than the hardware's workgroup dispatch (M = 64: 1.8x
     // slower), so smaller batches keep one tile per workgroup.
+    if constexpr (S == 4 && TNW == 1 && TMW == 2) if (queue != nullptr) {
+        // Work-queue form: every resident wave starts on a tile of its own and
+        // takes further ones from the queue.
+        static const uint32_t resident = mma_resident_wgs(gemm_mma_queue_kernel<L, TMW, XA>);
+        if (tiles >= (uint64_t)resident * 4u * MMA_QUEUE_MIN_TILES_PER_WAVE) {
+            Q8_LAUNCH((gemm_mma_queue_kernel<L, TMW, XA>), dim3(resident), dim3(256), 0, stream, stop,
+                      args, queue);
+            return hipGetLastError();
+        }
+    }
     if constexpr (S == 4 && TNW == 1) if (min_batch >= 256u) {
         // Persistent form: as many workgroups as stay resident (a multiple of
         // 8), each walking a strided list of tiles.
-        static const uint32_t resident = [] {
-            int per_cu = 0, dev = 0, cus = 0;
-            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                    &per_cu, (const void *)gemm_mma_persistent_kernel<L, TMW, XA>, 256, 0) != hipSuccess ||
-                hipGetDevice(&dev) != hipSuccess ||
-                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-                per_cu <= 0 || cus <= 0) {
-                (void)hipGetLastError();
-                return 512u;
-            }
-            return ((uint32_t)per_cu * (uint32_t)cus) & ~7u;
-        }();
+        static const uint32_t resident = mma_resident_wgs(gemm_mma_persistent_kernel<L, TMW, XA>);
         const uint32_t wgs = groups < resident ? groups : resident;
         if (wgs == groups || wgs % 8u == 0u) {
             Q8_LAUNCH((gemm_mma_persistent_kernel<L, TMW, XA>), dim3(wgs), dim3(256), 0, stream, stop,
@@ -542,11 +752,11 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
 
 template <int L, bool XA>
 inline hipError_t launch_mma_layout(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods,
-                                    int n, const MmaConfig *forced) {
+                                    int n, const MmaConfig *forced, uint32_t *queue) {
     const MmaConfig c = forced != nullptr ? *forced : pick_mma_config(prods, n);
 #define TM_MMA_CASE(A, B, C)                                                  \
     if (c.tmw == A && c.tnw == B && c.s == C) {                               \
-        return launch_mma_cfg<L, A, B, C, XA>(stream, stop, prods, n);              \
+        return launch_mma_cfg<L, A, B, C, XA>(stream, stop, prods, n, queue);       \
     }
     TM_MMA_CASE(2, 1, 1)
     TM_MMA_CASE(1, 1, 1)
@@ -559,19 +769,22 @@ inline hipError_t launch_mma_layout(hipStream_t stream, hipEvent_t stop, const M
 }
 
 // All products of one call share the weight layout and the 16-byte alignment
-// class of their activations (the caller groups them so).
+// class of their activations (the caller groups them so). `queue`: two zeroed
+// uint32 counters in device memory owned by the stream's context (see
+// gemm_mma_queue_kernel), or null to do without that kernel.
 inline hipError_t launch_gemm_mma_list(hipStream_t stream, hipEvent_t stop, bool packed,
                                        bool xaligned, const MmaProduct *prods, int n,
-                                       const MmaConfig *forced = nullptr) {
+                                       const MmaConfig *forced = nullptr,
+                                       uint32_t *queue = nullptr) {
     if (n <= 0 || n > MMA_MAX_DESCS) {
         return hipErrorInvalidValue;
     }
     if (packed) {
-        return xaligned ? launch_mma_layout<PACKED, true>(stream, stop, prods, n, forced)
-                        : launch_mma_layout<PACKED, false>(stream, stop, prods, n, forced);
+        return xaligned ? launch_mma_layout<PACKED, true>(stream, stop, prods, n, forced, queue)
+                        : launch_mma_layout<PACKED, false>(stream, stop, prods, n, forced, queue);
     }
-    return xaligned ? launch_mma_layout<RAW, true>(stream, stop, prods, n, forced)
-                    : launch_mma_layout<RAW, false>(stream, stop, prods, n, forced);
+    return xaligned ? launch_mma_layout<RAW, true>(stream, stop, prods, n, forced, queue)
+                    : launch_mma_layout<RAW, false>(stream, stop, prods, n, forced, queue);
 }
 
 } // namespace q8

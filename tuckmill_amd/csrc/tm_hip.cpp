@@ -97,6 +97,7 @@ struct tm_hip_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     hipStream_t copy_stream = nullptr;
+    uint32_t *mma_queue = nullptr; // two counters of the work-queue MFMA kernel, zero between launches
     std::atomic<uint64_t> allocated{0};
     std::atomic<uint64_t> leased{0};
     std::atomic<uint64_t> committed{0};
@@ -437,7 +438,8 @@ hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<c
                                     op->batch};
     }
     const q8::MmaConfig c{key.p0, key.p1, key.p2};
-    return q8::launch_gemm_mma_list(ctx->stream, stop, key.packed, key.flag, prods, n, &c);
+    return q8::launch_gemm_mma_list(ctx->stream, stop, key.packed, key.flag, prods, n, &c,
+                                    ctx->mma_queue);
 }
 
 hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
@@ -1072,6 +1074,15 @@ tm_hip_ctx *tm_hip_create(char *err, size_t err_cap) {
         tm_hip_destroy(ctx);
         return nullptr;
     }
+    e = hipMalloc((void **)&ctx->mma_queue, 256);
+    if (e == hipSuccess) {
+        e = hipMemset(ctx->mma_queue, 0, 256);
+    }
+    if (e != hipSuccess) {
+        hip_fail(err, err_cap, "work-queue counters", e);
+        tm_hip_destroy(ctx);
+        return nullptr;
+    }
     // Fail at creation, not at first use, when the device code is missing.
     hipFuncAttributes attr;
     e = hipFuncGetAttributes(&attr, (const void *)q8::gemv_list_kernel<q8::PACKED, kGemvR1, 1, true, 0>);
@@ -1119,6 +1130,9 @@ void tm_hip_destroy(tm_hip_ctx *ctx) {
             (void)hipEventDestroy(e);
         }
         ctx->event_pool.clear();
+    }
+    if (ctx->mma_queue != nullptr) {
+        (void)hipFree(ctx->mma_queue);
     }
     if (ctx->copy_stream != nullptr) {
         (void)hipStreamDestroy(ctx->copy_stream);
