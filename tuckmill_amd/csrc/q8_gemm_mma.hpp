@@ -684,20 +684,51 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
     constexpr int P = 4 / S;
     MmaArgs args;
     args.n = (uint32_t)n;
-    uint64_t tiles = 0;
     const MmaConfig c{TMW, TNW, S};
-    // Longest K first: the work-queue kernel hands tiles out in list order, and
-    // the long ones must not be the last to start. (The order of the list does
-    // not change any product's result.)
+    uint64_t tiles = 0;
+    uint32_t min_batch = 0xffffffffu;
+    for (int i = 0; i < n; ++i) {
+        tiles += mma_tiles(prods_in[i], c);
+        min_batch = prods_in[i].batch < min_batch ? prods_in[i].batch : min_batch;
+    }
+    // Which form runs (see the kernels): the work queue from 8 wave tiles per
+    // resident wave, else persistent workgroups from 256 tokens (measured on the
+    // 2B-class shapes: below that their static tile lists balance worse than the
+    // hardware's workgroup dispatch, M = 64 was 1.8x slower), else one tile per
+    // workgroup.
+    bool use_queue = false, use_persistent = false;
+    uint32_t launch_wgs = 0;
+    const uint32_t groups = (uint32_t)((tiles + P - 1) / P);
+    if constexpr (S == 4 && TNW == 1 && TMW == 2) if (queue != nullptr) {
+        static const uint32_t resident = mma_resident_wgs(gemm_mma_queue_kernel<L, TMW, XA>);
+        if (tiles >= (uint64_t)resident * 4u * MMA_QUEUE_MIN_TILES_PER_WAVE) {
+            use_queue = true;
+            launch_wgs = resident;
+        }
+    }
+    if constexpr (S == 4 && TNW == 1) if (!use_queue && min_batch >= 256u) {
+        static const uint32_t resident = mma_resident_wgs(gemm_mma_persistent_kernel<L, TMW, XA>);
+        const uint32_t wgs = groups < resident ? groups : resident;
+        if (wgs == groups || wgs % 8u == 0u) {
+            use_persistent = true;
+            launch_wgs = wgs;
+        }
+    }
+    // Longest K first where tiles are handed out in list order (the work queue,
+    // the hardware's workgroup dispatch): the long ones must not be the last to
+    // start (M = 64 on the 2B shapes: 87 -> 98 TFLOP/s). The persistent form's
+    // strided lists did better in the caller's order. The order of the list
+    // does not change any product's result.
     MmaProduct prods[MMA_MAX_DESCS];
     for (int i = 0; i < n; ++i) {
         int at = i;
-        while (at > 0 && prods[at - 1].cols < prods_in[i].cols) {
+        while (!use_persistent && at > 0 && prods[at - 1].cols < prods_in[i].cols) {
             prods[at] = prods[at - 1];
             --at;
         }
         prods[at] = prods_in[i];
     }
+    tiles = 0;
     for (int i = 0; i < n; ++i) {
         MmaDesc &d = args.d[i];
         d.w = prods[i].w;
@@ -714,35 +745,15 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
     args.total_tiles = (uint32_t)tiles;
     args.chunk_wgs = args.d[0].tiles_t >= (uint32_t)P ? args.d[0].tiles_t / P : 1u;
     args.pad = 0;
-    const uint32_t groups = (uint32_t)((tiles + P - 1) / P);
-    uint32_t min_batch = 0xffffffffu;
-    for (int i = 0; i < n; ++i) {
-        min_batch = prods[i].batch < min_batch ? prods[i].batch : min_batch;
+    if constexpr (S == 4 && TNW == 1 && TMW == 2) if (use_queue) {
+        Q8_LAUNCH((gemm_mma_queue_kernel<L, TMW, XA>), dim3(launch_wgs), dim3(256), 0, stream, stop,
+                  args, queue);
+        return hipGetLastError();
     }
-    // Measured on the 2B-class shapes: the persistent form wins from 256 tokens
-    // up (several token tiles per weight row tile); below that its static tile
-    // lists balance worse than the hardware's workgroup dispatch (M = 64: 1.8x
-    // slower), so smaller batches keep one tile per workgroup.
-    if constexpr (S == 4 && TNW == 1 && TMW == 2) if (queue != nullptr) {
-        // Work-queue form: every resident wave starts on a tile of its own and
-        // takes further ones from the queue.
-        static const uint32_t resident = mma_resident_wgs(gemm_mma_queue_kernel<L, TMW, XA>);
-        if (tiles >= (uint64_t)resident * 4u * MMA_QUEUE_MIN_TILES_PER_WAVE) {
-            Q8_LAUNCH((gemm_mma_queue_kernel<L, TMW, XA>), dim3(resident), dim3(256), 0, stream, stop,
-                      args, queue);
-            return hipGetLastError();
-        }
-    }
-    if constexpr (S == 4 && TNW == 1) if (min_batch >= 256u) {
-        // Persistent form: as many workgroups as stay resident (a multiple of
-        // 8), each walking a strided list of tiles.
-        static const uint32_t resident = mma_resident_wgs(gemm_mma_persistent_kernel<L, TMW, XA>);
-        const uint32_t wgs = groups < resident ? groups : resident;
-        if (wgs == groups || wgs % 8u == 0u) {
-            Q8_LAUNCH((gemm_mma_persistent_kernel<L, TMW, XA>), dim3(wgs), dim3(256), 0, stream, stop,
-                      args);
-            return hipGetLastError();
-        }
+    if constexpr (S == 4 && TNW == 1) if (use_persistent) {
+        Q8_LAUNCH((gemm_mma_persistent_kernel<L, TMW, XA>), dim3(launch_wgs), dim3(256), 0, stream,
+                  stop, args);
+        return hipGetLastError();
     }
     const size_t lds = S > 1 ? (size_t)P * (S - 1) * TMW * TNW * 16 * WAVE * sizeof(float) : 0;
     Q8_LAUNCH((gemm_mma_kernel<L, TMW, TNW, S, XA>), dim3(groups), dim3(256), lds, stream, stop,
