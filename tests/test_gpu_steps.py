@@ -146,6 +146,11 @@ def test_a_recorded_prefill_chunk_replays_every_product_kernel(ctx):
         ys += [(y, batch), (y8, batch)]
         calls.append((x, y, y8, xq, batch))
 
+    # and an F16 matrix with its row lookup
+    w16 = upload_new(ctx, (S.make_activations(96 * cols, 5) * np.float32(0.02)).astype(np.float16).view(np.uint8))
+    y16, row16 = ctx.buffer(4 * 96 * 4), ctx.buffer(cols * 4)
+    ys += [(y16, 4), (row16, 0)]
+
     def encode():
         for x, y, y8, xq, batch in calls:
             if batch <= H.GEMM_MAX_BATCH:
@@ -154,9 +159,11 @@ def test_a_recorded_prefill_chunk_replays_every_product_kernel(ctx):
                 ctx.q8_0_gemm_mma(w, x, y, rows, cols, batch)
             ctx.q8_0_quantize_act(x, xq, cols, batch)
             ctx.q8_0_gemm_i8(w, xq, y8, rows, cols, batch)
+        ctx.f16_gemm(w16, calls[0][0], y16, 96, cols, 4)
+        ctx.f16_row(w16, row16, 7, cols, 0)
 
     def outputs():
-        return [bits(b.download_f32(0, n * rows)).copy() for b, n in ys]
+        return [bits(b.download_f32(0, len(b) // 4)).copy() for b, n in ys]
 
     ctx.begin_group()
     encode()
@@ -169,7 +176,7 @@ def test_a_recorded_prefill_chunk_replays_every_product_kernel(ctx):
     step = ctx.end_group_recorded()
     for replay in range(3):
         for b, n in ys:
-            b.zero(0, n * rows * 4)
+            b.zero(0, len(b))
         step.run()
         ctx.fence()
         got = outputs()
