@@ -3,7 +3,7 @@
 // :638-668 tm_f16_gemm), single-row conversion (:409-419) and the indirect row
 // lookup (:257-269). They serve F16-weight artifacts (model fixtures, F16 twins
 // of quantized tensors), not the headline decode path, but are HBM-bound just
-// the same: 2 bytes per weight, streamed once per group of TB tokens.
+// the same: 2 bytes per weight, streamed once per group of TB tokens (up to 8).
 //
 // Summation order (fixed; tolerance-qualified against the CPU's sequential sum
 // like the reference's own kernel): a lane owns 8 consecutive columns of every
@@ -202,7 +202,7 @@ __global__ __launch_bounds__(256) void f16_row_indirect_kernel(const uint16_t *_
     out[i] = row < rows ? f16_bits_to_f32(w[(size_t)row * cols + i]) : 0.0f;
 }
 
-inline int f16_tokens(uint32_t batch) { return batch == 1u ? 1 : (batch == 2u ? 2 : 4); }
+inline int f16_tokens(uint32_t batch) { return batch == 1u ? 1 : (batch == 2u ? 2 : (batch <= 4u ? 4 : 8)); }
 
 // About 16 KiB of weights per wave, at least one pass of 8 rows; a matrix that
 // would give fewer than 1024 tiles gets one-pass tiles so that it still spreads.
@@ -285,6 +285,9 @@ inline hipError_t launch_f16_list(hipStream_t stream, hipEvent_t stop, int tb, b
     case 4:
         return vec ? launch_f16_list_cfg<4, true>(stream, stop, prods, n)
                    : launch_f16_list_cfg<4, false>(stream, stop, prods, n);
+    case 8:
+        return vec ? launch_f16_list_cfg<8, true>(stream, stop, prods, n)
+                   : launch_f16_list_cfg<8, false>(stream, stop, prods, n);
     default:
         return hipErrorInvalidValue;
     }
