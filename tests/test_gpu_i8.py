@@ -147,11 +147,15 @@ def test_independent_i8_products_in_a_group_share_one_launch(ctx):
 
 @pytest.mark.parametrize("rows,cols,batch", [(128, 1024, 64), (129, 2048, 65), (300, 1152, 200),
                                              (64, 96, 77), (1000, 64, 512), (257, 6144, 129),
-                                             (70, 32, 64), (513, 3072, 300)])
+                                             (70, 32, 64), (513, 3072, 300),
+                                             # one to three token tiles of 16
+                                             (300, 1152, 5), (65, 96, 16), (129, 2080, 9),
+                                             (300, 1152, 17), (256, 2048, 32), (65, 96, 20),
+                                             (100, 352, 48), (70, 1024, 33), (513, 160, 41)])
 def test_lds_staged_i8_gemm_is_bit_exact(ctx, rows, cols, batch):
-    # Prefill-sized batches over sealed weights without the verification output
+    # Batches of five and more over sealed weights without the verification output
     # take the LDS-staged kernel: partial token and row tiles, K stages that end
-    # inside the last stage, both workgroup shapes.
+    # inside the last stage, every workgroup shape.
     w = S.make_weights(rows, cols, 3 * rows + cols)
     x = S.make_activations(cols * batch, batch + 1)
     wb = weights_buffer(ctx, w, rows, cols, True)

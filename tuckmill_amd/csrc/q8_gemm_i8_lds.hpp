@@ -1,5 +1,5 @@
-// int8-activation GEMM for prefill-sized batches over sealed weights: operand
-// tiles staged through LDS.
+// int8-activation GEMM for batches of five tokens and more over sealed weights:
+// operand tiles staged through LDS.
 //
 // Same arithmetic as gemm_i8_kernel (q8_gemm_i8.hpp): one
 // v_mfma_i32_16x16x32_i8 per Q8_0 block and 16x16 tile gives the exact sumi,
@@ -9,24 +9,32 @@
 // What changes is how the operands arrive. The register-fed kernel lets every
 // lane fetch 8 bytes of its own token / weight row per block: 16 cache lines
 // per load instruction, a quarter of each used, re-fetched from L2 by every
-// wave. Here a workgroup of WM x WN waves owns (WM*64 tokens) x (WN*64 rows) and
-// walks K in stages of KS blocks; per stage every operand byte is fetched once
+// wave. Here a workgroup of WM x WN waves owns (WM*TM*16 tokens) x (WN*TN*16 rows)
+// and walks K in stages of KS blocks; per stage every operand byte is fetched once
 // per workgroup as whole 16-byte pieces of full rows (buffer_load ... lds, no
 // registers held in flight), double-buffered. Pieces are stored XOR-swizzled
 // (the fetching lane chooses which piece of its row it brings, its LDS slot is
 // fixed by the instruction) so that the MFMA operand reads, 8 bytes per lane
 // with 16 lanes on 16 different rows, touch every bank once.
+//
+// One fetch instruction moves 1 KiB: 64 / (2*KS) operand rows of 32*KS bytes each.
+// How that kilobyte is spread over cache lines matters more than anything else
+// when the batch is small and the kernel lives off the weight stream: with
+// stages of 2 blocks an instruction touches 16 lines for 64 bytes each and the
+// fetch runs at about a quarter of HBM speed; with 4 blocks it takes 8 whole
+// lines (i8_lds_shape below picks the stage depth per batch).
 #pragma once
 
 #include "q8_gemm_i8.hpp"
 
 namespace q8 {
 
-template <int WM, int WN, int KS> struct I8LdsShape {
-    static constexpr int tokens = WM * 64, rows = WN * 64;
+template <int WM, int WN, int KS, int TM = 4, int TN = 4> struct I8LdsShape {
+    static constexpr int tokens = WM * TM * 16, rows = WN * TN * 16;
     static constexpr int row_bytes = KS * 32;           // one operand row of a stage
     static constexpr int pieces = KS * 2;               // 16-byte pieces per operand row
-    static constexpr int rows_per_bankrow = 16 / pieces; // operand rows per 256 bytes of LDS
+    // operand rows per 256 bytes of LDS (rows of 256 bytes or more: one)
+    static constexpr int rows_per_bankrow = pieces >= 16 ? 1 : 16 / pieces;
     static constexpr int a_bytes = tokens * row_bytes;
     static constexpr int b_bytes = rows * row_bytes;
     // [block][token] f32, rounded up to whole 1 KiB fetch instructions
@@ -39,15 +47,14 @@ template <int WM, int WN, int KS> struct I8LdsShape {
 // is an involution on the piece index).
 template <int WM, int WN, int KS>
 __device__ __forceinline__ uint32_t i8_swz(uint32_t r, uint32_t p) {
-    using Sh = I8LdsShape<WM, WN, KS>;
-    return p ^ ((r / Sh::rows_per_bankrow) % Sh::pieces);
+    using Sh = I8LdsShape<WM, WN, KS>; // the swizzle does not depend on the wave tile
+    return p ^ ((r / Sh::rows_per_bankrow) % (Sh::pieces < 16 ? Sh::pieces : 16));
 }
 
-template <int WM, int WN, int KS>
+template <int WM, int WN, int KS, int TM = 4, int TN = 4>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_i8_lds_kernel(const I8Args args) {
-    using Sh = I8LdsShape<WM, WN, KS>;
-    constexpr int NW = WM * WN;
-    constexpr int TM = 4, TN = 4; // 16x16 tiles per wave: 64 tokens x 64 rows
+    using Sh = I8LdsShape<WM, WN, KS, TM, TN>;
+    constexpr int NW = WM * WN; // 16x16 tiles per wave: 16*TM tokens x 16*TN rows
     // two stage buffers as separate objects (reads of one provably do not alias
     // the fetch into the other)
     __shared__ __attribute__((aligned(16))) uint8_t stage_a[Sh::stage_bytes];
@@ -176,13 +183,13 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_i8_lds_kernel(const I8Args 
             float dw[TN];
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                const uint32_t r = wm * 64u + 16u * i + i16;
+                const uint32_t r = wm * (16u * TM) + 16u * i + i16;
                 a[i] = *(const long *)(sa + r * Sh::row_bytes + i8_swz<WM, WN, KS>(r, p) * 16u + half);
-                dx[i] = *(const float4 *)(sdx + kb * Sh::tokens + wm * 64u + 16u * i + 4u * g);
+                dx[i] = *(const float4 *)(sdx + kb * Sh::tokens + wm * (16u * TM) + 16u * i + 4u * g);
             }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const uint32_t r = wn * 64u + 16u * j + i16;
+                const uint32_t r = wn * (16u * TN) + 16u * j + i16;
                 b[j] = *(const long *)(sb + r * Sh::row_bytes + i8_swz<WM, WN, KS>(r, p) * 16u + half);
                 dw[j] = f16_bits_to_f32(sdw[r * KS + kb] & 0xffffu);
             }
@@ -224,8 +231,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_i8_lds_kernel(const I8Args 
         for (int j = 0; j < TN; ++j) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const uint32_t t = t0 + wm * 64u + 16u * i + 4u * g + v;
-                const uint32_t n = n0 + wn * 64u + 16u * j + i16;
+                const uint32_t t = t0 + wm * (16u * TM) + 16u * i + 4u * g + v;
+                const uint32_t n = n0 + wn * (16u * TN) + 16u * j + i16;
                 if (t < batch && n < rows) {
                     d.y[(size_t)t * rows + n] = acc[i][j][v];
                 }
@@ -234,10 +241,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_i8_lds_kernel(const I8Args 
     }
 }
 
-template <int WM, int WN, int KS>
+template <int WM, int WN, int KS, int TM = 4, int TN = 4>
 inline hipError_t launch_i8_lds_cfg(hipStream_t stream, hipEvent_t stop, const I8Product *prods,
                                     int n) {
-    using Sh = I8LdsShape<WM, WN, KS>;
+    using Sh = I8LdsShape<WM, WN, KS, TM, TN>;
     I8Args args;
     args.n = (uint32_t)n;
     uint64_t tiles = 0;
@@ -258,22 +265,39 @@ inline hipError_t launch_i8_lds_cfg(hipStream_t stream, hipEvent_t stop, const I
     args.total_tiles = (uint32_t)tiles;
     args.chunk_wgs = args.d[0].tiles_t;
     args.pad = 0;
-    Q8_LAUNCH((gemm_i8_lds_kernel<WM, WN, KS>), dim3((unsigned)tiles), dim3(WM * WN * 64), 0, stream,
-              stop, args);
+    Q8_LAUNCH((gemm_i8_lds_kernel<WM, WN, KS, TM, TN>), dim3((unsigned)tiles), dim3(WM * WN * 64), 0,
+              stream, stop, args);
     return hipGetLastError();
 }
 
 // Sealed weights, no verification output, every region below 4 GiB (32-bit
 // buffer offsets): the caller checks these before choosing this kernel.
-constexpr uint32_t GEMM_I8_LDS_MIN_BATCH = 17; // below: the streaming kernel (q8_gemv_i8.hpp)
+constexpr uint32_t GEMM_I8_LDS_MIN_BATCH = 5; // below: the streaming kernel (q8_gemv_i8.hpp)
 
-inline hipError_t launch_gemm_i8_lds_list(hipStream_t stream, hipEvent_t stop,
+// Workgroup shape for a batch. The bits do not depend on the shape.
+//   0..3  batches up to 64: four waves side by side, each 16 rows for all of the
+//         batch's tokens (1..4 token tiles of 16). A weight byte is used once per
+//         token tile here, so what counts is the weight stream: whole 128-byte
+//         lines per fetched row piece (stages of 4 blocks; 8 for one token tile,
+//         where LDS leaves room), and many small workgroups per CU so that many
+//         stages are in flight.
+//   4     larger batches: 2x2 waves over 128 tokens x 128 rows, stages of 2 blocks
+//         (bound by the epilogue's f32 operations, not by the fetch).
+inline int i8_lds_shape(uint32_t batch) { return batch <= 64u ? (int)((batch - 1u) / 16u) : 4; }
+
+inline hipError_t launch_gemm_i8_lds_list(hipStream_t stream, hipEvent_t stop, int shape,
                                           const I8Product *prods, int n) {
     if (n <= 0 || n > I8_MAX_DESCS) {
         return hipErrorInvalidValue;
     }
-    return prods[0].batch <= 64u ? launch_i8_lds_cfg<1, 4, 2>(stream, stop, prods, n)
-                                 : launch_i8_lds_cfg<2, 2, 2>(stream, stop, prods, n);
+    switch (shape) {
+    case 0: return launch_i8_lds_cfg<1, 4, 8, 1, 1>(stream, stop, prods, n);
+    case 1: return launch_i8_lds_cfg<1, 4, 4, 2, 1>(stream, stop, prods, n);
+    case 2: return launch_i8_lds_cfg<1, 4, 4, 3, 1>(stream, stop, prods, n);
+    case 3: return launch_i8_lds_cfg<1, 4, 4, 4, 1>(stream, stop, prods, n);
+    case 4: return launch_i8_lds_cfg<2, 2, 2, 4, 4>(stream, stop, prods, n);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 } // namespace q8

@@ -272,7 +272,7 @@ enum Variant : uint8_t {
     V_MMA,        // f32 MFMA GEMM: p0 = tmw, p1 = tnw, p2 = K split
     V_I8_TILE,    // register-fed int8 MFMA GEMM: p0 = tile configuration
     V_I8_STREAM,  // int8 streaming kernel: p0 = tokens per pass
-    V_I8_LDS,     // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (0: 1x4 waves, 1: 2x2)
+    V_I8_LDS,     // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (q8::i8_lds_shape)
     V_F16         // F16-weight list kernel: p0 = tokens per sweep, flag = every row 16-byte aligned
 };
 
@@ -296,14 +296,15 @@ GemvKey gemv_key(const Op &op) {
     k.packed = op.packed;
     if (op.kind == OP_I8) {
         k.flag = op.a[3] != nullptr;
-        if (op.packed && op.batch <= q8::GEMV_I8_MAX_BATCH) {
+        const bool small_regions = (uint64_t)op.rows * op.cols < (1ull << 32) &&
+                                   (uint64_t)op.batch * op.cols < (1ull << 32);
+        if (op.packed && op.a[3] == nullptr && op.batch >= q8::GEMM_I8_LDS_MIN_BATCH &&
+            small_regions) {
+            k.variant = V_I8_LDS;
+            k.p0 = (uint8_t)q8::i8_lds_shape(op.batch);
+        } else if (op.packed && op.batch <= q8::GEMV_I8_MAX_BATCH) {
             k.variant = V_I8_STREAM;
             k.p0 = (uint8_t)q8::gemv_i8_tokens(op.batch);
-        } else if (op.packed && op.a[3] == nullptr && op.batch >= q8::GEMM_I8_LDS_MIN_BATCH &&
-                   (uint64_t)op.rows * op.cols < (1ull << 32) &&
-                   (uint64_t)op.batch * op.cols < (1ull << 32)) {
-            k.variant = V_I8_LDS;
-            k.p0 = op.batch <= 64u ? 0 : 1;
         } else {
             k.variant = V_I8_TILE;
             k.p0 = (uint8_t)q8::pick_i8_config(op.batch);
@@ -453,7 +454,7 @@ hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<co
                                    op->rows, op->cols, op->batch};
     }
     if (key.variant == V_I8_LDS) {
-        return q8::launch_gemm_i8_lds_list(ctx->stream, stop, prods, n);
+        return q8::launch_gemm_i8_lds_list(ctx->stream, stop, key.p0, prods, n);
     }
     if (key.variant == V_I8_STREAM) {
         return q8::launch_gemv_i8_list(ctx->stream, stop, key.flag, key.p0, prods, n);
