@@ -293,7 +293,7 @@ def bench_sweep(host, ctx, steps, warmup):
             paths.append(("f32 mfma", TMH_GEMM_MMA, M))
         if M > 512:
             paths.append(("f32 mfma (slices of 512)", TMH_GEMM_MMA, 512))
-        paths.append(("i8 streaming dot4" if M <= 16 else "i8 mfma", TMH_GEMM_I8, M))
+        paths.append(("i8 streaming dot4" if M <= 4 else "i8 mfma", TMH_GEMM_I8, M))
         for label, kind, mb in paths:
             prods = []
             slices = (M + mb - 1) // mb
