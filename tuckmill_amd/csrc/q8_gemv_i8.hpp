@@ -1,5 +1,7 @@
 // The int8-activation profile at decode-sized batches (1 <= batch <= 16, sealed
 // weights): a bandwidth-bound streaming kernel instead of the MFMA tile kernel.
+// It is the fastest form up to 4 tokens; from 5 the LDS-staged MFMA kernel
+// (q8_gemm_i8_lds.hpp) takes over unless the caller asks for the block dots.
 //
 // Reference arithmetic (crates/tuckcore/src/kernels.rs:206-221) per row:
 //     for each block in order:  sum += (d_w * d_x) * (float)sumi
@@ -223,7 +225,7 @@ inline hipError_t launch_gemv_i8_cfg(hipStream_t stream, hipEvent_t stop, const 
     return hipGetLastError();
 }
 
-constexpr uint32_t GEMV_I8_MAX_BATCH = 16; // above this the MFMA tile kernel takes over
+constexpr uint32_t GEMV_I8_MAX_BATCH = 16; // above this the MFMA kernels only
 
 inline int gemv_i8_tokens(uint32_t batch) {
     return batch == 1u ? 1 : (batch == 2u ? 2 : (batch <= 4u ? 4 : 8));
