@@ -279,7 +279,7 @@ def bench_sweep(host, ctx, steps, warmup):
     widths = sorted({c for _, _, c, _ in pool})
     xqs = {c: ctx.buffer(H.xq_bytes(c, maxM)) for c in widths}
     ys = [ctx.buffer(maxM * maxr * 4) for _ in pool]
-    for M in (1, 2, 4, 8, 16, 32, 64, 512, 2048):
+    for M in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 2048):
         n = max(3, steps // (10 if M < 64 else 200 if M < 512 else 1000))
         w = max(2, n // 5)
         flops = sum(2.0 * M * r * c for _, r, c, _ in pool)

@@ -151,7 +151,10 @@ def test_independent_i8_products_in_a_group_share_one_launch(ctx):
                                              # one to three token tiles of 16
                                              (300, 1152, 5), (65, 96, 16), (129, 2080, 9),
                                              (300, 1152, 17), (256, 2048, 32), (65, 96, 20),
-                                             (100, 352, 48), (70, 1024, 33), (513, 160, 41)])
+                                             (100, 352, 48), (70, 1024, 33), (513, 160, 41),
+                                             # several token tiles of equal height, and the
+                                             # first batch of the 128-token shape
+                                             (200, 1024, 96), (64, 1152, 256), (100, 1024, 257)])
 def test_lds_staged_i8_gemm_is_bit_exact(ctx, rows, cols, batch):
     # Batches of five and more over sealed weights without the verification output
     # take the LDS-staged kernel: partial token and row tiles, K stages that end
