@@ -35,6 +35,7 @@ from tuckmill_amd import synth as S  # noqa: E402
 HBM_PEAK_GBS = 8000.0      # MI355X published HBM3E bandwidth
 MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X published dense f32 matrix rate
 MFMA_I8_PEAK_TOPS = 5000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 # HBM bytes per launch of the decode step's GEMV list kernel, from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in profiles/gemv_list_kernel__decode_step__pmc_traffic.txt
 # (fetch counter x 2.000 + write counter x 1.000, factors from a plain copy kernel).
@@ -182,8 +183,26 @@ def bench_gemm(host, ctx, steps, warmup):
     out["flops_per_step"] = flops_total
     out["mfma_f32_peak_tflops"] = MFMA_F32_PEAK_TFLOPS
     out["frac"] = out["tflops"] / MFMA_F32_PEAK_TFLOPS
-    out["kernel"] = "q8::gemm_mma_kernel"
-    for b in keep:
+    out["kernel"] = "q8::gemm_mma_persistent_kernel"
+    # The same model's vocabulary projection at M = 512: large enough on its own
+    # for the kernel that runs on the bf16 matrix cores (every f32 activation
+    # split into three exact bf16 pieces, so the products stay exact).
+    rows, cols = S.QWEN3_0_6B_LM_HEAD[1], S.QWEN3_0_6B_LM_HEAD[2]
+    m = H.Matrix.load(ctx, S.make_weights(rows, cols, S.tensor_seed(2, 0, "lm_head")), cols, rows)
+    xb = ctx.buffer(M * cols * 4)
+    xb.upload(0, S.make_activations(M * cols, 5))
+    yb = ctx.buffer(M * rows * 4)
+    n = max(5, steps // 20)
+    t = run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA)],
+                  max(2, warmup // 20), n, grouped=False)
+    us = t.gpu_ms / n * 1e3
+    flops = 2.0 * M * rows * cols
+    out["lm_head"] = {"rows": rows, "cols": cols, "us": us, "launches_per_step": t.launches / n,
+                      "tflops_f32_equivalent": flops / us / 1e6,
+                      "kernel": "q8::split_act_list_kernel + q8::gemm_bf16x3_kernel",
+                      "bf16_mfma_tflops_issued": 3.0 * flops / us / 1e6,
+                      "frac_of_bf16_mfma_peak": 3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS}
+    for b in keep + [m.buf, xb, yb]:
         b.free()
     return out
 

@@ -1,0 +1,153 @@
+"""GPU parity: the prefill GEMM from 384 tokens over sealed weights large enough
+to fill the chip with 128-token x 256-row tiles, which runs on the bf16 matrix
+cores with every f32 activation split into three exact bf16 pieces (contract: native/metal/tm_metal.h:172-175, tolerance-qualified like
+every matrix-core kernel; crates/metal/src/tests.rs:1169-1233 for the shapes).
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from tuckmill_amd import hip as H
+from tuckmill_amd import synth as S
+
+from q8util import bits, norm_err, ref_scale, require_gpu, upload_new, weights_buffer
+
+pytestmark = pytest.mark.gpu
+
+M0 = H.GEMM_MMA_BF16_MIN_BATCH
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = require_gpu()
+    yield c
+    c.close()
+
+
+def product(ctx, wb, x, rows, cols, batch, x_off=0, y_off=0):
+    xs = np.zeros(x_off + batch * cols, np.float32)
+    xs[x_off:] = x
+    xb = upload_new(ctx, xs)
+    yb = ctx.buffer((y_off + batch * rows) * 4)
+    yb.zero(0, (y_off + batch * rows) * 4)
+    ctx.q8_0_gemm_mma(wb, xb, yb, rows, cols, batch, x_off, y_off)
+    ctx.fence()
+    out = yb.download_f32(0, y_off + batch * rows).copy()
+    xb.free()
+    yb.free()
+    return out
+
+
+# K of 1, 3, 32, 33 (two K chunks of 17 and 16 blocks), 36, 64 and 96 blocks;
+# ragged rows; a ragged last token tile; the smallest batch of the kernel and
+# the largest; every product has at least 128 work units of its own.
+SHAPES = [(8192, 1024, 512), (11000, 96, M0), (8300, 1056, 500), (4096, 3072, 512),
+          (5000, 2048, M0 + 1), (33000, 32, 512), (8500, 1152, 450)]
+
+
+@pytest.mark.parametrize("rows,cols,batch", SHAPES)
+def test_gaussian_products_within_1e5(ctx, rows, cols, batch):
+    w = S.make_weights(rows, cols, 5 * rows + cols)
+    x = S.make_activations(batch * cols, batch + cols)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    launches = ctx.kernel_launches()
+    got = product(ctx, wb, x, rows, cols, batch, 32, 8)
+    assert ctx.kernel_launches() == launches + 2  # the split of x, then the product
+    assert not got[:8].any(), "nothing before y_off"
+    want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+    assert norm_err(got[8:].reshape(batch, rows), want) <= 1e-5
+    wb.free()
+
+
+def test_boundary_values_and_wide_ranges(ctx):
+    # crates/metal/src/tests.rs:1169-1233 (boundary weights and inputs), and
+    # activations that span 60 binades: every piece of the split is exact, so the
+    # large terms do not swamp the small ones any more than in the CPU's sum.
+    rows, cols, batch = 11000, 1024, M0
+    w = O.boundary_weights(rows, cols, 11)
+    x = O.boundary_input(cols * batch, 13)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    launches = ctx.kernel_launches()
+    got = product(ctx, wb, x, rows, cols, batch).reshape(batch, rows)
+    assert ctx.kernel_launches() == launches + 2
+    cpu = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+    for b in range(batch):
+        assert np.max(np.abs(got[b] - cpu[b])) <= 1e-4 * ref_scale(cpu[b]), f"token {b}"
+    rng = np.random.default_rng(3)
+    x = (S.make_activations(batch * cols, 9) *
+         np.exp2(rng.integers(-30, 30, batch * cols)).astype(np.float32)).astype(np.float32)
+    x[::97] = 0.0
+    x[5::101] = np.float32(1e-41)  # subnormal
+    got = product(ctx, wb, x, rows, cols, batch).reshape(batch, rows)
+    cpu = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+    assert norm_err(got, cpu) <= 1e-5
+    wb.free()
+
+
+def test_activations_off_a_16_byte_boundary_take_the_f32_kernels(ctx):
+    rows, cols, batch = 8192, 1024, M0
+    w = S.make_weights(rows, cols, 77)
+    x = S.make_activations(batch * cols, 78)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    launches = ctx.kernel_launches()
+    got = product(ctx, wb, x, rows, cols, batch, 3, 0)
+    assert ctx.kernel_launches() == launches + 1
+    want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+    assert norm_err(got.reshape(batch, rows), want) <= 1e-5
+    wb.free()
+
+
+def test_a_group_splits_each_input_once_and_has_the_bits_of_its_products_alone(ctx):
+    # q/k/v share their activations, o and down have their own (K of 2 and 3
+    # chunks: partial tiles added by whichever chunk arrives last, in chunk
+    # order). Twice: the second launch finds the arrival counters as the first
+    # left them. A replayed recording of the group gives the same bits again.
+    batch = 512
+    xs = {c: S.make_activations(batch * c, c) for c in (1024, 2048, 3072)}
+    xbs = {c: upload_new(ctx, x) for c, x in xs.items()}
+    mats = []
+    # (the last one is too small to fill the chip and runs on the f32 matrix
+    # cores, in a launch of its own)
+    for i, (rows, cols) in enumerate([(8192, 1024), (9000, 1024), (8192, 1024), (4096, 2048),
+                                      (4100, 3072), (1024, 1024)]):
+        w = S.make_weights(rows, cols, 600 + i)
+        mats.append((w, rows, cols, weights_buffer(ctx, w, rows, cols, True),
+                     ctx.buffer(batch * rows * 4)))
+
+    def encode():
+        for w, rows, cols, wb, yb in mats:
+            ctx.q8_0_gemm_mma(wb, xbs[cols], yb, rows, cols, batch, 0, 0)
+
+    launches = ctx.kernel_launches()
+    for _ in range(2):
+        for m in mats:
+            m[4].zero(0, batch * m[1] * 4)
+        ctx.begin_group()
+        encode()
+        ctx.end_group()
+        ctx.fence()
+    assert ctx.kernel_launches() == launches + 6
+    grouped = [m[4].download_f32(0, batch * m[1]).copy() for m in mats]
+    for i, (w, rows, cols, wb, yb) in enumerate(mats):
+        alone = product(ctx, wb, xs[cols], rows, cols, batch)
+        assert np.array_equal(bits(grouped[i]), bits(alone)), f"product {i}"
+        if i in (1, 4):
+            want = O.gemm_q8_0_f32(w, rows, cols, xs[cols], batch, threads=8)
+            assert norm_err(grouped[i].reshape(batch, rows), want) <= 1e-5
+
+    ctx.begin_group()
+    encode()
+    step = ctx.end_group_recorded()
+    assert step.launches == 3
+    for replay in range(3):
+        for m in mats:
+            m[4].zero(0, batch * m[1] * 4)
+        step.run()
+        ctx.fence()
+        for i, m in enumerate(mats):
+            assert np.array_equal(bits(m[4].download_f32(0, batch * m[1])), bits(grouped[i])), \
+                f"replay {replay}, product {i}"
+    step.free()
+    for m in mats:
+        m[3].free()
+        m[4].free()

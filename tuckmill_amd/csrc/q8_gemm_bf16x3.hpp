@@ -1,0 +1,610 @@
+// Q8_0 prefill GEMM with f32 activations on the bf16 matrix cores, exact
+// products ("split-float" form).
+//
+//   Y[t][n] = sum_b d[n][b] * sum_{k in block b} q[n][k] * X[t][k]
+//
+// The f32 MFMA kernel (q8_gemm_mma.hpp) is bound by the f32 matrix rate, which
+// on this part equals the vector rate (157 TFLOP/s); bf16 MFMA is 16 times
+// faster per instruction. An f32 activation is the exact sum of three bf16
+// numbers (its 24-bit significand cut into 8 + 8 + 8 bits: h = trunc(x),
+// m = trunc(x - h), l = x - h - m), a Q8_0 quant is exact in bf16, and an
+// 8-bit by 8-bit product is exact in the MFMA's f32 accumulator. So
+//     S = sum_k q*l + sum_k q*m + sum_k q*h        (three bf16 MFMAs per 16 k)
+// accumulates, in f32, exactly the products q*x of one block, smallest pieces
+// first, and  y += d * S  applies the block scale in f32 per output: no
+// activation is rounded anywhere (unlike the int8-activation profile), only the
+// order of the f32 additions differs from the CPU's, as for every MFMA kernel
+// (contract: native/metal/tm_metal.h:172-175, tolerance-qualified).
+// Non-finite activations give non-finite outputs, not necessarily the same
+// kind (inf - inf in the split).
+//
+// Two kernels: split_act_list_kernel writes the three bf16 planes of every
+// distinct X of a launch once; gemm_bf16x3_kernel is LDS-staged like the int8 GEMM
+// (q8_gemm_i8_lds.hpp): a workgroup of WM x WN waves owns (WM*64 tokens) x
+// (WN*64 rows) of one K chunk of at most 1024 columns (a tile with a longer K
+// is the sum of its chunks' partial tiles, added in chunk order by whichever
+// chunk finishes last), walks K one Q8_0 block per stage, fetches every operand byte
+// once per workgroup as 16-byte pieces straight into LDS (a ring of four
+// stages, XOR-swizzled so that the operand reads are conflict-free) and each
+// wave computes a 64 x 64 tile as 2 x 2 MFMA tiles of 32 x 32.
+#pragma once
+
+#include "q8_common.hpp"
+
+namespace q8 {
+
+typedef float floatx16_t __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+// xs holds, per Q8_0 block kb and piece p (0 = h, 1 = m, 2 = l), the 32 bf16
+// values of every token: [cols / 32][3][batch][32]. A workgroup's tokens of one
+// block and piece are then one contiguous run, which its fetches read as whole
+// cache lines.
+struct SplitDesc {
+    const float *x;   // [batch][cols], 16-byte aligned
+    uint16_t *xs;
+    uint32_t batch, cols;
+    uint32_t wg_begin; // first workgroup of this input in the launch
+    uint32_t pad;
+};
+
+constexpr int SPLIT_MAX_DESCS = 16;
+
+struct SplitArgs {
+    uint32_t n;
+    uint32_t pad;
+    SplitDesc d[SPLIT_MAX_DESCS];
+};
+
+// The distinct inputs of a launch's products, split once each (q/k/v and
+// gate/up share theirs).
+__global__ __launch_bounds__(256) void split_act_list_kernel(const SplitArgs args) {
+    uint32_t which = 0;
+    while (which + 1u < args.n && args.d[which + 1u].wg_begin <= blockIdx.x) {
+        ++which;
+    }
+    const SplitDesc &d = args.d[which];
+    const uint32_t batch = d.batch, cols = d.cols;
+    const uint32_t i = ((blockIdx.x - d.wg_begin) * 256u + threadIdx.x) * 4u; // element of [batch][cols]
+    if (i >= batch * cols) {
+        return;
+    }
+    const uint32_t t = i / cols, k = i % cols; // cols is a multiple of 32: the 4 share a block
+    const float4 v = *(const float4 *)(d.x + i);
+    const float in[4] = {v.x, v.y, v.z, v.w};
+    uint32_t h[4], m[4], l[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint32_t hb = __builtin_bit_cast(uint32_t, in[e]) & 0xffff0000u;
+        const float r1 = in[e] - __builtin_bit_cast(float, hb); // exact
+        const uint32_t mb = __builtin_bit_cast(uint32_t, r1) & 0xffff0000u;
+        const float r2 = r1 - __builtin_bit_cast(float, mb);    // exact, at most 8 significant bits
+        h[e] = hb >> 16;
+        m[e] = mb >> 16;
+        l[e] = __builtin_bit_cast(uint32_t, r2) >> 16;
+    }
+    const size_t piece = (size_t)batch * 32u;
+    uint16_t *dst = d.xs + ((size_t)(k >> 5) * 3u * batch + t) * 32u + (k & 31u);
+    *(uint2 *)dst = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+    *(uint2 *)(dst + piece) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
+    *(uint2 *)(dst + 2u * piece) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
+}
+
+struct Bx3Desc {
+    const uint8_t *w;    // sealed weights
+    const uint16_t *xs;  // the split activations of this product, [cols/32][3][batch][32] bf16
+    float *y;            // y_off already applied
+    uint32_t rows, cols, batch;
+    uint32_t tile_begin; // first work unit of this product in the launch
+    uint32_t tiles_t;    // token tiles per row tile
+    uint32_t chunks;     // K chunks per output tile (work units per tile)
+    uint32_t chunk_blocks; // Q8_0 blocks per chunk
+    uint32_t part_begin; // first arrival counter of this product (one per output tile)
+    uint32_t part_tile;  // first partial tile of this product in `partials`
+};
+
+constexpr int BX3_MAX_DESCS = 64;
+constexpr uint32_t BX3_CHUNK_BLOCKS = 32;   // K is cut into chunks of 1024 columns or more
+constexpr uint32_t BX3_MAX_SPLIT_TILES = 16384; // arrival counters per context
+
+struct Bx3Args {
+    uint32_t n;
+    uint32_t total_tiles; // work units
+    uint32_t chunk_wgs;
+    uint32_t pad;
+    float *partials;      // partial tiles [tile][chunk] of the products with chunks > 1
+    uint32_t *arrivals;   // one counter per split tile, zero between launches
+    Bx3Desc d[BX3_MAX_DESCS];
+};
+
+template <int WM, int WN, int TM> struct Bx3Shape {
+    static constexpr int tokens = WM * TM * 32, rows = WN * 64;
+    static constexpr int a_plane = tokens * 64;          // one plane: 32 bf16 = 64 bytes per token
+    static constexpr int a_bytes = 3 * a_plane;
+    static constexpr int b_bytes = rows * 32;            // 32 int8 per row
+    static constexpr int dw_bytes = rows * 4;            // per row the dword that holds its f16 scale
+    static constexpr int stage_bytes = a_bytes + b_bytes + dw_bytes;
+};
+
+// 8 signed bytes (two dwords) -> 8 bf16: the conversion to f32 is exact and
+// its upper half is the bf16.
+__device__ __forceinline__ bf16x8_t sbytes_to_bf16x8(uint32_t lo, uint32_t hi) {
+    uint32_t p[4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t f0 = __builtin_bit_cast(uint32_t, sbyte_to_float(lo, 2 * i));
+        const uint32_t f1 = __builtin_bit_cast(uint32_t, sbyte_to_float(lo, 2 * i + 1));
+        p[i] = __builtin_amdgcn_perm(f1, f0, 0x07060302u);
+        const uint32_t g0 = __builtin_bit_cast(uint32_t, sbyte_to_float(hi, 2 * i));
+        const uint32_t g1 = __builtin_bit_cast(uint32_t, sbyte_to_float(hi, 2 * i + 1));
+        p[2 + i] = __builtin_amdgcn_perm(g1, g0, 0x07060302u);
+    }
+    const u32x4 v = {p[0], p[1], p[2], p[3]};
+    return __builtin_bit_cast(bf16x8_t, v);
+}
+
+template <int WM, int WN, int TM>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_bf16x3_kernel(const Bx3Args args) {
+    using Sh = Bx3Shape<WM, WN, TM>;
+    constexpr int NW = WM * WN;
+    constexpr int TN = 2; // a wave computes TM x 2 tiles of 32 x 32: 32*TM tokens x 64 rows
+    // A ring of four stage buffers, separate objects so that reads of one
+    // provably do not alias the fetches into the others: three blocks are in
+    // flight while one is being used (a fetch takes about three stages' worth
+    // of MFMAs to arrive).
+    __shared__ __attribute__((aligned(16))) uint8_t stage_0[Sh::stage_bytes];
+    __shared__ __attribute__((aligned(16))) uint8_t stage_1[Sh::stage_bytes];
+    __shared__ __attribute__((aligned(16))) uint8_t stage_2[Sh::stage_bytes];
+    __shared__ __attribute__((aligned(16))) uint8_t stage_3[Sh::stage_bytes];
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const uint32_t idx = lane & 31u, half = lane >> 5;
+
+    uint32_t gidx = blockIdx.x;
+    {
+        const uint32_t cw = args.chunk_wgs;
+        const uint32_t span = 8u * cw;
+        const uint32_t g_full = (gridDim.x / span) * span;
+        if (gidx < g_full) {
+            const uint32_t xcd = gidx & 7u, j = gidx >> 3;
+            gidx = ((j / cw) * 8u + xcd) * cw + (j % cw);
+        }
+    }
+    const uint32_t tile = gidx; // one work unit (output tile x K chunk) per workgroup
+    uint32_t lo = 0, hi = args.n;
+    while (hi - lo > 1u) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (args.d[mid].tile_begin <= tile) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    const Bx3Desc &d = args.d[lo];
+    const uint32_t rows = d.rows, cols = d.cols, batch = d.batch;
+    const uint32_t unit = tile - d.tile_begin;
+    const uint32_t chunks = d.chunks, chunk = unit % chunks, local = unit / chunks;
+    const uint32_t t0 = (local % d.tiles_t) * Sh::tokens, n0 = (local / d.tiles_t) * Sh::rows;
+    const uint32_t blocks = cols >> 5;
+    const uint32_t kb_first = chunk * d.chunk_blocks;
+    const uint32_t kb_last = kb_first + d.chunk_blocks < blocks ? kb_first + d.chunk_blocks : blocks;
+
+    // Buffer descriptors (base, no stride, size in bytes, raw 32-bit format;
+    // 32-bit offsets: the caller keeps every region below 4 GiB). Reads past a
+    // region's end return zero instead of faulting.
+    auto descriptor = [](const void *base, size_t bytes) {
+        const uint64_t a = (uint64_t)(uintptr_t)base;
+        const u32x4 r = {(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+        return r;
+    };
+    const u32x4 rs_wq = descriptor(d.w, (size_t)rows * cols);
+    // (an odd number of scales ends inside the last dword: the two bytes behind
+    // it are allocation slack, never a fault, and never used)
+    const u32x4 rs_ws = descriptor(d.w + (size_t)rows * cols, (((size_t)rows * blocks + 1u) >> 1) * 4u);
+    const u32x4 rs_x = descriptor(d.xs, (size_t)batch * cols * 6u);
+
+    // The fetches are issued from inline assembly so that the compiler does not
+    // order LDS reads after them itself: its bookkeeping for loads that land in
+    // LDS waits for every such load in flight once a read cannot be matched to
+    // one fetch, which would drain the ring at every stage. The kernel waits
+    // by hand instead (`landed` below); there is no other vector memory
+    // operation between the first fetch and the last wait.
+    auto dma16 = [](const u32x4 &r, const uint8_t *lds, uint32_t lane_bytes, uint32_t block_bytes) {
+        const uint32_t m = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)lds;
+        asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :
+                     : "s"(m), "v"(lane_bytes), "s"(r), "s"(block_bytes)
+                     : "memory", "m0");
+    };
+    auto dma4 = [](const u32x4 &r, const uint8_t *lds, uint32_t lane_bytes) {
+        const uint32_t m = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)lds;
+        asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds"
+                     :
+                     : "s"(m), "v"(lane_bytes), "s"(r)
+                     : "memory", "m0");
+    };
+    // What a lane fetches does not change from block to block except for the
+    // block's byte offset, which rides in the instruction's scalar offset.
+    constexpr int NA = 3 * Sh::tokens / 16 / NW, NB = Sh::rows / 32 / NW;
+    uint32_t a_lane[NA], b_lane[NB], dw_first;
+#pragma unroll
+    for (int u = 0; u < NA; ++u) {
+        const uint32_t i = wave + (uint32_t)(u * NW);
+        const uint32_t pl = i / (Sh::tokens / 16), ri = i % (Sh::tokens / 16);
+        const uint32_t r = ri * 16u + (lane >> 2);
+        uint32_t t = t0 + r;
+        t = t < batch ? t : batch - 1u;
+        const uint32_t piece = (lane & 3u) ^ ((r >> 2) & 3u);
+        a_lane[u] = ((pl * batch + t) * 32u + piece * 8u) * 2u;
+    }
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+        const uint32_t i = wave + (uint32_t)(u * NW);
+        const uint32_t r = i * 32u + (lane >> 1);
+        uint32_t n = n0 + r;
+        n = n < rows ? n : rows - 1u;
+        const uint32_t piece = (lane & 1u) ^ ((r >> 3) & 1u);
+        b_lane[u] = n * cols + piece * 16u;
+    }
+    {
+        // Weight scales: per row the aligned dword that contains the f16 scale of
+        // the block (element e = row * blocks + kb lives in dword e / 2, half
+        // e % 2), one row per lane. Every wave issues one such fetch per block
+        // (waves beyond rows / 64 repeat a piece: same bytes, same place).
+        uint32_t n = n0 + (wave % (uint32_t)(Sh::rows / 64)) * 64u + lane;
+        n = n < rows ? n : rows - 1u;
+        dw_first = n * blocks;
+    }
+    const uint32_t a_block_bytes = __builtin_amdgcn_readfirstlane(batch * 192u);
+    auto fetch = [&](uint32_t kb_in, uint8_t *stage) {
+        // (fully unrolled: the number of fetch instructions per block is a
+        // compile-time constant, which the wait counters below rely on)
+        const uint32_t kb = __builtin_amdgcn_readfirstlane(kb_in); // scalar operand of the fetches
+#pragma unroll
+        for (int u = 0; u < NA; ++u) {
+            dma16(rs_x, stage + (wave + (uint32_t)(u * NW)) * 1024u, a_lane[u], kb * a_block_bytes);
+        }
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            dma16(rs_wq, stage + Sh::a_bytes + (wave + (uint32_t)(u * NW)) * 1024u, b_lane[u], kb * 32u);
+        }
+        dma4(rs_ws, stage + Sh::a_bytes + Sh::b_bytes + (wave % (uint32_t)(Sh::rows / 64)) * 256u,
+             ((dw_first + kb) >> 1) * 4u);
+    };
+
+    floatx16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                acc[i][j][v] = 0.0f;
+            }
+        }
+    }
+
+    uint32_t row_odd[TN]; // parity of this lane's first scale element per row tile
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        uint32_t n = n0 + wn * 64u + 32u * j + idx;
+        n = n < rows ? n : rows - 1u;
+        row_odd[j] = (n * blocks) & 1u;
+    }
+
+    // MFMA step m (k = 16m .. 16m+15) takes from lane (idx, half) the 8 values
+    // k = 16m + 8*half + 0..7 of token / weight row idx.
+    auto compute = [&](const uint8_t *stage, uint32_t kb) {
+        const uint32_t *sdw = (const uint32_t *)(stage + Sh::a_bytes + Sh::b_bytes);
+        const uint8_t *sb = stage + Sh::a_bytes;
+        bf16x8_t b[TN][2];
+        float dw[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const uint32_t r = wn * 64u + 32u * j + idx;
+#pragma unroll
+            for (int m = 0; m < 2; ++m) {
+                const uint32_t slot = (uint32_t)m ^ ((r >> 3) & 1u);
+                const u32x2 raw = *(const u32x2 *)(sb + r * 32u + slot * 16u + half * 8u);
+                b[j][m] = sbytes_to_bf16x8(raw.x, raw.y);
+            }
+            {
+                const uint32_t pair = sdw[r];
+                dw[j] = f16_bits_to_f32(((row_odd[j] + kb) & 1u) ? pair >> 16 : pair & 0xffffu);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const uint32_t r = wm * (32u * TM) + 32u * i + idx;
+            bf16x8_t a[3][2];
+#pragma unroll
+            for (int pl = 0; pl < 3; ++pl) {
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {
+                    const uint32_t slot = (uint32_t)(2 * m + (int)half) ^ ((r >> 2) & 3u);
+                    a[pl][m] = *(const bf16x8_t *)(stage + pl * Sh::a_plane + r * 64u + slot * 16u);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                floatx16_t s = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
+                                0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int pl = 2; pl >= 0; --pl) { // smallest pieces first
+#pragma unroll
+                    for (int m = 0; m < 2; ++m) {
+                        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[pl][m], b[j][m], s, 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    acc[i][j][v] = __builtin_fmaf(dw[j], s[v], acc[i][j][v]);
+                }
+            }
+        }
+    };
+
+    // Every wave issues the same number of fetch instructions per block, so
+    // "all but the newest two blocks have landed" is one counter value.
+    constexpr int F = NA + NB + 1;
+    static_assert((3 * Sh::tokens / 16) % NW == 0 && (Sh::rows / 32) % NW == 0, "uniform fetch");
+    constexpr int WAIT_TWO_BLOCKS = ((2 * F) & 15) | (((2 * F) >> 4) << 14) | (7 << 4) | (15 << 8);
+    auto landed = [&]() {
+        // this wave's fetch of the block about to be used is complete ...
+        __builtin_amdgcn_s_waitcnt(WAIT_TWO_BLOCKS);
+        // ... everybody's is, and everybody is done with the previous block's buffer
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    auto at = [&](uint32_t kb) { return kb < kb_last ? kb : kb_last - 1u; };
+    fetch(at(kb_first), stage_0);
+    fetch(at(kb_first + 1u), stage_1);
+    fetch(at(kb_first + 2u), stage_2);
+    for (uint32_t kb = kb_first; kb < kb_last; kb += 4u) {
+        landed();
+        fetch(at(kb + 3u), stage_3);
+        compute(stage_0, kb);
+        if (kb + 1u < kb_last) {
+            landed();
+            fetch(at(kb + 4u), stage_0);
+            compute(stage_1, kb + 1u);
+        }
+        if (kb + 2u < kb_last) {
+            landed();
+            fetch(at(kb + 5u), stage_1);
+            compute(stage_2, kb + 2u);
+        }
+        if (kb + 3u < kb_last) {
+            landed();
+            fetch(at(kb + 6u), stage_2);
+            compute(stage_3, kb + 3u);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); // vmcnt(0): every fetch has landed
+    __syncthreads(); // ... before the workgroup gives up its LDS
+
+    // A tile whose K is cut into chunks: every chunk's workgroup parks its
+    // partial tile; the one that arrives last adds the partial tiles in chunk
+    // order (whoever it is: the result does not depend on the order of arrival)
+    // and stores the sum. The arrival counter goes back to zero for the next launch.
+    if (chunks > 1u) {
+        constexpr uint32_t TILE_FLOATS = (uint32_t)NW * TM * TN * 16u * 64u;
+        const uint32_t slot = d.part_begin + local;
+        const size_t first_tile = (size_t)d.part_tile + (size_t)local * chunks;
+        float *mine = args.partials + (first_tile + chunk) * TILE_FLOATS +
+                      (size_t)wave * (TM * TN * 16u * 64u) + lane;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    __hip_atomic_store(mine + ((i * TN + j) * 16 + v) * 64, acc[i][j][v], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        // The partial tiles go to memory and come back from it with device-scope
+        // accesses that bypass this XCD's L2, so all it takes to publish them is
+        // to wait for the stores before the arrival is counted: no fence, which
+        // would write back and invalidate the whole L2 under the other
+        // workgroups' feet (measured: 14336 x 4096 in four chunks 481 us with
+        // fences).
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); // vmcnt(0)
+        asm volatile("" ::: "memory");
+        __shared__ uint32_t arrived;
+        __syncthreads();
+        if (threadIdx.x == 0u) {
+            arrived = __hip_atomic_fetch_add(&args.arrivals[slot], 1u, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (arrived != chunks - 1u) {
+            return;
+        }
+        if (threadIdx.x == 0u) {
+            __hip_atomic_store(&args.arrivals[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        const float *first = args.partials + first_tile * TILE_FLOATS +
+                             (size_t)wave * (TM * TN * 16u * 64u) + lane;
+        for (uint32_t c = 0; c < chunks; ++c) {
+            const float *part = first + (size_t)c * TILE_FLOATS;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const float pv = __hip_atomic_load(part + ((i * TN + j) * 16 + v) * 64,
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        acc[i][j][v] = c == 0u ? pv : acc[i][j][v] + pv;
+                    }
+                }
+            }
+        }
+    }
+
+    // acc[v] of a 32x32 tile is (token 8*(v/4) + 4*half + v%4, row idx).
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const uint32_t n = n0 + wn * 64u + 32u * j + idx;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t t = t0 + wm * (32u * TM) + 32u * i + 8u * (v / 4) + 4u * half + (v % 4);
+                if (t < batch && n < rows) {
+                    d.y[(size_t)t * rows + n] = acc[i][j][v];
+                }
+            }
+        }
+    }
+}
+
+struct Bx3Product {
+    const uint8_t *w;
+    const uint16_t *xs;
+    float *y;
+    uint32_t rows, cols, batch;
+};
+
+// The workgroup tile: 128 tokens x 256 rows (2 x 4 waves).
+constexpr uint32_t BX3_TILE_TOKENS = 128;
+constexpr uint32_t BX3_TILE_ROWS = 256;
+
+inline uint64_t bx3_tiles(uint32_t rows, uint32_t batch) {
+    return (uint64_t)((batch + BX3_TILE_TOKENS - 1u) / BX3_TILE_TOKENS) *
+           ((rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS);
+}
+// Q8_0 blocks per K chunk of a product. A product with few output tiles cuts K
+// into chunks of 1024 columns and more, as many as it takes to give the chip
+// about BX3_UNITS_WANTED work units; one with many tiles does not cut K at all
+// (14336 x 4096 at 512 tokens: 295 TFLOP/s whole, less in chunks; chunks shorter
+// than 1024 columns made the 0.6B projections slower, alone and together). A function of the
+// product's shape only: its result does not depend on what shares its launch.
+constexpr uint32_t BX3_UNITS_WANTED = 192;
+inline uint32_t bx3_chunk_blocks(uint32_t rows, uint32_t cols, uint32_t batch) {
+    const uint32_t blocks = cols / 32u;
+    const uint64_t tiles = bx3_tiles(rows, batch);
+    const uint32_t most = (blocks + BX3_CHUNK_BLOCKS - 1u) / BX3_CHUNK_BLOCKS;
+    const uint64_t want = (BX3_UNITS_WANTED + tiles - 1u) / tiles;
+    const uint32_t chunks = want < most ? (uint32_t)want : most;
+    return (blocks + chunks - 1u) / chunks;
+}
+// Work units (output tile x K chunk) of a product.
+inline uint64_t bx3_units(uint32_t rows, uint32_t cols, uint32_t batch);
+inline uint32_t bx3_chunks(uint32_t rows, uint32_t cols, uint32_t batch) {
+    const uint32_t cb = bx3_chunk_blocks(rows, cols, batch);
+    return (cols / 32u + cb - 1u) / cb;
+}
+inline uint64_t bx3_units(uint32_t rows, uint32_t cols, uint32_t batch) {
+    return bx3_tiles(rows, batch) * bx3_chunks(rows, cols, batch);
+}
+// Tiles of a product that need an arrival counter, and the floats of partial
+// tiles it needs (none for a single chunk).
+inline uint64_t bx3_split_tiles(uint32_t rows, uint32_t cols, uint32_t batch) {
+    return bx3_chunks(rows, cols, batch) > 1u ? bx3_tiles(rows, batch) : 0u;
+}
+inline uint64_t bx3_partial_floats(uint32_t rows, uint32_t cols, uint32_t batch) {
+    return bx3_split_tiles(rows, cols, batch) * bx3_chunks(rows, cols, batch) * BX3_TILE_TOKENS *
+           BX3_TILE_ROWS;
+}
+
+template <int WM, int WN, int TM>
+inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3Product *prods_in,
+                                 int n, float *partials, uint32_t *arrivals) {
+    using Sh = Bx3Shape<WM, WN, TM>;
+    static_assert(Sh::rows == (int)BX3_TILE_ROWS && Sh::tokens == (int)BX3_TILE_TOKENS, "tile");
+    Bx3Args args;
+    args.n = (uint32_t)n;
+    args.partials = partials;
+    args.arrivals = arrivals;
+    // Longest K first (the order of the list changes no product's result).
+    Bx3Product prods[BX3_MAX_DESCS];
+    for (int i = 0; i < n; ++i) {
+        int at = i;
+        while (at > 0 && prods[at - 1].cols < prods_in[i].cols) {
+            prods[at] = prods[at - 1];
+            --at;
+        }
+        prods[at] = prods_in[i];
+    }
+    uint64_t units = 0, split_tiles = 0, partial_tiles = 0;
+    for (int i = 0; i < n; ++i) {
+        Bx3Desc &d = args.d[i];
+        d.w = prods[i].w;
+        d.xs = prods[i].xs;
+        d.y = prods[i].y;
+        d.rows = prods[i].rows;
+        d.cols = prods[i].cols;
+        d.batch = prods[i].batch;
+        d.tile_begin = (uint32_t)units;
+        d.tiles_t = (prods[i].batch + Sh::tokens - 1) / Sh::tokens;
+        d.chunk_blocks = bx3_chunk_blocks(prods[i].rows, prods[i].cols, prods[i].batch);
+        d.chunks = bx3_chunks(prods[i].rows, prods[i].cols, prods[i].batch);
+        d.part_begin = (uint32_t)split_tiles;
+        d.part_tile = (uint32_t)partial_tiles;
+        const uint64_t tiles = (uint64_t)d.tiles_t * ((prods[i].rows + Sh::rows - 1) / Sh::rows);
+        units += tiles * d.chunks;
+        if (d.chunks > 1u) {
+            split_tiles += tiles;
+            partial_tiles += tiles * d.chunks;
+        }
+    }
+    if (units == 0 || units > 0x7fffffffull || split_tiles > BX3_MAX_SPLIT_TILES ||
+        (split_tiles > 0 && (partials == nullptr || arrivals == nullptr))) {
+        return hipErrorInvalidValue;
+    }
+    args.total_tiles = (uint32_t)units;
+    args.chunk_wgs = args.d[0].tiles_t * args.d[0].chunks;
+    args.pad = 0;
+    Q8_LAUNCH((gemm_bf16x3_kernel<WM, WN, TM>), dim3((unsigned)units), dim3(WM * WN * 64), 0, stream,
+              stop, args);
+    return hipGetLastError();
+}
+
+// Sealed weights, every region below 4 GiB (32-bit buffer offsets): the caller
+// checks these before choosing this kernel. `partials` holds the sum of the
+// products' bx3_partial_floats() floats, `arrivals` BX3_MAX_SPLIT_TILES counters
+// that are zero between launches (both may be null when no product has more than
+// 1024 columns).
+inline hipError_t launch_gemm_bf16x3_list(hipStream_t stream, hipEvent_t stop,
+                                          const Bx3Product *prods, int n, float *partials,
+                                          uint32_t *arrivals) {
+    if (n <= 0 || n > BX3_MAX_DESCS) {
+        return hipErrorInvalidValue;
+    }
+    return launch_bx3_cfg<2, 4, 2>(stream, stop, prods, n, partials, arrivals);
+}
+
+struct SplitInput {
+    const float *x;
+    uint16_t *xs;
+    uint32_t batch, cols;
+};
+
+// Every input: cols a positive multiple of 32, x 16-byte aligned, batch * cols below 2^30.
+inline hipError_t launch_split_act_list(hipStream_t stream, const SplitInput *in, int n) {
+    if (n <= 0 || n > SPLIT_MAX_DESCS) {
+        return hipErrorInvalidValue;
+    }
+    SplitArgs args;
+    args.n = (uint32_t)n;
+    args.pad = 0;
+    uint32_t wgs = 0;
+    for (int i = 0; i < n; ++i) {
+        if (in[i].batch == 0 || in[i].cols == 0 || (in[i].cols & 31u) != 0u ||
+            (uint64_t)in[i].batch * in[i].cols >= (1ull << 30)) {
+            return hipErrorInvalidValue;
+        }
+        args.d[i] = SplitDesc{in[i].x, in[i].xs, in[i].batch, in[i].cols, wgs, 0};
+        wgs += (in[i].batch * in[i].cols / 4u + 255u) / 256u;
+    }
+    hipLaunchKernelGGL(split_act_list_kernel, dim3(wgs), dim3(256), 0, stream, args);
+    return hipGetLastError();
+}
+
+} // namespace q8

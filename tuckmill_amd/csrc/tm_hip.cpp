@@ -23,6 +23,7 @@
 
 #include "q8_gemm_i8.hpp"
 #include "q8_gemv_i8.hpp"
+#include "q8_gemm_bf16x3.hpp"
 #include "q8_gemm_i8_lds.hpp"
 #include "q8_gemm_mma.hpp"
 #include "q8_gemv.hpp"
@@ -98,6 +99,16 @@ struct tm_hip_ctx {
     hipStream_t stream = nullptr;
     hipStream_t copy_stream = nullptr;
     uint32_t *mma_queue = nullptr; // two counters of the work-queue MFMA kernel, zero between launches
+    // Workspace of the bf16 split-float GEMM (split activations, partial tiles of
+    // products with K above 1024, their arrival counters): grown on demand, never
+    // shrunk. A buffer that was outgrown stays allocated until the context goes:
+    // recorded steps may still point at it.
+    uint8_t *bx3_xs = nullptr;
+    size_t bx3_xs_bytes = 0;
+    float *bx3_partials = nullptr;
+    size_t bx3_partial_bytes = 0;
+    uint32_t *bx3_arrivals = nullptr;
+    std::vector<void *> bx3_retired;
     std::atomic<uint64_t> allocated{0};
     std::atomic<uint64_t> leased{0};
     std::atomic<uint64_t> committed{0};
@@ -270,6 +281,7 @@ enum Variant : uint8_t {
     V_GENERAL,    // gemv_list_kernel, four tokens per pass (raw layout / narrow small batches)
     V_SPLIT,      // gemm_split_list_kernel: p0 = waves, p1 = tokens per wave, p2 = column tail
     V_MMA,        // f32 MFMA GEMM: p0 = tmw, p1 = tnw, p2 = K split
+    V_BF16X3,     // prefill GEMM on the bf16 matrix cores, activations split in three
     V_I8_TILE,    // register-fed int8 MFMA GEMM: p0 = tile configuration
     V_I8_STREAM,  // int8 streaming kernel: p0 = tokens per pass
     V_I8_LDS,     // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (q8::i8_lds_shape)
@@ -289,6 +301,31 @@ struct GemvKey {
     // one token, sealed weights, aligned activations: the kernel the planner's fusions target
     bool decode() const { return kind == OP_GEMV_LIST && variant == V_DECODE && packed && flag; }
 };
+
+// Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 384
+// tokens, and with at least 128 work units of 128 tokens x 256 rows (x K chunk)
+// of their own. The kernel is two to three times as fast as the f32 one when it
+// fills the chip (at 512 tokens 14336 x 4096: 204 us against 640 us, 6144 x 2048:
+// 69 against 133) but its units are large: 1024 x 1024 alone takes 48 us against
+// 15 us, and 33 us with K in four chunks. Measured at 512 tokens, alone: 64 units
+// 52 against 49 us, 128 units 57 against 94 us (K = 1024), 66 against 91 us
+// (K = 4096). A product's kernel depends on nothing but its own shape and
+// alignment, so its result does not depend on what shares its launch (the seven
+// 0.6B projections together would take 78 us instead of 144 us on this kernel,
+// and 359 us instead of 183 us one by one).
+constexpr uint32_t kBx3MinBatch = 384;
+constexpr uint64_t kBx3MinUnits = 128;
+constexpr uint64_t kBx3MaxPartialFloats = 1ull << 29; // 2 GiB of partial tiles per launch
+
+bool bx3_eligible(const Op &op, bool x_aligned) {
+    return op.packed && x_aligned && op.batch >= kBx3MinBatch &&
+           q8::bx3_units(op.rows, op.cols, op.batch) >= kBx3MinUnits &&
+           (uint64_t)op.rows * op.cols < (1ull << 32) &&
+           (uint64_t)op.batch * op.cols * 6u < (1ull << 32) &&
+           (uint64_t)op.batch * op.cols < (1ull << 30) &&
+           q8::bx3_split_tiles(op.rows, op.cols, op.batch) <= q8::BX3_MAX_SPLIT_TILES &&
+           q8::bx3_partial_floats(op.rows, op.cols, op.batch) <= kBx3MaxPartialFloats;
+}
 
 GemvKey gemv_key(const Op &op) {
     GemvKey k;
@@ -319,6 +356,10 @@ GemvKey gemv_key(const Op &op) {
     }
     const uintptr_t xp = (uintptr_t)op.a[1]->ptr + (uintptr_t)op.x_off * 4u;
     k.flag = (xp % 16u == 0);
+    if (op.kind == OP_MMA && bx3_eligible(op, k.flag)) {
+        k.variant = V_BF16X3;
+        return k;
+    }
     if (op.kind == OP_MMA) {
         // The tile shape and K split are chosen per product, so a product's
         // result does not depend on what else shares its launch.
@@ -426,7 +467,16 @@ struct Launch {
     const Op *norm = nullptr;         // an RMSNorm fused in front of the flagged entries
     GemvKey key{};
     const Op *single = nullptr;
+    // V_BF16X3: what the listed products need of the context's workspace
+    uint64_t bx3_split_tiles = 0, bx3_partial_floats = 0, bx3_xs_bytes = 0;
+    int bx3_inputs = 0;
 };
+
+// Two products read the same activations (and can share their split form).
+bool same_input(const Op &a, const Op &b) {
+    return a.a[1] == b.a[1] && a.x_off == b.x_off && a.batch == b.batch && a.cols == b.cols;
+}
+size_t bx3_xs_bytes_of(const Op &op) { return ((size_t)op.batch * op.cols * 6u + 255u) & ~(size_t)255u; }
 
 hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
                            GemvKey key) {
@@ -441,6 +491,87 @@ hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<c
     const q8::MmaConfig c{key.p0, key.p1, key.p2};
     return q8::launch_gemm_mma_list(ctx->stream, stop, key.packed, key.flag, prods, n, &c,
                                     ctx->mma_queue);
+}
+
+// The split-float GEMM: one launch that splits every distinct input of the list
+// into its three bf16 planes, then the product list. The workspace was sized by
+// ensure_bx3_workspace() when the launches were planned.
+hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch) {
+    const std::vector<const Op *> &ops = launch.list;
+    if (launch.bx3_xs_bytes > ctx->bx3_xs_bytes ||
+        launch.bx3_partial_floats * 4u > ctx->bx3_partial_bytes) {
+        return hipErrorInvalidValue;
+    }
+    q8::SplitInput inputs[q8::SPLIT_MAX_DESCS];
+    const Op *input_of[q8::SPLIT_MAX_DESCS];
+    q8::Bx3Product prods[q8::BX3_MAX_DESCS];
+    int n_in = 0, n = 0;
+    size_t xs_used = 0;
+    for (const Op *op : ops) {
+        int at = 0;
+        while (at < n_in && !same_input(*input_of[at], *op)) {
+            ++at;
+        }
+        if (at == n_in) {
+            if (n_in == q8::SPLIT_MAX_DESCS) {
+                return hipErrorInvalidValue;
+            }
+            input_of[n_in] = op;
+            inputs[n_in] = q8::SplitInput{(const float *)op->a[1]->ptr + op->x_off,
+                                          (uint16_t *)(ctx->bx3_xs + xs_used), op->batch, op->cols};
+            xs_used += bx3_xs_bytes_of(*op);
+            ++n_in;
+        }
+        prods[n++] = q8::Bx3Product{(const uint8_t *)op->a[0]->ptr, inputs[at].xs,
+                                    (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
+                                    op->batch};
+    }
+    hipError_t e = q8::launch_split_act_list(ctx->stream, inputs, n_in);
+    if (e != hipSuccess) {
+        return e;
+    }
+    return q8::launch_gemm_bf16x3_list(ctx->stream, stop, prods, n, ctx->bx3_partials,
+                                       ctx->bx3_arrivals);
+}
+
+// Kernel launches a planned launch stands for.
+uint32_t kernel_launches_of(const Launch &l) {
+    return l.single == nullptr && l.key.variant == V_BF16X3 ? 2u : 1u;
+}
+
+// Grow the split-float GEMM's workspace to what the largest of the planned
+// launches needs (launches on the context's stream run one after the other and
+// share it).
+hipError_t ensure_bx3_workspace(tm_hip_ctx *ctx, const std::vector<Launch> &plan) {
+    size_t xs = 0, partial = 0;
+    for (const Launch &l : plan) {
+        if (l.single == nullptr && l.key.variant == V_BF16X3) {
+            xs = l.bx3_xs_bytes > xs ? (size_t)l.bx3_xs_bytes : xs;
+            partial = l.bx3_partial_floats * 4u > partial ? (size_t)(l.bx3_partial_floats * 4u) : partial;
+        }
+    }
+    auto grow = [&](void **buf, size_t *have, size_t need) -> hipError_t {
+        if (need <= *have) {
+            return hipSuccess;
+        }
+        need += need / 4u; // some room, so that a slightly larger chunk does not allocate again
+        void *fresh = nullptr;
+        hipError_t e = hipMalloc(&fresh, need);
+        if (e != hipSuccess) {
+            return e;
+        }
+        if (*buf != nullptr) {
+            ctx->bx3_retired.push_back(*buf);
+        }
+        *buf = fresh;
+        *have = need;
+        return hipSuccess;
+    };
+    hipError_t e = grow((void **)&ctx->bx3_xs, &ctx->bx3_xs_bytes, xs);
+    if (e == hipSuccess) {
+        e = grow((void **)&ctx->bx3_partials, &ctx->bx3_partial_bytes, partial);
+    }
+    return e;
 }
 
 hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
@@ -466,6 +597,9 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     const std::vector<const Op *> &ops = launch.list;
     const std::vector<const Op *> &residual = launch.residual;
     const GemvKey key = launch.key;
+    if (key.variant == V_BF16X3) {
+        return launch_bx3_list(ctx, stop, launch);
+    }
     if (key.kind == OP_MMA) {
         return launch_mma_list(ctx, stop, ops, key);
     }
@@ -743,9 +877,32 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 conflict = conflict || op.a[3]->read_epoch == epoch || op.a[3]->write_epoch == epoch;
             }
             const bool open = !cur.list.empty() || cur.norm != nullptr;
+            bool new_input = true;
+            if (key.variant == V_BF16X3 && !cur.list.empty() && key == cur.key) {
+                for (const Op *other : cur.list) {
+                    new_input = new_input && !same_input(*other, op);
+                }
+                // the launch's share of the workspace stays within its limits
+                conflict = conflict ||
+                           cur.bx3_split_tiles + q8::bx3_split_tiles(op.rows, op.cols, op.batch) >
+                               q8::BX3_MAX_SPLIT_TILES ||
+                           cur.bx3_partial_floats +
+                                   q8::bx3_partial_floats(op.rows, op.cols, op.batch) >
+                               kBx3MaxPartialFloats ||
+                           (new_input && cur.bx3_inputs == q8::SPLIT_MAX_DESCS);
+            }
             if (open && (conflict || (!cur.list.empty() && !(key == cur.key)) ||
                          (int)cur.list.size() == cap)) {
                 flush();
+                new_input = true;
+            }
+            if (key.variant == V_BF16X3) {
+                cur.bx3_split_tiles += q8::bx3_split_tiles(op.rows, op.cols, op.batch);
+                cur.bx3_partial_floats += q8::bx3_partial_floats(op.rows, op.cols, op.batch);
+                if (new_input) {
+                    cur.bx3_inputs += 1;
+                    cur.bx3_xs_bytes += bx3_xs_bytes_of(op);
+                }
             }
             const bool takes_norm = normed && cur.norm != nullptr; // still pending after a flush?
             cur.key = key;
@@ -833,6 +990,10 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, hipEvent_t sto
                      bool *stop_attached) {
     const std::vector<Launch> plan = plan_launches(ctx, ops);
     *stop_attached = false;
+    hipError_t ws = ensure_bx3_workspace(ctx, plan);
+    if (ws != hipSuccess) {
+        return ws;
+    }
     for (size_t i = 0; i < plan.size(); ++i) {
         const bool last = i + 1 == plan.size();
         const hipEvent_t ev = last ? stop : nullptr;
@@ -842,7 +1003,7 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, hipEvent_t sto
         if (e != hipSuccess) {
             return e;
         }
-        ctx->launches.fetch_add(1, std::memory_order_relaxed);
+        ctx->launches.fetch_add(kernel_launches_of(l), std::memory_order_relaxed);
         if (last) {
             *stop_attached = true;
         }
@@ -1079,8 +1240,14 @@ tm_hip_ctx *tm_hip_create(char *err, size_t err_cap) {
     if (e == hipSuccess) {
         e = hipMemset(ctx->mma_queue, 0, 256);
     }
+    if (e == hipSuccess) {
+        e = hipMalloc((void **)&ctx->bx3_arrivals, q8::BX3_MAX_SPLIT_TILES * sizeof(uint32_t));
+    }
+    if (e == hipSuccess) {
+        e = hipMemset(ctx->bx3_arrivals, 0, q8::BX3_MAX_SPLIT_TILES * sizeof(uint32_t));
+    }
     if (e != hipSuccess) {
-        hip_fail(err, err_cap, "work-queue counters", e);
+        hip_fail(err, err_cap, "device-side counters", e);
         tm_hip_destroy(ctx);
         return nullptr;
     }
@@ -1134,6 +1301,14 @@ void tm_hip_destroy(tm_hip_ctx *ctx) {
     }
     if (ctx->mma_queue != nullptr) {
         (void)hipFree(ctx->mma_queue);
+    }
+    for (void *p : {(void *)ctx->bx3_arrivals, (void *)ctx->bx3_xs, (void *)ctx->bx3_partials}) {
+        if (p != nullptr) {
+            (void)hipFree(p);
+        }
+    }
+    for (void *p : ctx->bx3_retired) {
+        (void)hipFree(p);
     }
     if (ctx->copy_stream != nullptr) {
         (void)hipStreamDestroy(ctx->copy_stream);
@@ -1573,8 +1748,13 @@ int tm_hip_end_group_recorded(tm_hip_ctx *ctx, tm_hip_step **out, char *err, siz
     step->owner = ctx;
     step->operators = (uint32_t)ops.size();
     const std::vector<Launch> plan = plan_launches(ctx, ops);
+    hipError_t e = ensure_bx3_workspace(ctx, plan); // allocates: before the stream records
+    if (e != hipSuccess) {
+        delete step;
+        return hip_fail(err, err_cap, "end_group_recorded: workspace", e);
+    }
     // Relaxed mode: the launchers may query occupancy while the stream records.
-    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed);
+    e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed);
     if (e != hipSuccess) {
         delete step;
         return hip_fail(err, err_cap, "end_group_recorded: begin capture", e);
@@ -1604,7 +1784,10 @@ int tm_hip_end_group_recorded(tm_hip_ctx *ctx, tm_hip_step **out, char *err, siz
         delete step;
         return hip_fail(err, err_cap, "end_group_recorded: graph instantiation", e);
     }
-    step->launches = (uint32_t)plan.size();
+    step->launches = 0;
+    for (const Launch &l : plan) {
+        step->launches += kernel_launches_of(l);
+    }
     step->keep = allocs_of(ctx, ops);
     for (Alloc *a : step->keep) {
         a->refs.fetch_add(1, std::memory_order_relaxed);

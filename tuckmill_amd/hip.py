@@ -24,6 +24,9 @@ LIB_PATH = os.path.join(_HERE, "libtm_hip.so")
 ERR_CAP = 512  # crates/metal/src/lib.rs:32
 GEMM_MAX_BATCH = 32  # crates/metal/src/lib.rs:28-30
 GEMM_MMA_MAX_BATCH = 512
+# From this batch on tm_hip_q8_0_gemm_mma over sealed weights with 16-byte aligned activations
+# runs on the bf16 matrix cores (activations split into three exact bf16 pieces).
+GEMM_MMA_BF16_MIN_BATCH = 384
 GEMM_I8_MAX_BATCH = 2048
 ARGMAX_NONE = 0xFFFFFFFF  # crates/metal/src/lib.rs (ARGMAX_NONE), native/metal/kernels.metal:143
 ARGMAX_PARTIAL_BYTES = 512
