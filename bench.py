@@ -197,11 +197,8 @@ def bench_gemm(host, ctx, steps, warmup):
                   max(2, warmup // 20), n, grouped=False)
     us = t.gpu_ms / n * 1e3
     flops = 2.0 * M * rows * cols
-    out["lm_head"] = {"rows": rows, "cols": cols, "us": us, "launches_per_step": t.launches / n,
-                      "tflops_f32_equivalent": flops / us / 1e6,
-                      "kernel": "q8::split_act_list_kernel + q8::gemm_bf16x3_kernel",
-                      "bf16_mfma_tflops_issued": 3.0 * flops / us / 1e6,
-                      "frac_of_bf16_mfma_peak": 3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS}
+    out["lm_head"] = dict(_bf16_gemm_point(flops, us), rows=rows, cols=cols,
+                          launches_per_step=t.launches / n)
     for b in keep + [m.buf, xb, yb]:
         b.free()
     return out
@@ -215,6 +212,16 @@ def _weights_pool(ctx, shapes, copies, seed_base):
             raw = S.make_weights(rows, cols, seed_base + 17 * c + len(pool))
             pool.append((name, rows, cols, H.Matrix.load(ctx, raw, cols, rows)))
     return pool
+
+
+def _bf16_gemm_point(flops, us):
+    """A prefill GEMM that ran on the bf16 matrix cores: `flops` = 2*M*N*K of the
+    f32 product it stands for; the kernel issues three bf16 MFMA products per
+    f32 one (the activation's three exact pieces)."""
+    return {"flops": flops, "us": us, "tflops_f32_equivalent": flops / us / 1e6,
+            "kernel": "q8::split_act_list_kernel + q8::gemm_bf16x3_kernel",
+            "bf16_mfma_tflops_issued": 3.0 * flops / us / 1e6,
+            "frac_of_bf16_mfma_peak": 3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS}
 
 
 def bench_gemma(host, ctx, steps, warmup):
@@ -259,8 +266,7 @@ def bench_gemma(host, ctx, steps, warmup):
     flops = sum(2.0 * M * p.rows * p.cols for p in gp)
     t = run_steps(host, ctx, gp, gwarm, gsteps, grouped=True)
     us = t.gpu_ms / gsteps * 1e3
-    out["ffn_gemm_m512"] = {"flops": flops, "us": us, "tflops": flops / us / 1e6,
-                            "frac_of_f32_mfma_peak": flops / us / 1e6 / MFMA_F32_PEAK_TFLOPS}
+    out["ffn_gemm_m512"] = _bf16_gemm_point(flops, us)
     name, rows, cols, m = pool[-1]
     xb = ctx.buffer(M * cols * 4)
     xb.upload(0, S.make_activations(M * cols, 7))
@@ -270,8 +276,7 @@ def bench_gemma(host, ctx, steps, warmup):
     t = run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA)],
                   2, 5, grouped=False)
     us = t.gpu_ms / 5 * 1e3
-    out["lm_head_gemm_m512"] = {"flops": flops, "us": us, "tflops": flops / us / 1e6,
-                                "frac_of_f32_mfma_peak": flops / us / 1e6 / MFMA_F32_PEAK_TFLOPS}
+    out["lm_head_gemm_m512"] = _bf16_gemm_point(flops, us)
     for b in keep:
         b.free()
     for _, _, _, m in pool:
@@ -337,6 +342,12 @@ def bench_sweep(host, ctx, steps, warmup):
                 "frac_of_mfma_peak": flops / us / 1e6 / (MFMA_I8_PEAK_TOPS if kind == TMH_GEMM_I8
                                                         else MFMA_F32_PEAK_TFLOPS),
                 "quantize_act_us": quant_us})
+            if kind == TMH_GEMM_MMA and mb >= H.GEMM_MMA_BF16_MIN_BATCH:
+                # both sweep shapes are large enough for the kernel on the bf16
+                # matrix cores, which issues three bf16 products per f32 one
+                pt = out["points"][-1]
+                pt["path"] = label.replace("f32 mfma", "bf16 mfma x3")
+                pt["frac_of_mfma_peak"] = 3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS
     for b in [xb] + list(xqs.values()) + ys:
         b.free()
     for _, _, _, m in pool:
