@@ -1,4 +1,4 @@
-"""GPU parity: the prefill GEMM from 384 tokens over sealed weights large enough
+"""GPU parity: the prefill GEMM from 65 tokens over sealed weights large enough
 to fill the chip with 128-token x 256-row tiles, which runs on the bf16 matrix
 cores with every f32 activation split into three exact bf16 pieces (contract: native/metal/tm_metal.h:172-175, tolerance-qualified like
 every matrix-core kernel; crates/metal/src/tests.rs:1169-1233 for the shapes).
@@ -41,8 +41,9 @@ def product(ctx, wb, x, rows, cols, batch, x_off=0, y_off=0):
 # K of 1, 3, 32, 33 (two K chunks of 17 and 16 blocks), 36, 64 and 96 blocks;
 # ragged rows; a ragged last token tile; the smallest batch of the kernel and
 # the largest; every product has at least 128 work units of its own.
-SHAPES = [(8192, 1024, 512), (11000, 96, M0), (8300, 1056, 500), (4096, 3072, 512),
-          (5000, 2048, M0 + 1), (33000, 32, 512), (8500, 1152, 450)]
+SHAPES = [(8192, 1024, 512), (33000, 96, M0), (8300, 1056, 500), (4096, 3072, 512),
+          (33000, 2048, M0 + 1), (33000, 32, 512), (8500, 1152, 450), (11000, 1024, 384),
+          (16500, 1024, 129)]
 
 
 @pytest.mark.parametrize("rows,cols,batch", SHAPES)
@@ -63,7 +64,7 @@ def test_boundary_values_and_wide_ranges(ctx):
     # crates/metal/src/tests.rs:1169-1233 (boundary weights and inputs), and
     # activations that span 60 binades: every piece of the split is exact, so the
     # large terms do not swamp the small ones any more than in the CPU's sum.
-    rows, cols, batch = 11000, 1024, M0
+    rows, cols, batch = 33000, 1024, M0
     w = O.boundary_weights(rows, cols, 11)
     x = O.boundary_input(cols * batch, 13)
     wb = weights_buffer(ctx, w, rows, cols, True)
@@ -85,7 +86,7 @@ def test_boundary_values_and_wide_ranges(ctx):
 
 
 def test_activations_off_a_16_byte_boundary_take_the_f32_kernels(ctx):
-    rows, cols, batch = 8192, 1024, M0
+    rows, cols, batch = 8192, 1024, 512
     w = S.make_weights(rows, cols, 77)
     x = S.make_activations(batch * cols, 78)
     wb = weights_buffer(ctx, w, rows, cols, True)
@@ -151,3 +152,19 @@ def test_a_group_splits_each_input_once_and_has_the_bits_of_its_products_alone(c
     for m in mats:
         m[3].free()
         m[4].free()
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(8192, 1024, 512), (8191, 1024, 512), (7936, 1024, 512),
+                                             (32768, 1024, 65), (32768, 1024, 64), (32513, 1024, 65),
+                                             (4096, 4096, 128), (4096, 4096, 129), (6144, 2048, 512),
+                                             (6144, 2048, 256), (1024, 1024, 512), (2048, 6144, 384)])
+def test_the_choice_of_kernel_follows_the_documented_rule(ctx, rows, cols, batch):
+    # two launches (split, multiply) on the bf16 matrix cores, one on the f32 ones
+    wb = weights_buffer(ctx, S.make_weights(rows, cols, 1), rows, cols, True)
+    xb, yb = ctx.buffer(batch * cols * 4), ctx.buffer(batch * rows * 4)
+    launches = ctx.kernel_launches()
+    ctx.q8_0_gemm_mma(wb, xb, yb, rows, cols, batch, 0, 0)
+    ctx.fence()
+    assert ctx.kernel_launches() - launches == (2 if H.gemm_mma_on_bf16(rows, cols, batch) else 1)
+    for b in (wb, xb, yb):
+        b.free()

@@ -302,18 +302,19 @@ struct GemvKey {
     bool decode() const { return kind == OP_GEMV_LIST && variant == V_DECODE && packed && flag; }
 };
 
-// Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 384
+// Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 65
 // tokens, and with at least 128 work units of 128 tokens x 256 rows (x K chunk)
 // of their own. The kernel is two to three times as fast as the f32 one when it
 // fills the chip (at 512 tokens 14336 x 4096: 204 us against 640 us, 6144 x 2048:
-// 69 against 133) but its units are large: 1024 x 1024 alone takes 48 us against
-// 15 us, and 33 us with K in four chunks. Measured at 512 tokens, alone: 64 units
-// 52 against 49 us, 128 units 57 against 94 us (K = 1024), 66 against 91 us
-// (K = 4096). A product's kernel depends on nothing but its own shape and
-// alignment, so its result does not depend on what shares its launch (the seven
-// 0.6B projections together would take 78 us instead of 144 us on this kernel,
-// and 359 us instead of 183 us one by one).
-constexpr uint32_t kBx3MinBatch = 384;
+// 69 against 133; at 96 tokens 14336 x 4096: 73 against 173) but its units are
+// large: 1024 x 1024 at 512 tokens takes 48 us against 15 us, and 33 us with K in
+// four chunks. Measured alone at 512 tokens: 64 units 52 against 49 us, 128 units
+// 57 against 94 us (K = 1024), 66 against 91 us (K = 4096); at 64 tokens and
+// below the f32 kernels win or tie on most shapes. A product's kernel depends on
+// nothing but its own shape and alignment, so its result does not depend on
+// what shares its launch (the seven 0.6B projections together would take 78 us
+// instead of 144 us on this kernel, and 359 us instead of 183 us one by one).
+constexpr uint32_t kBx3MinBatch = 65;
 constexpr uint64_t kBx3MinUnits = 128;
 constexpr uint64_t kBx3MaxPartialFloats = 1ull << 29; // 2 GiB of partial tiles per launch
 

@@ -24,9 +24,29 @@ LIB_PATH = os.path.join(_HERE, "libtm_hip.so")
 ERR_CAP = 512  # crates/metal/src/lib.rs:32
 GEMM_MAX_BATCH = 32  # crates/metal/src/lib.rs:28-30
 GEMM_MMA_MAX_BATCH = 512
-# From this batch on tm_hip_q8_0_gemm_mma over sealed weights with 16-byte aligned activations
-# runs on the bf16 matrix cores (activations split into three exact bf16 pieces).
-GEMM_MMA_BF16_MIN_BATCH = 384
+# From this batch on tm_hip_q8_0_gemm_mma over a large sealed matrix (128 or more tiles of
+# 128 tokens x 256 rows, K chunks counted) with 16-byte aligned activations runs on the bf16
+# matrix cores (activations split into three exact bf16 pieces).
+GEMM_MMA_BF16_MIN_BATCH = 65
+
+
+def gemm_mma_bf16_units(rows: int, cols: int, batch: int) -> int:
+    """Work units (128 tokens x 256 rows x one K chunk) the bf16 matrix-core GEMM
+    makes of a product: K is cut into chunks of 1024 columns or more, as many as
+    give about 192 units (mirror of q8::bx3_units, csrc/q8_gemm_bf16x3.hpp)."""
+    tiles = -(-batch // 128) * -(-rows // 256)
+    blocks = cols // 32
+    chunks = min(-(-192 // tiles), -(-blocks // 32))
+    per_chunk = -(-blocks // chunks)
+    return tiles * -(-blocks // per_chunk)
+
+
+def gemm_mma_on_bf16(rows: int, cols: int, batch: int, x_off: int = 0) -> bool:
+    """Whether tm_hip_q8_0_gemm_mma over sealed weights takes the bf16 matrix-core
+    kernel for this product (mirror of bx3_eligible, csrc/tm_hip.cpp; the limits
+    on region sizes beyond 4 GiB are left out)."""
+    return (batch >= GEMM_MMA_BF16_MIN_BATCH and x_off % 4 == 0 and
+            gemm_mma_bf16_units(rows, cols, batch) >= 128)
 GEMM_I8_MAX_BATCH = 2048
 ARGMAX_NONE = 0xFFFFFFFF  # crates/metal/src/lib.rs (ARGMAX_NONE), native/metal/kernels.metal:143
 ARGMAX_PARTIAL_BYTES = 512
