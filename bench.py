@@ -303,6 +303,7 @@ def bench_sweep(host, ctx, steps, warmup):
     widths = sorted({c for _, _, c, _ in pool})
     xqs = {c: ctx.buffer(H.xq_bytes(c, maxM)) for c in widths}
     ys = [ctx.buffer(maxM * maxr * 4) for _ in pool]
+    slice_x, slice_y = [], []
     for M in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 2048):
         n = max(3, steps // (10 if M < 64 else 200 if M < 512 else 1000))
         w = max(2, n // 5)
@@ -330,9 +331,19 @@ def bench_sweep(host, ctx, steps, warmup):
                 for (name, r, c, m), yb in zip(pool, ys):
                     prods.append(tmh_product(m.buf.raw, xqs[c].raw, yb.raw, r, c, M, kind))
             else:
-                for (name, r, c, m), yb in zip(pool, ys):
-                    for _ in range(slices):
-                        prods.append(tmh_product(m.buf.raw, xb.raw, yb.raw, r, c, mb, kind))
+                # a batch above the largest one of a call goes in slices, each with
+                # its own rows of X and of Y (buffers of their own here: the step
+                # runner's products carry no offsets)
+                while len(slice_x) < slices - 1:
+                    sx = ctx.buffer(mb * maxc * 4)
+                    sx.upload(0, S.make_activations(mb * maxc, 100 + len(slice_x)))
+                    slice_x.append(sx)
+                    slice_y.append([ctx.buffer(mb * maxr * 4) for _ in pool])
+                for i, ((name, r, c, m), yb) in enumerate(zip(pool, ys)):
+                    prods.append(tmh_product(m.buf.raw, xb.raw, yb.raw, r, c, mb, kind))
+                    for sl in range(slices - 1):
+                        prods.append(tmh_product(m.buf.raw, slice_x[sl].raw, slice_y[sl][i].raw,
+                                                 r, c, mb, kind))
             t = run_steps(host, ctx, prods, w, n, grouped=True)
             us = t.gpu_ms / n * 1e3
             out["points"].append({
@@ -348,7 +359,7 @@ def bench_sweep(host, ctx, steps, warmup):
                 pt = out["points"][-1]
                 pt["path"] = label.replace("f32 mfma", "bf16 mfma x3")
                 pt["frac_of_mfma_peak"] = 3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS
-    for b in [xb] + list(xqs.values()) + ys:
+    for b in [xb] + list(xqs.values()) + ys + slice_x + [y for per in slice_y for y in per]:
         b.free()
     for _, _, _, m in pool:
         m.buf.free()
