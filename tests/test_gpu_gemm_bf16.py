@@ -82,6 +82,22 @@ def test_boundary_values_and_wide_ranges(ctx):
     got = product(ctx, wb, x, rows, cols, batch).reshape(batch, rows)
     cpu = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
     assert norm_err(got, cpu) <= 1e-5
+    # An infinite or NaN activation reaches the outputs as through f32 products:
+    # +-inf where the weight is not zero, NaN where it is (0 * inf) and for NaN.
+    x = S.make_activations(batch * cols, 10)
+    x[3 * cols + 17] = np.inf
+    x[5 * cols + 200] = np.nan
+    x[7 * cols + 999] = -np.inf
+    x[9 * cols + 40] = np.float32(np.uint32(0x7F800001).view(np.float32))  # a NaN in the low bits only
+    got = product(ctx, wb, x, rows, cols, batch).reshape(batch, rows)
+    with np.errstate(invalid="ignore", over="ignore"):
+        cpu = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
+    assert np.array_equal(np.isnan(got), np.isnan(cpu))
+    assert np.array_equal(np.isposinf(got), np.isposinf(cpu))
+    assert np.array_equal(np.isneginf(got), np.isneginf(cpu))
+    assert np.isnan(got[5]).all() and np.isnan(got[9]).all() and np.isinf(got[3]).any()
+    ok = np.isfinite(cpu)
+    assert np.max(np.abs(got[ok] - cpu[ok])) <= 1e-5 * np.max(np.abs(cpu[ok]))
     wb.free()
 
 

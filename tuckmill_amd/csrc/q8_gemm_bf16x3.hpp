@@ -15,18 +15,18 @@
 // activation is rounded anywhere (unlike the int8-activation profile), only the
 // order of the f32 additions differs from the CPU's, as for every MFMA kernel
 // (contract: native/metal/tm_metal.h:172-175, tolerance-qualified).
-// Non-finite activations give non-finite outputs, not necessarily the same
-// kind (inf - inf in the split).
+// An infinite or NaN activation goes into the first piece whole (the other two
+// are zero), so it reaches the outputs as it would through f32 products.
 //
 // Two kernels: split_act_list_kernel writes the three bf16 planes of every
 // distinct X of a launch once; gemm_bf16x3_kernel is LDS-staged like the int8 GEMM
-// (q8_gemm_i8_lds.hpp): a workgroup of WM x WN waves owns (WM*64 tokens) x
-// (WN*64 rows) of one K chunk of at most 1024 columns (a tile with a longer K
-// is the sum of its chunks' partial tiles, added in chunk order by whichever
-// chunk finishes last), walks K one Q8_0 block per stage, fetches every operand byte
-// once per workgroup as 16-byte pieces straight into LDS (a ring of four
-// stages, XOR-swizzled so that the operand reads are conflict-free) and each
-// wave computes a 64 x 64 tile as 2 x 2 MFMA tiles of 32 x 32.
+// (q8_gemm_i8_lds.hpp): a workgroup of WM x WN waves owns (WM*TM*32 tokens) x
+// (WN*64 rows) of one K chunk (a tile whose K is cut into chunks is the sum of
+// its chunks' partial tiles, added in chunk order by whichever chunk finishes
+// last), walks K one Q8_0 block per stage, fetches every operand byte once per
+// workgroup as 16-byte pieces straight into LDS (a ring of four stages,
+// XOR-swizzled so that the operand reads are conflict-free) and each wave
+// computes a (TM*32) x 64 tile as TM x 2 MFMA tiles of 32 x 32.
 #pragma once
 
 #include "q8_common.hpp"
@@ -75,8 +75,11 @@ __global__ __launch_bounds__(256) void split_act_list_kernel(const SplitArgs arg
     uint32_t h[4], m[4], l[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        const uint32_t hb = __builtin_bit_cast(uint32_t, in[e]) & 0xffff0000u;
-        const float r1 = in[e] - __builtin_bit_cast(float, hb); // exact
+        const uint32_t xb = __builtin_bit_cast(uint32_t, in[e]);
+        const bool finite = (xb & 0x7f800000u) != 0x7f800000u;
+        // (a NaN whose payload sits in the low 16 bits only must stay a NaN)
+        const uint32_t hb = finite ? xb & 0xffff0000u : xb | ((xb & 0xffffu) ? 0x00400000u : 0u);
+        const float r1 = finite ? in[e] - __builtin_bit_cast(float, hb) : 0.0f; // exact
         const uint32_t mb = __builtin_bit_cast(uint32_t, r1) & 0xffff0000u;
         const float r2 = r1 - __builtin_bit_cast(float, mb);    // exact, at most 8 significant bits
         h[e] = hb >> 16;
