@@ -186,10 +186,14 @@ def test_independent_mma_products_in_a_group_share_one_launch(ctx):
 
 @pytest.mark.parametrize("packed", [True, False])
 def test_a_large_mma_group_has_the_bits_of_its_products_alone(ctx, packed):
-    # Enough wave tiles in one launch for the work-queue kernel (a wave owns a
-    # tile over the whole of K and takes tiles from a device-side counter);
-    # each product alone has too few and runs the K-split kernels. Same bits,
-    # for K of 32, 33, 64 and 96 blocks, ragged rows and a ragged last token tile.
+    # Raw weights: enough wave tiles in one launch for the work-queue kernel (a
+    # wave owns a tile over the whole of K and takes tiles from a device-side
+    # counter); each product alone has too few and runs the K-split kernels.
+    # Sealed weights: the larger products run on the bf16 matrix cores (one
+    # launch splits their inputs, one multiplies), the others on the f32 ones,
+    # in runs of consecutive products of one kind. Same bits as alone either
+    # way, for K of 32, 33, 64 and 96 blocks, ragged rows and a ragged last
+    # token tile.
     shapes = [(4100, 1024, 500), (2048, 2048, 512), (1024, 3072, 512), (3000, 1056, 450),
               (4096, 1024, 512), (1024, 3072, 200)]
     mats = []
@@ -207,7 +211,12 @@ def test_a_large_mma_group_has_the_bits_of_its_products_alone(ctx, packed):
             ctx.q8_0_gemm_mma(wb, xb, yb, rows, cols, batch, 0, 0)
         ctx.end_group()
         ctx.fence()
-    assert ctx.kernel_launches() == launches + 2
+    per_group, prev = 0, None
+    for rows, cols, batch in shapes:
+        kind = "bf16" if packed and H.gemm_mma_on_bf16(rows, cols, batch) else "f32"
+        per_group += (2 if kind == "bf16" else 1) if kind != prev else 0
+        prev = kind
+    assert ctx.kernel_launches() == launches + 2 * per_group
     for i, (w, x, rows, cols, batch, wb, xb, yb) in enumerate(mats):
         grouped = yb.download_f32(0, batch * rows).copy()
         alone = run_gemm(ctx, ctx.q8_0_gemm_mma, wb, x, rows, cols, batch)

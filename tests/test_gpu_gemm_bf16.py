@@ -38,7 +38,7 @@ def product(ctx, wb, x, rows, cols, batch, x_off=0, y_off=0):
     return out
 
 
-# K of 1, 3, 32, 33 (two K chunks of 17 and 16 blocks), 36, 64 and 96 blocks;
+# K of 1, 3, 32 (whole, or two chunks of 16 blocks), 33 (17 + 16), 36, 64 and 96 blocks;
 # ragged rows; a ragged last token tile; the smallest batch of the kernel and
 # the largest; every product has at least 128 work units of its own.
 SHAPES = [(8192, 1024, 512), (33000, 96, M0), (8300, 1056, 500), (4096, 3072, 512),

@@ -107,7 +107,7 @@ struct Bx3Desc {
 };
 
 constexpr int BX3_MAX_DESCS = 64;
-constexpr uint32_t BX3_CHUNK_BLOCKS = 32;   // K is cut into chunks of 1024 columns or more
+constexpr uint32_t BX3_CHUNK_BLOCKS = 16;   // K is cut into chunks of 512 columns or more
 constexpr uint32_t BX3_MAX_SPLIT_TILES = 16384; // arrival counters per context
 
 struct Bx3Args {
@@ -483,16 +483,26 @@ inline uint64_t bx3_tiles(uint32_t rows, uint32_t batch) {
            ((rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS);
 }
 // Q8_0 blocks per K chunk of a product. A product with few output tiles cuts K
-// into chunks of 1024 columns and more, as many as it takes to give the chip
-// about BX3_UNITS_WANTED work units; one with many tiles does not cut K at all
-// (14336 x 4096 at 512 tokens: 295 TFLOP/s whole, less in chunks; chunks shorter
-// than 1024 columns made the 0.6B projections slower, alone and together). A function of the
-// product's shape only: its result does not depend on what shares its launch.
+// into at most BX3_MAX_CHUNKS chunks of 512 columns or more, as many as it takes
+// to give the chip about BX3_UNITS_WANTED work units; one with many tiles does
+// not cut K at all (14336 x 4096 at 512 tokens: 295 TFLOP/s whole, less in
+// chunks). Measured alone: chunks of 512 instead of 1024 columns make 6144 x 2048
+// at 256 tokens 47 us instead of 59 (f32 kernel: 69) and 8192 x 1024 at 512
+// tokens 49 instead of 56 (f32: 93). With eight chunks a product of 16 tiles is
+// about even with the f32 kernel alone (1024 x 4096 at 512 tokens: 52 against
+// 46 us, 2048 x 6144 at 256 tokens: 56 against 67) and far ahead in a group
+// (the Gemma FFN at 512 tokens: 145 us instead of 227 with its down projection
+// on the f32 kernel); chunks of 256 columns and less made the 0.6B projections
+// slower, alone and together. A
+// function of the product's shape only: its result does not depend on what
+// shares its launch.
 constexpr uint32_t BX3_UNITS_WANTED = 192;
+constexpr uint32_t BX3_MAX_CHUNKS = 8;
 inline uint32_t bx3_chunk_blocks(uint32_t rows, uint32_t cols, uint32_t batch) {
     const uint32_t blocks = cols / 32u;
     const uint64_t tiles = bx3_tiles(rows, batch);
-    const uint32_t most = (blocks + BX3_CHUNK_BLOCKS - 1u) / BX3_CHUNK_BLOCKS;
+    uint32_t most = (blocks + BX3_CHUNK_BLOCKS - 1u) / BX3_CHUNK_BLOCKS;
+    most = most < BX3_MAX_CHUNKS ? most : BX3_MAX_CHUNKS;
     const uint64_t want = (BX3_UNITS_WANTED + tiles - 1u) / tiles;
     const uint32_t chunks = want < most ? (uint32_t)want : most;
     return (blocks + chunks - 1u) / chunks;

@@ -32,11 +32,12 @@ GEMM_MMA_BF16_MIN_BATCH = 65
 
 def gemm_mma_bf16_units(rows: int, cols: int, batch: int) -> int:
     """Work units (128 tokens x 256 rows x one K chunk) the bf16 matrix-core GEMM
-    makes of a product: K is cut into chunks of 1024 columns or more, as many as
-    give about 192 units (mirror of q8::bx3_units, csrc/q8_gemm_bf16x3.hpp)."""
+    makes of a product: K is cut into at most eight chunks of 512 columns or more,
+    as many as give about 192 units (mirror of q8::bx3_units,
+    csrc/q8_gemm_bf16x3.hpp)."""
     tiles = -(-batch // 128) * -(-rows // 256)
     blocks = cols // 32
-    chunks = min(-(-192 // tiles), -(-blocks // 32))
+    chunks = min(-(-192 // tiles), -(-blocks // 16), 8)
     per_chunk = -(-blocks // chunks)
     return tiles * -(-blocks // per_chunk)
 
