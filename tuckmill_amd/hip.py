@@ -48,6 +48,8 @@ def gemm_mma_on_bf16(rows: int, cols: int, batch: int, x_off: int = 0) -> bool:
     on region sizes beyond 4 GiB are left out)."""
     return (batch >= GEMM_MMA_BF16_MIN_BATCH and x_off % 4 == 0 and
             gemm_mma_bf16_units(rows, cols, batch) >= 128)
+
+
 GEMM_I8_MAX_BATCH = 2048
 ARGMAX_NONE = 0xFFFFFFFF  # crates/metal/src/lib.rs (ARGMAX_NONE), native/metal/kernels.metal:143
 ARGMAX_PARTIAL_BYTES = 512
