@@ -582,8 +582,8 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
 // Sealed weights, every region below 4 GiB (32-bit buffer offsets): the caller
 // checks these before choosing this kernel. `partials` holds the sum of the
 // products' bx3_partial_floats() floats, `arrivals` BX3_MAX_SPLIT_TILES counters
-// that are zero between launches (both may be null when no product has more than
-// 1024 columns).
+// that are zero between launches (both may be null when no product's K is cut
+// into chunks).
 inline hipError_t launch_gemm_bf16x3_list(hipStream_t stream, hipEvent_t stop,
                                           const Bx3Product *prods, int n, float *partials,
                                           uint32_t *arrivals) {

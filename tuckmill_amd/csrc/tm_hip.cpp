@@ -100,7 +100,7 @@ struct tm_hip_ctx {
     hipStream_t copy_stream = nullptr;
     uint32_t *mma_queue = nullptr; // two counters of the work-queue MFMA kernel, zero between launches
     // Workspace of the bf16 split-float GEMM (split activations, partial tiles of
-    // products with K above 1024, their arrival counters): grown on demand, never
+    // products whose K is cut into chunks, their arrival counters): grown on demand, never
     // shrunk. A buffer that was outgrown stays allocated until the context goes:
     // recorded steps may still point at it.
     uint8_t *bx3_xs = nullptr;
