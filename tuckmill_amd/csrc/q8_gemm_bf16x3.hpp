@@ -297,8 +297,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16x3_kernel(const Bx3Args
         row_odd[j] = (n * blocks) & 1u;
     }
 
-    // MFMA step m (k = 16m .. 16m+15) takes from lane (idx, half) the 8 values
-    // k = 16m + 8*half + 0..7 of token / weight row idx.
+    // MFMA step m takes from lane (idx, half) the 8 values k = 16*half + 8m + 0..7
+    // of token / weight row idx (any assignment of a block's 32 k to the two
+    // steps' lanes does, as long as both operands use it): a lane's 16 quants of
+    // a weight row are then one 16-byte piece, read in one go.
     auto compute = [&](const uint8_t *stage, uint32_t kb) {
         const uint32_t *sdw = (const uint32_t *)(stage + Sh::a_bytes + Sh::b_bytes);
         const uint8_t *sb = stage + Sh::a_bytes;
@@ -307,11 +309,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16x3_kernel(const Bx3Args
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const uint32_t r = wn * 64u + 32u * j + idx;
-#pragma unroll
-            for (int m = 0; m < 2; ++m) {
-                const uint32_t slot = (uint32_t)m ^ ((r >> 3) & 1u);
-                const u32x2 raw = *(const u32x2 *)(sb + r * 32u + slot * 16u + half * 8u);
-                b[j][m] = sbytes_to_bf16x8(raw.x, raw.y);
+            {
+                const uint32_t slot = half ^ ((r >> 3) & 1u);
+                const u32x4 raw = *(const u32x4 *)(sb + r * 32u + slot * 16u);
+                b[j][0] = sbytes_to_bf16x8(raw.x, raw.y);
+                b[j][1] = sbytes_to_bf16x8(raw.z, raw.w);
             }
             {
                 const uint32_t pair = sdw[r];
@@ -326,7 +328,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16x3_kernel(const Bx3Args
             for (int pl = 0; pl < 3; ++pl) {
 #pragma unroll
                 for (int m = 0; m < 2; ++m) {
-                    const uint32_t slot = (uint32_t)(2 * m + (int)half) ^ ((r >> 2) & 3u);
+                    const uint32_t slot = (2u * half + (uint32_t)m) ^ ((r >> 2) & 3u);
                     a[pl][m] = *(const bf16x8_t *)(stage + pl * Sh::a_plane + r * 64u + slot * 16u);
                 }
             }
