@@ -190,8 +190,8 @@ def test_a_large_mma_group_has_the_bits_of_its_products_alone(ctx, packed):
     # wave owns a tile over the whole of K and takes tiles from a device-side
     # counter); each product alone has too few and runs the K-split kernels.
     # Sealed weights: the larger products run on the bf16 matrix cores (one
-    # launch splits their inputs, one multiplies), the others on the f32 ones,
-    # in runs of consecutive products of one kind. Same bits as alone either
+    # launch splits their inputs, one multiplies; tiles of 128 or of 64 tokens),
+    # the others on the f32 ones, one launch per kernel. Same bits as alone either
     # way, for K of 32, 33, 64 and 96 blocks, ragged rows and a ragged last
     # token tile.
     shapes = [(4100, 1024, 500), (2048, 2048, 512), (1024, 3072, 512), (3000, 1056, 450),
@@ -211,11 +211,11 @@ def test_a_large_mma_group_has_the_bits_of_its_products_alone(ctx, packed):
             ctx.q8_0_gemm_mma(wb, xb, yb, rows, cols, batch, 0, 0)
         ctx.end_group()
         ctx.fence()
-    per_group, prev = 0, None
+    kinds = set()  # one launch per kernel (two on the bf16 cores), whatever the order
     for rows, cols, batch in shapes:
-        kind = "bf16" if packed and H.gemm_mma_on_bf16(rows, cols, batch) else "f32"
-        per_group += (2 if kind == "bf16" else 1) if kind != prev else 0
-        prev = kind
+        on_bf16 = packed and H.gemm_mma_on_bf16(rows, cols, batch)
+        kinds.add(("bf16", H.gemm_mma_bf16_plan(rows, cols, batch)[0]) if on_bf16 else "f32")
+    per_group = sum(1 if kind == "f32" else 2 for kind in kinds)
     assert ctx.kernel_launches() == launches + 2 * per_group
     for i, (w, x, rows, cols, batch, wb, xb, yb) in enumerate(mats):
         grouped = yb.download_f32(0, batch * rows).copy()

@@ -6,29 +6,41 @@ from tuckmill_amd import synth as S
 
 
 def test_work_units_of_the_bf16_gemm():
+    plan = H.gemm_mma_bf16_plan
     # tiles of 128 tokens x 256 rows; K whole when the tiles alone give 192 units
-    assert H.gemm_mma_bf16_units(14336, 4096, 512) == 4 * 56
+    assert plan(14336, 4096, 512) == (128, 4 * 56, True)
     # else in chunks of 512 columns or more, at most eight, about 192 units
-    assert H.gemm_mma_bf16_units(6144, 2048, 512) == 4 * 24 * 2
-    assert H.gemm_mma_bf16_units(2048, 6144, 512) == 4 * 8 * 6
-    assert H.gemm_mma_bf16_units(1024, 4096, 512) == 4 * 4 * 8
-    assert H.gemm_mma_bf16_units(1024, 1024, 512) == 4 * 4 * 2
-    assert H.gemm_mma_bf16_units(33000, 96, 65) == 129
+    assert plan(6144, 2048, 512) == (128, 4 * 24 * 2, True)
+    assert plan(2048, 6144, 512) == (128, 4 * 8 * 6, True)
     # 33 blocks in two chunks of 17 and 16
-    assert H.gemm_mma_bf16_units(8300, 1056, 500) == 4 * 33 * 2
+    assert plan(8300, 1056, 500) == (128, 4 * 33 * 2, True)
+    # fewer than 192 such units: tiles of 64 tokens, if 4 chunks are enough ...
+    assert plan(4096, 1024, 512) == (64, 8 * 16 * 2, True)
+    assert plan(2048, 2048, 512) == (64, 8 * 8 * 3, True)
+    assert plan(33000, 96, 65) == (64, 2 * 129, True)
+    # ... else the large tile with 128 units or more, or none
+    assert plan(1024, 4096, 512) == (128, 4 * 4 * 8, True)
+    assert plan(1152, 6912, 512) == (128, 4 * 5 * 8, True)
+    assert plan(1024, 3072, 512) == (128, 4 * 4 * 6, False)
+    assert plan(1024, 1024, 512) == (128, 4 * 4 * 2, False)
 
 
 def test_which_products_take_the_bf16_matrix_cores():
-    # the 0.6B projections are too small on their own at any batch ...
-    for _, rows, cols in S.QWEN3_0_6B_LAYER:
-        assert not H.gemm_mma_on_bf16(rows, cols, 512)
-    # ... the vocabulary projections and the 2B-class FFN are not
+    # the 0.6B attention and down projections are too small on their own,
+    # the vocabulary projections and the 2B-class FFN are not
+    for name, rows, cols in S.QWEN3_0_6B_LAYER:
+        if name in ("q", "k", "v", "o", "down"):
+            assert not H.gemm_mma_on_bf16(rows, cols, 512)
     _, rows, cols = S.QWEN3_0_6B_LM_HEAD
     assert H.gemm_mma_on_bf16(rows, cols, H.GEMM_MMA_BF16_MIN_BATCH)
     assert not H.gemm_mma_on_bf16(rows, cols, H.GEMM_MMA_BF16_MIN_BATCH - 1)
     for _, rows, cols in S.SWEEP_2B:
         assert H.gemm_mma_on_bf16(rows, cols, 256)
-        assert not H.gemm_mma_on_bf16(rows, cols, 128)
+    # 192 units of the small tile in at most 4 chunks are the least that pays: q
+    # (128 units) and down (6 chunks) stay on the f32 kernels, gate and up do not
+    assert not H.gemm_mma_on_bf16(2048, 1024, 512)
+    assert not H.gemm_mma_on_bf16(1024, 3072, 512)
+    assert H.gemm_mma_on_bf16(3072, 1024, 512)
     # activations must start on a 16-byte boundary
     assert not H.gemm_mma_on_bf16(8192, 1024, 512, x_off=3)
     assert H.gemm_mma_on_bf16(8192, 1024, 512, x_off=32)

@@ -476,63 +476,89 @@ struct Bx3Product {
     uint32_t rows, cols, batch;
 };
 
-// The workgroup tile: 128 tokens x 256 rows (2 x 4 waves).
-constexpr uint32_t BX3_TILE_TOKENS = 128;
+// How a product is cut into work units (output tile x K chunk). A function of
+// the product's shape only: its result does not depend on what shares its launch.
+//
+// Tile: 256 rows x 128 tokens (2 x 4 waves, two per SIMD), or x 64 tokens (1 x 4
+// waves, one per SIMD) for some products that would make fewer than 192 units
+// of the large tile (bx3_plan below). Measured alone, the small tile is 1.1-1.6 times as fast on such
+// products (4096 x 1024 at 512 tokens: 35 against 40 us, 6144 x 2048 at 128
+// tokens: 33 us against 48 on the f32 kernel) and 10-25 % slower on large ones
+// (a quarter more operand bytes per product).
+//
+// K chunks: a product with few output tiles cuts K into at most BX3_MAX_CHUNKS
+// chunks of 512 columns or more, as many as it takes to give the chip about
+// BX3_UNITS_WANTED work units; one with many tiles does not cut K at all
+// (14336 x 4096 at 512 tokens: 295 TFLOP/s whole, less in chunks). Measured
+// alone with the large tile: chunks of 512 instead of 1024 columns make
+// 6144 x 2048 at 256 tokens 47 us instead of 59 (f32 kernel: 69) and 8192 x 1024
+// at 512 tokens 49 instead of 56 (f32: 93); chunks of 256 columns and less made
+// the 0.6B projections slower, alone and together.
 constexpr uint32_t BX3_TILE_ROWS = 256;
-
-inline uint64_t bx3_tiles(uint32_t rows, uint32_t batch) {
-    return (uint64_t)((batch + BX3_TILE_TOKENS - 1u) / BX3_TILE_TOKENS) *
-           ((rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS);
-}
-// Q8_0 blocks per K chunk of a product. A product with few output tiles cuts K
-// into at most BX3_MAX_CHUNKS chunks of 512 columns or more, as many as it takes
-// to give the chip about BX3_UNITS_WANTED work units; one with many tiles does
-// not cut K at all (14336 x 4096 at 512 tokens: 295 TFLOP/s whole, less in
-// chunks). Measured alone: chunks of 512 instead of 1024 columns make 6144 x 2048
-// at 256 tokens 47 us instead of 59 (f32 kernel: 69) and 8192 x 1024 at 512
-// tokens 49 instead of 56 (f32: 93). With eight chunks a product of 16 tiles is
-// about even with the f32 kernel alone (1024 x 4096 at 512 tokens: 52 against
-// 46 us, 2048 x 6144 at 256 tokens: 56 against 67) and far ahead in a group
-// (the Gemma FFN at 512 tokens: 145 us instead of 227 with its down projection
-// on the f32 kernel); chunks of 256 columns and less made the 0.6B projections
-// slower, alone and together. A
-// function of the product's shape only: its result does not depend on what
-// shares its launch.
 constexpr uint32_t BX3_UNITS_WANTED = 192;
 constexpr uint32_t BX3_MAX_CHUNKS = 8;
-inline uint32_t bx3_chunk_blocks(uint32_t rows, uint32_t cols, uint32_t batch) {
+
+struct Bx3Plan {
+    uint32_t tile_tokens;  // 128 or 64
+    uint32_t chunk_blocks; // Q8_0 blocks per K chunk
+    uint32_t chunks;
+    uint64_t tiles;        // output tiles
+    uint64_t units;        // tiles x chunks
+    uint64_t split_tiles;  // tiles that need an arrival counter (chunks > 1)
+    uint64_t partial_floats; // floats of partial tiles (chunks > 1)
+};
+
+inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint32_t tile_tokens) {
+    Bx3Plan p;
+    p.tile_tokens = tile_tokens;
     const uint32_t blocks = cols / 32u;
-    const uint64_t tiles = bx3_tiles(rows, batch);
+    p.tiles = (uint64_t)((batch + tile_tokens - 1u) / tile_tokens) *
+              ((rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS);
     uint32_t most = (blocks + BX3_CHUNK_BLOCKS - 1u) / BX3_CHUNK_BLOCKS;
     most = most < BX3_MAX_CHUNKS ? most : BX3_MAX_CHUNKS;
-    const uint64_t want = (BX3_UNITS_WANTED + tiles - 1u) / tiles;
+    const uint64_t want = (BX3_UNITS_WANTED + p.tiles - 1u) / p.tiles;
     const uint32_t chunks = want < most ? (uint32_t)want : most;
-    return (blocks + chunks - 1u) / chunks;
+    p.chunk_blocks = (blocks + chunks - 1u) / chunks;
+    p.chunks = (blocks + p.chunk_blocks - 1u) / p.chunk_blocks;
+    p.units = p.tiles * p.chunks;
+    p.split_tiles = p.chunks > 1u ? p.tiles : 0u;
+    p.partial_floats = p.split_tiles * p.chunks * tile_tokens * BX3_TILE_ROWS;
+    return p;
 }
-// Work units (output tile x K chunk) of a product.
-inline uint64_t bx3_units(uint32_t rows, uint32_t cols, uint32_t batch);
-inline uint32_t bx3_chunks(uint32_t rows, uint32_t cols, uint32_t batch) {
-    const uint32_t cb = bx3_chunk_blocks(rows, cols, batch);
-    return (cols / 32u + cb - 1u) / cb;
+
+// The plan of a product, and whether the kernel pays for it on its own
+// (`worth`). In order of preference: the large tile with 192 units or more; the
+// small tile with 192 units or more in at most 4 K chunks (1024 x 3072 at 512
+// tokens in six chunks: 40 us against 32 on the f32 kernel); the large tile with
+// 128 units or more (alone about even with the f32 kernel, far ahead when
+// products share a launch). Measured alone at 512 tokens against the f32
+// kernel: small tile 3072 x 1024 34 against 35 us, 2048 x 2048 39 against 49,
+// 4096 x 1024 36 against 48, 2048 x 1024 (128 units) 31 against 28; large tile
+// 8192 x 1024 49 against 93, 6144 x 2048 69 against 133.
+inline Bx3Plan bx3_plan(uint32_t rows, uint32_t cols, uint32_t batch, bool *worth) {
+    const Bx3Plan large = bx3_plan_with(rows, cols, batch, 128u);
+    if (large.units >= BX3_UNITS_WANTED) {
+        *worth = true;
+        return large;
+    }
+    const Bx3Plan small = bx3_plan_with(rows, cols, batch, 64u);
+    if (small.units >= BX3_UNITS_WANTED && small.chunks <= 4u) {
+        *worth = true;
+        return small;
+    }
+    *worth = large.units >= 128u;
+    return large;
 }
-inline uint64_t bx3_units(uint32_t rows, uint32_t cols, uint32_t batch) {
-    return bx3_tiles(rows, batch) * bx3_chunks(rows, cols, batch);
-}
-// Tiles of a product that need an arrival counter, and the floats of partial
-// tiles it needs (none for a single chunk).
-inline uint64_t bx3_split_tiles(uint32_t rows, uint32_t cols, uint32_t batch) {
-    return bx3_chunks(rows, cols, batch) > 1u ? bx3_tiles(rows, batch) : 0u;
-}
-inline uint64_t bx3_partial_floats(uint32_t rows, uint32_t cols, uint32_t batch) {
-    return bx3_split_tiles(rows, cols, batch) * bx3_chunks(rows, cols, batch) * BX3_TILE_TOKENS *
-           BX3_TILE_ROWS;
+inline Bx3Plan bx3_plan(uint32_t rows, uint32_t cols, uint32_t batch) {
+    bool worth;
+    return bx3_plan(rows, cols, batch, &worth);
 }
 
 template <int WM, int WN, int TM>
 inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3Product *prods_in,
                                  int n, float *partials, uint32_t *arrivals) {
     using Sh = Bx3Shape<WM, WN, TM>;
-    static_assert(Sh::rows == (int)BX3_TILE_ROWS && Sh::tokens == (int)BX3_TILE_TOKENS, "tile");
+    static_assert(Sh::rows == (int)BX3_TILE_ROWS, "tile");
     Bx3Args args;
     args.n = (uint32_t)n;
     args.partials = partials;
@@ -557,9 +583,13 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
         d.cols = prods[i].cols;
         d.batch = prods[i].batch;
         d.tile_begin = (uint32_t)units;
+        const Bx3Plan plan = bx3_plan(prods[i].rows, prods[i].cols, prods[i].batch);
+        if (plan.tile_tokens != (uint32_t)Sh::tokens) {
+            return hipErrorInvalidValue; // the caller lists products of one tile shape
+        }
         d.tiles_t = (prods[i].batch + Sh::tokens - 1) / Sh::tokens;
-        d.chunk_blocks = bx3_chunk_blocks(prods[i].rows, prods[i].cols, prods[i].batch);
-        d.chunks = bx3_chunks(prods[i].rows, prods[i].cols, prods[i].batch);
+        d.chunk_blocks = plan.chunk_blocks;
+        d.chunks = plan.chunks;
         d.part_begin = (uint32_t)split_tiles;
         d.part_tile = (uint32_t)partial_tiles;
         const uint64_t tiles = (uint64_t)d.tiles_t * ((prods[i].rows + Sh::rows - 1) / Sh::rows);
@@ -581,18 +611,22 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
     return hipGetLastError();
 }
 
-// Sealed weights, every region below 4 GiB (32-bit buffer offsets): the caller
-// checks these before choosing this kernel. `partials` holds the sum of the
-// products' bx3_partial_floats() floats, `arrivals` BX3_MAX_SPLIT_TILES counters
-// that are zero between launches (both may be null when no product's K is cut
-// into chunks).
-inline hipError_t launch_gemm_bf16x3_list(hipStream_t stream, hipEvent_t stop,
+// Sealed weights, every region below 4 GiB (32-bit buffer offsets), every
+// product's plan with `tile_tokens`: the caller checks these before choosing
+// this kernel. `partials` holds the sum of the products' partial_floats,
+// `arrivals` BX3_MAX_SPLIT_TILES counters that are zero between launches (both
+// may be null when no product's K is cut into chunks).
+inline hipError_t launch_gemm_bf16x3_list(hipStream_t stream, hipEvent_t stop, uint32_t tile_tokens,
                                           const Bx3Product *prods, int n, float *partials,
                                           uint32_t *arrivals) {
     if (n <= 0 || n > BX3_MAX_DESCS) {
         return hipErrorInvalidValue;
     }
-    return launch_bx3_cfg<2, 4, 2>(stream, stop, prods, n, partials, arrivals);
+    switch (tile_tokens) {
+    case 128: return launch_bx3_cfg<2, 4, 2>(stream, stop, prods, n, partials, arrivals);
+    case 64: return launch_bx3_cfg<1, 4, 2>(stream, stop, prods, n, partials, arrivals);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 struct SplitInput {

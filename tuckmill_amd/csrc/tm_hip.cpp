@@ -281,7 +281,8 @@ enum Variant : uint8_t {
     V_GENERAL,    // gemv_list_kernel, four tokens per pass (raw layout / narrow small batches)
     V_SPLIT,      // gemm_split_list_kernel: p0 = waves, p1 = tokens per wave, p2 = column tail
     V_MMA,        // f32 MFMA GEMM: p0 = tmw, p1 = tnw, p2 = K split
-    V_BF16X3,     // prefill GEMM on the bf16 matrix cores, activations split in three
+    V_BF16X3,     // prefill GEMM on the bf16 matrix cores, activations split in three:
+                  // p0 = tokens per tile / 64
     V_I8_TILE,    // register-fed int8 MFMA GEMM: p0 = tile configuration
     V_I8_STREAM,  // int8 streaming kernel: p0 = tokens per pass
     V_I8_LDS,     // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (q8::i8_lds_shape)
@@ -303,29 +304,29 @@ struct GemvKey {
 };
 
 // Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 65
-// tokens, and with at least 128 work units of 128 tokens x 256 rows (x K chunk)
-// of their own. The kernel is two to three times as fast as the f32 one when it
-// fills the chip (at 512 tokens 14336 x 4096: 204 us against 640 us, 6144 x 2048:
-// 69 against 133; at 96 tokens 14336 x 4096: 73 against 173) but its units are
-// large: 1024 x 1024 at 512 tokens takes 48 us against 15 us, and 33 us with K in
-// four chunks. Measured alone at 512 tokens: 64 units 52 against 49 us, 128 units
-// 57 against 94 us (K = 1024), 66 against 91 us (K = 4096); at 64 tokens and
-// below the f32 kernels win or tie on most shapes. A product's kernel depends on
-// nothing but its own shape and alignment, so its result does not depend on
-// what shares its launch (the seven 0.6B projections together would take 78 us
-// instead of 144 us on this kernel, and 359 us instead of 183 us one by one).
+// tokens, and with enough work units (256 rows x 128 or 64 tokens x K chunk)
+// of their own for the kernel to pay (q8::bx3_plan has the rule and the
+// measurements behind it). The kernel is two to three times as fast as the f32
+// one when it fills the chip (at 512 tokens 14336 x 4096: 204 us against 640 us,
+// 6144 x 2048: 69 against 133; at 96 tokens 14336 x 4096: 73 against 173) but its
+// units are large: 1024 x 1024 at 512 tokens takes 48 us against 15 us, and 33 us
+// with K in four chunks; at 64 tokens and below the f32 kernels win or tie on
+// most shapes. A product's kernel depends on nothing but its own shape and
+// alignment, so its result does not depend on what shares its launch.
 constexpr uint32_t kBx3MinBatch = 65;
-constexpr uint64_t kBx3MinUnits = 128;
 constexpr uint64_t kBx3MaxPartialFloats = 1ull << 29; // 2 GiB of partial tiles per launch
 
 bool bx3_eligible(const Op &op, bool x_aligned) {
-    return op.packed && x_aligned && op.batch >= kBx3MinBatch &&
-           q8::bx3_units(op.rows, op.cols, op.batch) >= kBx3MinUnits &&
-           (uint64_t)op.rows * op.cols < (1ull << 32) &&
-           (uint64_t)op.batch * op.cols * 6u < (1ull << 32) &&
-           (uint64_t)op.batch * op.cols < (1ull << 30) &&
-           q8::bx3_split_tiles(op.rows, op.cols, op.batch) <= q8::BX3_MAX_SPLIT_TILES &&
-           q8::bx3_partial_floats(op.rows, op.cols, op.batch) <= kBx3MaxPartialFloats;
+    if (!op.packed || !x_aligned || op.batch < kBx3MinBatch ||
+        (uint64_t)op.rows * op.cols >= (1ull << 32) ||
+        (uint64_t)op.batch * op.cols * 6u >= (1ull << 32) ||
+        (uint64_t)op.batch * op.cols >= (1ull << 30)) {
+        return false;
+    }
+    bool worth = false;
+    const q8::Bx3Plan plan = q8::bx3_plan(op.rows, op.cols, op.batch, &worth);
+    return worth && plan.split_tiles <= q8::BX3_MAX_SPLIT_TILES &&
+           plan.partial_floats <= kBx3MaxPartialFloats;
 }
 
 GemvKey gemv_key(const Op &op) {
@@ -359,6 +360,7 @@ GemvKey gemv_key(const Op &op) {
     k.flag = (xp % 16u == 0);
     if (op.kind == OP_MMA && bx3_eligible(op, k.flag)) {
         k.variant = V_BF16X3;
+        k.p0 = (uint8_t)(q8::bx3_plan(op.rows, op.cols, op.batch).tile_tokens / 64u); // 2 or 1
         return k;
     }
     if (op.kind == OP_MMA) {
@@ -531,8 +533,8 @@ hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launc
     if (e != hipSuccess) {
         return e;
     }
-    return q8::launch_gemm_bf16x3_list(ctx->stream, stop, prods, n, ctx->bx3_partials,
-                                       ctx->bx3_arrivals);
+    return q8::launch_gemm_bf16x3_list(ctx->stream, stop, launch.key.p0 * 64u, prods, n,
+                                       ctx->bx3_partials, ctx->bx3_arrivals);
 }
 
 // Kernel launches a planned launch stands for.
@@ -828,10 +830,17 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
 std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
     std::vector<Launch> plan;
     Launch cur;
+    // Open prefill launches set aside while a product of another kernel is
+    // listed (see below); closed together with `cur`.
+    std::vector<Launch> parked;
     // Hazards are tracked per allocation with an epoch stamp, so planning a
     // step of n products costs O(n), not O(n^2).
     uint64_t epoch = ++ctx->plan_epoch;
     auto flush = [&]() {
+        for (Launch &l : parked) {
+            plan.push_back(std::move(l));
+        }
+        parked.clear();
         if (cur.norm != nullptr) {
             bool used = false;
             for (bool b : cur.normed) {
@@ -877,6 +886,23 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             if (op.a[3] != nullptr) {
                 conflict = conflict || op.a[3]->read_epoch == epoch || op.a[3]->write_epoch == epoch;
             }
+            // The prefill products of a layer alternate between kernels (f32 and
+            // bf16 matrix cores, tile shapes). As long as nothing depends on
+            // anything since the last closed launch, each kernel keeps one
+            // open launch: the open one is set aside, not closed, when a
+            // product of another kernel arrives, and taken up again later.
+            if (key.kind == OP_MMA && !conflict && cur.norm == nullptr && !cur.list.empty() &&
+                cur.key.kind == OP_MMA && !(key == cur.key)) {
+                parked.push_back(std::move(cur));
+                cur = Launch();
+                for (size_t i = 0; i < parked.size(); ++i) {
+                    if (parked[i].key == key) {
+                        cur = std::move(parked[i]);
+                        parked.erase(parked.begin() + (long)i);
+                        break;
+                    }
+                }
+            }
             const bool open = !cur.list.empty() || cur.norm != nullptr;
             bool new_input = true;
             if (key.variant == V_BF16X3 && !cur.list.empty() && key == cur.key) {
@@ -884,12 +910,10 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                     new_input = new_input && !same_input(*other, op);
                 }
                 // the launch's share of the workspace stays within its limits
+                const q8::Bx3Plan mine = q8::bx3_plan(op.rows, op.cols, op.batch);
                 conflict = conflict ||
-                           cur.bx3_split_tiles + q8::bx3_split_tiles(op.rows, op.cols, op.batch) >
-                               q8::BX3_MAX_SPLIT_TILES ||
-                           cur.bx3_partial_floats +
-                                   q8::bx3_partial_floats(op.rows, op.cols, op.batch) >
-                               kBx3MaxPartialFloats ||
+                           cur.bx3_split_tiles + mine.split_tiles > q8::BX3_MAX_SPLIT_TILES ||
+                           cur.bx3_partial_floats + mine.partial_floats > kBx3MaxPartialFloats ||
                            (new_input && cur.bx3_inputs == q8::SPLIT_MAX_DESCS);
             }
             if (open && (conflict || (!cur.list.empty() && !(key == cur.key)) ||
@@ -898,8 +922,9 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 new_input = true;
             }
             if (key.variant == V_BF16X3) {
-                cur.bx3_split_tiles += q8::bx3_split_tiles(op.rows, op.cols, op.batch);
-                cur.bx3_partial_floats += q8::bx3_partial_floats(op.rows, op.cols, op.batch);
+                const q8::Bx3Plan mine = q8::bx3_plan(op.rows, op.cols, op.batch);
+                cur.bx3_split_tiles += mine.split_tiles;
+                cur.bx3_partial_floats += mine.partial_floats;
                 if (new_input) {
                     cur.bx3_inputs += 1;
                     cur.bx3_xs_bytes += bx3_xs_bytes_of(op);

@@ -30,16 +30,27 @@ GEMM_MMA_MAX_BATCH = 512
 GEMM_MMA_BF16_MIN_BATCH = 65
 
 
-def gemm_mma_bf16_units(rows: int, cols: int, batch: int) -> int:
-    """Work units (128 tokens x 256 rows x one K chunk) the bf16 matrix-core GEMM
-    makes of a product: K is cut into at most eight chunks of 512 columns or more,
-    as many as give about 192 units (mirror of q8::bx3_units,
-    csrc/q8_gemm_bf16x3.hpp)."""
-    tiles = -(-batch // 128) * -(-rows // 256)
-    blocks = cols // 32
-    chunks = min(-(-192 // tiles), -(-blocks // 16), 8)
-    per_chunk = -(-blocks // chunks)
-    return tiles * -(-blocks // per_chunk)
+def gemm_mma_bf16_plan(rows: int, cols: int, batch: int):
+    """(tokens per tile, work units, worth it) for the bf16 matrix-core GEMM on a
+    product. A unit is 256 rows x 128 or 64 tokens x one K chunk; K is cut into
+    at most eight chunks of 512 columns or more, as many as give about 192
+    units. In order of preference: the large tile with 192 units or more, the
+    small tile with 192 units or more in at most 4 chunks, the large tile with
+    128 units or more (mirror of q8::bx3_plan, csrc/q8_gemm_bf16x3.hpp)."""
+    def plan(tokens):
+        tiles = -(-batch // tokens) * -(-rows // 256)
+        blocks = cols // 32
+        chunks = min(-(-192 // tiles), -(-blocks // 16), 8)
+        per_chunk = -(-blocks // chunks)
+        chunks = -(-blocks // per_chunk)
+        return tiles * chunks, chunks
+    large, _ = plan(128)
+    if large >= 192:
+        return 128, large, True
+    small, chunks = plan(64)
+    if small >= 192 and chunks <= 4:
+        return 64, small, True
+    return 128, large, large >= 128
 
 
 def gemm_mma_on_bf16(rows: int, cols: int, batch: int, x_off: int = 0) -> bool:
@@ -47,7 +58,7 @@ def gemm_mma_on_bf16(rows: int, cols: int, batch: int, x_off: int = 0) -> bool:
     kernel for this product (mirror of bx3_eligible, csrc/tm_hip.cpp; the limits
     on region sizes beyond 4 GiB are left out)."""
     return (batch >= GEMM_MMA_BF16_MIN_BATCH and x_off % 4 == 0 and
-            gemm_mma_bf16_units(rows, cols, batch) >= 128)
+            gemm_mma_bf16_plan(rows, cols, batch)[2])
 
 
 GEMM_I8_MAX_BATCH = 2048
