@@ -171,7 +171,9 @@ def bench_gemm(host, ctx, steps, warmup):
         ms = t.gpu_ms / steps
         ms_sum += ms
         out["shapes"].append({"name": name, "rows": rows, "cols": cols, "us": ms * 1e3,
-                              "tflops": 2.0 * M * rows * cols / (ms * 1e-3) / 1e12})
+                              "tflops": 2.0 * M * rows * cols / (ms * 1e-3) / 1e12,
+                              "matrix_cores": "bf16 x3" if H.gemm_mma_on_bf16(rows, cols, M)
+                              else "f32"})
     t = run_steps(host, ctx, products, warmup, steps, grouped=True)
     ms_group = t.gpu_ms / steps
     out["one_commit_per_product"] = {"us": ms_sum * 1e3,
@@ -183,7 +185,11 @@ def bench_gemm(host, ctx, steps, warmup):
     out["flops_per_step"] = flops_total
     out["mfma_f32_peak_tflops"] = MFMA_F32_PEAK_TFLOPS
     out["frac"] = out["tflops"] / MFMA_F32_PEAK_TFLOPS
-    out["kernel"] = "q8::gemm_mma_persistent_kernel"
+    on_bf16 = [n for n, r, c in S.QWEN3_0_6B_LAYER if H.gemm_mma_on_bf16(r, c, M)]
+    out["kernel"] = ("q8::gemm_mma_persistent_kernel (f32 matrix cores)" +
+                     (f"; q8::gemm_bf16x3_kernel for {', '.join(on_bf16)} (large enough on their "
+                      "own for the bf16 matrix cores, three exact bf16 pieces per activation)"
+                      if on_bf16 else ""))
     # The same model's vocabulary projection at M = 512: large enough on its own
     # for the kernel that runs on the bf16 matrix cores (every f32 activation
     # split into three exact bf16 pieces, so the products stay exact).
