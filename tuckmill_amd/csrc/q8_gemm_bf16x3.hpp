@@ -146,19 +146,16 @@ __device__ __forceinline__ bf16x8_t sbytes_to_bf16x8(uint32_t lo, uint32_t hi) {
     return __builtin_bit_cast(bf16x8_t, v);
 }
 
-template <int WM, int WN, int TM>
+template <int WM, int WN, int TM, int NS>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16x3_kernel(const Bx3Args args) {
     using Sh = Bx3Shape<WM, WN, TM>;
     constexpr int NW = WM * WN;
     constexpr int TN = 2; // a wave computes TM x 2 tiles of 32 x 32: 32*TM tokens x 64 rows
-    // A ring of four stage buffers, separate objects so that reads of one
-    // provably do not alias the fetches into the others: three blocks are in
-    // flight while one is being used (a fetch takes about three stages' worth
-    // of MFMAs to arrive).
-    __shared__ __attribute__((aligned(16))) uint8_t stage_0[Sh::stage_bytes];
-    __shared__ __attribute__((aligned(16))) uint8_t stage_1[Sh::stage_bytes];
-    __shared__ __attribute__((aligned(16))) uint8_t stage_2[Sh::stage_bytes];
-    __shared__ __attribute__((aligned(16))) uint8_t stage_3[Sh::stage_bytes];
+    // A ring of NS stage buffers: NS - 1 blocks are in flight while one is being
+    // used (a fetch takes about three stages' worth of MFMAs to arrive on the
+    // large tile, with one workgroup per CU; the small tile runs two workgroups
+    // per CU with three buffers each).
+    __shared__ __attribute__((aligned(16))) uint8_t stage_mem[NS][Sh::stage_bytes];
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -352,40 +349,34 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bf16x3_kernel(const Bx3Args
     };
 
     // Every wave issues the same number of fetch instructions per block, so
-    // "all but the newest two blocks have landed" is one counter value.
+    // "all but the newest NS - 2 blocks have landed" is one counter value.
     constexpr int F = NA + NB + 1;
     static_assert((3 * Sh::tokens / 16) % NW == 0 && (Sh::rows / 32) % NW == 0, "uniform fetch");
-    constexpr int WAIT_TWO_BLOCKS = ((2 * F) & 15) | (((2 * F) >> 4) << 14) | (7 << 4) | (15 << 8);
+    constexpr int IN_FLIGHT = (NS - 2) * F; // fetches of the newest NS - 2 blocks
+    static_assert(IN_FLIGHT < 64, "vmcnt field");
+    constexpr int WAIT_OLDEST_BLOCK =
+        (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14) | (7 << 4) | (15 << 8);
     auto landed = [&]() {
         // this wave's fetch of the block about to be used is complete ...
-        __builtin_amdgcn_s_waitcnt(WAIT_TWO_BLOCKS);
+        __builtin_amdgcn_s_waitcnt(WAIT_OLDEST_BLOCK);
         // ... everybody's is, and everybody is done with the previous block's buffer
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
     auto at = [&](uint32_t kb) { return kb < kb_last ? kb : kb_last - 1u; };
-    fetch(at(kb_first), stage_0);
-    fetch(at(kb_first + 1u), stage_1);
-    fetch(at(kb_first + 2u), stage_2);
-    for (uint32_t kb = kb_first; kb < kb_last; kb += 4u) {
-        landed();
-        fetch(at(kb + 3u), stage_3);
-        compute(stage_0, kb);
-        if (kb + 1u < kb_last) {
-            landed();
-            fetch(at(kb + 4u), stage_0);
-            compute(stage_1, kb + 1u);
-        }
-        if (kb + 2u < kb_last) {
-            landed();
-            fetch(at(kb + 5u), stage_1);
-            compute(stage_2, kb + 2u);
-        }
-        if (kb + 3u < kb_last) {
-            landed();
-            fetch(at(kb + 6u), stage_2);
-            compute(stage_3, kb + 3u);
+#pragma unroll
+    for (int u = 0; u < NS - 1; ++u) {
+        fetch(at(kb_first + (uint32_t)u), stage_mem[u]);
+    }
+    for (uint32_t kb = kb_first; kb < kb_last; kb += (uint32_t)NS) {
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+            if (kb + (uint32_t)u < kb_last) { // (uniform over the workgroup)
+                landed();
+                fetch(at(kb + (uint32_t)(u + NS - 1)), stage_mem[(u + NS - 1) % NS]);
+                compute(stage_mem[u], kb + (uint32_t)u);
+            }
         }
     }
     __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); // vmcnt(0): every fetch has landed
@@ -554,7 +545,7 @@ inline Bx3Plan bx3_plan(uint32_t rows, uint32_t cols, uint32_t batch) {
     return bx3_plan(rows, cols, batch, &worth);
 }
 
-template <int WM, int WN, int TM>
+template <int WM, int WN, int TM, int NS>
 inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3Product *prods_in,
                                  int n, float *partials, uint32_t *arrivals) {
     using Sh = Bx3Shape<WM, WN, TM>;
@@ -606,7 +597,7 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
     args.total_tiles = (uint32_t)units;
     args.chunk_wgs = args.d[0].tiles_t * args.d[0].chunks;
     args.pad = 0;
-    Q8_LAUNCH((gemm_bf16x3_kernel<WM, WN, TM>), dim3((unsigned)units), dim3(WM * WN * 64), 0, stream,
+    Q8_LAUNCH((gemm_bf16x3_kernel<WM, WN, TM, NS>), dim3((unsigned)units), dim3(WM * WN * 64), 0, stream,
               stop, args);
     return hipGetLastError();
 }
@@ -623,8 +614,8 @@ inline hipError_t launch_gemm_bf16x3_list(hipStream_t stream, hipEvent_t stop, u
         return hipErrorInvalidValue;
     }
     switch (tile_tokens) {
-    case 128: return launch_bx3_cfg<2, 4, 2>(stream, stop, prods, n, partials, arrivals);
-    case 64: return launch_bx3_cfg<1, 4, 2>(stream, stop, prods, n, partials, arrivals);
+    case 128: return launch_bx3_cfg<2, 4, 2, 4>(stream, stop, prods, n, partials, arrivals);
+    case 64: return launch_bx3_cfg<1, 4, 2, 3>(stream, stop, prods, n, partials, arrivals);
     default: return hipErrorInvalidValue;
     }
 }
