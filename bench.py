@@ -205,6 +205,11 @@ def bench_gemm(host, ctx, steps, warmup):
     flops = 2.0 * M * rows * cols
     out["lm_head"] = dict(_bf16_gemm_point(flops, us), rows=rows, cols=cols,
                           launches_per_step=t.launches / n)
+    # ... and at 64 tokens (one 64-token tile of the same kernel)
+    t = run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, 64, TMH_GEMM_MMA)],
+                  max(2, warmup // 20), n, grouped=False)
+    us = t.gpu_ms / n * 1e3
+    out["lm_head_m64"] = dict(_bf16_gemm_point(2.0 * 64 * rows * cols, us), rows=rows, cols=cols, M=64)
     for b in keep + [m.buf, xb, yb]:
         b.free()
     return out

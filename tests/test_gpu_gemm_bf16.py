@@ -1,4 +1,4 @@
-"""GPU parity: the prefill GEMM from 65 tokens over sealed weights large enough
+"""GPU parity: the prefill GEMM from 33 tokens over sealed weights large enough
 to fill the chip with 128-token x 256-row tiles, which runs on the bf16 matrix
 cores with every f32 activation split into three exact bf16 pieces (contract: native/metal/tm_metal.h:172-175, tolerance-qualified like
 every matrix-core kernel; crates/metal/src/tests.rs:1169-1233 for the shapes).
@@ -14,7 +14,7 @@ from q8util import bits, norm_err, ref_scale, require_gpu, upload_new, weights_b
 
 pytestmark = pytest.mark.gpu
 
-M0 = H.GEMM_MMA_BF16_MIN_BATCH
+M0 = H.GEMM_MMA_BF16_MIN_BATCH  # 33: one 64-token tile up to 64 tokens
 
 
 @pytest.fixture(scope="module")
@@ -41,12 +41,14 @@ def product(ctx, wb, x, rows, cols, batch, x_off=0, y_off=0):
 # K of 1, 3, 32 (whole, or two chunks of 16 blocks), 33 (17 + 16), 36, 64 and 96 blocks;
 # ragged rows; a ragged last token tile; the smallest batch of the kernel and
 # the largest; every product has at least 128 work units of its own.
-SHAPES = [(8192, 1024, 512), (33000, 96, M0), (8300, 1056, 500), (4096, 3072, 512),
-          (33000, 2048, M0 + 1), (33000, 32, 512), (8500, 1152, 450), (11000, 1024, 384),
+SHAPES = [(8192, 1024, 512), (33000, 96, 65), (8300, 1056, 500), (4096, 3072, 512),
+          (33000, 2048, 66), (33000, 32, 512), (8500, 1152, 450), (11000, 1024, 384),
           (16500, 1024, 129),
           # tiles of 64 tokens (fewer than 192 units of the large tile)
           (4096, 1024, 512), (2048, 2048, 512), (1024, 4096, 512), (6144, 2048, 128),
-          (4100, 1056, 200), (33000, 96, M0)]
+          (4100, 1056, 200), (33000, 96, 80),
+          # one tile of 64 tokens (matrices of 16 M weights and more)
+          (33000, 1024, M0), (4096, 4096, 64), (16500, 1056, 40)]
 
 
 @pytest.mark.parametrize("rows,cols,batch", SHAPES)
@@ -67,7 +69,7 @@ def test_boundary_values_and_wide_ranges(ctx):
     # crates/metal/src/tests.rs:1169-1233 (boundary weights and inputs), and
     # activations that span 60 binades: every piece of the split is exact, so the
     # large terms do not swamp the small ones any more than in the CPU's sum.
-    rows, cols, batch = 33000, 1024, M0
+    rows, cols, batch = 33000, 1024, 65
     w = O.boundary_weights(rows, cols, 11)
     x = O.boundary_input(cols * batch, 13)
     wb = weights_buffer(ctx, w, rows, cols, True)
@@ -178,7 +180,9 @@ def test_a_group_splits_each_input_once_and_has_the_bits_of_its_products_alone(c
                                              (4096, 4096, 128), (4096, 4096, 129), (6144, 2048, 512),
                                              (6144, 2048, 256), (1024, 1024, 512), (2048, 6144, 384),
                                              (2048, 1024, 512), (3072, 1024, 512), (1024, 3072, 512),
-                                             (1024, 2048, 512), (6144, 2048, 128), (2048, 4096, 128)])
+                                             (1024, 2048, 512), (6144, 2048, 128), (2048, 4096, 128),
+                                             (16384, 1024, 64), (16383, 1024, 64), (16384, 1024, 33),
+                                             (16384, 1024, 32), (8192, 4096, 48), (6144, 2048, 64)])
 def test_the_choice_of_kernel_follows_the_documented_rule(ctx, rows, cols, batch):
     # two launches (split, multiply) on the bf16 matrix cores, one on the f32 ones
     wb = weights_buffer(ctx, S.make_weights(rows, cols, 1), rows, cols, True)

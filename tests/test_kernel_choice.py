@@ -41,6 +41,8 @@ def test_which_products_take_the_bf16_matrix_cores():
     assert not H.gemm_mma_on_bf16(2048, 1024, 512)
     assert not H.gemm_mma_on_bf16(1024, 3072, 512)
     assert H.gemm_mma_on_bf16(3072, 1024, 512)
+    # up to 64 tokens: matrices of 16 M weights and more
+    assert H.gemm_mma_on_bf16(4096, 4096, 64) and not H.gemm_mma_on_bf16(6144, 2048, 64)
     # activations must start on a 16-byte boundary
     assert not H.gemm_mma_on_bf16(8192, 1024, 512, x_off=3)
     assert H.gemm_mma_on_bf16(8192, 1024, 512, x_off=32)

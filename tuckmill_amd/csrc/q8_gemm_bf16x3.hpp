@@ -518,7 +518,7 @@ inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint3
 }
 
 // The plan of a product, and whether the kernel pays for it on its own
-// (`worth`). In order of preference: the large tile with 192 units or more; the
+// (`worth`). Above 64 tokens, in order of preference: the large tile with 192 units or more; the
 // small tile with 192 units or more in at most 4 K chunks (1024 x 3072 at 512
 // tokens in six chunks: 40 us against 32 on the f32 kernel); the large tile with
 // 128 units or more (alone about even with the f32 kernel, far ahead when
@@ -527,6 +527,17 @@ inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint3
 // 4096 x 1024 36 against 48, 2048 x 1024 (128 units) 31 against 28; large tile
 // 8192 x 1024 49 against 93, 6144 x 2048 69 against 133.
 inline Bx3Plan bx3_plan(uint32_t rows, uint32_t cols, uint32_t batch, bool *worth) {
+    if (batch <= 64u) {
+        // One small tile of tokens. The kernel's time hardly depends on the
+        // batch here (27 us for 8192 x 1024, 97 us for 151936 x 1024), the f32
+        // kernel's does: from 33 tokens (its 64-token tile) a matrix of 16 M
+        // weights is the break-even (16384 x 1024 at 64 tokens: 30 against 29 us;
+        // 4096 x 4096: 34 against 47; 151936 x 1024: 97 against 219). At 32
+        // tokens and below only the largest matrices would gain, and little.
+        const Bx3Plan one = bx3_plan_with(rows, cols, batch, 64u);
+        *worth = (uint64_t)rows * cols >= (1ull << 24) && one.units >= 128u;
+        return one;
+    }
     const Bx3Plan large = bx3_plan_with(rows, cols, batch, 128u);
     if (large.units >= BX3_UNITS_WANTED) {
         *worth = true;

@@ -303,17 +303,17 @@ struct GemvKey {
     bool decode() const { return kind == OP_GEMV_LIST && variant == V_DECODE && packed && flag; }
 };
 
-// Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 65
+// Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 33
 // tokens, and with enough work units (256 rows x 128 or 64 tokens x K chunk)
 // of their own for the kernel to pay (q8::bx3_plan has the rule and the
 // measurements behind it). The kernel is two to three times as fast as the f32
 // one when it fills the chip (at 512 tokens 14336 x 4096: 204 us against 640 us,
 // 6144 x 2048: 69 against 133; at 96 tokens 14336 x 4096: 73 against 173) but its
 // units are large: 1024 x 1024 at 512 tokens takes 48 us against 15 us, and 33 us
-// with K in four chunks; at 64 tokens and below the f32 kernels win or tie on
+// with K in four chunks; at 32 tokens and below the f32 kernels win or tie on
 // most shapes. A product's kernel depends on nothing but its own shape and
 // alignment, so its result does not depend on what shares its launch.
-constexpr uint32_t kBx3MinBatch = 65;
+constexpr uint32_t kBx3MinBatch = 33;
 constexpr uint64_t kBx3MaxPartialFloats = 1ull << 29; // 2 GiB of partial tiles per launch
 
 bool bx3_eligible(const Op &op, bool x_aligned) {

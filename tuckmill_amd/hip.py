@@ -27,14 +27,15 @@ GEMM_MMA_MAX_BATCH = 512
 # From this batch on tm_hip_q8_0_gemm_mma over a large sealed matrix (128 or more tiles of
 # 128 tokens x 256 rows, K chunks counted) with 16-byte aligned activations runs on the bf16
 # matrix cores (activations split into three exact bf16 pieces).
-GEMM_MMA_BF16_MIN_BATCH = 65
+GEMM_MMA_BF16_MIN_BATCH = 33
 
 
 def gemm_mma_bf16_plan(rows: int, cols: int, batch: int):
     """(tokens per tile, work units, worth it) for the bf16 matrix-core GEMM on a
     product. A unit is 256 rows x 128 or 64 tokens x one K chunk; K is cut into
     at most eight chunks of 512 columns or more, as many as give about 192
-    units. In order of preference: the large tile with 192 units or more, the
+    units. Up to 64 tokens the small tile, for matrices of 16 M weights and more
+    with 128 units or more; above, in order of preference: the large tile with 192 units or more, the
     small tile with 192 units or more in at most 4 chunks, the large tile with
     128 units or more (mirror of q8::bx3_plan, csrc/q8_gemm_bf16x3.hpp)."""
     def plan(tokens):
@@ -44,6 +45,9 @@ def gemm_mma_bf16_plan(rows: int, cols: int, batch: int):
         per_chunk = -(-blocks // chunks)
         chunks = -(-blocks // per_chunk)
         return tiles * chunks, chunks
+    if batch <= 64:  # one small tile of tokens: a matrix of 16 M weights is the break-even
+        units, _ = plan(64)
+        return 64, units, rows * cols >= 1 << 24 and units >= 128
     large, _ = plan(128)
     if large >= 192:
         return 128, large, True
