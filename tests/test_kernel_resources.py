@@ -18,23 +18,50 @@ from tuckmill_amd import build as B
 DECODE_KERNEL = re.compile(r"Function Name: _ZN2q816gemv_list_kernelILi1ELi8ELi1ELb1ELi0ELi\d+ELb0EEE")
 
 
-def test_decode_kernel_keeps_four_waves_per_simd(tmp_path):
+@pytest.fixture(scope="module")
+def resource_remarks(tmp_path_factory):
+    """The compiler's per-kernel resource remarks for the whole library, as lines."""
     hipcc = shutil.which(B.HIPCC) or (B.HIPCC if os.path.exists(B.HIPCC) else None)
     if hipcc is None:
         pytest.skip("hipcc not available")
+    out = tmp_path_factory.mktemp("resources") / "device.o"
     cmd = [hipcc, "-x", "hip", "-std=c++17", "-O3", *B.DEVICE_FLAGS, "--cuda-device-only",
            "-I", os.path.join(B.ROOT, "include"), "-I", B.CSRC,
            "-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(B.CSRC, "tm_hip.cpp"),
-           "-o", str(tmp_path / "device.o")]
+           "-o", str(out)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     assert res.returncode == 0, res.stderr[-2000:]
-    lines = res.stderr.splitlines()
-    start = [i for i, l in enumerate(lines) if DECODE_KERNEL.search(l)]
-    assert start, "decode kernel not found in the resource remarks"
-    for at in start:  # the long- and the short-list instantiation
-        block = "\n".join(lines[at:at + 14])
+    return res.stderr.splitlines()
+
+
+def _blocks(lines, pattern):
+    start = [i for i, l in enumerate(lines) if pattern.search(l)]
+    return ["\n".join(lines[at:at + 14]) for at in start]
+
+
+def test_decode_kernel_keeps_four_waves_per_simd(resource_remarks):
+    blocks = _blocks(resource_remarks, DECODE_KERNEL)
+    assert blocks, "decode kernel not found in the resource remarks"
+    for block in blocks:  # the long- and the short-list instantiation
         vgprs = int(re.search(r" VGPRs: (\d+)", block).group(1))
         spill = int(re.search(r"VGPRs Spill: (\d+)", block).group(1))
         occupancy = int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", block).group(1))
         assert spill == 0
         assert vgprs <= 128 and occupancy >= 4, f"{vgprs} VGPRs, {occupancy} waves/SIMD"
+
+
+# gemm_bf16x3_kernel<WM, 4, 2, NS>: the 128-token and the 64-token tile
+BF16_KERNEL = re.compile(r"Function Name: _ZN2q818gemm_bf16x3_kernelILi[12]ELi4ELi2ELi[34]EEE")
+
+
+def test_bf16_gemm_keeps_its_results_in_vector_registers(resource_remarks):
+    """Both tiles run two waves per SIMD and rescale every MFMA result once per
+    Q8_0 block: the results must sit in ordinary vector registers (no
+    accumulation registers, which cost a move per result), unspilled."""
+    blocks = _blocks(resource_remarks, BF16_KERNEL)
+    assert len(blocks) >= 2, "bf16 GEMM kernels not found in the resource remarks"
+    for block in blocks:
+        agprs = int(re.search(r"AGPRs: (\d+)", block).group(1))
+        spill = int(re.search(r"VGPRs Spill: (\d+)", block).group(1))
+        occupancy = int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", block).group(1))
+        assert agprs == 0 and spill == 0 and occupancy >= 2, block

@@ -147,7 +147,12 @@ __device__ __forceinline__ bf16x8_t sbytes_to_bf16x8(uint32_t lo, uint32_t hi) {
 }
 
 template <int WM, int WN, int TM, int NS>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_bf16x3_kernel(const Bx3Args args) {
+// (Two waves per SIMD, declared: with a register budget of 256 the compiler keeps
+// the MFMA results in ordinary vector registers, which the rescale reads
+// directly. With a single wave's budget it parked the small tile's results in
+// accumulation registers and paid a v_accvgpr_read per result and block, 64 of
+// the tile's 184 vector instructions per stage: 5-7 % slower.)
+__global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3Args args) {
     using Sh = Bx3Shape<WM, WN, TM>;
     constexpr int NW = WM * WN;
     constexpr int TN = 2; // a wave computes TM x 2 tiles of 32 x 32: 32*TM tokens x 64 rows
