@@ -110,6 +110,44 @@ def test_copy_contract_synchronizes_with_in_flight_compute(ctx):
     assert np.all(yb.download_f32(0, 4) == 320.0)
 
 
+def test_copy_f32_moves_exact_slices_and_refuses_out_of_range(ctx):
+    # crates/metal/src/tests.rs:1076-1115
+    src = (np.sin(np.arange(64, dtype=np.float32)) * np.float32(1e-30)
+           + np.arange(64, dtype=np.float32)).astype(np.float32)
+    a, b = ctx.buffer(64 * 4), ctx.buffer(64 * 4)
+    a.upload(0, src)
+    ctx.copy_f32(a, 8, b, 40, 16)
+    ctx.fence()
+    out = b.download_f32(0, 64)
+    assert np.array_equal(bits(out[40:56]), bits(src[8:24])), "bit-exact slice"
+    assert not out[:40].view(np.uint32).any() and not out[56:].view(np.uint32).any()
+    for args in [(a, 60, b, 0, 8), (a, 0, b, 60, 8), (a, 0, b, 0, 0)]:
+        with pytest.raises(H.TuckmillError) as e:
+            ctx.copy_f32(*args)
+        assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS
+    # every bit pattern survives (NaN payloads, infinities, subnormals, -0), at
+    # odd offsets and a ragged length that spans many workgroups
+    n = (1 << 20) + 3
+    raw = np.random.default_rng(9).integers(0, 1 << 32, n + 5, dtype=np.uint64).astype(np.uint32)
+    big, dst = ctx.buffer((n + 5) * 4), ctx.buffer((n + 7) * 4)
+    big.upload(0, raw.view(np.float32))
+    ctx.copy_f32(big, 5, dst, 7, n)
+    got = dst.download_f32(0, n + 7).view(np.uint32)
+    assert np.array_equal(got[7:], raw[5:]) and not got[:7].any()
+
+
+def test_copy_f32_inside_a_group_follows_the_product_that_wrote_its_source(ctx):
+    wb, xb, yb = ones_problem(ctx, xval=3.0)
+    keep = ctx.buffer(8 * 4)
+    ctx.begin_group()
+    ctx.q8_0_gemv(wb, xb, yb, 4, 64)
+    ctx.copy_f32(yb, 0, keep, 2, 4)
+    ctx.end_group()
+    ctx.fence()
+    out = keep.download_f32(0, 8)
+    assert np.all(out[2:6] == 192.0) and not out[:2].any() and not out[6:].any()
+
+
 def test_dropping_buffers_before_fence_is_safe(ctx):
     wb, xb, yb = ones_problem(ctx, xval=7.0)
     ctx.q8_0_gemv(wb, xb, yb, 4, 64)
