@@ -298,6 +298,17 @@ uint64_t tm_hip_kernel_launches(const tm_hip_ctx *ctx);
 int tm_hip_profile_set(tm_hip_ctx *ctx, int enabled);
 int tm_hip_profile_read(tm_hip_ctx *ctx, uint32_t index, char *name, size_t name_cap,
                         uint64_t *nanos, uint64_t *count);
+/* Per-commit GPU times, for benchmarks that report a robust statistic the way
+ * the reference's isolated timings do (crates/metal/src/tests.rs:1057-1066,
+ * benchmarks/tools/ggml-mul-mat.c:69-75). While enabled, every commit that
+ * completes appends its GPU nanoseconds (the value last_gpu_ms reports for it)
+ * to a log kept by the context; the log holds the most recent
+ * TM_HIP_COMMIT_LOG_CAP entries. read copies up to `cap` entries in completion
+ * order into `nanos`, removes them and returns their number. set(…, 0) stops
+ * logging and clears the log. No counterpart in the reference. */
+#define TM_HIP_COMMIT_LOG_CAP 65536u
+int tm_hip_commit_log_set(tm_hip_ctx *ctx, int enabled);
+size_t tm_hip_commit_log_read(tm_hip_ctx *ctx, uint64_t *nanos, size_t cap);
 /* Live bytes in handles of this context. */
 uint64_t tm_hip_allocated_bytes(const tm_hip_ctx *ctx);
 /* Bytes leased by commits that have not completed yet. */

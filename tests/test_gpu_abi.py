@@ -11,7 +11,7 @@ import oracle as O
 from tuckmill_amd import hip as H
 from tuckmill_amd import synth as S
 
-from q8util import bits, gemv, require_gpu, upload_new, weights_buffer
+from q8util import bits, gemv, norm_err, require_gpu, upload_new, weights_buffer
 
 pytestmark = pytest.mark.gpu
 
@@ -158,6 +158,55 @@ def test_dropping_buffers_before_fence_is_safe(ctx):
     yb.free()
     assert ctx.allocated_bytes() == 0
     assert ctx.in_flight_bytes() == 0
+
+
+def test_buffers_freed_inside_an_open_group_stay_alive_until_the_commit_completes(ctx):
+    # native/metal/tm_metal.m:673, :707-739: a group leases every buffer when the
+    # operation is encoded, so handles may be dropped before end_group.
+    rows, cols = 151_936, 1024
+    w = S.make_weights(rows, cols, 12)
+    x = S.make_activations(cols, 13)
+    want = O.gemv_q8_0_f32(w, rows, cols, x, threads=8)
+    for recorded in (False, True):
+        wb = weights_buffer(ctx, w, rows, cols, True)
+        xb = upload_new(ctx, x)
+        tb = ctx.buffer(rows * 4)   # written by the first product, read by the copy
+        keep = ctx.buffer(rows * 4)
+        ctx.fence()
+        total = wb.len() + xb.len() + tb.len()
+        ctx.begin_group()
+        ctx.q8_0_gemv(wb, xb, tb, rows, cols)
+        ctx.copy_f32(tb, 0, keep, 0, rows)
+        wb.free()
+        xb.free()
+        tb.free()
+        assert ctx.allocated_bytes() == rows * 4, "only the kept output is handle-live"
+        # fresh (zero-filled) allocations of the same sizes must not land on the
+        # group's memory
+        spoil = [ctx.buffer(n) for n in (total - rows * 4 - cols * 4, cols * 4, rows * 4)]
+        if recorded:
+            step = ctx.end_group_recorded()
+            step.run()
+        else:
+            ctx.end_group()
+            assert ctx.in_flight_bytes() >= total or ctx.completed_dispatches() == \
+                ctx.committed_dispatches()
+        ctx.fence()
+        assert norm_err(keep.download_f32(0, rows), want) <= 1e-5
+        if recorded:
+            step.free()
+        assert ctx.in_flight_bytes() == 0
+        for b in spoil + [keep]:
+            b.free()
+        assert ctx.allocated_bytes() == 0
+    # an aborted group gives its references back
+    wb, xb, yb = ones_problem(ctx)
+    ctx.begin_group()
+    ctx.q8_0_gemv(wb, xb, yb, 4, 64)
+    for b in (wb, xb, yb):
+        b.free()
+    ctx.abort_group()
+    assert ctx.allocated_bytes() == 0 and ctx.in_flight_bytes() == 0
 
 
 def test_in_flight_bytes_stay_visible_until_completion(ctx):
@@ -317,8 +366,19 @@ def test_row_indirect_reads_the_id_on_the_device(ctx, packed):
         ctx.row_indirect_f32(wb, 8, rows, cols, ids, slot, ob)
         ctx.fence()
         assert not ob.download(0, cols * 4).any()
-    with pytest.raises(H.TuckmillError):
-        ctx.row_indirect_f32(wb, 1, rows, cols, ids, 0, ob)   # F16 twin is not built
+    # Type 1 (F16) on this buffer: it is too short for rows x cols halves
+    # (BOUNDS); with few enough rows to fit, a sealed buffer is still refused,
+    # because it holds Q8_0 in the device layout (UNSUPPORTED).
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.row_indirect_f32(wb, 1, rows, cols, ids, 0, ob)
+    assert e.value.abi_code == H.TM_HIP_ERR_BOUNDS
+    if packed:
+        with pytest.raises(H.TuckmillError) as e:
+            ctx.row_indirect_f32(wb, 1, 19, cols, ids, 0, ob)
+        assert e.value.abi_code == H.TM_HIP_ERR_UNSUPPORTED
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.row_indirect_f32(wb, 2, rows, cols, ids, 0, ob)   # neither Q8_0 nor F16
+    assert e.value.abi_code == H.TM_HIP_ERR_UNSUPPORTED
     with pytest.raises(H.TuckmillError):
         ctx.row_indirect_f32(wb, 8, rows, cols, ids, 4, ob)   # slot past ids
     with pytest.raises(H.TuckmillError):
@@ -343,8 +403,13 @@ def test_matrix_serves_lm_head_and_embedding_from_one_buffer(ctx):
     assert np.max(np.abs(got - want)) / np.max(np.abs(want)) <= 1e-5
     assert np.array_equal(bits(ob.download_f32(0, cols)),
                           bits(O.dequant_q8_0(w).reshape(rows, cols)[514]))
-    with pytest.raises(H.TuckmillError):
+    # the same bytes declared as F16: the length does not match rows x cols halves
+    with pytest.raises(H.TuckmillError) as e:
         H.Matrix.load(ctx, w, cols, rows, type_id=1)
+    assert e.value.code == "InvalidArtifact"
+    with pytest.raises(H.TuckmillError) as e:  # crates/tuckcore/src/engine/metal.rs:126-131
+        H.Matrix.load(ctx, w, cols, rows, type_id=2)
+    assert e.value.code == "UnsupportedQuantization"
 
 
 # ------------------------------------------------------------------ seal --

@@ -212,18 +212,26 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_i8_lds_kernel(const I8Args 
         }
     };
 
+    // A wave fetches only its share of a stage and every wave reads all of it:
+    // each wave waits for its own fetch (the only vector memory operations it
+    // has in flight; the barrier alone does not wait for loads that land in
+    // LDS), then all meet.
+    auto landed = [&]() {
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); // vmcnt(0)
+        __syncthreads();
+    };
     fetch(0, stage_a);
     for (uint32_t st = 0; st < nstages; st += 2u) {
-        __syncthreads(); // stage st has landed everywhere; stage_b is free
+        landed(); // stage st is there for everyone; stage_b is free
         fetch(st + 1u < nstages ? st + 1u : st, stage_b);
         compute(st, stage_a);
         if (st + 1u < nstages) {
-            __syncthreads();
+            landed();
             fetch(st + 2u < nstages ? st + 2u : st + 1u, stage_a);
             compute(st + 1u, stage_b);
         }
     }
-    __syncthreads(); // no fetch may be in flight when the workgroup gives up its LDS
+    landed(); // no fetch may be in flight when the workgroup gives up its LDS
 
 #pragma unroll
     for (int i = 0; i < TM; ++i) {

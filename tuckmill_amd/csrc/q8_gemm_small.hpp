@@ -111,8 +111,11 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
     uint32_t r0 = row_first, c = 0;
     float acc[R][TW];
     auto do_step = [&](uint32_t step, uint8_t *cur, uint8_t *nxt) {
-        // The fetch of this step has landed (each wave waits for its own part,
-        // then all meet), and every wave has finished reading the other buffer.
+        // The fetch of this step has landed: each wave waits for its own part
+        // (the barrier alone does not wait for loads that land in LDS; the
+        // scale loads requested with them are as old and come back with them),
+        // then all meet, and every wave has finished reading the other buffer.
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); // vmcnt(0)
         __syncthreads();
         uint32_t cn = c + 1u, rn = r0;
         if (cn == full) {
@@ -225,7 +228,9 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
             do_step(step + 1u, stage_b, stage_a);
         }
     }
-    __syncthreads(); // no fetch may still be in flight when the workgroup gives up its LDS
+    // no fetch may still be in flight when the workgroup gives up its LDS
+    __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); // vmcnt(0)
+    __syncthreads();
 }
 
 } // namespace q8

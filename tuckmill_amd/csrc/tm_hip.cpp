@@ -73,6 +73,29 @@ struct Op {
     const char *what = "";     // static operator name
 };
 
+// An operation recorded into an open group holds a reference on every
+// allocation it names from the moment it is recorded (the reference's group
+// leases its buffers at encode time, native/metal/tm_metal.m:673, :707-739): a
+// handle may be freed before end_group and the memory lives on. The references
+// are dropped once the commit (or the recorded step) has taken its own, or when
+// the group is aborted.
+void ops_hold(const Op &op) {
+    for (int i = 0; i < op.n_alloc; ++i) {
+        if (op.a[i] != nullptr) {
+            op.a[i]->refs.fetch_add(1, std::memory_order_relaxed);
+        }
+    }
+}
+
+void ops_drop(std::vector<Op> &ops) {
+    for (const Op &op : ops) {
+        for (int i = 0; i < op.n_alloc; ++i) {
+            alloc_release(op.a[i]);
+        }
+    }
+    ops.clear();
+}
+
 // `start` is either an event recorded just before the commit's work or, when
 // the stream was still busy with the previous commit, that commit's stop
 // event (the new work starts when the old one ends; one event fewer on the
@@ -127,6 +150,8 @@ struct tm_hip_ctx {
     std::vector<hipEvent_t> event_pool;
     ProfileSlot profile[kProfileSlots];
     uint32_t profile_used = 0;
+    bool commit_log_on = false;       // under q_mu
+    std::deque<uint64_t> commit_log;  // GPU nanoseconds per completed commit, oldest first
 };
 
 struct tm_hip_buffer {
@@ -243,6 +268,12 @@ void settle(tm_hip_ctx *ctx) {
             ctx->last_gpu_nanos.store(nanos, std::memory_order_relaxed);
             ctx->gpu_nanos_total.fetch_add(nanos, std::memory_order_relaxed);
             account_profile(ctx, c.label, nanos);
+            if (ctx->commit_log_on) {
+                if (ctx->commit_log.size() >= TM_HIP_COMMIT_LOG_CAP) {
+                    ctx->commit_log.pop_front();
+                }
+                ctx->commit_log.push_back(nanos);
+            }
             ctx->leased.fetch_sub(c.leased, std::memory_order_relaxed);
             ctx->event_pool.push_back(c.start);
             if (!c.stop_lent) {
@@ -1124,6 +1155,7 @@ int commit_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, const char *label, c
 int submit(tm_hip_ctx *ctx, Op &op, const char *what, char *err, size_t cap) {
     op.what = what;
     if (ctx->group_active) {
+        ops_hold(op);
         ctx->group_ops.push_back(op);
         return TM_HIP_OK;
     }
@@ -1294,10 +1326,7 @@ void tm_hip_destroy(tm_hip_ctx *ctx) {
         return;
     }
     if (ctx->group_active) {
-        for (Op &op : ctx->group_ops) {
-            (void)op;
-        }
-        ctx->group_ops.clear();
+        ops_drop(ctx->group_ops);
         ctx->group_active = false;
     }
     if (ctx->stream != nullptr) {
@@ -1745,7 +1774,9 @@ int tm_hip_end_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {
     std::vector<Op> ops;
     ops.swap(ctx->group_ops);
     // An empty group still commits once, like an empty command buffer.
-    return commit_ops(ctx, ops, "group", "group", err, err_cap);
+    const int rc = commit_ops(ctx, ops, "group", "group", err, err_cap);
+    ops_drop(ops); // the commit holds its own leases now
+    return rc;
 }
 
 int tm_hip_end_group_recorded(tm_hip_ctx *ctx, tm_hip_step **out, char *err, size_t err_cap) {
@@ -1763,6 +1794,11 @@ int tm_hip_end_group_recorded(tm_hip_ctx *ctx, tm_hip_step **out, char *err, siz
     ctx->group_active = false;
     std::vector<Op> ops;
     ops.swap(ctx->group_ops);
+    // The group's references go on every way out; a recorded step takes its own.
+    struct DropOnExit {
+        std::vector<Op> &ops;
+        ~DropOnExit() { ops_drop(ops); }
+    } drop_on_exit{ops};
     if (ops.empty()) {
         return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
                     "end_group_recorded: the group holds no operation");
@@ -1882,7 +1918,7 @@ int tm_hip_abort_group(tm_hip_ctx *ctx, char *err, size_t err_cap) {
     if (!ctx->group_active) {
         return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED, "abort_group: no dispatch group is open");
     }
-    ctx->group_ops.clear();
+    ops_drop(ctx->group_ops);
     ctx->group_active = false;
     return TM_HIP_OK;
 }
@@ -2361,6 +2397,31 @@ int tm_hip_profile_read(tm_hip_ctx *ctx, uint32_t index, char *name, size_t name
         *count = ctx->profile[index].count;
     }
     return 1;
+}
+
+int tm_hip_commit_log_set(tm_hip_ctx *ctx, int enabled) {
+    if (ctx == nullptr) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    settle(ctx);
+    std::lock_guard<std::mutex> g(ctx->q_mu);
+    ctx->commit_log_on = enabled != 0;
+    ctx->commit_log.clear();
+    return TM_HIP_OK;
+}
+
+size_t tm_hip_commit_log_read(tm_hip_ctx *ctx, uint64_t *nanos, size_t cap) {
+    if (ctx == nullptr || nanos == nullptr) {
+        return 0;
+    }
+    settle(ctx);
+    std::lock_guard<std::mutex> g(ctx->q_mu);
+    size_t n = 0;
+    while (n < cap && !ctx->commit_log.empty()) {
+        nanos[n++] = ctx->commit_log.front();
+        ctx->commit_log.pop_front();
+    }
+    return n;
 }
 
 uint64_t tm_hip_allocated_bytes(const tm_hip_ctx *ctx) {

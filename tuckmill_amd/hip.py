@@ -187,6 +187,9 @@ _SIGS = {
     "tm_hip_profile_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_char_p,
                                            ctypes.c_size_t, ctypes.POINTER(ctypes.c_uint64),
                                            ctypes.POINTER(ctypes.c_uint64)]),
+    "tm_hip_commit_log_set": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "tm_hip_commit_log_read": (ctypes.c_size_t, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64),
+                                                 ctypes.c_size_t]),
     "tm_hip_allocated_bytes": (ctypes.c_uint64, [ctypes.c_void_p]),
     "tm_hip_in_flight_bytes": (ctypes.c_uint64, [ctypes.c_void_p]),
 }
@@ -426,6 +429,19 @@ class HipContext:
 
     def live_gpu_bytes(self) -> int:
         return self.allocated_bytes() + self.in_flight_bytes()
+
+    def set_commit_log(self, enabled: bool):
+        """Starts (and clears) or stops the per-commit GPU time log."""
+        with self._inner.lock:
+            self._lib.tm_hip_commit_log_set(self._inner.raw, 1 if enabled else 0)
+
+    def read_commit_log(self) -> np.ndarray:
+        """GPU nanoseconds of the commits completed since the last read, oldest first."""
+        out = np.empty(65536, dtype=np.uint64)
+        with self._inner.lock:
+            n = self._lib.tm_hip_commit_log_read(
+                self._inner.raw, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint64)), out.size)
+        return out[:int(n)].copy()
 
     def set_profiling(self, enabled: bool):
         with self._inner.lock:
