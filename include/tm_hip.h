@@ -217,6 +217,36 @@ int tm_hip_q8_0_gemm_mma(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm
                          uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off,
                          uint32_t y_off, char *err, size_t err_cap);
 
+/* tm_hip_q8_0_gemm_mma for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc. No counterpart in the reference. Same arguments, refusals, kernels
+ * and results as tm_hip_q8_0_gemm_mma (bit for bit), with these differences:
+ *   - Nothing is allocated or freed on the device, in this call or later because
+ *     of it: the workspace of the large-product form lies in a static device
+ *     array of TM_HIP_NOALLOC_WORKSPACE_BYTES that every GPU the library runs on
+ *     holds from load to process exit. A product whose split activations
+ *     (6 bytes x batch x cols, at most TM_HIP_NOALLOC_XS_BYTES) or partial tiles
+ *     do not fit is refused with TM_HIP_ERR_UNSUPPORTED and a message that says
+ *     what it needs; tm_hip_q8_0_gemm_mma takes it.
+ *   - The kernels are launched at once on the context's stream, in order with
+ *     everything committed before and after; the call is not a commit (no
+ *     events, not counted by committed_dispatches) and is refused while a
+ *     dispatch group is open. tm_hip_fence and host copies wait for it like for
+ *     any other work.
+ *   - w, x and y stay leased (visible in tm_hip_in_flight_bytes, safe to free)
+ *     until the next commit of the context completes or a fence has passed;
+ *     after TM_HIP_NOALLOC_MAX_PENDING calls without either, the call is refused.
+ *   - All calls on one GPU share the one array, which keeps the last call's
+ *     contents (what must start at zero is cleared by the call itself): calls
+ *     that overlap on one GPU, from two contexts or two processes' worth of
+ *     streams in one process, race. One context orders its own calls. */
+#define TM_HIP_NOALLOC_WORKSPACE_BYTES (64u << 20)
+#define TM_HIP_NOALLOC_XS_BYTES (20u << 20)
+#define TM_HIP_NOALLOC_MAX_PENDING 1024u
+int tm_hip_q8_0_gemm_mma_noalloc(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x,
+                                 tm_hip_buffer *y, uint32_t rows, uint32_t cols, uint32_t batch,
+                                 uint32_t x_off, uint32_t y_off, char *err, size_t err_cap);
+
 /* out[out_off + i] = d * q of row `row`, i < cols; exact
  * (native/metal/tm_metal.h:137-139). */
 int tm_hip_q8_0_row_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *out, uint32_t row,

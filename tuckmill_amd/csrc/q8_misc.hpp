@@ -75,4 +75,12 @@ __global__ __launch_bounds__(256) void copy_f32_kernel(const float *src, float *
     }
 }
 
+// Clears n dwords (counters that must read zero when the next kernel starts).
+__global__ __launch_bounds__(256) void zero_u32_kernel(uint32_t *dst, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        dst[i] = 0u;
+    }
+}
+
 } // namespace q8

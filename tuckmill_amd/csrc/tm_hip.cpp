@@ -32,7 +32,64 @@
 #include "q8_neighbors.hpp"
 #include "f16_gemv.hpp"
 
+// Workspace of tm_hip_q8_0_gemm_mma_noalloc, the entry point that allocates
+// nothing: device memory that exists from the moment the library is loaded, one
+// copy per GPU, held until the process ends. Layout (byte offsets):
+//   [0, 256)                 the two counters of the work-queue MFMA kernel
+//   [256, 256 + 64 KiB)      arrival counters of the bf16 GEMM's K chunks
+//   [128 KiB, +20 MiB)       split activations (6 bytes per activation element)
+//   [128 KiB + 20 MiB, end)  partial tiles of products whose K is cut into chunks
+constexpr size_t kScratchBytes = TM_HIP_NOALLOC_WORKSPACE_BYTES;
+constexpr size_t kScratchQueueOff = 0;
+constexpr size_t kScratchArrivalsOff = 256;
+constexpr size_t kScratchCounterDwords = 64u + q8::BX3_MAX_SPLIT_TILES;
+constexpr size_t kScratchXsOff = 128u << 10;
+constexpr size_t kScratchXsBytes = TM_HIP_NOALLOC_XS_BYTES;
+constexpr size_t kScratchPartialOff = kScratchXsOff + kScratchXsBytes;
+constexpr size_t kScratchPartialBytes = kScratchBytes - kScratchPartialOff;
+static_assert(kScratchArrivalsOff + q8::BX3_MAX_SPLIT_TILES * 4u <= kScratchXsOff, "counters");
+static __device__ __align__(256) uint8_t scratch[kScratchBytes];
+
 namespace {
+
+// In host code `scratch` is only a stand-in for the device array: its address on
+// a GPU comes from hipGetSymbolAddress, asked once per device with that device
+// current (every GPU holds its own copy at its own address).
+constexpr int kMaxDevices = 64;
+uint8_t *g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mu;
+
+hipError_t scratch_on_current_device(int device, uint8_t **out) {
+    if (device < 0 || device >= kMaxDevices) {
+        return hipErrorInvalidDevice;
+    }
+    std::lock_guard<std::mutex> g(g_scratch_mu);
+    if (g_scratch_ptr[device] == nullptr) {
+        void *ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) {
+            return e;
+        }
+        if (ptr == nullptr) {
+            return hipErrorInvalidSymbol;
+        }
+        g_scratch_ptr[device] = (uint8_t *)ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return hipSuccess;
+}
+
+// Device memory the kernels use beyond a product's own buffers.
+struct Workspace {
+    uint32_t *mma_queue = nullptr; // two counters of the work-queue MFMA kernel, zero between launches
+    // The bf16 split-float GEMM: split activations, partial tiles of products
+    // whose K is cut into chunks, their arrival counters (zero between launches).
+    uint8_t *xs = nullptr;
+    size_t xs_bytes = 0;
+    float *partials = nullptr;
+    size_t partial_bytes = 0;
+    uint32_t *arrivals = nullptr;
+};
 
 constexpr int kProfileSlots = 128;
 constexpr int kProfileName = 48;
@@ -121,17 +178,17 @@ struct tm_hip_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     hipStream_t copy_stream = nullptr;
-    uint32_t *mma_queue = nullptr; // two counters of the work-queue MFMA kernel, zero between launches
-    // Workspace of the bf16 split-float GEMM (split activations, partial tiles of
-    // products whose K is cut into chunks, their arrival counters): grown on demand, never
-    // shrunk. A buffer that was outgrown stays allocated until the context goes:
-    // recorded steps may still point at it.
-    uint8_t *bx3_xs = nullptr;
-    size_t bx3_xs_bytes = 0;
-    float *bx3_partials = nullptr;
-    size_t bx3_partial_bytes = 0;
-    uint32_t *bx3_arrivals = nullptr;
+    // The workspace of ordinary commits: grown on demand, never shrunk. A buffer
+    // that was outgrown stays allocated until the context goes: recorded steps may
+    // still point at it.
+    Workspace ws;
     std::vector<void *> bx3_retired;
+    // The fixed workspace inside the device's static array, and the allocations
+    // that launches of tm_hip_q8_0_gemm_mma_noalloc still use: the next commit
+    // adopts them (it completes after those launches), a fence releases them.
+    Workspace fixed;
+    std::vector<Alloc *> noalloc_keep;
+    uint64_t noalloc_leased = 0;
     std::atomic<uint64_t> allocated{0};
     std::atomic<uint64_t> leased{0};
     std::atomic<uint64_t> committed{0};
@@ -214,6 +271,21 @@ int hip_fail(char *err, size_t cap, const char *what, hipError_t e) {
 
 // ------------------------------------------------ completion accounting --
 
+// Launches of tm_hip_q8_0_gemm_mma_noalloc hold at most this many allocations
+// between two commits or fences (the list never grows: the call is refused).
+constexpr size_t kNoallocKeepCap = 3u * TM_HIP_NOALLOC_MAX_PENDING;
+
+// The stream has passed every launch of the allocation-free entry point (the
+// caller has just synchronized it): give their allocations back.
+void noalloc_release(tm_hip_ctx *ctx) {
+    for (Alloc *a : ctx->noalloc_keep) {
+        alloc_release(a);
+    }
+    ctx->noalloc_keep.clear();
+    ctx->leased.fetch_sub(ctx->noalloc_leased, std::memory_order_relaxed);
+    ctx->noalloc_leased = 0;
+}
+
 hipEvent_t take_event(tm_hip_ctx *ctx) {
     // q_mu held by the caller
     if (!ctx->event_pool.empty()) {
@@ -294,6 +366,7 @@ int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
     if (e != hipSuccess) {
         return hip_fail(err, cap, "stream synchronize", e);
     }
+    noalloc_release(ctx);
     settle(ctx);
     if (ctx->completed.load(std::memory_order_acquire) <
         ctx->committed.load(std::memory_order_relaxed)) {
@@ -513,7 +586,7 @@ bool same_input(const Op &a, const Op &b) {
 size_t bx3_xs_bytes_of(const Op &op) { return ((size_t)op.batch * op.cols * 6u + 255u) & ~(size_t)255u; }
 
 hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
-                           GemvKey key) {
+                           GemvKey key, const Workspace &ws) {
     q8::MmaProduct prods[q8::MMA_MAX_DESCS];
     int n = 0;
     for (const Op *op : ops) {
@@ -524,16 +597,16 @@ hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<c
     }
     const q8::MmaConfig c{key.p0, key.p1, key.p2};
     return q8::launch_gemm_mma_list(ctx->stream, stop, key.packed, key.flag, prods, n, &c,
-                                    ctx->mma_queue);
+                                    ws.mma_queue);
 }
 
 // The split-float GEMM: one launch that splits every distinct input of the list
 // into its three bf16 planes, then the product list. The workspace was sized by
 // ensure_bx3_workspace() when the launches were planned.
-hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch) {
+hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch,
+                           const Workspace &ws) {
     const std::vector<const Op *> &ops = launch.list;
-    if (launch.bx3_xs_bytes > ctx->bx3_xs_bytes ||
-        launch.bx3_partial_floats * 4u > ctx->bx3_partial_bytes) {
+    if (launch.bx3_xs_bytes > ws.xs_bytes || launch.bx3_partial_floats * 4u > ws.partial_bytes) {
         return hipErrorInvalidValue;
     }
     q8::SplitInput inputs[q8::SPLIT_MAX_DESCS];
@@ -552,7 +625,7 @@ hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launc
             }
             input_of[n_in] = op;
             inputs[n_in] = q8::SplitInput{(const float *)op->a[1]->ptr + op->x_off,
-                                          (uint16_t *)(ctx->bx3_xs + xs_used), op->batch, op->cols};
+                                          (uint16_t *)(ws.xs + xs_used), op->batch, op->cols};
             xs_used += bx3_xs_bytes_of(*op);
             ++n_in;
         }
@@ -565,7 +638,7 @@ hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launc
         return e;
     }
     return q8::launch_gemm_bf16x3_list(ctx->stream, stop, launch.key.p0 * 64u, prods, n,
-                                       ctx->bx3_partials, ctx->bx3_arrivals);
+                                       ws.partials, ws.arrivals);
 }
 
 // Kernel launches a planned launch stands for.
@@ -601,9 +674,9 @@ hipError_t ensure_bx3_workspace(tm_hip_ctx *ctx, const std::vector<Launch> &plan
         *have = need;
         return hipSuccess;
     };
-    hipError_t e = grow((void **)&ctx->bx3_xs, &ctx->bx3_xs_bytes, xs);
+    hipError_t e = grow((void **)&ctx->ws.xs, &ctx->ws.xs_bytes, xs);
     if (e == hipSuccess) {
-        e = grow((void **)&ctx->bx3_partials, &ctx->bx3_partial_bytes, partial);
+        e = grow((void **)&ctx->ws.partials, &ctx->ws.partial_bytes, partial);
     }
     return e;
 }
@@ -627,15 +700,16 @@ hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<co
     return q8::launch_gemm_i8_list(ctx->stream, stop, key.packed, key.flag, key.p0, prods, n);
 }
 
-hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch) {
+hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch,
+                            const Workspace &ws) {
     const std::vector<const Op *> &ops = launch.list;
     const std::vector<const Op *> &residual = launch.residual;
     const GemvKey key = launch.key;
     if (key.variant == V_BF16X3) {
-        return launch_bx3_list(ctx, stop, launch);
+        return launch_bx3_list(ctx, stop, launch, ws);
     }
     if (key.kind == OP_MMA) {
-        return launch_mma_list(ctx, stop, ops, key);
+        return launch_mma_list(ctx, stop, ops, key, ws);
     }
     if (key.kind == OP_I8) {
         return launch_i8_list(ctx, stop, ops, key);
@@ -1056,7 +1130,7 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, hipEvent_t sto
         const hipEvent_t ev = last ? stop : nullptr;
         const Launch &l = plan[i];
         hipError_t e = l.single != nullptr ? launch_single(ctx, ev, *l.single)
-                                           : launch_gemv_list(ctx, ev, l);
+                                           : launch_gemv_list(ctx, ev, l, ctx->ws);
         if (e != hipSuccess) {
             return e;
         }
@@ -1096,6 +1170,13 @@ int commit_work(tm_hip_ctx *ctx, std::vector<Alloc *> keep, const char *label, c
         a->refs.fetch_add(1, std::memory_order_relaxed);
         c.leased += a->len;
     }
+    // Allocations still used by launches of the allocation-free entry point go
+    // with this commit: it completes after them. Their bytes are in the ledger
+    // already, and their references pass on as they are.
+    const uint64_t adopted = ctx->noalloc_leased;
+    c.keep.insert(c.keep.end(), ctx->noalloc_keep.begin(), ctx->noalloc_keep.end());
+    ctx->noalloc_keep.clear();
+    ctx->noalloc_leased = 0;
     if (ctx->profiling.load(std::memory_order_relaxed)) {
         snprintf(c.label, sizeof c.label, "%s", label);
     }
@@ -1112,6 +1193,7 @@ int commit_work(tm_hip_ctx *ctx, std::vector<Alloc *> keep, const char *label, c
     }
     c.seq = ctx->committed.fetch_add(1, std::memory_order_relaxed) + 1;
     ctx->leased.fetch_add(c.leased, std::memory_order_relaxed);
+    c.leased += adopted;
     {
         std::lock_guard<std::mutex> g(ctx->q_mu);
         ctx->pending.push_back(std::move(c));
@@ -1247,6 +1329,30 @@ int check_product(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_bu
     return TM_HIP_OK;
 }
 
+// The operation tm_hip_q8_0_gemm_mma records for a product.
+Op mma_op(tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y, uint32_t rows, uint32_t cols,
+          uint32_t batch, uint32_t x_off, uint32_t y_off) {
+    Op op;
+    // Below this batch a 32-token MFMA tile is mostly padding and the vector
+    // kernels (GEMV arithmetic, which is within any tolerance of itself) are
+    // faster: 1 token -> the decode kernel, 2..16 -> the token-split kernel.
+    const bool small = w->alloc->packed && (batch == 1 || (batch <= 16 && cols >= 1024u));
+    op.kind = small ? OP_GEMV_LIST : OP_MMA;
+    op.a[0] = w->alloc;
+    op.a[1] = x->alloc;
+    op.a[2] = y->alloc;
+    op.n_alloc = 3;
+    op.writes_mask = 4;
+    op.rows = rows;
+    op.cols = cols;
+    op.batch = batch;
+    op.x_off = x_off;
+    op.y_off = y_off;
+    op.packed = w->alloc->packed;
+    op.what = "q8_0_gemm_mma";
+    return op;
+}
+
 // The stream must be idle with respect to the step's replays.
 void step_dispose(tm_hip_step *step) {
     (void)hipGraphExecDestroy(step->exec);
@@ -1294,21 +1400,38 @@ tm_hip_ctx *tm_hip_create(char *err, size_t err_cap) {
         tm_hip_destroy(ctx);
         return nullptr;
     }
-    e = hipMalloc((void **)&ctx->mma_queue, 256);
+    e = hipMalloc((void **)&ctx->ws.mma_queue, 256);
     if (e == hipSuccess) {
-        e = hipMemset(ctx->mma_queue, 0, 256);
+        e = hipMemset(ctx->ws.mma_queue, 0, 256);
     }
     if (e == hipSuccess) {
-        e = hipMalloc((void **)&ctx->bx3_arrivals, q8::BX3_MAX_SPLIT_TILES * sizeof(uint32_t));
+        e = hipMalloc((void **)&ctx->ws.arrivals, q8::BX3_MAX_SPLIT_TILES * sizeof(uint32_t));
     }
     if (e == hipSuccess) {
-        e = hipMemset(ctx->bx3_arrivals, 0, q8::BX3_MAX_SPLIT_TILES * sizeof(uint32_t));
+        e = hipMemset(ctx->ws.arrivals, 0, q8::BX3_MAX_SPLIT_TILES * sizeof(uint32_t));
     }
     if (e != hipSuccess) {
         hip_fail(err, err_cap, "device-side counters", e);
         tm_hip_destroy(ctx);
         return nullptr;
     }
+    // The static workspace of the entry point that allocates nothing: this
+    // device's address of the array, asked here, with the device current.
+    uint8_t *fixed = nullptr;
+    e = scratch_on_current_device(ctx->device, &fixed);
+    if (e != hipSuccess) {
+        fail(err, err_cap, TM_HIP_ERR_SOURCE, "static workspace of this device is missing: %s",
+             hipGetErrorString(e));
+        tm_hip_destroy(ctx);
+        return nullptr;
+    }
+    ctx->fixed.mma_queue = (uint32_t *)(fixed + kScratchQueueOff);
+    ctx->fixed.arrivals = (uint32_t *)(fixed + kScratchArrivalsOff);
+    ctx->fixed.xs = fixed + kScratchXsOff;
+    ctx->fixed.xs_bytes = kScratchXsBytes;
+    ctx->fixed.partials = (float *)(fixed + kScratchPartialOff);
+    ctx->fixed.partial_bytes = kScratchPartialBytes;
+    ctx->noalloc_keep.reserve(kNoallocKeepCap);
     // Fail at creation, not at first use, when the device code is missing.
     hipFuncAttributes attr;
     e = hipFuncGetAttributes(&attr, (const void *)q8::gemv_list_kernel<q8::PACKED, kGemvR1, 1, true, 0>);
@@ -1354,10 +1477,9 @@ void tm_hip_destroy(tm_hip_ctx *ctx) {
         }
         ctx->event_pool.clear();
     }
-    if (ctx->mma_queue != nullptr) {
-        (void)hipFree(ctx->mma_queue);
-    }
-    for (void *p : {(void *)ctx->bx3_arrivals, (void *)ctx->bx3_xs, (void *)ctx->bx3_partials}) {
+    noalloc_release(ctx);
+    for (void *p : {(void *)ctx->ws.mma_queue, (void *)ctx->ws.arrivals, (void *)ctx->ws.xs,
+                    (void *)ctx->ws.partials}) {
         if (p != nullptr) {
             (void)hipFree(p);
         }
@@ -1824,7 +1946,7 @@ int tm_hip_end_group_recorded(tm_hip_ctx *ctx, tm_hip_step **out, char *err, siz
     hipError_t launch_err = hipSuccess;
     for (const Launch &l : plan) {
         launch_err = l.single != nullptr ? launch_single(ctx, nullptr, *l.single)
-                                         : launch_gemv_list(ctx, nullptr, l);
+                                         : launch_gemv_list(ctx, nullptr, l, ctx->ws);
         if (launch_err != hipSuccess) {
             break;
         }
@@ -1984,24 +2106,83 @@ int tm_hip_q8_0_gemm_mma(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm
     if (rc != TM_HIP_OK) {
         return rc;
     }
-    Op op;
-    // Below this batch a 32-token MFMA tile is mostly padding and the vector
-    // kernels (GEMV arithmetic, which is within any tolerance of itself) are
-    // faster: 1 token -> the decode kernel, 2..16 -> the token-split kernel.
-    const bool small = w->alloc->packed && (batch == 1 || (batch <= 16 && cols >= 1024u));
-    op.kind = small ? OP_GEMV_LIST : OP_MMA;
-    op.a[0] = w->alloc;
-    op.a[1] = x->alloc;
-    op.a[2] = y->alloc;
-    op.n_alloc = 3;
-    op.writes_mask = 4;
-    op.rows = rows;
-    op.cols = cols;
-    op.batch = batch;
-    op.x_off = x_off;
-    op.y_off = y_off;
-    op.packed = w->alloc->packed;
+    Op op = mma_op(w, x, y, rows, cols, batch, x_off, y_off);
     return submit(ctx, op, "q8_0_gemm_mma", err, err_cap);
+}
+
+int tm_hip_q8_0_gemm_mma_noalloc(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x,
+                                 tm_hip_buffer *y, uint32_t rows, uint32_t cols, uint32_t batch,
+                                 uint32_t x_off, uint32_t y_off, char *err, size_t err_cap) {
+    const char *what = "q8_0_gemm_mma_noalloc";
+    int rc = check_product(ctx, w, x, y, rows, cols, batch, TM_HIP_GEMM_MMA_MAX_BATCH, x_off, y_off,
+                           err, err_cap, what);
+    if (rc != TM_HIP_OK) {
+        return rc;
+    }
+    if (ctx->group_active) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "%s: launches at once, not into the open dispatch group; close the group first",
+                    what);
+    }
+    const Op op = mma_op(w, x, y, rows, cols, batch, x_off, y_off);
+    Launch launch;
+    launch.key = gemv_key(op);
+    launch.list.push_back(&op);
+    launch.residual.push_back(nullptr);
+    launch.glu.push_back(nullptr);
+    launch.normed.push_back(false);
+    bool counters = launch.key.kind == OP_MMA; // the work-queue form of the f32 kernel may run
+    if (launch.key.variant == V_BF16X3) {
+        const q8::Bx3Plan plan = q8::bx3_plan(rows, cols, batch);
+        launch.bx3_split_tiles = plan.split_tiles;
+        launch.bx3_partial_floats = plan.partial_floats;
+        launch.bx3_xs_bytes = bx3_xs_bytes_of(op);
+        launch.bx3_inputs = 1;
+        if (launch.bx3_xs_bytes > ctx->fixed.xs_bytes ||
+            launch.bx3_partial_floats * 4u > ctx->fixed.partial_bytes) {
+            return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                        "%s: %u tokens x %u columns on %u rows need %llu bytes of split activations "
+                        "and %llu bytes of partial tiles, the static workspace holds %zu and %zu; "
+                        "use q8_0_gemm_mma, or fewer tokens per call",
+                        what, batch, cols, rows, (unsigned long long)launch.bx3_xs_bytes,
+                        (unsigned long long)(launch.bx3_partial_floats * 4u), ctx->fixed.xs_bytes,
+                        ctx->fixed.partial_bytes);
+        }
+        counters = plan.split_tiles > 0;
+    }
+    if (ctx->noalloc_keep.size() + 3u > kNoallocKeepCap) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "%s: %zu buffers of earlier calls are still held; commit other work or call "
+                    "fence first",
+                    what, ctx->noalloc_keep.size());
+    }
+    // Held until the next commit adopts them or a fence has passed them (the list
+    // has its capacity from tm_hip_create on).
+    for (int i = 0; i < 3; ++i) {
+        op.a[i]->refs.fetch_add(1, std::memory_order_relaxed);
+        ctx->noalloc_keep.push_back(op.a[i]);
+        ctx->noalloc_leased += op.a[i]->len;
+        ctx->leased.fetch_add(op.a[i]->len, std::memory_order_relaxed);
+    }
+    if (counters) {
+        // The array keeps what the last call left in it, and every call on this
+        // GPU shares it: the counters start from zero whatever came before. A
+        // fill kernel, not a memset, so that a caller may record the call.
+        hipLaunchKernelGGL(q8::zero_u32_kernel, dim3((unsigned)((kScratchCounterDwords + 255u) / 256u)),
+                           dim3(256), 0, ctx->stream, (uint32_t *)ctx->fixed.mma_queue,
+                           (uint32_t)kScratchCounterDwords);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            return hip_fail(err, err_cap, what, e);
+        }
+        ctx->launches.fetch_add(1, std::memory_order_relaxed);
+    }
+    const hipError_t e = launch_gemv_list(ctx, nullptr, launch, ctx->fixed);
+    if (e != hipSuccess) {
+        return hip_fail(err, err_cap, what, e);
+    }
+    ctx->launches.fetch_add(kernel_launches_of(launch), std::memory_order_relaxed);
+    return TM_HIP_OK;
 }
 
 int tm_hip_q8_0_row_f32(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *out, uint32_t row,

@@ -65,6 +65,8 @@ def gemm_mma_on_bf16(rows: int, cols: int, batch: int, x_off: int = 0) -> bool:
             gemm_mma_bf16_plan(rows, cols, batch)[2])
 
 
+NOALLOC_WORKSPACE_BYTES = 64 << 20  # TM_HIP_NOALLOC_WORKSPACE_BYTES
+NOALLOC_XS_BYTES = 20 << 20
 GEMM_I8_MAX_BATCH = 2048
 ARGMAX_NONE = 0xFFFFFFFF  # crates/metal/src/lib.rs (ARGMAX_NONE), native/metal/kernels.metal:143
 ARGMAX_PARTIAL_BYTES = 512
@@ -160,6 +162,8 @@ _SIGS = {
                          [ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_q8_0_gemm_mma": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_uint32] * 5 +
                              [ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_q8_0_gemm_mma_noalloc": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_uint32] * 5 +
+                                     [ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_q8_0_row_f32": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_uint32] * 3 +
                             [ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_f16_gemv": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_uint32] * 2 +
@@ -339,6 +343,13 @@ class HipContext:
         self._check_owned(w, x, y)
         self._operate("q8_0_gemm_mma", self._lib.tm_hip_q8_0_gemm_mma, w.raw, x.raw, y.raw, rows,
                       cols, batch, x_off, y_off)
+
+    def q8_0_gemm_mma_noalloc(self, w, x, y, rows, cols, batch, x_off=0, y_off=0):
+        """q8_0_gemm_mma launched at once out of the library's static device
+        workspace: allocates nothing, is not a commit."""
+        self._check_owned(w, x, y)
+        self._operate("q8_0_gemm_mma_noalloc", self._lib.tm_hip_q8_0_gemm_mma_noalloc, w.raw, x.raw,
+                      y.raw, rows, cols, batch, x_off, y_off)
 
     def q8_0_row(self, w, out, row: int, cols: int, out_off: int = 0):
         self._check_owned(w, out)

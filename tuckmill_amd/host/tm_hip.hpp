@@ -275,6 +275,16 @@ class HipContext {
                                         y_off, e, ERR_CAP);
         });
     }
+    // q8_0_gemm_mma out of the library's static device workspace: allocates
+    // nothing on the device, launches at once, is not a commit.
+    void q8_0_gemm_mma_noalloc(const HipBuffer &w, const HipBuffer &x, const HipBuffer &y,
+                               uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off,
+                               uint32_t y_off) const {
+        operate("q8_0_gemm_mma_noalloc", [&](char *e) {
+            return tm_hip_q8_0_gemm_mma_noalloc(raw(), w.raw(), x.raw(), y.raw(), rows, cols, batch,
+                                                x_off, y_off, e, ERR_CAP);
+        });
+    }
     void q8_0_row(const HipBuffer &w, const HipBuffer &out, uint32_t row, uint32_t cols,
                   uint32_t out_off) const {
         operate("q8_0_row", [&](char *e) {
