@@ -206,13 +206,16 @@ int tm_hip_q8_0_gemm(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip
 
 /* Same contract for batch 1..=TM_HIP_GEMM_MMA_MAX_BATCH on the MFMA matrix
  * cores: every product q*x is exact (f32 operand tiles with W dequantized
- * exactly as d*q; or, for large products over sealed weights from 33
- * tokens, bf16 tiles with every activation split into three exact bf16
- * pieces). Summation order differs from the GEMV: tolerance-qualified, not
- * bit-identical (native/metal/tm_metal.h:172-178). A product's result does not
- * depend on what shares its dispatch group. The large-product form keeps a
- * workspace in the context (6 bytes per activation element plus partial
- * tiles), grown on first use and freed with the context. */
+ * exactly as d*q; or, from 33 tokens over sealed weights, bf16 tiles with
+ * every activation split into three exact bf16 pieces). Summation order
+ * differs from the GEMV: tolerance-qualified, not bit-identical
+ * (native/metal/tm_metal.h:172-178). Which of the two forms runs, and how K is
+ * cut, is decided per launch from the products that share it (independent
+ * products of one dispatch group): the same group gives the same bits every
+ * time, on every replay of a recorded step too, but a product's last bits may
+ * differ between groupings. The bf16 form keeps a workspace in the context
+ * (6 bytes per activation element plus partial tiles), grown on first use and
+ * freed with the context. */
 int tm_hip_q8_0_gemm_mma(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y,
                          uint32_t rows, uint32_t cols, uint32_t batch, uint32_t x_off,
                          uint32_t y_off, char *err, size_t err_cap);

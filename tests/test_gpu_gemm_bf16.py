@@ -119,19 +119,22 @@ def test_activations_off_a_16_byte_boundary_take_the_f32_kernels(ctx):
     wb.free()
 
 
-def test_a_group_splits_each_input_once_and_has_the_bits_of_its_products_alone(ctx):
+def test_a_group_splits_each_input_once_and_is_deterministic(ctx):
     # q/k/v share their activations, o and down have their own (K of 2 and 3
     # chunks: partial tiles added by whichever chunk arrives last, in chunk
-    # order). Twice: the second launch finds the arrival counters as the first
-    # left them. A replayed recording of the group gives the same bits again.
+    # order). The second product would be too small on its own; the launch
+    # decides for all of them together, so all six share one launch (plus the one
+    # that splits the three distinct inputs). Three times: every launch finds the
+    # arrival counters as the last left them and gives the same bits; a replayed
+    # recording of the group gives them again.
     batch = 512
     xs = {c: S.make_activations(batch * c, c) for c in (1024, 2048, 3072)}
     xbs = {c: upload_new(ctx, x) for c, x in xs.items()}
     mats = []
-    # (the second one is too small to fill the chip and runs on the f32 matrix
-    # cores, in a launch of its own; the others still share theirs)
-    for i, (rows, cols) in enumerate([(8192, 1024), (1024, 1024), (9000, 1024), (8192, 1024),
-                                      (4096, 2048), (4100, 3072)]):
+    shapes = [(8192, 1024), (1024, 1024), (9000, 1024), (8192, 1024), (4096, 2048), (4100, 3072)]
+    assert not H.gemm_mma_on_bf16(1024, 1024, batch)
+    assert H.gemm_mma_launch_tile([(r, c, batch) for r, c in shapes]) == 128
+    for i, (rows, cols) in enumerate(shapes):
         w = S.make_weights(rows, cols, 600 + i)
         mats.append((w, rows, cols, weights_buffer(ctx, w, rows, cols, True),
                      ctx.buffer(batch * rows * 4)))
@@ -141,26 +144,33 @@ def test_a_group_splits_each_input_once_and_has_the_bits_of_its_products_alone(c
             ctx.q8_0_gemm_mma(wb, xbs[cols], yb, rows, cols, batch, 0, 0)
 
     launches = ctx.kernel_launches()
-    for _ in range(2):
+    runs = []
+    for _ in range(3):
         for m in mats:
             m[4].zero(0, batch * m[1] * 4)
         ctx.begin_group()
         encode()
         ctx.end_group()
         ctx.fence()
-    assert ctx.kernel_launches() == launches + 6
-    grouped = [m[4].download_f32(0, batch * m[1]).copy() for m in mats]
+        runs.append([m[4].download_f32(0, batch * m[1]).copy() for m in mats])
+    assert ctx.kernel_launches() == launches + 3 * 2
+    grouped = runs[0]
+    picked = [0, 1, 77, 255, 256, 510, 511]
     for i, (w, rows, cols, wb, yb) in enumerate(mats):
-        alone = product(ctx, wb, xs[cols], rows, cols, batch)
-        assert np.array_equal(bits(grouped[i]), bits(alone)), f"product {i}"
+        assert np.array_equal(bits(grouped[i]), bits(runs[1][i])), f"product {i}"
+        assert np.array_equal(bits(grouped[i]), bits(runs[2][i])), f"product {i}"
         if i in (2, 5):
             want = O.gemm_q8_0_f32(w, rows, cols, xs[cols], batch, threads=8)
             assert norm_err(grouped[i].reshape(batch, rows), want) <= 1e-5
+        else:
+            x = np.ascontiguousarray(xs[cols].reshape(batch, cols)[picked]).reshape(-1)
+            want = O.gemm_q8_0_f32(w, rows, cols, x, len(picked), threads=8)
+            assert norm_err(grouped[i].reshape(batch, rows)[picked], want) <= 1e-5
 
     ctx.begin_group()
     encode()
     step = ctx.end_group_recorded()
-    assert step.launches == 3
+    assert step.launches == 2
     for replay in range(3):
         for m in mats:
             m[4].zero(0, batch * m[1] * 4)

@@ -46,3 +46,22 @@ def test_which_products_take_the_bf16_matrix_cores():
     # activations must start on a 16-byte boundary
     assert not H.gemm_mma_on_bf16(8192, 1024, 512, x_off=3)
     assert H.gemm_mma_on_bf16(8192, 1024, 512, x_off=32)
+
+
+def test_products_that_share_a_launch_decide_together():
+    tile = H.gemm_mma_launch_tile
+    M = 512
+    layer = {name: (rows, cols, M) for name, rows, cols in S.QWEN3_0_6B_LAYER}
+    # alone, only gate and up are large enough (tiles of 64 tokens) ...
+    assert [tile([layer[n]]) for n in ("q", "k", "v", "o", "gate", "up", "down")] == \
+        [0, 0, 0, 0, 64, 64, 0]
+    # ... all seven in one launch have 480 units of the large tile between them
+    assert tile(list(layer.values())) == 128
+    # the dependent layer's launches: q, k, v together and gate, up together take
+    # the small tile; o and down, alone in theirs, stay on the f32 matrix cores
+    assert tile([layer["q"], layer["k"], layer["v"]]) == 64
+    assert tile([layer["gate"], layer["up"]]) == 128
+    assert tile([layer["o"]]) == 0 and tile([layer["down"]]) == 0
+    # up to 64 tokens: 16 M weights between them
+    assert tile([(6144, 2048, 64)]) == 0 and tile([(6144, 2048, 64), (6144, 2048, 64)]) == 64
+    assert tile([]) == 0

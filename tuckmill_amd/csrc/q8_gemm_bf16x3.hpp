@@ -472,8 +472,8 @@ struct Bx3Product {
     uint32_t rows, cols, batch;
 };
 
-// How a product is cut into work units (output tile x K chunk). A function of
-// the product's shape only: its result does not depend on what shares its launch.
+// How a product is cut into work units (output tile x K chunk): a function of
+// the product's shape and of the tile its launch uses.
 //
 // Tile: 256 rows x 128 tokens (2 x 4 waves, two per SIMD), or x 64 tokens (1 x 4
 // waves, one per SIMD) for some products that would make fewer than 192 units
@@ -522,39 +522,63 @@ inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint3
     return p;
 }
 
-// The plan of a product, and whether the kernel pays for it on its own
-// (`worth`). Above 64 tokens, in order of preference: the large tile with 192 units or more; the
-// small tile with 192 units or more in at most 4 K chunks (1024 x 3072 at 512
-// tokens in six chunks: 40 us against 32 on the f32 kernel); the large tile with
-// 128 units or more (alone about even with the f32 kernel, far ahead when
-// products share a launch). Measured alone at 512 tokens against the f32
-// kernel: small tile 3072 x 1024 34 against 35 us, 2048 x 2048 39 against 49,
-// 4096 x 1024 36 against 48, 2048 x 1024 (128 units) 31 against 28; large tile
-// 8192 x 1024 49 against 93, 6144 x 2048 69 against 133.
+// Which tile the products of one launch take together, or 0 when the kernel does
+// not pay for them: the rule of a single product, with the launch's sums in the
+// place of the product's own figures (`shapes` = rows, cols, batch of every
+// product; all with batch <= 64 or all above).
+//
+// Up to 64 tokens there is one small tile of tokens. The kernel's time hardly
+// depends on the batch here (27 us for 8192 x 1024, 97 us for 151936 x 1024), the
+// f32 kernel's does: from 33 tokens (its 64-token tile) 16 M weights are the
+// break-even (16384 x 1024 at 64 tokens: 30 against 29 us; 4096 x 4096: 34 against
+// 47; 151936 x 1024: 97 against 219). At 32 tokens and below only the largest
+// matrices would gain, and little.
+//
+// Above 64 tokens, in order of preference: the large tile with 192 units or more;
+// the small tile with 192 units or more in at most 4 K chunks per product (1024 x
+// 3072 at 512 tokens in six chunks: 40 us against 32 on the f32 kernel); the large
+// tile with 128 units or more (a product alone is then about even with the f32
+// kernel, products that share a launch far ahead). Measured alone at 512 tokens
+// against the f32 kernel: small tile 3072 x 1024 34 against 35 us, 2048 x 2048 39
+// against 49, 4096 x 1024 36 against 48, 2048 x 1024 (128 units) 31 against 28;
+// large tile 8192 x 1024 49 against 93, 6144 x 2048 69 against 133. Together: the
+// seven Qwen3-0.6B projections at 512 tokens 78 us on the large tile against 144
+// on the f32 kernel.
+struct Bx3Shape3 {
+    uint32_t rows, cols, batch;
+};
+
+inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
+    if (n <= 0) {
+        return 0;
+    }
+    uint64_t large = 0, small = 0, weights = 0;
+    uint32_t small_chunks = 0;
+    for (int i = 0; i < n; ++i) {
+        const Bx3Plan s = bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 64u);
+        small += s.units;
+        small_chunks = s.chunks > small_chunks ? s.chunks : small_chunks;
+        large += bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 128u).units;
+        weights += (uint64_t)shapes[i].rows * shapes[i].cols;
+    }
+    if (shapes[0].batch <= 64u) {
+        return weights >= (1ull << 24) && small >= 128u ? 64u : 0u;
+    }
+    if (large >= BX3_UNITS_WANTED) {
+        return 128u;
+    }
+    if (small >= BX3_UNITS_WANTED && small_chunks <= 4u) {
+        return 64u;
+    }
+    return large >= 128u ? 128u : 0u;
+}
+
+// A product on its own: its plan, and whether the kernel pays for it (`worth`).
 inline Bx3Plan bx3_plan(uint32_t rows, uint32_t cols, uint32_t batch, bool *worth) {
-    if (batch <= 64u) {
-        // One small tile of tokens. The kernel's time hardly depends on the
-        // batch here (27 us for 8192 x 1024, 97 us for 151936 x 1024), the f32
-        // kernel's does: from 33 tokens (its 64-token tile) a matrix of 16 M
-        // weights is the break-even (16384 x 1024 at 64 tokens: 30 against 29 us;
-        // 4096 x 4096: 34 against 47; 151936 x 1024: 97 against 219). At 32
-        // tokens and below only the largest matrices would gain, and little.
-        const Bx3Plan one = bx3_plan_with(rows, cols, batch, 64u);
-        *worth = (uint64_t)rows * cols >= (1ull << 24) && one.units >= 128u;
-        return one;
-    }
-    const Bx3Plan large = bx3_plan_with(rows, cols, batch, 128u);
-    if (large.units >= BX3_UNITS_WANTED) {
-        *worth = true;
-        return large;
-    }
-    const Bx3Plan small = bx3_plan_with(rows, cols, batch, 64u);
-    if (small.units >= BX3_UNITS_WANTED && small.chunks <= 4u) {
-        *worth = true;
-        return small;
-    }
-    *worth = large.units >= 128u;
-    return large;
+    const Bx3Shape3 one{rows, cols, batch};
+    const uint32_t tile = bx3_launch_tile(&one, 1);
+    *worth = tile != 0u;
+    return bx3_plan_with(rows, cols, batch, tile != 0u ? tile : (batch <= 64u ? 64u : 128u));
 }
 inline Bx3Plan bx3_plan(uint32_t rows, uint32_t cols, uint32_t batch) {
     bool worth;
@@ -590,10 +614,9 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
         d.cols = prods[i].cols;
         d.batch = prods[i].batch;
         d.tile_begin = (uint32_t)units;
-        const Bx3Plan plan = bx3_plan(prods[i].rows, prods[i].cols, prods[i].batch);
-        if (plan.tile_tokens != (uint32_t)Sh::tokens) {
-            return hipErrorInvalidValue; // the caller lists products of one tile shape
-        }
+        // K chunks as the product's shape and the launch's tile say
+        const Bx3Plan plan = bx3_plan_with(prods[i].rows, prods[i].cols, prods[i].batch,
+                                           (uint32_t)Sh::tokens);
         d.tiles_t = (prods[i].batch + Sh::tokens - 1) / Sh::tokens;
         d.chunk_blocks = plan.chunk_blocks;
         d.chunks = plan.chunks;
@@ -618,9 +641,9 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
     return hipGetLastError();
 }
 
-// Sealed weights, every region below 4 GiB (32-bit buffer offsets), every
-// product's plan with `tile_tokens`: the caller checks these before choosing
-// this kernel. `partials` holds the sum of the products' partial_floats,
+// Sealed weights, every region below 4 GiB (32-bit buffer offsets): the caller
+// checks these before choosing this kernel; every product is planned with
+// bx3_plan_with(..., tile_tokens). `partials` holds the sum of the products' partial_floats,
 // `arrivals` BX3_MAX_SPLIT_TILES counters that are zero between launches (both
 // may be null when no product's K is cut into chunks).
 inline hipError_t launch_gemm_bf16x3_list(hipStream_t stream, hipEvent_t stop, uint32_t tile_tokens,

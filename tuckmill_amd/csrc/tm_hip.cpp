@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <chrono>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -362,6 +363,23 @@ void settle(tm_hip_ctx *ctx) {
 }
 
 int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
+    // A decode step lasts about 0.1 ms and its token is wanted at once: poll the
+    // last commit's stop event for a while before handing the wait to the
+    // runtime, whose wake-up alone costs tens of microseconds.
+    hipEvent_t last = nullptr;
+    {
+        std::lock_guard<std::mutex> g(ctx->q_mu);
+        if (!ctx->pending.empty()) {
+            last = ctx->pending.back().stop;
+        }
+    }
+    if (last != nullptr) {
+        const auto t0 = std::chrono::steady_clock::now();
+        while (hipEventQuery(last) == hipErrorNotReady &&
+               std::chrono::steady_clock::now() - t0 < std::chrono::milliseconds(2)) {
+        }
+        (void)hipGetLastError(); // "not ready" is not an error to keep
+    }
     hipError_t e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
         return hip_fail(err, cap, "stream synchronize", e);
@@ -408,31 +426,66 @@ struct GemvKey {
 };
 
 // Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 33
-// tokens, and with enough work units (256 rows x 128 or 64 tokens x K chunk)
-// of their own for the kernel to pay (q8::bx3_plan has the rule and the
-// measurements behind it). The kernel is two to three times as fast as the f32
-// one when it fills the chip (at 512 tokens 14336 x 4096: 204 us against 640 us,
-// 6144 x 2048: 69 against 133; at 96 tokens 14336 x 4096: 73 against 173) but its
-// units are large: 1024 x 1024 at 512 tokens takes 48 us against 15 us, and 33 us
-// with K in four chunks; at 32 tokens and below the f32 kernels win or tie on
-// most shapes. A product's kernel depends on nothing but its own shape and
-// alignment, so its result does not depend on what shares its launch.
+// tokens, and when the products that share the launch have enough work units
+// (256 rows x 128 or 64 tokens x K chunk) between them for the kernel to pay
+// (q8::bx3_launch_tile has the rule and the measurements behind it). The kernel
+// is two to three times as fast as the f32 one when it fills the chip (at 512
+// tokens 14336 x 4096: 204 us against 640 us, 6144 x 2048: 69 against 133; at 96
+// tokens 14336 x 4096: 73 against 173) but its units are large: 1024 x 1024 at 512
+// tokens takes 48 us alone against 15 us, while the seven projections of a
+// Qwen3-0.6B layer together take 78 us against 144. The choice is made per launch:
+// the same group gives the same bits every time, but a product's bits may depend
+// on what shares its launch (the entry point is tolerance-qualified,
+// native/metal/tm_metal.h:172-175; bit-identity claims belong to q8_0_gemm).
 constexpr uint32_t kBx3MinBatch = 33;
 constexpr uint64_t kBx3MaxPartialFloats = 1ull << 29; // 2 GiB of partial tiles per launch
 
-bool bx3_eligible(const Op &op, bool x_aligned) {
-    if (!op.packed || !x_aligned || op.batch < kBx3MinBatch ||
-        (uint64_t)op.rows * op.cols >= (1ull << 32) ||
-        (uint64_t)op.batch * op.cols * 6u >= (1ull << 32) ||
-        (uint64_t)op.batch * op.cols >= (1ull << 30)) {
-        return false;
-    }
-    bool worth = false;
-    const q8::Bx3Plan plan = q8::bx3_plan(op.rows, op.cols, op.batch, &worth);
-    return worth && plan.split_tiles <= q8::BX3_MAX_SPLIT_TILES &&
-           plan.partial_floats <= kBx3MaxPartialFloats;
+bool x_aligned_of(const Op &op) {
+    return ((uintptr_t)op.a[1]->ptr + (uintptr_t)op.x_off * 4u) % 16u == 0;
 }
 
+// The product could run on the bf16 matrix cores at all (its launch decides
+// whether it does).
+bool bx3_admissible(const Op &op) {
+    return op.kind == OP_MMA && op.packed && x_aligned_of(op) && op.batch >= kBx3MinBatch &&
+           (uint64_t)op.rows * op.cols < (1ull << 32) &&
+           (uint64_t)op.batch * op.cols * 6u < (1ull << 32) &&
+           (uint64_t)op.batch * op.cols < (1ull << 30);
+}
+
+bool bx3_fits(const Op &op, uint32_t tile_tokens) {
+    const q8::Bx3Plan plan = q8::bx3_plan_with(op.rows, op.cols, op.batch, tile_tokens);
+    return plan.split_tiles <= q8::BX3_MAX_SPLIT_TILES && plan.partial_floats <= kBx3MaxPartialFloats;
+}
+
+GemvKey bx3_key(uint32_t tile_tokens) {
+    GemvKey k;
+    k.kind = OP_MMA;
+    k.variant = V_BF16X3;
+    k.p0 = (uint8_t)(tile_tokens / 64u); // 2 or 1
+    k.packed = true;
+    k.flag = true;
+    return k;
+}
+
+// The f32 matrix-core kernel's key: tile shape and K split are chosen per
+// product, so its result does not depend on what else shares the launch.
+GemvKey mma_f32_key(const Op &op) {
+    GemvKey k;
+    k.kind = OP_MMA;
+    k.packed = op.packed;
+    k.flag = x_aligned_of(op);
+    const q8::MmaProduct p{nullptr, nullptr, nullptr, op.rows, op.cols, op.batch};
+    const q8::MmaConfig c = q8::pick_mma_config(&p, 1);
+    k.variant = V_MMA;
+    k.p0 = (uint8_t)c.tmw;
+    k.p1 = (uint8_t)c.tnw;
+    k.p2 = (uint8_t)c.s;
+    return k;
+}
+
+// The key of a product that launches on its own (for OP_MMA products inside a
+// group, assign_mma_keys decides per launch instead).
 GemvKey gemv_key(const Op &op) {
     GemvKey k;
     k.kind = op.kind;
@@ -460,23 +513,18 @@ GemvKey gemv_key(const Op &op) {
         k.flag = (op.cols & 7u) == 0u;
         return k;
     }
-    const uintptr_t xp = (uintptr_t)op.a[1]->ptr + (uintptr_t)op.x_off * 4u;
-    k.flag = (xp % 16u == 0);
-    if (op.kind == OP_MMA && bx3_eligible(op, k.flag)) {
-        k.variant = V_BF16X3;
-        k.p0 = (uint8_t)(q8::bx3_plan(op.rows, op.cols, op.batch).tile_tokens / 64u); // 2 or 1
-        return k;
-    }
     if (op.kind == OP_MMA) {
-        // The tile shape and K split are chosen per product, so a product's
-        // result does not depend on what else shares its launch.
-        const q8::MmaProduct p{nullptr, nullptr, nullptr, op.rows, op.cols, op.batch};
-        const q8::MmaConfig c = q8::pick_mma_config(&p, 1);
-        k.variant = V_MMA;
-        k.p0 = (uint8_t)c.tmw;
-        k.p1 = (uint8_t)c.tnw;
-        k.p2 = (uint8_t)c.s;
-    } else if (op.batch == 1) {
+        if (bx3_admissible(op)) {
+            const q8::Bx3Shape3 one{op.rows, op.cols, op.batch};
+            const uint32_t tile = q8::bx3_launch_tile(&one, 1);
+            if (tile != 0u && bx3_fits(op, tile)) {
+                return bx3_key(tile);
+            }
+        }
+        return mma_f32_key(op);
+    }
+    k.flag = x_aligned_of(op);
+    if (op.batch == 1) {
         k.variant = V_DECODE;
     } else if (op.packed && op.cols >= 1024u) {
         // waves x tokens per wave, measured on 2B-class shapes (the
@@ -929,11 +977,73 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
     return hipGetLastError();
 }
 
+// The kernel of every matrix-core product (OP_MMA) of a sequence, decided per
+// launch: consecutive products that do not depend on each other will share
+// launches, and whether the ones that could run on the bf16 matrix cores do is
+// decided on their sums (products of up to 64 tokens and of more form two pools,
+// each with the one tile q8::bx3_launch_tile gives it). The rest take the f32
+// kernels. Entries of other operations are left unset.
+std::vector<GemvKey> assign_mma_keys(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
+    std::vector<GemvKey> keys(ops.size());
+    std::vector<size_t> run;
+    uint64_t epoch = ++ctx->plan_epoch;
+    auto close = [&]() {
+        if (run.empty()) {
+            return;
+        }
+        for (size_t i : run) {
+            keys[i] = mma_f32_key(ops[i]);
+        }
+        for (int small_batch = 0; small_batch < 2; ++small_batch) {
+            std::vector<size_t> pool;
+            std::vector<q8::Bx3Shape3> shapes;
+            for (size_t i : run) {
+                const Op &op = ops[i];
+                if (bx3_admissible(op) && (op.batch <= 64u) == (small_batch != 0)) {
+                    pool.push_back(i);
+                    shapes.push_back(q8::Bx3Shape3{op.rows, op.cols, op.batch});
+                }
+            }
+            const uint32_t tile = q8::bx3_launch_tile(shapes.data(), (int)shapes.size());
+            if (tile == 0u) {
+                continue;
+            }
+            for (size_t i : pool) {
+                if (bx3_fits(ops[i], tile)) {
+                    keys[i] = bx3_key(tile);
+                }
+            }
+        }
+        run.clear();
+        epoch = ++ctx->plan_epoch;
+    };
+    for (size_t i = 0; i < ops.size(); ++i) {
+        const Op &op = ops[i];
+        if (op.kind != OP_MMA) {
+            close();
+            continue;
+        }
+        // the planner's own rule for sharing a launch (plan_launches below)
+        const bool conflict = op.a[2]->read_epoch == epoch || op.a[2]->write_epoch == epoch ||
+                              op.a[1]->write_epoch == epoch || op.a[0]->write_epoch == epoch;
+        if (conflict || (int)run.size() == q8::MMA_MAX_DESCS) {
+            close();
+        }
+        run.push_back(i);
+        op.a[0]->read_epoch = epoch;
+        op.a[1]->read_epoch = epoch;
+        op.a[2]->write_epoch = epoch;
+    }
+    close();
+    return keys;
+}
+
 // Plan the launches of a sequence of recorded operations. Consecutive
 // list-kernel products that neither read nor overwrite each other's outputs
 // share one launch; everything else launches on its own, in order.
 std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
     std::vector<Launch> plan;
+    const std::vector<GemvKey> mma_keys = assign_mma_keys(ctx, ops);
     Launch cur;
     // Open prefill launches set aside while a product of another kernel is
     // listed (see below); closed together with `cur`.
@@ -964,10 +1074,11 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
         cur = Launch();
         epoch = ++ctx->plan_epoch;
     };
-    for (const Op &op : ops) {
+    for (size_t op_index = 0; op_index < ops.size(); ++op_index) {
+        const Op &op = ops[op_index];
         if (op.kind == OP_GEMV_LIST || op.kind == OP_MMA || op.kind == OP_I8 ||
             op.kind == OP_F16_GEMM) {
-            const GemvKey key = gemv_key(op);
+            const GemvKey key = op.kind == OP_MMA ? mma_keys[op_index] : gemv_key(op);
             const int cap = key.kind == OP_MMA  ? q8::MMA_MAX_DESCS
                             : key.kind == OP_I8 ? q8::I8_MAX_DESCS
                                                 : q8::GEMV_MAX_DESCS;
@@ -1015,7 +1126,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                     new_input = new_input && !same_input(*other, op);
                 }
                 // the launch's share of the workspace stays within its limits
-                const q8::Bx3Plan mine = q8::bx3_plan(op.rows, op.cols, op.batch);
+                const q8::Bx3Plan mine = q8::bx3_plan_with(op.rows, op.cols, op.batch, key.p0 * 64u);
                 conflict = conflict ||
                            cur.bx3_split_tiles + mine.split_tiles > q8::BX3_MAX_SPLIT_TILES ||
                            cur.bx3_partial_floats + mine.partial_floats > kBx3MaxPartialFloats ||
@@ -1027,7 +1138,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 new_input = true;
             }
             if (key.variant == V_BF16X3) {
-                const q8::Bx3Plan mine = q8::bx3_plan(op.rows, op.cols, op.batch);
+                const q8::Bx3Plan mine = q8::bx3_plan_with(op.rows, op.cols, op.batch, key.p0 * 64u);
                 cur.bx3_split_tiles += mine.split_tiles;
                 cur.bx3_partial_floats += mine.partial_floats;
                 if (new_input) {
@@ -2133,7 +2244,7 @@ int tm_hip_q8_0_gemm_mma_noalloc(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffe
     launch.normed.push_back(false);
     bool counters = launch.key.kind == OP_MMA; // the work-queue form of the f32 kernel may run
     if (launch.key.variant == V_BF16X3) {
-        const q8::Bx3Plan plan = q8::bx3_plan(rows, cols, batch);
+        const q8::Bx3Plan plan = q8::bx3_plan_with(rows, cols, batch, launch.key.p0 * 64u);
         launch.bx3_split_tiles = plan.split_tiles;
         launch.bx3_partial_floats = plan.partial_floats;
         launch.bx3_xs_bytes = bx3_xs_bytes_of(op);

@@ -30,37 +30,55 @@ GEMM_MMA_MAX_BATCH = 512
 GEMM_MMA_BF16_MIN_BATCH = 33
 
 
-def gemm_mma_bf16_plan(rows: int, cols: int, batch: int):
-    """(tokens per tile, work units, worth it) for the bf16 matrix-core GEMM on a
-    product. A unit is 256 rows x 128 or 64 tokens x one K chunk; K is cut into
-    at most eight chunks of 512 columns or more, as many as give about 192
-    units. Up to 64 tokens the small tile, for matrices of 16 M weights and more
-    with 128 units or more; above, in order of preference: the large tile with 192 units or more, the
-    small tile with 192 units or more in at most 4 chunks, the large tile with
-    128 units or more (mirror of q8::bx3_plan, csrc/q8_gemm_bf16x3.hpp)."""
-    def plan(tokens):
-        tiles = -(-batch // tokens) * -(-rows // 256)
-        blocks = cols // 32
-        chunks = min(-(-192 // tiles), -(-blocks // 16), 8)
-        per_chunk = -(-blocks // chunks)
-        chunks = -(-blocks // per_chunk)
-        return tiles * chunks, chunks
-    if batch <= 64:  # one small tile of tokens: a matrix of 16 M weights is the break-even
-        units, _ = plan(64)
-        return 64, units, rows * cols >= 1 << 24 and units >= 128
-    large, _ = plan(128)
+def _bf16_units(rows: int, cols: int, batch: int, tokens: int):
+    """(work units, K chunks) of a product on the bf16 matrix-core GEMM with tiles
+    of `tokens` tokens x 256 rows: K is cut into at most eight chunks of 512
+    columns or more, as many as give the product about 192 units of its own
+    (mirror of q8::bx3_plan_with, csrc/q8_gemm_bf16x3.hpp)."""
+    tiles = -(-batch // tokens) * -(-rows // 256)
+    blocks = cols // 32
+    chunks = min(-(-192 // tiles), -(-blocks // 16), 8)
+    per_chunk = -(-blocks // chunks)
+    chunks = -(-blocks // per_chunk)
+    return tiles * chunks, chunks
+
+
+def gemm_mma_launch_tile(shapes) -> int:
+    """Tokens per tile (128 or 64) with which the products `shapes` = [(rows, cols,
+    batch), ...] that share one launch run on the bf16 matrix cores, or 0 when they
+    stay on the f32 ones (mirror of q8::bx3_launch_tile). All batches up to 64, or
+    all above. Up to 64 tokens: 16 M weights and 128 units of the small tile between
+    them. Above, in order of preference: 192 units or more of the large tile; 192 or
+    more of the small tile in at most 4 chunks per product; 128 or more of the large
+    tile."""
+    shapes = list(shapes)
+    if not shapes:
+        return 0
+    small = sum(_bf16_units(r, c, b, 64)[0] for r, c, b in shapes)
+    small_chunks = max(_bf16_units(r, c, b, 64)[1] for r, c, b in shapes)
+    large = sum(_bf16_units(r, c, b, 128)[0] for r, c, b in shapes)
+    if shapes[0][2] <= 64:
+        return 64 if sum(r * c for r, c, _ in shapes) >= 1 << 24 and small >= 128 else 0
     if large >= 192:
-        return 128, large, True
-    small, chunks = plan(64)
-    if small >= 192 and chunks <= 4:
-        return 64, small, True
-    return 128, large, large >= 128
+        return 128
+    if small >= 192 and small_chunks <= 4:
+        return 64
+    return 128 if large >= 128 else 0
+
+
+def gemm_mma_bf16_plan(rows: int, cols: int, batch: int):
+    """(tokens per tile, work units, worth it) of a product that launches alone."""
+    tile = gemm_mma_launch_tile([(rows, cols, batch)])
+    tokens = tile or (64 if batch <= 64 else 128)
+    return tokens, _bf16_units(rows, cols, batch, tokens)[0], tile != 0
 
 
 def gemm_mma_on_bf16(rows: int, cols: int, batch: int, x_off: int = 0) -> bool:
     """Whether tm_hip_q8_0_gemm_mma over sealed weights takes the bf16 matrix-core
-    kernel for this product (mirror of bx3_eligible, csrc/tm_hip.cpp; the limits
-    on region sizes beyond 4 GiB are left out)."""
+    kernel for this product when it launches alone (mirror of gemv_key,
+    csrc/tm_hip.cpp; the limits on region sizes beyond 4 GiB are left out). In a
+    dispatch group the products that share a launch decide together
+    (gemm_mma_launch_tile)."""
     return (batch >= GEMM_MMA_BF16_MIN_BATCH and x_off % 4 == 0 and
             gemm_mma_bf16_plan(rows, cols, batch)[2])
 

@@ -6,6 +6,7 @@
 // one commit per product when `grouped` is 0; `grouped` 2 records the group
 // once and replays it every step. The loop lives in native code so that the
 // measured time is the library's, not an interpreter's.
+#include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <cstring>
@@ -37,6 +38,10 @@ struct tmh_timing {
     double host_ms;     // host time spent issuing the timed steps (before the final fence)
     uint64_t launches;  // kernel launches issued by the timed steps
     uint64_t commits;
+    // GPU time per step from the commits' own events (a step's commits added up),
+    // as order statistics over the timed steps: the robust figures beside the mean
+    // gpu_ms / steps. Zero when a step's commits could not be told apart.
+    double step_us_median, step_us_min, step_us_p10, step_us_p90;
 };
 
 struct Bound {
@@ -91,6 +96,7 @@ int tmh_run_steps(tm_hip_ctx *ctx, const tmh_product *products, uint32_t n, uint
             one_step();
         }
         gpu.fence();
+        tm_hip_commit_log_set(ctx, 1);
         const uint64_t nanos0 = gpu.gpu_nanos_total();
         const uint64_t launches0 = gpu.kernel_launches();
         const uint64_t commits0 = gpu.committed_dispatches();
@@ -107,9 +113,26 @@ int tmh_run_steps(tm_hip_ctx *ctx, const tmh_product *products, uint32_t n, uint
             out->gpu_ms = (double)(gpu.gpu_nanos_total() - nanos0) / 1e6;
             out->launches = gpu.kernel_launches() - launches0;
             out->commits = gpu.committed_dispatches() - commits0;
+            out->step_us_median = out->step_us_min = out->step_us_p10 = out->step_us_p90 = 0.0;
+            std::vector<uint64_t> log(TM_HIP_COMMIT_LOG_CAP);
+            const size_t got = tm_hip_commit_log_read(ctx, log.data(), log.size());
+            const uint64_t per_step = steps > 0 ? out->commits / steps : 0;
+            if (steps > 0 && per_step > 0 && got == out->commits && per_step * steps == out->commits) {
+                std::vector<double> us(steps, 0.0);
+                for (size_t i = 0; i < got; ++i) {
+                    us[i / per_step] += (double)log[i] / 1e3;
+                }
+                std::sort(us.begin(), us.end());
+                out->step_us_min = us.front();
+                out->step_us_median = steps % 2 ? us[steps / 2] : 0.5 * (us[steps / 2 - 1] + us[steps / 2]);
+                out->step_us_p10 = us[(size_t)((steps - 1) * 0.1)];
+                out->step_us_p90 = us[(size_t)((steps - 1) * 0.9)];
+            }
         }
+        tm_hip_commit_log_set(ctx, 0);
         return 0;
     } catch (const TuckmillError &e) {
+        tm_hip_commit_log_set(ctx, 0);
         if (err != nullptr && err_cap > 0) {
             snprintf(err, err_cap, "%s", e.what());
         }
