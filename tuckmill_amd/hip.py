@@ -24,6 +24,7 @@ LIB_PATH = os.path.join(_HERE, "libtm_hip.so")
 ERR_CAP = 512  # crates/metal/src/lib.rs:32
 GEMM_MAX_BATCH = 32  # crates/metal/src/lib.rs:28-30
 GEMM_MMA_MAX_BATCH = 512
+PREFILL_BATCH = 128  # crates/tuckcore/src/engine/metal.rs:25 (the engine's prefill chunk)
 # From this batch on tm_hip_q8_0_gemm_mma over a large sealed matrix (128 or more tiles of
 # 128 tokens x 256 rows, K chunks counted) with 16-byte aligned activations runs on the bf16
 # matrix cores (activations split into three exact bf16 pieces).
@@ -117,6 +118,96 @@ def hip_error(abi_code: int, text: str, what: str) -> TuckmillError:
     else:
         code = "Internal"
     return TuckmillError(code, f"hip {what}: {text}", abi_code)
+
+
+# ---- kernel selection (crates/tuckcore/src/kernels.rs:36-113) -----------------
+
+class ResolvedKernels:
+    """A concrete kernel implementation actually used at runtime."""
+    SCALAR, NEON, METAL, HIP = "scalar", "neon", "metal", "hip"
+
+    @staticmethod
+    def default_for_target() -> str:
+        import platform
+        return ResolvedKernels.NEON if platform.machine() in ("aarch64", "arm64") \
+            else ResolvedKernels.SCALAR
+
+
+class KernelSelection:
+    """``--kernels`` as the reference parses it, with ``hip`` beside ``metal``. A
+    forced selection never falls back silently: ``hip`` without a usable gfx950
+    device is a typed refusal at load."""
+    NAMES = ("auto", "scalar", "neon", "metal", "hip")
+
+    def __init__(self, name: str):
+        self.name = name
+
+    def __eq__(self, other):
+        return isinstance(other, KernelSelection) and other.name == self.name
+
+    def __repr__(self):
+        return f"KernelSelection({self.name!r})"
+
+    @staticmethod
+    def parse(s: str):
+        """kernels.rs:46-54: None for an unknown name."""
+        return KernelSelection(s) if s in KernelSelection.NAMES else None
+
+    def resolve(self, device: "Probe | None" = None) -> str:
+        """kernels.rs:58-86. ``device`` stands in for the library's probe."""
+        import platform
+        import sys
+        if self.name == "scalar":
+            return ResolvedKernels.SCALAR
+        if self.name == "auto":  # never a GPU path unasked
+            return ResolvedKernels.default_for_target()
+        if self.name == "metal":
+            if sys.platform == "darwin":
+                return ResolvedKernels.METAL
+            raise TuckmillError("Unavailable", "the Metal kernel implementation requires macOS; "
+                                "select --kernels auto, hip, neon, or scalar on this machine")
+        if self.name == "neon":
+            if platform.machine() in ("aarch64", "arm64"):
+                return ResolvedKernels.NEON
+            raise TuckmillError("InvalidRequest", "the NEON kernel implementation requires an "
+                                "aarch64 target; select --kernels auto or --kernels scalar on this "
+                                "machine")
+        device = device if device is not None else probe()
+        if not device.available:
+            raise TuckmillError("Unavailable", "the HIP kernel implementation requires a gfx950 "
+                                f"device ({device.info}); select --kernels auto or scalar on this "
+                                "machine", TM_HIP_ERR_NO_DEVICE)
+        return ResolvedKernels.HIP
+
+
+# ---- numerical profile (crates/tuckcore/src/forward.rs:284-311) ---------------
+
+class NumericalProfile:
+    """``oracle-f32``: f32 activations, weights dequantized exactly. ``llama-cpu``:
+    activations quantized per 32 to Q8_0 for Q8_0 weights, int8 block dots."""
+    ORACLE_F32, LLAMA_CPU = "oracle-f32", "llama-cpu"
+
+    @staticmethod
+    def parse(s: str):
+        return s if s in (NumericalProfile.ORACLE_F32, NumericalProfile.LLAMA_CPU) else None
+
+
+def check_engine_options(kernels: str, profile: str, prefill_batch_given: bool = False):
+    """The load-time checks of crates/tuckcore/src/executor.rs:294-314 with a
+    device mode that covers Metal and HIP. The Metal path implements oracle-f32
+    only (typed refusal); the HIP path also implements llama-cpu for Q8_0 weights."""
+    device_mode = kernels in (ResolvedKernels.METAL, ResolvedKernels.HIP)
+    if not device_mode and prefill_batch_given:
+        raise TuckmillError("InvalidRequest", "prefill_batch applies only to the device kernel "
+                            "paths (metal, hip); the resolved CPU kernels execute single-token "
+                            "steps and must not silently ignore it")
+    if NumericalProfile.parse(profile) is None:
+        raise TuckmillError("InvalidRequest", f"unknown numerical profile {profile!r} "
+                            "(oracle-f32, llama-cpu)")
+    if kernels == ResolvedKernels.METAL and profile != NumericalProfile.ORACLE_F32:
+        raise TuckmillError("UnsupportedArchitecture", "the Metal path implements the oracle-f32 "
+                            "numerical profile only; select --numerical-profile oracle-f32, or "
+                            "--kernels hip for llama-cpu on a GPU")
 
 
 _lib = None
@@ -615,13 +706,22 @@ def xq_split(raw: np.ndarray, cols: int, batch: int):
 class Matrix:
     """A device projection matrix: the HIP form of the reference's ``Matrix``
     (crates/tuckcore/src/engine/metal.rs:106-226): Q8_0 blocks (type 8) or
-    F16 halves (type 1), uploaded raw."""
+    F16 halves (type 1), uploaded raw, with the numerical profile its products
+    run under (crates/tuckcore/src/forward.rs:606-645 switches per matvec):
+    ``oracle-f32`` (default), or ``llama-cpu`` for Q8_0 weights — activations
+    quantized per 32 on the device, int8 block dots, the f32 sum of
+    kernels.rs:206-221 bit for bit; the matrix owns and sizes the
+    quantized-activation buffer. F16 weights under ``llama-cpu`` have no device
+    kernel here: a typed refusal at load, never a substitution."""
 
-    def __init__(self, buf: HipBuffer, type_id: int, in_dim: int, out_dim: int):
+    def __init__(self, buf: HipBuffer, type_id: int, in_dim: int, out_dim: int,
+                 profile: str = NumericalProfile.ORACLE_F32):
         self.buf = buf
         self.type_id = type_id
         self.in_dim = in_dim
         self.out_dim = out_dim
+        self.profile = profile
+        self._xq = None  # quantized activations of the llama-cpu profile
 
     @staticmethod
     def plan(in_dim: int, out_dim: int, type_id: int = 8) -> int:
@@ -629,7 +729,7 @@ class Matrix:
 
     @staticmethod
     def load(ctx: HipContext, raw, in_dim: int, out_dim: int, type_id: int = 8,
-             seal: bool = True) -> "Matrix":
+             seal: bool = True, profile: str = NumericalProfile.ORACLE_F32) -> "Matrix":
         """Staged raw upload in 4 MiB slices (engine/metal.rs:138-147), then
         the seal step that re-lays the weights out for the device."""
         if out_dim <= 1:
@@ -637,6 +737,14 @@ class Matrix:
         if type_id not in (1, 8):
             raise TuckmillError("UnsupportedQuantization",
                                 f"engine matrices must be F16 or Q8_0; got type {type_id}")
+        if NumericalProfile.parse(profile) is None:
+            raise TuckmillError("InvalidRequest", f"unknown numerical profile {profile!r} "
+                                "(oracle-f32, llama-cpu)", TM_HIP_ERR_UNSUPPORTED)
+        if profile == NumericalProfile.LLAMA_CPU and type_id != 8:
+            raise TuckmillError("UnsupportedArchitecture",
+                                "the HIP path implements the llama-cpu numerical profile for Q8_0 "
+                                "weights only; F16 weights run under oracle-f32",
+                                TM_HIP_ERR_UNSUPPORTED)
         raw = np.ascontiguousarray(np.frombuffer(raw, dtype=np.uint8) if not
                                    isinstance(raw, np.ndarray) else raw).view(np.uint8).ravel()
         total = Matrix.plan(in_dim, out_dim, type_id)
@@ -651,16 +759,38 @@ class Matrix:
             off += n
         if seal and type_id == 8:
             ctx.q8_0_pack(buf, out_dim, in_dim)
-        return Matrix(buf, type_id, in_dim, out_dim)
+        return Matrix(buf, type_id, in_dim, out_dim, profile)
+
+    def _gemm_llama_cpu(self, ctx: HipContext, x: HipBuffer, y: HipBuffer, batch: int):
+        """forward.rs:783-821 on the device: quantize the activations once per
+        product, then the int8 product, in slices of GEMM_I8_MAX_BATCH tokens."""
+        rows, cols = self.out_dim, self.in_dim
+        t0 = 0
+        while t0 < batch:
+            n = min(batch - t0, GEMM_I8_MAX_BATCH)
+            need = xq_bytes(cols, n)
+            if self._xq is None or self._xq.len() < need:
+                # (a buffer replaced while an open group still names it stays alive:
+                # the group holds its memory)
+                self._xq = ctx.buffer(need, True)
+            ctx.q8_0_quantize_act(x, self._xq, cols, n, t0 * cols)
+            ctx.q8_0_gemm_i8(self.buf, self._xq, y, rows, cols, n, t0 * rows)
+            t0 += n
 
     def gemv(self, ctx: HipContext, x: HipBuffer, y: HipBuffer):
-        if self.type_id == 1:
+        if self.profile == NumericalProfile.LLAMA_CPU:
+            self._gemm_llama_cpu(ctx, x, y, 1)
+        elif self.type_id == 1:
             ctx.f16_gemv(self.buf, x, y, self.out_dim, self.in_dim)
         else:
             ctx.q8_0_gemv(self.buf, x, y, self.out_dim, self.in_dim)
 
     def gemm(self, ctx: HipContext, x: HipBuffer, y: HipBuffer, batch: int, exact: bool):
         rows, cols = self.out_dim, self.in_dim
+        if self.profile == NumericalProfile.LLAMA_CPU:
+            # exact whatever the batch: the int8 products are bit-identical to the CPU's
+            self._gemm_llama_cpu(ctx, x, y, batch)
+            return
         if not exact and self.type_id == 8 and 2 <= batch <= GEMM_MMA_MAX_BATCH:
             ctx.q8_0_gemm_mma(self.buf, x, y, rows, cols, batch, 0, 0)
             return

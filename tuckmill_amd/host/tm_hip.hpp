@@ -25,9 +25,14 @@ namespace tuckmill_hip {
 constexpr size_t ERR_CAP = 512;               // crates/metal/src/lib.rs:32
 constexpr uint32_t GEMM_MAX_BATCH = TM_HIP_GEMM_MAX_BATCH;
 constexpr uint32_t GEMM_MMA_MAX_BATCH = TM_HIP_GEMM_MMA_MAX_BATCH;
+constexpr uint32_t GEMM_I8_MAX_BATCH = TM_HIP_GEMM_I8_MAX_BATCH;
+constexpr uint32_t PREFILL_BATCH = 128;        // crates/tuckcore/src/engine/metal.rs:25
 constexpr size_t STAGING_CHUNK_BYTES = 4u << 20; // crates/tuckcore/src/qwen35_gpu.rs:1176
 
-enum class ErrorCode { InvalidRequest, Unavailable, Internal, UnsupportedQuantization, InvalidArtifact };
+enum class ErrorCode {
+    InvalidRequest, Unavailable, Internal, UnsupportedQuantization, InvalidArtifact,
+    UnsupportedArchitecture
+};
 
 class TuckmillError : public std::runtime_error {
   public:
@@ -58,6 +63,128 @@ struct Probe {
 };
 
 inline Probe probe() { return Probe{tm_hip_available() != 0, tm_hip_runtime_info()}; }
+
+// ---- kernel selection (crates/tuckcore/src/kernels.rs:36-113) ---------------
+//
+// `--kernels hip` next to auto / scalar / neon / metal. A forced selection never
+// falls back silently: `hip` on a machine without a usable gfx950 device is a
+// typed refusal at load, like `metal` off macOS and `neon` off aarch64.
+enum class ResolvedKernels { Scalar, Neon, Metal, Hip };
+
+inline const char *as_str(ResolvedKernels k) {
+    switch (k) {
+    case ResolvedKernels::Scalar: return "scalar";
+    case ResolvedKernels::Neon: return "neon";
+    case ResolvedKernels::Metal: return "metal";
+    case ResolvedKernels::Hip: return "hip";
+    }
+    return "scalar";
+}
+
+inline ResolvedKernels default_kernels_for_target() {
+#if defined(__aarch64__)
+    return ResolvedKernels::Neon;
+#else
+    return ResolvedKernels::Scalar;
+#endif
+}
+
+class KernelSelection {
+  public:
+    enum Kind { Auto, Scalar, Neon, Metal, Hip };
+    KernelSelection(Kind kind = Auto) : kind_(kind) {}
+    Kind kind() const { return kind_; }
+    bool operator==(const KernelSelection &o) const { return kind_ == o.kind_; }
+
+    // kernels.rs:46-54, with the new arm. `ok` is false for an unknown name.
+    static KernelSelection parse(const std::string &s, bool *ok) {
+        *ok = true;
+        if (s == "auto") return Auto;
+        if (s == "scalar") return Scalar;
+        if (s == "neon") return Neon;
+        if (s == "metal") return Metal;
+        if (s == "hip") return Hip;
+        *ok = false;
+        return Auto;
+    }
+
+    // kernels.rs:58-86. `device` answers whether a HIP device is usable (the
+    // library's probe by default; tests pass their own).
+    ResolvedKernels resolve(Probe device = probe()) const {
+        switch (kind_) {
+        case Scalar: return ResolvedKernels::Scalar;
+        case Auto: return default_kernels_for_target(); // never a GPU path unasked
+        case Metal:
+#if defined(__APPLE__)
+            return ResolvedKernels::Metal;
+#else
+            throw TuckmillError(ErrorCode::Unavailable,
+                                "the Metal kernel implementation requires macOS; select --kernels "
+                                "auto, hip, neon, or scalar on this machine");
+#endif
+        case Neon:
+#if defined(__aarch64__)
+            return ResolvedKernels::Neon;
+#else
+            throw TuckmillError(ErrorCode::InvalidRequest,
+                                "the NEON kernel implementation requires an aarch64 target; select "
+                                "--kernels auto or --kernels scalar on this machine");
+#endif
+        case Hip:
+            if (!device.available) {
+                throw TuckmillError(ErrorCode::Unavailable,
+                                    "the HIP kernel implementation requires a gfx950 device (" +
+                                        device.info + "); select --kernels auto or scalar on this machine",
+                                    TM_HIP_ERR_NO_DEVICE);
+            }
+            return ResolvedKernels::Hip;
+        }
+        return ResolvedKernels::Scalar;
+    }
+
+  private:
+    Kind kind_;
+};
+
+// ---- numerical profile (crates/tuckcore/src/forward.rs:284-311) -------------
+enum class NumericalProfile { OracleF32, LlamaCpu };
+
+inline bool parse_numerical_profile(const std::string &s, NumericalProfile *out) {
+    if (s == "oracle-f32") {
+        *out = NumericalProfile::OracleF32;
+        return true;
+    }
+    if (s == "llama-cpu") {
+        *out = NumericalProfile::LlamaCpu;
+        return true;
+    }
+    return false;
+}
+
+inline const char *as_str(NumericalProfile p) {
+    return p == NumericalProfile::OracleF32 ? "oracle-f32" : "llama-cpu";
+}
+
+// The load-time checks of crates/tuckcore/src/executor.rs:294-314 with a device
+// mode that covers Metal and HIP: a prefill batch only means something on a
+// device path; the Metal path implements oracle-f32 only (typed refusal, never
+// a silent substitution), the HIP path also implements llama-cpu for Q8_0
+// weights (activations quantized per 32, int8 block dots).
+inline void check_engine_options(ResolvedKernels kernels, NumericalProfile profile,
+                                 bool prefill_batch_given) {
+    const bool device_mode = kernels == ResolvedKernels::Metal || kernels == ResolvedKernels::Hip;
+    if (!device_mode && prefill_batch_given) {
+        throw TuckmillError(ErrorCode::InvalidRequest,
+                            "prefill_batch applies only to the device kernel paths (metal, hip); the "
+                            "resolved CPU kernels execute single-token steps and must not silently "
+                            "ignore it");
+    }
+    if (kernels == ResolvedKernels::Metal && profile != NumericalProfile::OracleF32) {
+        throw TuckmillError(ErrorCode::UnsupportedArchitecture,
+                            "the Metal path implements the oracle-f32 numerical profile only; select "
+                            "--numerical-profile oracle-f32, or --kernels hip for llama-cpu on a GPU");
+    }
+}
 
 struct ContextInner {
     tm_hip_ctx *raw = nullptr;
@@ -398,8 +525,23 @@ class HipContext {
     std::shared_ptr<ContextInner> inner_;
 };
 
-// A device projection matrix of Q8_0 weights
-// (crates/tuckcore/src/engine/metal.rs:106-226).
+// Bytes of a quantized-activation buffer (tm_hip_q8_0_quantize_act): batch * cols
+// int8 quants, then (cols / 32) x (batch rounded up to 4) f32 scales.
+inline size_t xq_bytes(uint32_t cols, uint32_t batch) {
+    const size_t bpad = ((size_t)batch + 3u) & ~(size_t)3u;
+    return (size_t)batch * cols + (size_t)(cols / 32u) * bpad * 4u;
+}
+
+// A device projection matrix (crates/tuckcore/src/engine/metal.rs:106-226) with
+// the numerical profile its products run under
+// (crates/tuckcore/src/forward.rs:606-645 switches per matvec):
+//   oracle-f32  f32 activations, weights dequantized exactly (the default);
+//   llama-cpu   Q8_0 weights: activations quantized per 32 on the device
+//               (tensor.rs:184-206), int8 block dots, the f32 sum of
+//               kernels.rs:206-221, bit for bit; the matrix owns the quantized
+//               activation buffer and sizes it. F16 weights under llama-cpu
+//               (activations rounded to f16, forward.rs:823-870) have no device
+//               kernel here: a typed refusal at load, never a substitution.
 class Matrix {
   public:
     static uint64_t plan(uint64_t in_dim, uint64_t out_dim, uint32_t type_id = 8) {
@@ -409,13 +551,20 @@ class Matrix {
     // Staged raw upload in 4 MiB slices (engine/metal.rs:138-147), then the
     // seal step that re-lays the weights out for coalesced device loads.
     static Matrix load(const HipContext &gpu, const uint8_t *raw, uint64_t in_dim, uint64_t out_dim,
-                       uint32_t type_id = 8, bool seal = true) {
+                       uint32_t type_id = 8, bool seal = true,
+                       NumericalProfile profile = NumericalProfile::OracleF32) {
         if (out_dim <= 1) {
             throw TuckmillError(ErrorCode::Internal, "1-D tensors use the f32 path");
         }
         if (type_id != 1 && type_id != 8) {
             throw TuckmillError(ErrorCode::UnsupportedQuantization,
                                 "engine matrices must be F16 or Q8_0");
+        }
+        if (profile == NumericalProfile::LlamaCpu && type_id != 8) {
+            throw TuckmillError(ErrorCode::UnsupportedArchitecture,
+                                "the HIP path implements the llama-cpu numerical profile for Q8_0 "
+                                "weights only; F16 weights run under oracle-f32",
+                                TM_HIP_ERR_UNSUPPORTED);
         }
         const size_t total = (size_t)plan(in_dim, out_dim, type_id);
         Matrix m;
@@ -431,11 +580,14 @@ class Matrix {
         m.type_id = type_id;
         m.in_dim = in_dim;
         m.out_dim = out_dim;
+        m.profile = profile;
         return m;
     }
 
-    void gemv(const HipContext &gpu, const HipBuffer &x, const HipBuffer &y) const {
-        if (type_id == 1) {
+    void gemv(const HipContext &gpu, const HipBuffer &x, const HipBuffer &y) {
+        if (profile == NumericalProfile::LlamaCpu) {
+            gemm_llama_cpu(gpu, x, y, 1);
+        } else if (type_id == 1) {
             gpu.f16_gemv(buf, x, y, (uint32_t)out_dim, (uint32_t)in_dim);
         } else {
             gpu.q8_0_gemv(buf, x, y, (uint32_t)out_dim, (uint32_t)in_dim);
@@ -444,9 +596,15 @@ class Matrix {
 
     // engine/metal.rs:171-196: batch 1 and `exact` keep the GEMV's per-row
     // arithmetic in slices of GEMM_MAX_BATCH; other batches use the matrix cores.
+    // Under llama-cpu every batch is exact already (the int8 products are
+    // bit-identical to the CPU's whatever the batch).
     void gemm(const HipContext &gpu, const HipBuffer &x, const HipBuffer &y, uint32_t batch,
-              bool exact) const {
+              bool exact) {
         const uint32_t rows = (uint32_t)out_dim, cols = (uint32_t)in_dim;
+        if (profile == NumericalProfile::LlamaCpu) {
+            gemm_llama_cpu(gpu, x, y, batch);
+            return;
+        }
         if (!exact && type_id == 8 && batch >= 2 && batch <= GEMM_MMA_MAX_BATCH) {
             gpu.q8_0_gemm_mma(buf, x, y, rows, cols, batch, 0, 0);
             return;
@@ -478,6 +636,29 @@ class Matrix {
     HipBuffer buf;
     uint32_t type_id = 8;
     uint64_t in_dim = 0, out_dim = 0;
+    NumericalProfile profile = NumericalProfile::OracleF32;
+
+  private:
+    // forward.rs:783-821 on the device: quantize the activations once per
+    // product, then the int8 product, in slices of GEMM_I8_MAX_BATCH tokens. The
+    // quantized-activation buffer grows to the largest slice seen and is kept (a
+    // buffer that is replaced while a group still names it stays alive: the group
+    // holds its memory).
+    void gemm_llama_cpu(const HipContext &gpu, const HipBuffer &x, const HipBuffer &y,
+                        uint32_t batch) {
+        const uint32_t rows = (uint32_t)out_dim, cols = (uint32_t)in_dim;
+        for (uint32_t t0 = 0; t0 < batch;) {
+            const uint32_t n = std::min(batch - t0, GEMM_I8_MAX_BATCH);
+            const size_t need = xq_bytes(cols, n);
+            if (xq.len() < need) {
+                xq = gpu.buffer(need, true);
+            }
+            gpu.q8_0_quantize_act(x, xq, cols, n, t0 * cols);
+            gpu.q8_0_gemm_i8(buf, xq, y, rows, cols, n, t0 * rows);
+            t0 += n;
+        }
+    }
+    HipBuffer xq; // quantized activations of the llama-cpu profile
 };
 
 } // namespace tuckmill_hip

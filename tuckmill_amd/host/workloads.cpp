@@ -10,6 +10,7 @@
 #include <chrono>
 #include <cstdio>
 #include <cstring>
+#include <string>
 
 #include "tm_hip.hpp"
 
@@ -141,16 +142,26 @@ int tmh_run_steps(tm_hip_ctx *ctx, const tmh_product *products, uint32_t n, uint
 }
 
 // Self-check of the C++ handles (Matrix::load with its staged upload and
-// seal, gemv, gemm slices, row lookup, ledger == plan). Returns 0 and the
-// outputs for the caller to compare with its oracle.
-int tmh_matrix_roundtrip(const uint8_t *raw, uint32_t rows, uint32_t cols, const float *x,
-                         uint32_t batch, int exact, float *y_out, float *row_out, uint32_t row,
-                         char *err, size_t err_cap) {
+// seal, gemv, gemm slices, row lookup, ledger == plan) under a numerical
+// profile ("oracle-f32" or "llama-cpu"). Returns 0 and the outputs for the
+// caller to compare with its oracle.
+int tmh_matrix_roundtrip_profile(const uint8_t *raw, uint32_t rows, uint32_t cols, uint32_t type_id,
+                                 const char *profile_name, const float *x, uint32_t batch, int exact,
+                                 float *y_out, float *row_out, uint32_t row, char *err,
+                                 size_t err_cap) {
     try {
+        NumericalProfile profile;
+        if (!parse_numerical_profile(profile_name != nullptr ? profile_name : "", &profile)) {
+            throw TuckmillError(ErrorCode::InvalidRequest,
+                                std::string("unknown numerical profile '") +
+                                    (profile_name != nullptr ? profile_name : "") +
+                                    "' (oracle-f32, llama-cpu)",
+                                TM_HIP_ERR_UNSUPPORTED);
+        }
         HipContext gpu = HipContext::open();
         const uint64_t before = gpu.allocated_bytes();
-        Matrix m = Matrix::load(gpu, raw, cols, rows);
-        if (gpu.allocated_bytes() - before != Matrix::plan(cols, rows)) {
+        Matrix m = Matrix::load(gpu, raw, cols, rows, type_id, true, profile);
+        if (gpu.allocated_bytes() - before != Matrix::plan(cols, rows, type_id)) {
             throw TuckmillError(ErrorCode::Internal, "allocation ledger differs from the plan");
         }
         HipBuffer xb = gpu.buffer((size_t)batch * cols * 4);
@@ -173,6 +184,82 @@ int tmh_matrix_roundtrip(const uint8_t *raw, uint32_t rows, uint32_t cols, const
             snprintf(err, err_cap, "%s", e.what());
         }
         return e.abi_code() != 0 ? e.abi_code() : TM_HIP_ERR_INTERNAL;
+    }
+}
+
+int tmh_matrix_roundtrip(const uint8_t *raw, uint32_t rows, uint32_t cols, const float *x,
+                         uint32_t batch, int exact, float *y_out, float *row_out, uint32_t row,
+                         char *err, size_t err_cap) {
+    return tmh_matrix_roundtrip_profile(raw, rows, cols, 8, "oracle-f32", x, batch, exact, y_out,
+                                        row_out, row, err, err_cap);
+}
+
+// The selection types through a C surface, for callers that test them without a
+// GPU. Error classes: 0 ok, 1 unknown name, 2 InvalidRequest, 3 Unavailable,
+// 4 UnsupportedArchitecture, 5 other.
+static int error_class(const TuckmillError &e) {
+    switch (e.code()) {
+    case ErrorCode::InvalidRequest: return 2;
+    case ErrorCode::Unavailable: return 3;
+    case ErrorCode::UnsupportedArchitecture: return 4;
+    default: return 5;
+    }
+}
+
+// KernelSelection::parse(name).resolve() with `device_available` standing in
+// for the probe (-1: ask the library); the resolved name goes to `resolved`.
+int tmh_resolve_kernels(const char *name, int device_available, char *resolved, size_t cap,
+                        char *err, size_t err_cap) {
+    bool ok = false;
+    const KernelSelection sel = KernelSelection::parse(name != nullptr ? name : "", &ok);
+    if (!ok) {
+        snprintf(err, err_cap, "unknown kernel selection '%s'", name != nullptr ? name : "");
+        return 1;
+    }
+    try {
+        const Probe device = device_available < 0
+                                 ? probe()
+                                 : Probe{device_available != 0, device_available != 0
+                                                                    ? "test device"
+                                                                    : "no HIP device available"};
+        snprintf(resolved, cap, "%s", as_str(sel.resolve(device)));
+        return 0;
+    } catch (const TuckmillError &e) {
+        snprintf(err, err_cap, "%s", e.what());
+        return error_class(e);
+    }
+}
+
+// check_engine_options(resolved kernels, profile, prefill batch given).
+int tmh_check_engine_options(const char *kernels, const char *profile_name, int prefill_batch_given,
+                             char *err, size_t err_cap) {
+    ResolvedKernels k;
+    const std::string ks = kernels != nullptr ? kernels : "";
+    if (ks == "scalar") {
+        k = ResolvedKernels::Scalar;
+    } else if (ks == "neon") {
+        k = ResolvedKernels::Neon;
+    } else if (ks == "metal") {
+        k = ResolvedKernels::Metal;
+    } else if (ks == "hip") {
+        k = ResolvedKernels::Hip;
+    } else {
+        snprintf(err, err_cap, "unknown resolved kernels '%s'", ks.c_str());
+        return 1;
+    }
+    NumericalProfile profile;
+    if (!parse_numerical_profile(profile_name != nullptr ? profile_name : "", &profile)) {
+        snprintf(err, err_cap, "unknown numerical profile '%s'",
+                 profile_name != nullptr ? profile_name : "");
+        return 1;
+    }
+    try {
+        check_engine_options(k, profile, prefill_batch_given != 0);
+        snprintf(err, err_cap, "%s", as_str(profile));
+        return 0;
+    } catch (const TuckmillError &e) {
+        snprintf(err, err_cap, "%s", e.what());
+        return error_class(e);
     }
 }
 
