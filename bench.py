@@ -39,10 +39,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 # HBM bytes per launch of the decode step's GEMV list kernel, from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in profiles/gemv_list_kernel__decode_step__pmc_traffic.txt
 # (fetch counter x 2.000 + write counter x 1.000, factors from a plain copy kernel).
-DECODE_STEP_TRAFFIC_BYTES = 644.69e6
+DECODE_STEP_TRAFFIC_BYTES = 644.77e6
 DECODE_STEP_TRAFFIC_SOURCE = ("constant from profiles/gemv_list_kernel__decode_step__pmc_traffic.txt "
                               "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --workload "
-                              "traffic`); not measured in this run")
+                              "traffic` on q8::gemv_list_kernel<1, 8, 1, true, 0, 224, false>); not "
+                              "measured in this run")
 
 
 class tmh_product(ctypes.Structure):
@@ -603,26 +604,76 @@ def bench_chain(host, ctx, steps, warmup, recorded=True):
 
 
 def run_traffic(host, ctx):
-    """A short, fixed sequence for hardware-counter runs (rocprofv3 --pmc):
-    a plain f32 copy of known size (the calibration kernel: 256 MiB read,
-    256 MiB written per dispatch), five decode steps and three M = 512 GEMM
-    groups. Prints the algorithmic bytes of each so that the counter values
+    """A short, fixed sequence for hardware-counter runs (rocprofv3 --pmc) and
+    the kernel trace that goes with them: every kernel family a few times, each
+    preceded by enough untimed work of its own to be at its steady clocks.
+      1. a plain f32 copy of known size (the calibration kernel: 256 MiB read,
+         256 MiB written per dispatch)
+      2. the decode step (gemv_list_kernel, one dispatch per step)
+      3. the seven Qwen3-0.6B projections at M = 512 as one group over sealed
+         weights (split_act_list_kernel + gemm_bf16x3_kernel, 128-token tiles)
+      4. the same over raw weights (gemm_mma kernels, f32 matrix cores)
+      5. the Gemma-3-1B vocabulary projection at M = 512 (gemm_bf16x3_kernel)
+      6. 2B-class shapes, int8-activation profile at M = 512
+         (quantize_act_kernel + gemm_i8_lds_kernel), 8 copies of each matrix
+    Prints the algorithmic bytes / operations of each so that the counter values
     per dispatch can be set beside them."""
     n = 64 << 20  # f32 elements
     src, dst = ctx.buffer(n * 4), ctx.buffer(n * 4)
     for _ in range(3):
         ctx.copy_f32(src, 0, dst, 0, n)
     ctx.fence()
+    src.free()
+    dst.free()
+    report = {"copy_f32_kernel": {"read_bytes": n * 4, "written_bytes": n * 4, "dispatches": 3}}
     products, keep, _ = build_decode_step(ctx, keep_host=False)
     step_bytes = sum(S.gemv_bytes(pr.rows, pr.cols) for pr in products)
     run_steps(host, ctx, products, 0, 5, grouped=True)
-    g = bench_gemm(host, ctx, 3, 0)
-    print(json.dumps({"copy_f32_kernel": {"read_bytes": n * 4, "written_bytes": n * 4},
-                      "gemv_list_kernel": {"algorithmic_bytes_per_dispatch": step_bytes,
-                                           "weights_bytes": sum(S.q8_0_bytes(p.rows, p.cols)
-                                                                for p in products)},
-                      "gemm_mma_kernel": {"flops_per_group_dispatch": g["flops_per_step"]}}),
-          flush=True)
+    report["gemv_list_kernel"] = {
+        "algorithmic_bytes_per_dispatch": step_bytes, "timed_dispatches": 5,
+        "weights_bytes": sum(S.q8_0_bytes(p.rows, p.cols) for p in products)}
+    for obj in keep:
+        (obj.buf if isinstance(obj, H.Matrix) else obj).free()
+    M = 512
+    for label, seal in (("gemm_bf16x3_kernel, seven projections, sealed", True),
+                        ("gemm_mma kernels (f32), seven projections, raw", False)):
+        prods, keep = [], []
+        for name, rows, cols in S.QWEN3_0_6B_LAYER:
+            m = H.Matrix.load(ctx, S.make_weights(rows, cols, S.tensor_seed(2, 0, name)), cols, rows,
+                              seal=seal)
+            xb, yb = ctx.buffer(M * cols * 4), ctx.buffer(M * rows * 4)
+            xb.upload(0, S.make_activations(M * cols, rows))
+            keep += [m.buf, xb, yb]
+            prods.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA))
+        run_steps(host, ctx, prods, 0, 5, grouped=True)
+        report[label] = {"flops_per_group": sum(2.0 * M * p.rows * p.cols for p in prods),
+                         "timed_groups": 5}
+        for b in keep:
+            b.free()
+    rows, cols = [s for s in S.GEMMA3_1B if s[0] == "lm_head"][0][1:]
+    m = H.Matrix.load(ctx, S.make_weights(rows, cols, 3999), cols, rows)
+    xb, yb = ctx.buffer(M * cols * 4), ctx.buffer(M * rows * 4)
+    xb.upload(0, S.make_activations(M * cols, 7))
+    run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA)], 0, 5,
+              grouped=False)
+    report["gemm_bf16x3_kernel, Gemma lm_head"] = {"flops_per_dispatch": 2.0 * M * rows * cols,
+                                                   "timed_dispatches": 5}
+    for b in (m.buf, xb, yb):
+        b.free()
+    pool = _weights_pool(ctx, list(S.SWEEP_2B), 8, 4000)
+    widths = sorted({c for _, _, c, _ in pool})
+    xb = ctx.buffer(M * max(widths) * 4)
+    xb.upload(0, S.make_activations(M * max(widths), 99))
+    xqs = {c: ctx.buffer(H.xq_bytes(c, M)) for c in widths}
+    ys = [ctx.buffer(M * r * 4) for _, r, _, _ in pool]
+    prods = [tmh_product(None, xb.raw, xqs[c].raw, 1, c, M, TMH_QUANT) for c in widths]
+    prods += [tmh_product(m.buf.raw, xqs[c].raw, yb.raw, r, c, M, TMH_GEMM_I8)
+              for (_, r, c, m), yb in zip(pool, ys)]
+    run_steps(host, ctx, prods, 0, 5, grouped=True)
+    report["gemm_i8_lds_kernel, 2B shapes"] = {
+        "int8_ops_per_group": sum(2.0 * M * r * c for _, r, c, _ in pool), "timed_groups": 5,
+        "products_per_group": len(pool)}
+    print(json.dumps(report), flush=True)
 
 
 def main():
