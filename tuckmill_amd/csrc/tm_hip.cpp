@@ -199,12 +199,18 @@ struct tm_hip_ctx {
     std::atomic<uint64_t> launches{0};
     std::atomic<int> profiling{0};
     bool group_active = false;
+    // Work put on the stream outside any commit since the last synchronize (zero
+    // fills, the tail copy of a seal, launches of the allocation-free entry
+    // point): a fence has to ask the runtime, the last commit's event does not
+    // cover it. Under the caller's serialization.
+    bool loose_work = false;
     std::vector<Op> group_ops;
     std::vector<struct tm_hip_step *> steps; // recorded steps not yet freed
     uint64_t plan_epoch = 0;
     std::mutex q_mu; // pending commits, event pool, profile table
     std::mutex copy_mu;
     std::deque<Commit> pending;
+    std::deque<Commit> retired; // completed, GPU time not read yet (measure_retired)
     std::vector<hipEvent_t> event_pool;
     ProfileSlot profile[kProfileSlots];
     uint32_t profile_used = 0;
@@ -322,44 +328,72 @@ void account_profile(tm_hip_ctx *ctx, const char *label, uint64_t nanos) {
     }
 }
 
-// Retire every commit whose stop event has been reached, in order. May be
-// called from any thread.
-void settle(tm_hip_ctx *ctx) {
+// Take the GPU times of the retired commits (q_mu held by the caller): their
+// events are read here, not when the commits retire, so that retiring a long
+// queue at a fence costs nothing per commit beyond its leases; the measurement
+// entry points ask for the times when somebody wants them.
+void measure_retired(tm_hip_ctx *ctx) {
+    while (!ctx->retired.empty()) {
+        Commit &c = ctx->retired.front();
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, c.start, c.stop) != hipSuccess || ms < 0.0f) {
+            (void)hipGetLastError();
+            ms = 0.0f;
+        }
+        const uint64_t nanos = (uint64_t)((double)ms * 1e6);
+        ctx->last_gpu_nanos.store(nanos, std::memory_order_relaxed);
+        ctx->gpu_nanos_total.fetch_add(nanos, std::memory_order_relaxed);
+        account_profile(ctx, c.label, nanos);
+        if (ctx->commit_log_on) {
+            if (ctx->commit_log.size() >= TM_HIP_COMMIT_LOG_CAP) {
+                ctx->commit_log.pop_front();
+            }
+            ctx->commit_log.push_back(nanos);
+        }
+        ctx->event_pool.push_back(c.start);
+        if (!c.stop_lent) {
+            ctx->event_pool.push_back(c.stop);
+        }
+        ctx->retired.pop_front();
+    }
+}
+
+// Retire every commit whose stop event has been reached, in order: its leases
+// end and it counts as completed. `all_done`: the caller has just synchronized
+// the stream, nothing needs to be asked. May be called from any thread.
+constexpr size_t kMaxUnmeasured = 1024; // retired commits whose events wait to be read
+
+void settle(tm_hip_ctx *ctx, bool all_done = false) {
     std::vector<Alloc *> release;
     {
         std::lock_guard<std::mutex> g(ctx->q_mu);
         while (!ctx->pending.empty()) {
             Commit &c = ctx->pending.front();
-            if (hipEventQuery(c.stop) != hipSuccess) {
+            if (!all_done && hipEventQuery(c.stop) != hipSuccess) {
+                (void)hipGetLastError(); // "not ready" is not an error to keep
                 break;
             }
-            float ms = 0.0f;
-            if (hipEventElapsedTime(&ms, c.start, c.stop) != hipSuccess || ms < 0.0f) {
-                ms = 0.0f;
-            }
-            const uint64_t nanos = (uint64_t)((double)ms * 1e6);
-            ctx->last_gpu_nanos.store(nanos, std::memory_order_relaxed);
-            ctx->gpu_nanos_total.fetch_add(nanos, std::memory_order_relaxed);
-            account_profile(ctx, c.label, nanos);
-            if (ctx->commit_log_on) {
-                if (ctx->commit_log.size() >= TM_HIP_COMMIT_LOG_CAP) {
-                    ctx->commit_log.pop_front();
-                }
-                ctx->commit_log.push_back(nanos);
-            }
             ctx->leased.fetch_sub(c.leased, std::memory_order_relaxed);
-            ctx->event_pool.push_back(c.start);
-            if (!c.stop_lent) {
-                ctx->event_pool.push_back(c.stop);
-            }
             release.insert(release.end(), c.keep.begin(), c.keep.end());
+            c.keep.clear();
+            ctx->retired.push_back(std::move(c));
             ctx->pending.pop_front();
             ctx->completed.fetch_add(1, std::memory_order_release);
+        }
+        if (ctx->retired.size() > kMaxUnmeasured) {
+            measure_retired(ctx); // gives the events back to the pool
         }
     }
     for (Alloc *a : release) {
         alloc_release(a);
     }
+}
+
+// For the entry points that report GPU times.
+void settle_and_measure(tm_hip_ctx *ctx) {
+    settle(ctx);
+    std::lock_guard<std::mutex> g(ctx->q_mu);
+    measure_retired(ctx);
 }
 
 int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
@@ -373,19 +407,30 @@ int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
             last = ctx->pending.back().stop;
         }
     }
+    bool reached = false;
     if (last != nullptr) {
         const auto t0 = std::chrono::steady_clock::now();
-        while (hipEventQuery(last) == hipErrorNotReady &&
+        hipError_t q;
+        while ((q = hipEventQuery(last)) == hipErrorNotReady &&
                std::chrono::steady_clock::now() - t0 < std::chrono::milliseconds(2)) {
         }
         (void)hipGetLastError(); // "not ready" is not an error to keep
+        reached = q == hipSuccess;
     }
-    hipError_t e = hipStreamSynchronize(ctx->stream);
-    if (e != hipSuccess) {
-        return hip_fail(err, cap, "stream synchronize", e);
+    // The stream runs in order: once the last commit's stop event is reached and
+    // nothing was put on the stream outside a commit, everything is done, and
+    // the runtime's own synchronize (which retires its record of every launch
+    // since the last one, a few microseconds each) can be left for later.
+    const bool proven = !ctx->loose_work && (last == nullptr || reached);
+    if (!proven) {
+        const hipError_t e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) {
+            return hip_fail(err, cap, "stream synchronize", e);
+        }
+        ctx->loose_work = false;
     }
     noalloc_release(ctx);
-    settle(ctx);
+    settle(ctx, true);
     if (ctx->completed.load(std::memory_order_acquire) <
         ctx->committed.load(std::memory_order_relaxed)) {
         return fail(err, cap, TM_HIP_ERR_INTERNAL,
@@ -1583,6 +1628,7 @@ void tm_hip_destroy(tm_hip_ctx *ctx) {
             }
         }
         ctx->pending.clear();
+        measure_retired(ctx); // hands the retired commits' events back to the pool
         for (hipEvent_t e : ctx->event_pool) {
             (void)hipEventDestroy(e);
         }
@@ -1624,6 +1670,7 @@ tm_hip_buffer *tm_hip_buffer_new(tm_hip_ctx *ctx, size_t bytes, int shared, char
              bytes, hipGetErrorString(e));
         return nullptr;
     }
+    ctx->loose_work = true;
     e = hipMemsetAsync(ptr, 0, bytes, ctx->stream);
     if (e != hipSuccess) {
         (void)hipFree(ptr);
@@ -1698,6 +1745,7 @@ int tm_hip_buffer_zero(tm_hip_ctx *ctx, tm_hip_buffer *buffer, size_t off, size_
         return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
                     "buffer_zero: buffer holds sealed Q8_0 weights");
     }
+    ctx->loose_work = true;
     hipError_t e = hipMemsetAsync((uint8_t *)buffer->alloc->ptr + off, 0, len, ctx->stream);
     if (e != hipSuccess) {
         return hip_fail(err, err_cap, "buffer_zero", e);
@@ -2267,6 +2315,7 @@ int tm_hip_q8_0_gemm_mma_noalloc(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffe
                     "fence first",
                     what, ctx->noalloc_keep.size());
     }
+    ctx->loose_work = true; // launched outside any commit: a fence asks the runtime
     // Held until the next commit adopts them or a fence has passed them (the list
     // has its capacity from tm_hip_create on).
     for (int i = 0; i < 3; ++i) {
@@ -2517,6 +2566,7 @@ int tm_hip_q8_0_pack(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t rows, uint32_t 
     fresh->prows = rows;
     fresh->pcols = cols;
     if (w->len > need) {
+        ctx->loose_work = true;
         e = hipMemcpyAsync((uint8_t *)ptr + need, (const uint8_t *)w->alloc->ptr + need,
                            w->len - need, hipMemcpyDeviceToDevice, ctx->stream);
         if (e != hipSuccess) {
@@ -2643,7 +2693,7 @@ double tm_hip_last_gpu_ms(const tm_hip_ctx *ctx) {
     if (ctx == nullptr) {
         return 0.0;
     }
-    settle(const_cast<tm_hip_ctx *>(ctx));
+    settle_and_measure(const_cast<tm_hip_ctx *>(ctx));
     return (double)ctx->last_gpu_nanos.load(std::memory_order_relaxed) / 1e6;
 }
 
@@ -2651,7 +2701,7 @@ uint64_t tm_hip_gpu_nanos_total(const tm_hip_ctx *ctx) {
     if (ctx == nullptr) {
         return 0;
     }
-    settle(const_cast<tm_hip_ctx *>(ctx));
+    settle_and_measure(const_cast<tm_hip_ctx *>(ctx));
     return ctx->gpu_nanos_total.load(std::memory_order_relaxed);
 }
 
@@ -2663,7 +2713,9 @@ int tm_hip_profile_set(tm_hip_ctx *ctx, int enabled) {
     if (ctx == nullptr) {
         return TM_HIP_ERR_UNSUPPORTED;
     }
+    settle(ctx);
     std::lock_guard<std::mutex> g(ctx->q_mu);
+    measure_retired(ctx); // commits so far are accounted under the old setting
     ctx->profile_used = 0;
     ctx->profiling.store(enabled ? 1 : 0, std::memory_order_relaxed);
     return TM_HIP_OK;
@@ -2676,6 +2728,7 @@ int tm_hip_profile_read(tm_hip_ctx *ctx, uint32_t index, char *name, size_t name
     }
     settle(ctx);
     std::lock_guard<std::mutex> g(ctx->q_mu);
+    measure_retired(ctx);
     if (index >= ctx->profile_used) {
         return 0;
     }
@@ -2697,6 +2750,7 @@ int tm_hip_commit_log_set(tm_hip_ctx *ctx, int enabled) {
     }
     settle(ctx);
     std::lock_guard<std::mutex> g(ctx->q_mu);
+    measure_retired(ctx); // commits so far stay out of (or go into) the log as it was
     ctx->commit_log_on = enabled != 0;
     ctx->commit_log.clear();
     return TM_HIP_OK;
@@ -2708,6 +2762,7 @@ size_t tm_hip_commit_log_read(tm_hip_ctx *ctx, uint64_t *nanos, size_t cap) {
     }
     settle(ctx);
     std::lock_guard<std::mutex> g(ctx->q_mu);
+    measure_retired(ctx);
     size_t n = 0;
     while (n < cap && !ctx->commit_log.empty()) {
         nanos[n++] = ctx->commit_log.front();
