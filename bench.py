@@ -471,9 +471,10 @@ def bench_sweep(host, ctx, steps, warmup):
                 "frac_of_mfma_peak": flops / us / 1e6 / (MFMA_I8_PEAK_TOPS if kind == TMH_GEMM_I8
                                                         else MFMA_F32_PEAK_TFLOPS),
                 "quantize_act_us": quant_us})
-            if kind == TMH_GEMM_MMA and all(H.gemm_mma_on_bf16(r, c, mb) for _, r, c, _ in pool):
-                # every product is large enough at this batch for the kernel on the
-                # bf16 matrix cores, which issues three bf16 products per f32 one
+            if kind == TMH_GEMM_MMA and mb >= H.GEMM_MMA_BF16_MIN_BATCH and \
+                    H.gemm_mma_launch_tile([(r, c, mb) for _, r, c, _ in pool]):
+                # the products that share the launch are large enough together for the
+                # kernel on the bf16 matrix cores, which issues three bf16 products per f32 one
                 pt = out["points"][-1]
                 pt["path"] = label.replace("f32 mfma", "bf16 mfma x3")
                 pt["frac_of_mfma_peak"] = 3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS

@@ -206,7 +206,7 @@ int tm_hip_q8_0_gemm(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm_hip
 
 /* Same contract for batch 1..=TM_HIP_GEMM_MMA_MAX_BATCH on the MFMA matrix
  * cores: every product q*x is exact (f32 operand tiles with W dequantized
- * exactly as d*q; or, from 33 tokens over sealed weights, bf16 tiles with
+ * exactly as d*q; or, from 17 tokens over sealed weights, bf16 tiles with
  * every activation split into three exact bf16 pieces). Summation order
  * differs from the GEMV: tolerance-qualified, not bit-identical
  * (native/metal/tm_metal.h:172-178). Which of the two forms runs, and how K is

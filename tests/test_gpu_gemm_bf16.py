@@ -1,4 +1,4 @@
-"""GPU parity: the prefill GEMM from 33 tokens over sealed weights large enough
+"""GPU parity: the prefill GEMM from 17 tokens over sealed weights large enough
 to fill the chip with 128-token x 256-row tiles, which runs on the bf16 matrix
 cores with every f32 activation split into three exact bf16 pieces (contract: native/metal/tm_metal.h:172-175, tolerance-qualified like
 every matrix-core kernel; crates/metal/src/tests.rs:1169-1233 for the shapes).
@@ -14,7 +14,7 @@ from q8util import bits, norm_err, ref_scale, require_gpu, upload_new, weights_b
 
 pytestmark = pytest.mark.gpu
 
-M0 = H.GEMM_MMA_BF16_MIN_BATCH  # 33: one 64-token tile up to 64 tokens
+M0 = H.GEMM_MMA_BF16_MIN_BATCH  # 17: one 64-token tile up to 64 tokens
 
 
 @pytest.fixture(scope="module")

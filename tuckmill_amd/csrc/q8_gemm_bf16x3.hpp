@@ -525,14 +525,15 @@ inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint3
 // Which tile the products of one launch take together, or 0 when the kernel does
 // not pay for them: the rule of a single product, with the launch's sums in the
 // place of the product's own figures (`shapes` = rows, cols, batch of every
-// product; all with batch <= 64 or all above).
+// product; all with batch <= 32, all with 33..64, or all above).
 //
 // Up to 64 tokens there is one small tile of tokens. The kernel's time hardly
 // depends on the batch here (27 us for 8192 x 1024, 97 us for 151936 x 1024), the
 // f32 kernel's does: from 33 tokens (its 64-token tile) 16 M weights are the
 // break-even (16384 x 1024 at 64 tokens: 30 against 29 us; 4096 x 4096: 34 against
 // 47; 151936 x 1024: 97 against 219). At 32 tokens and below only the largest
-// matrices would gain, and little.
+// matrices would gain, and little: from 17 tokens (below, the exact small-batch
+// kernel serves the entry point) the bar is 32 M weights.
 //
 // Above 64 tokens, in order of preference: the large tile with 192 units or more;
 // the small tile with 192 units or more in at most 4 K chunks per product (1024 x
@@ -560,6 +561,12 @@ inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
         small_chunks = s.chunks > small_chunks ? s.chunks : small_chunks;
         large += bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 128u).units;
         weights += (uint64_t)shapes[i].rows * shapes[i].cols;
+    }
+    if (shapes[0].batch <= 32u) {
+        // half of the one token tile is padding: only twice the weights pay (the
+        // f32 kernel's own tile is 32 tokens here; 20 x (6144 x 2048 + 2048 x 6144) at
+        // 32 tokens: 385 us on the f32 kernels, about 300 us here)
+        return weights >= (1ull << 25) && small >= 128u ? 64u : 0u;
     }
     if (shapes[0].batch <= 64u) {
         return weights >= (1ull << 24) && small >= 128u ? 64u : 0u;

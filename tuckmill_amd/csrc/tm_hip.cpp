@@ -470,7 +470,7 @@ struct GemvKey {
     bool decode() const { return kind == OP_GEMV_LIST && variant == V_DECODE && packed && flag; }
 };
 
-// Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 33
+// Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 17
 // tokens, and when the products that share the launch have enough work units
 // (256 rows x 128 or 64 tokens x K chunk) between them for the kernel to pay
 // (q8::bx3_launch_tile has the rule and the measurements behind it). The kernel
@@ -482,7 +482,7 @@ struct GemvKey {
 // the same group gives the same bits every time, but a product's bits may depend
 // on what shares its launch (the entry point is tolerance-qualified,
 // native/metal/tm_metal.h:172-175; bit-identity claims belong to q8_0_gemm).
-constexpr uint32_t kBx3MinBatch = 33;
+constexpr uint32_t kBx3MinBatch = 17;
 constexpr uint64_t kBx3MaxPartialFloats = 1ull << 29; // 2 GiB of partial tiles per launch
 
 bool x_aligned_of(const Op &op) {
@@ -1025,8 +1025,8 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
 // The kernel of every matrix-core product (OP_MMA) of a sequence, decided per
 // launch: consecutive products that do not depend on each other will share
 // launches, and whether the ones that could run on the bf16 matrix cores do is
-// decided on their sums (products of up to 64 tokens and of more form two pools,
-// each with the one tile q8::bx3_launch_tile gives it). The rest take the f32
+// decided on their sums (products of up to 32, up to 64 and of more tokens form
+// three pools, each with the one tile q8::bx3_launch_tile gives it). The rest take the f32
 // kernels. Entries of other operations are left unset.
 std::vector<GemvKey> assign_mma_keys(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
     std::vector<GemvKey> keys(ops.size());
@@ -1039,12 +1039,13 @@ std::vector<GemvKey> assign_mma_keys(tm_hip_ctx *ctx, const std::vector<Op> &ops
         for (size_t i : run) {
             keys[i] = mma_f32_key(ops[i]);
         }
-        for (int small_batch = 0; small_batch < 2; ++small_batch) {
+        for (uint32_t batch_class = 0; batch_class < 3; ++batch_class) {
             std::vector<size_t> pool;
             std::vector<q8::Bx3Shape3> shapes;
             for (size_t i : run) {
                 const Op &op = ops[i];
-                if (bx3_admissible(op) && (op.batch <= 64u) == (small_batch != 0)) {
+                const uint32_t cls = op.batch <= 32u ? 0u : op.batch <= 64u ? 1u : 2u;
+                if (bx3_admissible(op) && cls == batch_class) {
                     pool.push_back(i);
                     shapes.push_back(q8::Bx3Shape3{op.rows, op.cols, op.batch});
                 }

@@ -25,10 +25,10 @@ ERR_CAP = 512  # crates/metal/src/lib.rs:32
 GEMM_MAX_BATCH = 32  # crates/metal/src/lib.rs:28-30
 GEMM_MMA_MAX_BATCH = 512
 PREFILL_BATCH = 128  # crates/tuckcore/src/engine/metal.rs:25 (the engine's prefill chunk)
-# From this batch on tm_hip_q8_0_gemm_mma over a large sealed matrix (128 or more tiles of
-# 128 tokens x 256 rows, K chunks counted) with 16-byte aligned activations runs on the bf16
-# matrix cores (activations split into three exact bf16 pieces).
-GEMM_MMA_BF16_MIN_BATCH = 33
+# From this batch on tm_hip_q8_0_gemm_mma over sealed weights with 16-byte aligned
+# activations may run on the bf16 matrix cores (activations split into three exact bf16
+# pieces), when the products of its launch are large enough together (gemm_mma_launch_tile).
+GEMM_MMA_BF16_MIN_BATCH = 17
 
 
 def _bf16_units(rows: int, cols: int, batch: int, tokens: int):
@@ -47,9 +47,9 @@ def _bf16_units(rows: int, cols: int, batch: int, tokens: int):
 def gemm_mma_launch_tile(shapes) -> int:
     """Tokens per tile (128 or 64) with which the products `shapes` = [(rows, cols,
     batch), ...] that share one launch run on the bf16 matrix cores, or 0 when they
-    stay on the f32 ones (mirror of q8::bx3_launch_tile). All batches up to 64, or
-    all above. Up to 64 tokens: 16 M weights and 128 units of the small tile between
-    them. Above, in order of preference: 192 units or more of the large tile; 192 or
+    stay on the f32 ones (mirror of q8::bx3_launch_tile). All batches up to 32, all
+    from 33 to 64, or all above. Up to 64 tokens: 16 M weights (32 M up to 32 tokens) and 128 units of
+    the small tile between them. Above, in order of preference: 192 units or more of the large tile; 192 or
     more of the small tile in at most 4 chunks per product; 128 or more of the large
     tile."""
     shapes = list(shapes)
@@ -58,6 +58,8 @@ def gemm_mma_launch_tile(shapes) -> int:
     small = sum(_bf16_units(r, c, b, 64)[0] for r, c, b in shapes)
     small_chunks = max(_bf16_units(r, c, b, 64)[1] for r, c, b in shapes)
     large = sum(_bf16_units(r, c, b, 128)[0] for r, c, b in shapes)
+    if shapes[0][2] <= 32:  # half of the one token tile is padding: twice the weights
+        return 64 if sum(r * c for r, c, _ in shapes) >= 1 << 25 and small >= 128 else 0
     if shapes[0][2] <= 64:
         return 64 if sum(r * c for r, c, _ in shapes) >= 1 << 24 and small >= 128 else 0
     if large >= 192:
