@@ -83,6 +83,57 @@ def test_dispatch_completion_accounting_is_exact(ctx):
     assert np.all(yb.download_f32(0, 4) == 128.0)
 
 
+def test_gpu_times_are_read_when_asked_for_and_the_commit_log_keeps_them_apart(ctx):
+    # A fence retires commits without reading their events; the measurement
+    # entry points read them. The per-commit log (no counterpart in the
+    # reference) holds one entry per commit completed while it was on.
+    wb, xb, yb = ones_problem(ctx, rows=64, cols=1024)
+    ctx.q8_0_gemv(wb, xb, yb, 64, 1024)      # before the log is on: must stay out of it
+    ctx.fence()
+    total0 = ctx.gpu_nanos_total()
+    ctx.set_commit_log(True)
+    n = 37
+    for _ in range(n):
+        ctx.q8_0_gemv(wb, xb, yb, 64, 1024)
+    ctx.fence()
+    assert ctx.completed_dispatches() == ctx.committed_dispatches()
+    log = ctx.read_commit_log()
+    assert log.size == n and (log > 0).all()
+    assert int(log.sum()) == ctx.gpu_nanos_total() - total0
+    assert ctx.last_gpu_ms() == pytest.approx(float(log[-1]) / 1e6)
+    assert ctx.read_commit_log().size == 0, "read drains the log"
+    ctx.set_commit_log(False)
+    ctx.q8_0_gemv(wb, xb, yb, 64, 1024)
+    ctx.fence()
+    assert ctx.read_commit_log().size == 0
+    # far more commits than the library keeps unmeasured: nothing is lost
+    total1 = ctx.gpu_nanos_total()
+    ctx.set_commit_log(True)
+    for _ in range(2500):
+        ctx.q8_0_gemv(wb, xb, yb, 64, 1024)
+    ctx.fence()
+    log = ctx.read_commit_log()
+    assert log.size == 2500 and int(log.sum()) == ctx.gpu_nanos_total() - total1
+    ctx.set_commit_log(False)
+
+
+def test_a_fence_waits_for_work_issued_outside_commits(ctx):
+    # zero fills and the allocation-free launches are not commits: the fence must
+    # not take the last commit's event for the whole stream
+    rows, cols = 151_936, 1024
+    w = S.make_weights(rows, cols, 21)
+    x = S.make_activations(cols, 22)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    xb, yb = upload_new(ctx, x), ctx.buffer(rows * 4)
+    big = upload_new(ctx, np.full(64 << 20, 0xAB, np.uint8))
+    for _ in range(5):
+        ctx.q8_0_gemv(wb, xb, yb, rows, cols)   # commits
+    big.zero(0, 64 << 20)                       # behind them, not a commit
+    ctx.fence()
+    assert not big.download(0, 64 << 20).any()
+    assert norm_err(yb.download_f32(0, rows), O.gemv_q8_0_f32(w, rows, cols, x, threads=8)) <= 1e-5
+
+
 def test_upload_download_respect_bounds_and_offsets(ctx):
     buf = ctx.buffer(16, True)
     buf.upload(8, bytes([9] * 8))
