@@ -185,6 +185,112 @@ def test_a_group_splits_each_input_once_and_is_deterministic(ctx):
         m[4].free()
 
 
+@pytest.mark.parametrize("kind", ["rmsnorm", "silu_mul", "gelu_tanh_mul"])
+@pytest.mark.parametrize("batch", [500, 64])
+def test_the_operator_in_front_writes_the_split_form_itself(ctx, kind, batch):
+    # A layer as the executor encodes it: the norm before q/k/v (or the gated
+    # activation before the down projection), then the products that read its
+    # result. Inside one group the operator writes the split form of its result
+    # as well and the products' launch does without its split pass: one kernel
+    # launch fewer, the same bits as with the operator committed on its own
+    # first (where the products' launch splits the input itself). A product
+    # that reads the result from an offset, or another buffer, keeps its pass.
+    cols = 1024
+    shapes = [(8192, cols), (2048, cols), (9000, cols)]
+    assert H.gemm_mma_launch_tile([(r, c, batch) for r, c in shapes]) != 0
+    src = [upload_new(ctx, S.make_activations(batch * cols, 40 + i)) for i in range(2)]
+    wn = upload_new(ctx, (1.0 + 0.1 * S.make_activations(cols, 9)).astype(np.float32))
+    xb = ctx.buffer((batch * cols + 32) * 4)
+    mats = []
+    for i, (rows, c) in enumerate(shapes):
+        w = S.make_weights(rows, c, 700 + i)
+        mats.append((w, rows, c, weights_buffer(ctx, w, rows, c, True), ctx.buffer(batch * rows * 4)))
+
+    def operator():
+        if kind == "rmsnorm":
+            ctx.rmsnorm(src[0], wn, xb, batch, cols, 1e-6)
+        elif kind == "silu_mul":
+            ctx.silu_mul(src[0], src[1], xb, batch * cols)
+        else:
+            ctx.gelu_tanh_mul(src[0], src[1], xb, batch * cols)
+
+    def products(x_off=0):
+        for w, rows, c, wb, yb in mats:
+            ctx.q8_0_gemm_mma(wb, xb, yb, rows, c, batch, x_off, 0)
+
+    def outputs():
+        ctx.fence()
+        return [m[4].download_f32(0, batch * m[1]).copy() for m in mats]
+
+    def clear():
+        xb.zero(0, (batch * cols + 32) * 4)
+        for m in mats:
+            m[4].zero(0, batch * m[1] * 4)
+
+    clear()
+    operator()
+    ctx.fence()
+    x = xb.download_f32(0, batch * cols).copy()
+    before = ctx.kernel_launches()
+    ctx.begin_group()
+    products()
+    ctx.end_group()
+    apart = outputs()
+    assert ctx.kernel_launches() == before + 2  # the split pass and the products
+
+    for attempt in range(2):  # the second run finds the workspace as the first left it
+        clear()
+        before = ctx.kernel_launches()
+        ctx.begin_group()
+        operator()
+        products()
+        ctx.end_group()
+        fused = outputs()
+        assert ctx.kernel_launches() == before + 2  # the operator and the products
+        assert np.array_equal(bits(xb.download_f32(0, batch * cols)), bits(x))
+        for i in range(len(mats)):
+            assert np.array_equal(bits(fused[i]), bits(apart[i])), f"attempt {attempt}, product {i}"
+    w, rows, c, wb, yb = mats[1]
+    want = O.gemm_q8_0_f32(w, rows, c, x, batch, threads=8)
+    assert norm_err(fused[1].reshape(batch, rows), want) <= 1e-5
+
+    # recorded and replayed
+    ctx.begin_group()
+    operator()
+    products()
+    step = ctx.end_group_recorded()
+    assert step.launches == 2
+    for replay in range(2):
+        clear()
+        step.run()
+        got = outputs()
+        for i in range(len(mats)):
+            assert np.array_equal(bits(got[i]), bits(apart[i])), f"replay {replay}, product {i}"
+    step.free()
+
+    # read from an offset: not the operator's whole result, so the launch splits it itself
+    clear()
+    operator()
+    ctx.fence()
+    before = ctx.kernel_launches()
+    ctx.begin_group()
+    operator()
+    products(x_off=32)
+    ctx.end_group()
+    off = outputs()
+    assert ctx.kernel_launches() == before + 3
+    full = xb.download_f32(0, batch * cols + 32)
+    w, rows, c, wb, yb = mats[1]
+    want = O.gemm_q8_0_f32(w, rows, c, np.ascontiguousarray(full[32:]), batch, threads=8)
+    assert norm_err(off[1].reshape(batch, rows), want) <= 1e-5
+
+    for b in src + [wn, xb]:
+        b.free()
+    for m in mats:
+        m[3].free()
+        m[4].free()
+
+
 @pytest.mark.parametrize("rows,cols,batch", [(8192, 1024, 512), (8191, 1024, 512), (7936, 1024, 512),
                                              (32768, 1024, 65), (32768, 1024, 64), (32513, 1024, 65),
                                              (4096, 4096, 128), (4096, 4096, 129), (6144, 2048, 512),

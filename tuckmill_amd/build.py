@@ -62,7 +62,7 @@ def build_host(verbose: bool = False) -> str:
 
 
 PROBE_DIR = os.path.join(HERE, "probes")
-PROBES = ("phase_barrier",)
+PROBES = ("phase_barrier", "mfma_coissue")
 
 
 def build_probes(verbose: bool = False) -> list[str]:

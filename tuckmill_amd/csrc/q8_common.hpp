@@ -37,6 +37,42 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
 
+// An f32 as the exact sum of three bf16 numbers: its 24-bit significand cut into
+// 8 + 8 + 8 bits (h = trunc(x), m = trunc(x - h), l = x - h - m; both
+// subtractions are exact). An infinity or NaN goes into h whole, m = l = 0.
+__device__ __forceinline__ void split3_bf16(float x, uint32_t &h, uint32_t &m, uint32_t &l) {
+    const uint32_t xb = __builtin_bit_cast(uint32_t, x);
+    const bool finite = (xb & 0x7f800000u) != 0x7f800000u;
+    // (a NaN whose payload sits in the low 16 bits only must stay a NaN)
+    const uint32_t hb = finite ? xb & 0xffff0000u : xb | ((xb & 0xffffu) ? 0x00400000u : 0u);
+    const float r1 = finite ? x - __builtin_bit_cast(float, hb) : 0.0f; // exact
+    const uint32_t mb = __builtin_bit_cast(uint32_t, r1) & 0xffff0000u;
+    const float r2 = r1 - __builtin_bit_cast(float, mb); // exact, at most 8 significant bits
+    h = hb >> 16;
+    m = mb >> 16;
+    l = __builtin_bit_cast(uint32_t, r2) >> 16;
+}
+
+// Where the pieces of element (token t, column k) of a [batch][cols] matrix live
+// in its split form [cols / 32][3][batch][32] (bf16 units): the h piece at the
+// returned index, m and l each batch * 32 further on.
+__device__ __forceinline__ size_t split_index(uint32_t batch, uint32_t t, uint32_t k) {
+    return ((size_t)(k >> 5) * 3u * batch + t) * 32u + (k & 31u);
+}
+
+// One element into the split form (for the operators that write a matrix product's
+// activations and its split form in one pass).
+__device__ __forceinline__ void split_store(uint16_t *xs, uint32_t batch, uint32_t t, uint32_t k,
+                                            float v) {
+    uint32_t h, m, l;
+    split3_bf16(v, h, m, l);
+    uint16_t *dst = xs + split_index(batch, t, k);
+    const size_t piece = (size_t)batch * 32u;
+    dst[0] = (uint16_t)h;
+    dst[piece] = (uint16_t)m;
+    dst[2u * piece] = (uint16_t)l;
+}
+
 // binary32 -> binary16 bits with the rounding of
 // crates/tuckcore/src/tensor.rs:145-178: round to nearest even, overflow and
 // NaN both become +-inf, magnitudes below 2^-25 become +-0.

@@ -75,19 +75,10 @@ __global__ __launch_bounds__(256) void split_act_list_kernel(const SplitArgs arg
     uint32_t h[4], m[4], l[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        const uint32_t xb = __builtin_bit_cast(uint32_t, in[e]);
-        const bool finite = (xb & 0x7f800000u) != 0x7f800000u;
-        // (a NaN whose payload sits in the low 16 bits only must stay a NaN)
-        const uint32_t hb = finite ? xb & 0xffff0000u : xb | ((xb & 0xffffu) ? 0x00400000u : 0u);
-        const float r1 = finite ? in[e] - __builtin_bit_cast(float, hb) : 0.0f; // exact
-        const uint32_t mb = __builtin_bit_cast(uint32_t, r1) & 0xffff0000u;
-        const float r2 = r1 - __builtin_bit_cast(float, mb);    // exact, at most 8 significant bits
-        h[e] = hb >> 16;
-        m[e] = mb >> 16;
-        l[e] = __builtin_bit_cast(uint32_t, r2) >> 16;
+        split3_bf16(in[e], h[e], m[e], l[e]);
     }
     const size_t piece = (size_t)batch * 32u;
-    uint16_t *dst = d.xs + ((size_t)(k >> 5) * 3u * batch + t) * 32u + (k & 31u);
+    uint16_t *dst = d.xs + split_index(batch, t, k);
     *(uint2 *)dst = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
     *(uint2 *)(dst + piece) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
     *(uint2 *)(dst + 2u * piece) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
@@ -303,29 +294,26 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
     // of token / weight row idx (any assignment of a block's 32 k to the two
     // steps' lanes does, as long as both operands use it): a lane's 16 quants of
     // a weight row are then one 16-byte piece, read in one go.
+    //
+    // The instruction order of a block is written out (scheduling barriers pin
+    // it): a wave's vector instructions hide under MFMAs only where they sit
+    // between the MFMAs of its own instruction stream. (Measured with a probe
+    // kernel: four to six independent vector instructions per 32-cycle MFMA cost
+    // nothing there, while a wave that only issues MFMAs keeps the SIMD's issue
+    // port and the partner wave's vector work waits.) So every MFMA is followed
+    // by a few conversions of the next weight rows or a few rescale FMAs of the
+    // chain before it: 1-2 % faster than the compiler's own order, which issues
+    // runs of eight and more MFMAs back to back.
     auto compute = [&](const uint8_t *stage, uint32_t kb) {
+        static_assert(TM == 2 && TN == 2, "written for 2 x 2 tiles per wave");
         const uint32_t *sdw = (const uint32_t *)(stage + Sh::a_bytes + Sh::b_bytes);
         const uint8_t *sb = stage + Sh::a_bytes;
-        bf16x8_t b[TN][2];
-        float dw[TN];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const uint32_t r = wn * 64u + 32u * j + idx;
-            {
-                const uint32_t slot = half ^ ((r >> 3) & 1u);
-                const u32x4 raw = *(const u32x4 *)(sb + r * 32u + slot * 16u);
-                b[j][0] = sbytes_to_bf16x8(raw.x, raw.y);
-                b[j][1] = sbytes_to_bf16x8(raw.z, raw.w);
-            }
-            {
-                const uint32_t pair = sdw[r];
-                dw[j] = f16_bits_to_f32(((row_odd[j] + kb) & 1u) ? pair >> 16 : pair & 0xffffu);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const uint32_t r = wm * (32u * TM) + 32u * i + idx;
-            bf16x8_t a[3][2];
+        const uint32_t r0 = wn * 64u + idx, r1 = r0 + 32u;
+        const u32x4 raw0 = *(const u32x4 *)(sb + r0 * 32u + (half ^ ((r0 >> 3) & 1u)) * 16u);
+        const u32x4 raw1 = *(const u32x4 *)(sb + r1 * 32u + (half ^ ((r1 >> 3) & 1u)) * 16u);
+        const uint32_t pair0 = sdw[r0], pair1 = sdw[r1];
+        bf16x8_t a0[3][2], a1[3][2];
+        auto load_a = [&](bf16x8_t (&a)[3][2], uint32_t r) {
 #pragma unroll
             for (int pl = 0; pl < 3; ++pl) {
 #pragma unroll
@@ -334,23 +322,70 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
                     a[pl][m] = *(const bf16x8_t *)(stage + pl * Sh::a_plane + r * 64u + slot * 16u);
                 }
             }
+        };
+        auto two = [](uint32_t w, int i) { // bytes 2i, 2i+1 of w as two bf16
+            const uint32_t f0 = __builtin_bit_cast(uint32_t, sbyte_to_float(w, 2 * i));
+            const uint32_t f1 = __builtin_bit_cast(uint32_t, sbyte_to_float(w, 2 * i + 1));
+            return __builtin_amdgcn_perm(f1, f0, 0x07060302u);
+        };
+        auto pack = [](uint32_t p0, uint32_t p1, uint32_t p2, uint32_t p3) {
+            const u32x4 v = {p0, p1, p2, p3};
+            return __builtin_bit_cast(bf16x8_t, v);
+        };
+        const floatx16_t zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
+                                 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+#define BX3_SB __builtin_amdgcn_sched_barrier(0)
+        load_a(a0, wm * 64u + idx);
+        const bf16x8_t b00 = pack(two(raw0.x, 0), two(raw0.x, 1), two(raw0.y, 0), two(raw0.y, 1));
+        const bf16x8_t b01 = pack(two(raw0.z, 0), two(raw0.z, 1), two(raw0.w, 0), two(raw0.w, 1));
+        const float dw0 = f16_bits_to_f32(((row_odd[0] + kb) & 1u) ? pair0 >> 16 : pair0 & 0xffffu);
+        BX3_SB;
+        // chain (0, 0), the second row tile's weights converted on the way
+        floatx16_t s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0[2][0], b00, zero, 0, 0, 0);
+        load_a(a1, wm * 64u + 32u + idx);
+        BX3_SB;
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0[2][1], b01, s, 0, 0, 0);
+        const uint32_t q0 = two(raw1.x, 0), q1 = two(raw1.x, 1);
+        BX3_SB;
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0[1][0], b00, s, 0, 0, 0);
+        const uint32_t q2 = two(raw1.y, 0), q3 = two(raw1.y, 1);
+        BX3_SB;
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0[1][1], b01, s, 0, 0, 0);
+        const uint32_t q4 = two(raw1.z, 0), q5 = two(raw1.z, 1);
+        BX3_SB;
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0[0][0], b00, s, 0, 0, 0);
+        const uint32_t q6 = two(raw1.w, 0), q7 = two(raw1.w, 1);
+        BX3_SB;
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0[0][1], b01, s, 0, 0, 0);
+        const bf16x8_t b10 = pack(q0, q1, q2, q3), b11 = pack(q4, q5, q6, q7);
+        const float dw1 = f16_bits_to_f32(((row_odd[1] + kb) & 1u) ? pair1 >> 16 : pair1 & 0xffffu);
+        BX3_SB;
+        // a chain of six MFMAs with the rescale of the chain before it in between
+        auto chain = [&](const bf16x8_t (&a)[3][2], const bf16x8_t &bA, const bf16x8_t &bB,
+                         const floatx16_t &prev, float prev_dw, floatx16_t &into) {
+            floatx16_t t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2][0], bA, zero, 0, 0, 0);
+            BX3_SB;
+            t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2][1], bB, t, 0, 0, 0);
+            BX3_SB;
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                floatx16_t s = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
-                                0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+            for (int g = 0; g < 4; ++g) {
+                t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1 - g / 2][g % 2], g % 2 ? bB : bA, t, 0, 0, 0);
 #pragma unroll
-                for (int pl = 2; pl >= 0; --pl) { // smallest pieces first
-#pragma unroll
-                    for (int m = 0; m < 2; ++m) {
-                        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[pl][m], b[j][m], s, 0, 0, 0);
-                    }
+                for (int v = 4 * g; v < 4 * g + 4; ++v) {
+                    into[v] = __builtin_fmaf(prev_dw, prev[v], into[v]);
                 }
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    acc[i][j][v] = __builtin_fmaf(dw[j], s[v], acc[i][j][v]);
-                }
+                BX3_SB;
             }
+            return t;
+        };
+        floatx16_t t = chain(a1, b00, b01, s, dw0, acc[0][0]); // chain (1, 0)
+        s = chain(a0, b10, b11, t, dw0, acc[1][0]);            // chain (0, 1)
+        t = chain(a1, b10, b11, s, dw1, acc[0][1]);            // chain (1, 1)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            acc[1][1][v] = __builtin_fmaf(dw1, t[v], acc[1][1][v]);
         }
+#undef BX3_SB
     };
 
     // Every wave issues the same number of fetch instructions per block, so

@@ -34,14 +34,25 @@ __global__ __launch_bounds__(256) void axpy_kernel(const float *a, float *y, flo
     }
 }
 
+// The three operators below can write, next to their f32 result, its split form
+// for the bf16 matrix cores (q8_gemm_bf16x3.hpp) when the product that reads
+// the result follows directly: `xs` non-null, the result taken as a
+// [n / cols][cols] matrix. That saves the product's own split pass, a dependent
+// launch of about 5 us.
+
 // out[i] = silu(gate[i]) * up[i],  silu(g) = g / (1 + exp(-g))
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float *gate, const float *up,
-                                                       float *out, uint32_t n) {
+                                                       float *out, uint32_t n, uint16_t *xs,
+                                                       uint32_t cols) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i < n) {
         const float g = gate[i];
         const float s = g / (1.0f + expf(-g));
-        out[i] = s * up[i];
+        const float v = s * up[i];
+        out[i] = v;
+        if (xs != nullptr) {
+            split_store(xs, n / cols, i / cols, i % cols, v);
+        }
     }
 }
 
@@ -49,24 +60,34 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float *gate, const 
 // 0.5 x (1 + tanh(sqrt(2/pi) x (1 + 0.044715 x^2))), evaluated in the order of
 // kernels.metal:391-395.
 __global__ __launch_bounds__(256) void gelu_tanh_mul_kernel(const float *gate, const float *up,
-                                                            float *out, uint32_t n) {
+                                                            float *out, uint32_t n, uint16_t *xs,
+                                                            uint32_t cols) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i < n) {
         const float x = gate[i];
         const float inner = 0.7978845608028654f * x * (1.0f + 0.044715f * x * x);
-        out[i] = 0.5f * x * (1.0f + tanhf(inner)) * up[i];
+        const float v = 0.5f * x * (1.0f + tanhf(inner)) * up[i];
+        out[i] = v;
+        if (xs != nullptr) {
+            split_store(xs, n / cols, i / cols, i % cols, v);
+        }
     }
 }
 
-// One wave per row (four rows per workgroup): y = (x * inv) * w with
+// One wave per row (RMSNORM_ROWS rows per workgroup: one, so that the few hundred
+// rows of a prefill chunk spread over the whole chip): y = (x * inv) * w with
 // inv = 1 / sqrt(mean(x^2) + eps). The sum of squares is q8::row_sumsq's: fixed
 // order, not the CPU's sequential one, hence tolerance-qualified like the
 // reference's own GPU kernel; the GEMV kernel's fused form computes the same
 // bits. In place (x == y) is safe: a lane rereads only what it writes itself.
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const float *x, const float *weight, float *y,
-                                                      uint32_t rows, uint32_t cols, float eps) {
+constexpr uint32_t RMSNORM_ROWS = 1;
+
+__global__ __launch_bounds__(64 * RMSNORM_ROWS) void rmsnorm_kernel(const float *x, const float *weight,
+                                                                    float *y, uint32_t rows,
+                                                                    uint32_t cols, float eps,
+                                                                    uint16_t *xs) {
     const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const uint32_t row = blockIdx.x * RMSNORM_ROWS + (threadIdx.x >> 6);
     if (row >= rows) {
         return;
     }
@@ -74,10 +95,36 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float *x, const floa
     float *yr = y + (size_t)row * cols;
     const float sumsq = row_sumsq(xr, cols, lane);
     const float inv = 1.0f / sqrtf(sumsq / (float)cols + eps);
-    for (uint32_t e0 = lane * 16u; e0 < cols; e0 += 1024u) {
-        const uint32_t e1 = e0 + 16u < cols ? e0 + 16u : cols;
-        for (uint32_t e = e0; e < e1; ++e) {
-            yr[e] = xr[e] * inv * weight[e];
+    const bool vec = (cols & 3u) == 0u && ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)weight)) & 15u) == 0u;
+    if (vec) {
+        // four consecutive elements per lane, a wave's 1 KiB in one piece
+        for (uint32_t e = lane * 4u; e < cols; e += 256u) {
+            const float4 xv = *(const float4 *)(xr + e);
+            const float4 wv = *(const float4 *)(weight + e);
+            const float4 v = make_float4(xv.x * inv * wv.x, xv.y * inv * wv.y, xv.z * inv * wv.z,
+                                         xv.w * inv * wv.w);
+            *(float4 *)(yr + e) = v;
+            if (xs != nullptr) {
+                const float in[4] = {v.x, v.y, v.z, v.w};
+                uint32_t h[4], m[4], l[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    split3_bf16(in[i], h[i], m[i], l[i]);
+                }
+                uint16_t *dst = xs + split_index(rows, row, e); // the four share a block of 32
+                const size_t piece = (size_t)rows * 32u;
+                *(uint2 *)dst = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+                *(uint2 *)(dst + piece) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
+                *(uint2 *)(dst + 2u * piece) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
+            }
+        }
+        return;
+    }
+    for (uint32_t e = lane; e < cols; e += 64u) {
+        const float v = xr[e] * inv * weight[e];
+        yr[e] = v;
+        if (xs != nullptr) {
+            split_store(xs, rows, row, e, v);
         }
     }
 }

@@ -670,6 +670,14 @@ struct Launch {
     // V_BF16X3: what the listed products need of the context's workspace
     uint64_t bx3_split_tiles = 0, bx3_partial_floats = 0, bx3_xs_bytes = 0;
     int bx3_inputs = 0;
+    // V_BF16X3: bit i set = the launch's i-th distinct input (in list order)
+    // arrives split already, written by the launch just before this one.
+    uint32_t bx3_presplit = 0;
+    // An RMSNorm or gated activation on its own whose result is the next
+    // launch's input: byte offset in the split workspace where it writes the
+    // split form as well, or -1.
+    int64_t split_xs_off = -1;
+    uint32_t split_cols = 0; // the row length that result is cut by
 };
 
 // Two products read the same activations (and can share their split form).
@@ -726,9 +734,20 @@ hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launc
                                     (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
                                     op->batch};
     }
-    hipError_t e = q8::launch_split_act_list(ctx->stream, inputs, n_in);
-    if (e != hipSuccess) {
-        return e;
+    // Inputs that the launch before this one has split already stay out of the
+    // split pass (none left: no split pass).
+    q8::SplitInput to_split[q8::SPLIT_MAX_DESCS];
+    int n_split = 0;
+    for (int i = 0; i < n_in; ++i) {
+        if (((launch.bx3_presplit >> i) & 1u) == 0u) {
+            to_split[n_split++] = inputs[i];
+        }
+    }
+    if (n_split > 0) {
+        hipError_t e = q8::launch_split_act_list(ctx->stream, to_split, n_split);
+        if (e != hipSuccess) {
+            return e;
+        }
     }
     return q8::launch_gemm_bf16x3_list(ctx->stream, stop, launch.key.p0 * 64u, prods, n,
                                        ws.partials, ws.arrivals);
@@ -736,7 +755,11 @@ hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launc
 
 // Kernel launches a planned launch stands for.
 uint32_t kernel_launches_of(const Launch &l) {
-    return l.single == nullptr && l.key.variant == V_BF16X3 ? 2u : 1u;
+    if (l.single != nullptr || l.key.variant != V_BF16X3) {
+        return 1u;
+    }
+    const uint32_t all = l.bx3_inputs >= 32 ? 0xffffffffu : (1u << l.bx3_inputs) - 1u;
+    return (l.bx3_presplit & all) == all ? 1u : 2u; // the split pass, unless nothing is left to it
 }
 
 // Grow the split-float GEMM's workspace to what the largest of the planned
@@ -925,7 +948,10 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
+// `split_to`: where an RMSNorm or gated activation writes the split form of its
+// result as well (the planner's fuse_split_passes), or null.
+hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op,
+                         uint16_t *split_to = nullptr, uint32_t split_cols = 0) {
     const uint8_t *w = op.a[0] ? (const uint8_t *)op.a[0]->ptr : nullptr;
     hipStream_t st = ctx->stream;
     switch (op.kind) {
@@ -972,17 +998,18 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op) {
     case OP_SILU_MUL:
         Q8_LAUNCH(q8::silu_mul_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
                   (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
-                  op.extra);
+                  op.extra, split_to, split_cols);
         break;
     case OP_GELU_MUL:
         Q8_LAUNCH(q8::gelu_tanh_mul_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
                   (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
-                  op.extra);
+                  op.extra, split_to, split_cols);
         break;
     case OP_RMSNORM:
-        Q8_LAUNCH(q8::rmsnorm_kernel, dim3((op.rows + 3u) / 4u), dim3(256), 0, st, stop,
+        Q8_LAUNCH(q8::rmsnorm_kernel, dim3((op.rows + q8::RMSNORM_ROWS - 1u) / q8::RMSNORM_ROWS),
+                  dim3(64u * q8::RMSNORM_ROWS), 0, st, stop,
                   (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
-                  op.rows, op.cols, op.scalar);
+                  op.rows, op.cols, op.scalar, split_to);
         break;
     case OP_ARGMAX: {
         float *part_v = (float *)op.a[1]->ptr;
@@ -1082,6 +1109,56 @@ std::vector<GemvKey> assign_mma_keys(tm_hip_ctx *ctx, const std::vector<Op> &ops
     }
     close();
     return keys;
+}
+
+// A bf16-matrix-core launch reads its activations in split form, which a pass
+// of its own makes first: a dependent launch of about 5 us. Where the launch
+// right before it is the RMSNorm or gated activation that writes those
+// activations (the norm before q/k/v and before gate/up, the activation before
+// the down projection), that operator writes the split form too, into the
+// place in the workspace where the product launch expects it, and the input
+// drops out of the split pass. Both launches are neighbours on one stream, so
+// nothing else touches the workspace in between.
+void fuse_split_passes(std::vector<Launch> &plan) {
+    for (size_t j = 1; j < plan.size(); ++j) {
+        Launch &cons = plan[j];
+        Launch &prod = plan[j - 1];
+        if (cons.single != nullptr || cons.key.variant != V_BF16X3 || prod.single == nullptr) {
+            continue;
+        }
+        const Op &p = *prod.single;
+        if (p.kind != OP_RMSNORM && p.kind != OP_SILU_MUL && p.kind != OP_GELU_MUL) {
+            continue;
+        }
+        // the launch's distinct inputs in list order, as launch_bx3_list lays them out
+        const Op *input_of[q8::SPLIT_MAX_DESCS];
+        int n_in = 0;
+        size_t off = 0;
+        for (const Op *op : cons.list) {
+            int at = 0;
+            while (at < n_in && !same_input(*input_of[at], *op)) {
+                ++at;
+            }
+            if (at < n_in) {
+                continue;
+            }
+            if (n_in == q8::SPLIT_MAX_DESCS) {
+                break;
+            }
+            input_of[n_in] = op;
+            const bool whole = op->a[1] == p.a[2] && op->x_off == 0;
+            const bool shape = p.kind == OP_RMSNORM
+                                   ? op->batch == p.rows && op->cols == p.cols
+                                   : (uint64_t)op->batch * op->cols == p.extra;
+            if (whole && shape && prod.split_xs_off < 0) {
+                prod.split_xs_off = (int64_t)off;
+                prod.split_cols = op->cols;
+                cons.bx3_presplit |= 1u << n_in;
+            }
+            off += bx3_xs_bytes_of(*op);
+            ++n_in;
+        }
+    }
 }
 
 // Plan the launches of a sequence of recorded operations. Consecutive
@@ -1270,7 +1347,20 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
         }
     }
     flush();
+    fuse_split_passes(plan);
     return plan;
+}
+
+// One planned launch on the stream (`ws`: the context's grown workspace).
+hipError_t issue_launch(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &l) {
+    if (l.single == nullptr) {
+        return launch_gemv_list(ctx, stop, l, ctx->ws);
+    }
+    if (l.split_xs_off >= 0) {
+        return launch_single(ctx, stop, *l.single, (uint16_t *)(ctx->ws.xs + l.split_xs_off),
+                             l.split_cols);
+    }
+    return launch_single(ctx, stop, *l.single);
 }
 
 // Issue the launches; the last one carries the commit's stop event.
@@ -1286,8 +1376,7 @@ hipError_t issue_ops(tm_hip_ctx *ctx, const std::vector<Op> &ops, hipEvent_t sto
         const bool last = i + 1 == plan.size();
         const hipEvent_t ev = last ? stop : nullptr;
         const Launch &l = plan[i];
-        hipError_t e = l.single != nullptr ? launch_single(ctx, ev, *l.single)
-                                           : launch_gemv_list(ctx, ev, l, ctx->ws);
+        hipError_t e = issue_launch(ctx, ev, l);
         if (e != hipSuccess) {
             return e;
         }
@@ -2105,8 +2194,7 @@ int tm_hip_end_group_recorded(tm_hip_ctx *ctx, tm_hip_step **out, char *err, siz
     }
     hipError_t launch_err = hipSuccess;
     for (const Launch &l : plan) {
-        launch_err = l.single != nullptr ? launch_single(ctx, nullptr, *l.single)
-                                         : launch_gemv_list(ctx, nullptr, l, ctx->ws);
+        launch_err = issue_launch(ctx, nullptr, l);
         if (launch_err != hipSuccess) {
             break;
         }
