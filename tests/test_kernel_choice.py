@@ -18,10 +18,12 @@ def test_work_units_of_the_bf16_gemm():
     assert plan(4096, 1024, 512) == (64, 8 * 16 * 2, True)
     assert plan(2048, 2048, 512) == (64, 8 * 8 * 3, True)
     assert plan(33000, 96, 65) == (64, 2 * 129, True)
-    # ... else the large tile with 128 units or more, or none
-    assert plan(1024, 4096, 512) == (128, 4 * 4 * 8, True)
-    assert plan(1152, 6912, 512) == (128, 4 * 5 * 8, True)
-    assert plan(1024, 3072, 512) == (128, 4 * 4 * 6, False)
+    # ... in however many K chunks (six here) ...
+    assert plan(1024, 4096, 512) == (64, 8 * 4 * 6, True)
+    assert plan(1152, 6912, 512) == (64, 8 * 5 * 5, True)
+    assert plan(1024, 3072, 512) == (64, 8 * 4 * 6, True)
+    # ... else none (the large tile's figures are what the plan reports then)
+    assert plan(1024, 2048, 512) == (128, 4 * 4 * 4, False)
     assert plan(1024, 1024, 512) == (128, 4 * 4 * 2, False)
 
 
@@ -29,17 +31,17 @@ def test_which_products_take_the_bf16_matrix_cores():
     # the 0.6B attention and down projections are too small on their own,
     # the vocabulary projections and the 2B-class FFN are not
     for name, rows, cols in S.QWEN3_0_6B_LAYER:
-        if name in ("q", "k", "v", "o", "down"):
+        if name in ("q", "k", "v", "o"):
             assert not H.gemm_mma_on_bf16(rows, cols, 512)
     _, rows, cols = S.QWEN3_0_6B_LM_HEAD
     assert H.gemm_mma_on_bf16(rows, cols, H.GEMM_MMA_BF16_MIN_BATCH)
     assert not H.gemm_mma_on_bf16(rows, cols, H.GEMM_MMA_BF16_MIN_BATCH - 1)
     for _, rows, cols in S.SWEEP_2B:
         assert H.gemm_mma_on_bf16(rows, cols, 256)
-    # 192 units of the small tile in at most 4 chunks are the least that pays: q
-    # (128 units) and down (6 chunks) stay on the f32 kernels, gate and up do not
+    # 192 units of the small tile are the least that pays: q (128 units) stays on
+    # the f32 kernels; gate, up and down (six K chunks) do not
     assert not H.gemm_mma_on_bf16(2048, 1024, 512)
-    assert not H.gemm_mma_on_bf16(1024, 3072, 512)
+    assert H.gemm_mma_on_bf16(1024, 3072, 512)
     assert H.gemm_mma_on_bf16(3072, 1024, 512)
     # up to 64 tokens: matrices of 16 M weights and more
     assert H.gemm_mma_on_bf16(4096, 4096, 64) and not H.gemm_mma_on_bf16(6144, 2048, 64)
@@ -52,16 +54,19 @@ def test_products_that_share_a_launch_decide_together():
     tile = H.gemm_mma_launch_tile
     M = 512
     layer = {name: (rows, cols, M) for name, rows, cols in S.QWEN3_0_6B_LAYER}
-    # alone, only gate and up are large enough (tiles of 64 tokens) ...
+    # alone, only gate, up and down are large enough (tiles of 64 tokens) ...
     assert [tile([layer[n]]) for n in ("q", "k", "v", "o", "gate", "up", "down")] == \
-        [0, 0, 0, 0, 64, 64, 0]
+        [0, 0, 0, 0, 64, 64, 64]
     # ... all seven in one launch have 480 units of the large tile between them
     assert tile(list(layer.values())) == 128
     # the dependent layer's launches: q, k, v together and gate, up together take
-    # the small tile; o and down, alone in theirs, stay on the f32 matrix cores
+    # the small and the large tile, down alone the small one; o, alone in its
+    # launch, stays on the f32 matrix cores
     assert tile([layer["q"], layer["k"], layer["v"]]) == 64
     assert tile([layer["gate"], layer["up"]]) == 128
-    assert tile([layer["o"]]) == 0 and tile([layer["down"]]) == 0
+    assert tile([layer["o"]]) == 0 and tile([layer["down"]]) == 64
+    # the engine's prefill chunk of 128 tokens: all seven on the small tile
+    assert tile([(r, c, 128) for _, r, c in S.QWEN3_0_6B_LAYER]) == 64
     # up to 64 tokens: 16 M weights between them
     assert tile([(6144, 2048, 64)]) == 0 and tile([(6144, 2048, 64), (6144, 2048, 64)]) == 64
     assert tile([]) == 0

@@ -571,10 +571,14 @@ inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint3
 // kernel serves the entry point) the bar is 32 M weights.
 //
 // Above 64 tokens, in order of preference: the large tile with 192 units or more;
-// the small tile with 192 units or more in at most 4 K chunks per product (1024 x
-// 3072 at 512 tokens in six chunks: 40 us against 32 on the f32 kernel); the large
-// tile with 128 units or more (a product alone is then about even with the f32
-// kernel, products that share a launch far ahead). Measured alone at 512 tokens
+// the small tile with 192 units or more, in however many K chunks (alone, split
+// pass included: 1024 x 4096 at 512 tokens in six chunks 37 us, against 47 on the
+// large tile and 46 on the f32 kernel; 896 x 4864 39 against 51; 2048 x 4096 at 256
+// tokens 35 against 45; 1024 x 3072 at 512 tokens 33 against 31 on the f32 kernel,
+// 28 when the gated activation in front of it has written its split form; the
+// seven Qwen3-0.6B projections at 128 tokens 34 us against 54 on the f32
+// kernels); the large tile with 128 units or more (a product alone is then
+// about even with the f32 kernel, products that share a launch far ahead). Measured alone at 512 tokens
 // against the f32 kernel: small tile 3072 x 1024 34 against 35 us, 2048 x 2048 39
 // against 49, 4096 x 1024 36 against 48, 2048 x 1024 (128 units) 31 against 28;
 // large tile 8192 x 1024 49 against 93, 6144 x 2048 69 against 133. Together: the
@@ -589,11 +593,8 @@ inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
         return 0;
     }
     uint64_t large = 0, small = 0, weights = 0;
-    uint32_t small_chunks = 0;
     for (int i = 0; i < n; ++i) {
-        const Bx3Plan s = bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 64u);
-        small += s.units;
-        small_chunks = s.chunks > small_chunks ? s.chunks : small_chunks;
+        small += bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 64u).units;
         large += bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 128u).units;
         weights += (uint64_t)shapes[i].rows * shapes[i].cols;
     }
@@ -609,7 +610,7 @@ inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
     if (large >= BX3_UNITS_WANTED) {
         return 128u;
     }
-    if (small >= BX3_UNITS_WANTED && small_chunks <= 4u) {
+    if (small >= BX3_UNITS_WANTED) {
         return 64u;
     }
     return large >= 128u ? 128u : 0u;

@@ -50,13 +50,11 @@ def gemm_mma_launch_tile(shapes) -> int:
     stay on the f32 ones (mirror of q8::bx3_launch_tile). All batches up to 32, all
     from 33 to 64, or all above. Up to 64 tokens: 16 M weights (32 M up to 32 tokens) and 128 units of
     the small tile between them. Above, in order of preference: 192 units or more of the large tile; 192 or
-    more of the small tile in at most 4 chunks per product; 128 or more of the large
-    tile."""
+    more of the small tile; 128 or more of the large tile."""
     shapes = list(shapes)
     if not shapes:
         return 0
     small = sum(_bf16_units(r, c, b, 64)[0] for r, c, b in shapes)
-    small_chunks = max(_bf16_units(r, c, b, 64)[1] for r, c, b in shapes)
     large = sum(_bf16_units(r, c, b, 128)[0] for r, c, b in shapes)
     if shapes[0][2] <= 32:  # half of the one token tile is padding: twice the weights
         return 64 if sum(r * c for r, c, _ in shapes) >= 1 << 25 and small >= 128 else 0
@@ -64,7 +62,7 @@ def gemm_mma_launch_tile(shapes) -> int:
         return 64 if sum(r * c for r, c, _ in shapes) >= 1 << 24 and small >= 128 else 0
     if large >= 192:
         return 128
-    if small >= 192 and small_chunks <= 4:
+    if small >= 192:
         return 64
     return 128 if large >= 128 else 0
 
