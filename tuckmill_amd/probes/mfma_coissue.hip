@@ -10,6 +10,7 @@
 //   mode 1  every wave: V FMAs per MFMA slot, no MFMAs
 //   mode 2  one wave per SIMD MFMAs only, its partner wave FMAs only
 //   mode 3  every wave: one MFMA, then V FMAs, repeated
+//   mode 5  the same with one wave per SIMD
 #include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstdlib>
@@ -18,7 +19,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 #define CHECK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("%s: %s\n", #x, hipGetErrorString(e)); exit(1); } } while (0)
 
 // mode 0: every wave MFMA only; 1: every wave VALU only; 2: waves 0-3 MFMA, 4-7 VALU;
-// 3: every wave 1 MFMA + V valu interleaved; 4: waves 0-3 MFMA only (4-7 exit)
+// 3: every wave 1 MFMA + V valu interleaved; 4: waves 0-3 MFMA only (4-7 exit);
+// 5: like 3 with one wave per SIMD (waves 4-7 exit)
 template <int MODE, int V>
 __global__ __launch_bounds__(512, 1) void k(float *out, int iters, float seed) {
     const int wave = threadIdx.x >> 6;
@@ -28,9 +30,12 @@ __global__ __launch_bounds__(512, 1) void k(float *out, int iters, float seed) {
     for (int i = 0; i < 8; ++i) f[i] = seed + i + threadIdx.x;
     bf16x8_t a, b;
     for (int i = 0; i < 8; ++i) { a[i] = (__bf16)(seed + i); b[i] = (__bf16)(seed - i); }
-    const bool do_mfma = MODE == 0 || MODE == 3 || ((MODE == 2 || MODE == 4) && wave < 4);
+    if (MODE == 5 && wave >= 4) {
+        return;
+    }
+    const bool do_mfma = MODE == 0 || MODE == 3 || MODE == 5 || ((MODE == 2 || MODE == 4) && wave < 4);
     const bool do_valu = MODE == 1 || MODE == 3 || (MODE == 2 && wave >= 4);
-    if (MODE == 3) {
+    if (MODE == 3 || MODE == 5) {
         for (int it = 0; it < iters; ++it) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
@@ -57,6 +62,44 @@ __global__ __launch_bounds__(512, 1) void k(float *out, int iters, float seed) {
     for (int c = 0; c < 4; ++c) for (int v = 0; v < 16; ++v) s += acc[c][v];
     for (int i = 0; i < 8; ++i) s += f[i];
     if (s == 12345.678f) out[threadIdx.x] = s;
+}
+
+// CH accumulators per wave, used round-robin: CH = 1 is one chain of dependent
+// MFMAs (each takes the one before as its C operand), CH = 4 four independent ones.
+// WAVES = 4: one wave per SIMD (the other four exit), 8: two.
+template <int CH, int WAVES>
+__global__ __launch_bounds__(512, 1) void chains(float *out, int iters, float seed) {
+    if ((int)(threadIdx.x >> 6) >= WAVES) {
+        return;
+    }
+    floatx16_t acc[CH];
+    for (int c = 0; c < CH; ++c) for (int v = 0; v < 16; ++v) acc[c][v] = seed * v;
+    bf16x8_t a, b;
+    for (int i = 0; i < 8; ++i) { a[i] = (__bf16)(seed + i); b[i] = (__bf16)(seed - i); }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            acc[m % CH] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[m % CH], 0, 0, 0);
+        }
+    }
+    float s = 0;
+    for (int c = 0; c < CH; ++c) for (int v = 0; v < 16; ++v) s += acc[c][v];
+    if (s == 12345.678f) out[threadIdx.x] = s;
+}
+
+template <int CH, int WAVES> void run_chains(float *out) {
+    const int iters = 20000;
+    hipEvent_t e0, e1;
+    CHECK(hipEventCreate(&e0)); CHECK(hipEventCreate(&e1));
+    for (int w = 0; w < 2; ++w) chains<CH, WAVES><<<256, 512>>>(out, iters, 0.5f);
+    CHECK(hipEventRecord(e0));
+    chains<CH, WAVES><<<256, 512>>>(out, iters, 0.5f);
+    CHECK(hipEventRecord(e1));
+    CHECK(hipEventSynchronize(e1));
+    float ms; CHECK(hipEventElapsedTime(&ms, e0, e1));
+    printf("%d wave(s) per SIMD, %d accumulator chain(s) per wave:   %8.1f us  %6.1f ns per 4 MFMAs of a wave\n",
+           WAVES / 4, CH, ms * 1e3, ms * 1e6 / iters);
+    fflush(stdout);
 }
 
 template <int MODE, int V> void run(const char *name, float *out) {
@@ -87,5 +130,14 @@ int main() {
     run<3, 6>("each wave MFMA + V VALU interleaved", out);
     run<3, 8>("each wave MFMA + V VALU interleaved", out);
     run<3, 16>("each wave MFMA + V VALU interleaved", out);
+    run<5, 2>("one wave per SIMD: MFMA + V VALU interleaved", out);
+    run<5, 4>("one wave per SIMD: MFMA + V VALU interleaved", out);
+    run<5, 6>("one wave per SIMD: MFMA + V VALU interleaved", out);
+    run<5, 8>("one wave per SIMD: MFMA + V VALU interleaved", out);
+    run_chains<1, 4>(out);
+    run_chains<2, 4>(out);
+    run_chains<4, 4>(out);
+    run_chains<1, 8>(out);
+    run_chains<2, 8>(out);
     return 0;
 }
