@@ -93,6 +93,35 @@ def test_every_token_of_the_small_gemm_equals_its_own_gemv(ctx, rows, cols, batc
         assert np.array_equal(bits(single), bits(got[b])), f"token {b}"
 
 
+def test_products_that_go_as_two_token_groups_share_launches_by_descriptor_count(ctx):
+    # 17 to 32 tokens over a matrix with a column tail go as two descriptors of up
+    # to 16 tokens each (the 8-tokens-per-wave form has no tail variant). A
+    # launch holds 224 descriptors: 120 such products in one group take two
+    # launches, and every one of them comes out as it does alone.
+    rows, cols, batch, n = 40, 1152, 20, 120
+    w = S.make_weights(rows, cols, 901)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    xs = [S.make_activations(cols * batch, 300 + i) for i in range(3)]
+    xbs = [upload_new(ctx, x) for x in xs]
+    ybs = [ctx.buffer(batch * rows * 4) for _ in range(n)]
+    alone = []
+    for x in xs:
+        alone.append(run_gemm(ctx, ctx.q8_0_gemm, wb, x, rows, cols, batch).reshape(batch, rows))
+        assert norm_err(alone[-1], O.gemm_q8_0_f32(w, rows, cols, x, batch)) <= 1e-5
+    before = ctx.kernel_launches()
+    ctx.begin_group()
+    for i, yb in enumerate(ybs):
+        ctx.q8_0_gemm(wb, xbs[i % 3], yb, rows, cols, batch, 0, 0)
+    ctx.end_group()
+    ctx.fence()
+    assert ctx.kernel_launches() == before + 2
+    for i, yb in enumerate(ybs):
+        got = yb.download_f32(0, batch * rows).reshape(batch, rows)
+        assert np.array_equal(bits(got), bits(alone[i % 3])), f"product {i}"
+    for b in [wb] + xbs + ybs:
+        b.free()
+
+
 def test_gemm_batch_limits(ctx):
     wb, xb, yb = ctx.buffer(64), ctx.buffer(64), ctx.buffer(64)
     with pytest.raises(H.TuckmillError) as e:

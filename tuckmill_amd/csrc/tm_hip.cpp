@@ -578,6 +578,13 @@ GemvKey gemv_key(const Op &op) {
         k.p0 = op.batch <= 4 ? 1 : op.batch <= 8 ? 2 : 4;
         k.p1 = op.batch <= 2 ? 2 : op.batch <= 16 ? 4 : 8;
         k.p2 = (op.cols & 1023u) != 0u; // the instantiation that also handles a column tail
+        if (k.p2 != 0 && k.p1 == 8) {
+            // With a column tail the 8-tokens-per-wave form keeps 72 dwords per
+            // lane in scratch: such a product goes as two groups of up to 16
+            // tokens instead (split_token_groups; a token's result does not
+            // depend on which tokens share its workgroup).
+            k.p1 = 4;
+        }
     } else {
         k.variant = V_GENERAL;
     }
@@ -670,6 +677,7 @@ struct Launch {
     // V_BF16X3: what the listed products need of the context's workspace
     uint64_t bx3_split_tiles = 0, bx3_partial_floats = 0, bx3_xs_bytes = 0;
     int bx3_inputs = 0;
+    uint32_t descs = 0; // descriptors the listed products take (token groups count one each)
     // V_BF16X3: bit i set = the launch's i-th distinct input (in list order)
     // arrives split already, written by the launch just before this one.
     uint32_t bx3_presplit = 0;
@@ -816,6 +824,16 @@ hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<co
     return q8::launch_gemm_i8_list(ctx->stream, stop, key.packed, key.flag, key.p0, prods, n);
 }
 
+// Descriptors a product takes in a list launch: one, or for the token-split
+// kernel as many groups of waves x tokens-per-wave tokens as its batch needs.
+uint32_t split_token_groups(const GemvKey &key, uint32_t batch) {
+    if (key.variant != V_SPLIT) {
+        return 1u;
+    }
+    const uint32_t group_tokens = (uint32_t)key.p0 * key.p1;
+    return (batch + group_tokens - 1u) / group_tokens;
+}
+
 hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch,
                             const Workspace &ws) {
     const std::vector<const Op *> &ops = launch.list;
@@ -861,16 +879,29 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     }
     const bool small_launch = launch_bytes < (16u << 20);
     bool tails = false; // some product has a column tail with a streaming path of its own
+    size_t at = 0; // the product's place in the launch's list (the fusions are recorded per product)
     for (const Op *op : ops) {
         const uint32_t tail = op->cols & 1023u;
         tails = tails || (op->cols >= 1024u && (tail == 128u || tail == 768u));
+        // The token-split kernel covers waves x tokens-per-wave tokens per
+        // descriptor: a larger batch goes as several descriptors over the same
+        // weights, each with its own rows of X and Y.
+        const uint32_t group_tokens = key.variant == V_SPLIT ? (uint32_t)key.p0 * key.p1 : op->batch;
+        const uint32_t groups = split_token_groups(key, op->batch);
+        if (args.n + groups > (uint32_t)q8::GEMV_MAX_DESCS) {
+            return hipErrorInvalidValue;
+        }
+      for (uint32_t grp = 0; grp < groups; ++grp) {
         q8::GemvDesc &d = args.d[args.n++];
         d.w = (const uint8_t *)op->a[0]->ptr;
-        d.x = (const float *)op->a[1]->ptr + op->x_off;
-        d.y = (float *)op->a[2]->ptr + op->y_off;
+        d.x = (const float *)op->a[1]->ptr + op->x_off + (size_t)grp * group_tokens * op->cols;
+        d.y = (float *)op->a[2]->ptr + op->y_off + (size_t)grp * group_tokens * op->rows;
         d.rows = op->rows;
         d.cols = op->cols;
-        d.batch = op->batch;
+        d.batch = groups == 1u ? op->batch
+                               : (op->batch - grp * group_tokens < group_tokens
+                                      ? op->batch - grp * group_tokens
+                                      : group_tokens);
         d.tile_begin = tiles;
         d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
         if (small_launch && key.decode() && d.rows_per_tile == (uint32_t)R &&
@@ -885,7 +916,6 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
             }
         }
         d.pad = 0;
-        const size_t at = args.n - 1;
         const bool pair_first = launch.glu[at] != nullptr;
         const bool pair_second = at > 0 && launch.glu[at - 1] != nullptr;
         if (pair_first) { // a tile covers the same rows of both matrices: half the rows each
@@ -893,12 +923,12 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
             d.pad |= q8::GEMV_PAIR;
             fused = true;
         }
-        if (launch.norm != nullptr && launch.normed[args.n - 1]) {
+        if (launch.norm != nullptr && launch.normed[at]) {
             d.x = args.norm_h; // not read through: the kernel normalises norm_h itself
             d.pad |= q8::GEMV_X_NORMED | (norm_written ? 0u : q8::GEMV_WRITES_NORM);
             norm_written = true;
         }
-        const Op *update = residual[args.n - 1];
+        const Op *update = residual[at];
         d.res = update != nullptr ? (float *)update->a[1]->ptr : nullptr;
         d.alpha = update != nullptr ? update->scalar : 0.0f;
         d.pad2 = 0;
@@ -909,6 +939,8 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         } else {
             tiles += (op->rows + d.rows_per_tile - 1) / d.rows_per_tile;
         }
+      }
+        ++at;
     }
     args.total_tiles = tiles;
 #define TM_SPLIT_CASE(W, T, A, TL)                                                           \
@@ -927,7 +959,9 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     TM_SPLIT_ALL(1, 4)
     TM_SPLIT_ALL(2, 4)
     TM_SPLIT_ALL(4, 4)
-    TM_SPLIT_ALL(4, 8)
+    // (eight tokens per wave: no column-tail form, see gemv_key)
+    TM_SPLIT_CASE(4, 8, true, false)
+    TM_SPLIT_CASE(4, 8, false, false)
 #undef TM_SPLIT_ALL
 #undef TM_SPLIT_CASE
 #define TM_GEMV_CASE(P, T, A)                                                                \
@@ -1255,8 +1289,9 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                            cur.bx3_partial_floats + mine.partial_floats > kBx3MaxPartialFloats ||
                            (new_input && cur.bx3_inputs == q8::SPLIT_MAX_DESCS);
             }
+            const uint32_t need = split_token_groups(key, op.batch); // descriptors of this product
             if (open && (conflict || (!cur.list.empty() && !(key == cur.key)) ||
-                         (int)cur.list.size() == cap)) {
+                         (int)(cur.descs + need) > cap)) {
                 flush();
                 new_input = true;
             }
@@ -1271,6 +1306,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             }
             const bool takes_norm = normed && cur.norm != nullptr; // still pending after a flush?
             cur.key = key;
+            cur.descs += need;
             cur.list.push_back(&op);
             cur.residual.push_back(nullptr);
             cur.glu.push_back(nullptr);
