@@ -302,27 +302,30 @@ def bench_gemm(host, ctx, steps, warmup):
     wn = ctx.buffer(hid * 4)
     wn.upload(0, (1.0 + 0.1 * S.make_activations(hid, 11)).astype(np.float32))
     bufs["h"].upload(0, S.make_activations(M * hid, 12))
-    def prod(name, x):
-        m, _, yb, rows, cols = mats[name]
-        return tmh_product(m.buf.raw, x.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA)
-    full = [tmh_product(wn.raw, bufs["h"].raw, bufs["xn"].raw, M, hid, M, TMH_RMSNORM),
-            prod("q", bufs["xn"]), prod("k", bufs["xn"]), prod("v", bufs["xn"]),
-            prod("o", mats["q"][2]),
-            tmh_product(bufs["h"].raw, mats["o"][2].raw, bufs["h"].raw, 1, M * hid, 1, TMH_AXPY),
-            tmh_product(wn.raw, bufs["h"].raw, bufs["xn2"].raw, M, hid, M, TMH_RMSNORM),
-            prod("gate", bufs["xn2"]), prod("up", bufs["xn2"]),
-            tmh_product(mats["gate"][2].raw, mats["up"][2].raw, bufs["act"].raw, 1, M * ffn, 1,
-                        TMH_SILU_MUL),
-            prod("down", bufs["act"]),
-            tmh_product(bufs["h"].raw, mats["down"][2].raw, bufs["h"].raw, 1, M * hid, 1, TMH_AXPY)]
-    t = run_steps(host, ctx, full, warmup, steps, grouped=True)
-    stats = step_stats(t, steps)
-    us = stats.get("median_us") or stats["mean_us"]
-    out["layer_with_operators"] = {
-        "us": us, "step_us": stats, "launches_per_step": t.launches / steps,
-        "tflops": flops_total / us / 1e6,
-        "order": "rmsnorm -> q,k,v -> o(q) -> axpy -> rmsnorm -> gate,up -> silu_mul -> down -> axpy; "
-                 "no attention"}
+    def layer(tokens):
+        def prod(name, x):
+            m, _, yb, rows, cols = mats[name]
+            return tmh_product(m.buf.raw, x.raw, yb.raw, rows, cols, tokens, TMH_GEMM_MMA)
+        return [tmh_product(wn.raw, bufs["h"].raw, bufs["xn"].raw, tokens, hid, tokens, TMH_RMSNORM),
+                prod("q", bufs["xn"]), prod("k", bufs["xn"]), prod("v", bufs["xn"]),
+                prod("o", mats["q"][2]),
+                tmh_product(bufs["h"].raw, mats["o"][2].raw, bufs["h"].raw, 1, tokens * hid, 1, TMH_AXPY),
+                tmh_product(wn.raw, bufs["h"].raw, bufs["xn2"].raw, tokens, hid, tokens, TMH_RMSNORM),
+                prod("gate", bufs["xn2"]), prod("up", bufs["xn2"]),
+                tmh_product(mats["gate"][2].raw, mats["up"][2].raw, bufs["act"].raw, 1, tokens * ffn, 1,
+                            TMH_SILU_MUL),
+                prod("down", bufs["act"]),
+                tmh_product(bufs["h"].raw, mats["down"][2].raw, bufs["h"].raw, 1, tokens * hid, 1,
+                            TMH_AXPY)]
+    for key, tokens in (("layer_with_operators", M), ("layer_with_operators_m128", 128)):
+        t = run_steps(host, ctx, layer(tokens), warmup, steps, grouped=True)
+        stats = step_stats(t, steps)
+        us = stats.get("median_us") or stats["mean_us"]
+        out[key] = {
+            "M": tokens, "us": us, "step_us": stats, "launches_per_step": t.launches / steps,
+            "tflops": flops_total * tokens / M / us / 1e6,
+            "order": "rmsnorm -> q,k,v -> o(q) -> axpy -> rmsnorm -> gate,up -> silu_mul -> down -> axpy; "
+                     "no attention"}
     keep += list(bufs.values()) + [wn]
     # the engine's prefill chunk
     m128 = [tmh_product(p.w, p.x, p.y, p.rows, p.cols, 128, TMH_GEMM_MMA) for p in products]

@@ -678,7 +678,11 @@ inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint3
 // 28 when the gated activation in front of it has written its split form; the
 // seven Qwen3-0.6B projections at 128 tokens 34 us against 54 on the f32
 // kernels); the large tile with 128 units or more (a product alone is then
-// about even with the f32 kernel, products that share a launch far ahead). Measured alone at 512 tokens
+// about even with the f32 kernel, products that share a launch far ahead);
+// the small tile again for products of 3072 columns and more with at least 32
+// units (alone, at 128 tokens: 1024 x 3072 29 us against 34 on the f32 kernel,
+// 1024 x 4096 32 against 44, 1152 x 6912 38 against 71, 1536 x 8960 45 against 90;
+// at 256 tokens 1024 x 4096 34 against 39; 2048 columns lose, 27 against 24). Measured alone at 512 tokens
 // against the f32 kernel: small tile 3072 x 1024 34 against 35 us, 2048 x 2048 39
 // against 49, 4096 x 1024 36 against 48, 2048 x 1024 (128 units) 31 against 28;
 // large tile 8192 x 1024 49 against 93, 6144 x 2048 69 against 133. Together: the
@@ -693,7 +697,9 @@ inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
         return 0;
     }
     uint64_t large = 0, small = 0, weights = 0;
+    uint32_t least_cols = shapes[0].cols;
     for (int i = 0; i < n; ++i) {
+        least_cols = shapes[i].cols < least_cols ? shapes[i].cols : least_cols;
         small += bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 64u).units;
         large += bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 128u).units;
         weights += (uint64_t)shapes[i].rows * shapes[i].cols;
@@ -713,7 +719,14 @@ inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
     if (small >= BX3_UNITS_WANTED) {
         return 64u;
     }
-    return large >= 128u ? 128u : 0u;
+    if (large >= 128u) {
+        return 128u;
+    }
+    // Few output tiles under a deep K: the f32 kernels walk K in one piece per
+    // workgroup (4.6 + 9.8 us per 1024 columns at 128 tokens and up to 4096 rows),
+    // this kernel cuts it into chunks (22.5 + 2.3 us per 1024 columns, its split
+    // pass included).
+    return least_cols >= 3072u && small >= 32u ? 64u : 0u;
 }
 
 // A product on its own: its plan, and whether the kernel pays for it (`worth`).

@@ -50,7 +50,8 @@ def gemm_mma_launch_tile(shapes) -> int:
     stay on the f32 ones (mirror of q8::bx3_launch_tile). All batches up to 32, all
     from 33 to 64, or all above. Up to 64 tokens: 16 M weights (32 M up to 32 tokens) and 128 units of
     the small tile between them. Above, in order of preference: 192 units or more of the large tile; 192 or
-    more of the small tile; 128 or more of the large tile."""
+    more of the small tile; 128 or more of the large tile; the small tile for products of 3072
+    columns and more with 32 units or more."""
     shapes = list(shapes)
     if not shapes:
         return 0
@@ -64,7 +65,10 @@ def gemm_mma_launch_tile(shapes) -> int:
         return 128
     if small >= 192:
         return 64
-    return 128 if large >= 128 else 0
+    if large >= 128:
+        return 128
+    # few output tiles under a deep K
+    return 64 if min(c for _, c, _ in shapes) >= 3072 and small >= 32 else 0
 
 
 def gemm_mma_bf16_plan(rows: int, cols: int, batch: int):
