@@ -135,7 +135,9 @@ def test_gemm_batch_limits(ctx):
 
 
 MMA_SHAPES = [(16, 1024, 16), (40, 64, 3), (3584, 1024, 16), (3584, 1024, 32), (40, 64, 27),
-              (1024, 3584, 64), (100, 96, 77), (40, 64, 512), (1024, 3584, 7), (6144, 1024, 1)]
+              (1024, 3584, 64), (100, 96, 77), (40, 64, 512), (1024, 3584, 7), (6144, 1024, 1),
+              # few output tiles at a wide batch: 32-token tiles (ragged last token and row tiles)
+              (500, 2048, 500), (1000, 1024, 130)]
 
 
 @pytest.mark.parametrize("packed", [False, True])

@@ -654,8 +654,18 @@ inline MmaConfig pick_mma_config(const MmaProduct *prods, int n) {
         const uint32_t blocks = prods[i].cols / 32u;
         min_blocks = blocks < min_blocks ? blocks : min_blocks;
     }
+    // Tokens per wave tile: 64, or 32 for narrow batches and for launches that
+    // would leave most of the chip idle with 64 (at most 128 output tiles of
+    // 64 tokens x 32 rows: twice the workgroups, each half as long; 1024 x 2048
+    // at 128 tokens 24 -> 15 us, 1024 x 1024 14 -> 9, 256 x 4096 43 -> 26,
+    // 512 x 2048 at 512 tokens 23 -> 15; at 192 tiles the 64-token tile is
+    // already ahead, 1536 x 1024 at 256 tokens 14 against 16).
+    uint64_t tiles64 = 0;
+    for (int i = 0; i < n; ++i) {
+        tiles64 += (uint64_t)((prods[i].batch + 63u) / 64u) * ((prods[i].rows + 31u) / 32u);
+    }
     MmaConfig c;
-    c.tmw = max_batch > 32u ? 2 : 1;
+    c.tmw = max_batch > 32u && tiles64 > 128u ? 2 : 1;
     c.tnw = 1;
     c.s = min_blocks >= 4u ? 4 : (min_blocks >= 2u ? 2 : 1);
     return c;
