@@ -654,18 +654,21 @@ inline MmaConfig pick_mma_config(const MmaProduct *prods, int n) {
         const uint32_t blocks = prods[i].cols / 32u;
         min_blocks = blocks < min_blocks ? blocks : min_blocks;
     }
-    // Tokens per wave tile: 64, or 32 for narrow batches and for launches that
-    // would leave most of the chip idle with 64 (at most 128 output tiles of
-    // 64 tokens x 32 rows: twice the workgroups, each half as long; 1024 x 2048
-    // at 128 tokens 24 -> 15 us, 1024 x 1024 14 -> 9, 256 x 4096 43 -> 26,
-    // 512 x 2048 at 512 tokens 23 -> 15; at 192 tiles the 64-token tile is
-    // already ahead, 1536 x 1024 at 256 tokens 14 against 16).
+    // Tokens per wave tile: 64, or 32 for narrow batches and for launches whose
+    // last round of workgroups would be less than half full with 64 (the chip
+    // runs 256 of these workgroups at a time; a 32-token tile makes twice the
+    // workgroups, each half as long). Up to 128 output tiles of 64 tokens x 32
+    // rows: 1024 x 2048 at 128 tokens 24 -> 15 us, 1024 x 1024 14 -> 9, 256 x 4096
+    // 43 -> 26, 512 x 2048 at 512 tokens 23 -> 15; 257 to 384 tiles: the 0.6B gate
+    // and up projections together at 128 tokens 27 -> 24; at 192 and at 256 tiles
+    // the 64-token tile is ahead (1536 x 1024 at 256 tokens 14 against 16 us).
     uint64_t tiles64 = 0;
     for (int i = 0; i < n; ++i) {
         tiles64 += (uint64_t)((prods[i].batch + 63u) / 64u) * ((prods[i].rows + 31u) / 32u);
     }
+    const bool short_last_round = tiles64 <= 128u || (tiles64 > 256u && tiles64 <= 384u);
     MmaConfig c;
-    c.tmw = max_batch > 32u && tiles64 > 128u ? 2 : 1;
+    c.tmw = max_batch > 32u && !short_last_round ? 2 : 1;
     c.tnw = 1;
     c.s = min_blocks >= 4u ? 4 : (min_blocks >= 2u ? 2 : 1);
     return c;

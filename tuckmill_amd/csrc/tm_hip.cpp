@@ -1121,6 +1121,33 @@ std::vector<GemvKey> assign_mma_keys(tm_hip_ctx *ctx, const std::vector<Op> &ops
                 }
             }
         }
+        // The products left to the f32 matrix cores choose their token tile
+        // together as well (q8::pick_mma_config: it depends on how many output
+        // tiles the launch has). Those that could share a launch: the first
+        // one's layout, alignment and K split.
+        std::vector<size_t> f32_pool;
+        std::vector<q8::MmaProduct> f32_shapes;
+        for (size_t i : run) {
+            const GemvKey &k = keys[i];
+            if (k.variant != V_MMA || ops[i].batch <= 32u) {
+                continue;
+            }
+            if (!f32_pool.empty()) {
+                const GemvKey &first = keys[f32_pool.front()];
+                if (k.packed != first.packed || k.flag != first.flag || k.p2 != first.p2) {
+                    continue;
+                }
+            }
+            f32_pool.push_back(i);
+            f32_shapes.push_back(q8::MmaProduct{nullptr, nullptr, nullptr, ops[i].rows, ops[i].cols,
+                                                ops[i].batch});
+        }
+        if (f32_pool.size() > 1) {
+            const q8::MmaConfig c = q8::pick_mma_config(f32_shapes.data(), (int)f32_shapes.size());
+            for (size_t i : f32_pool) {
+                keys[i].p0 = (uint8_t)c.tmw;
+            }
+        }
         run.clear();
         epoch = ++ctx->plan_epoch;
     };
