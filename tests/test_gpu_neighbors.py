@@ -356,3 +356,57 @@ def test_gated_activation_is_not_fused_when_out_is_the_up_buffer(ctx):
     g, u = O.gemv_q8_0_f32(wg, ffn, hidden, x), O.gemv_q8_0_f32(wu, ffn, hidden, x)
     want = O.silu_mul(g, u)
     assert np.all(np.abs(ub.download_f32(0, ffn) - want) <= 2e-5 * np.maximum(np.abs(want), 1.0))
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 1024), (37, 1152), (5, 1000), (3, 7), (512, 1024)])
+@pytest.mark.parametrize("in_place", [False, True])
+def test_a_norm_takes_the_residual_update_of_its_input_in_front_of_itself(ctx, rows, cols, in_place):
+    # h += alpha * t; xn = rmsnorm(h): between two blocks of a layer at prefill
+    # sizes. Inside a group the norm does the update on its way (one launch), with
+    # the same bits in h and in xn as the two launched one after the other.
+    # Aligned and unaligned widths, rows the size of a prefill chunk and a few.
+    n = rows * cols
+    h0 = S.make_activations(n, 5)
+    t = S.make_activations(n, 6)
+    w = (1.0 + 0.25 * S.make_activations(cols, 7)).astype(np.float32)
+    hb, tb, wb = upload_new(ctx, h0), upload_new(ctx, t), upload_new(ctx, w)
+    yb = hb if in_place else ctx.buffer(n * 4)
+    alpha, eps = 0.5, 1e-6
+
+    def run(grouped):
+        hb.upload(0, h0)
+        before = ctx.kernel_launches()
+        if grouped:
+            ctx.begin_group()
+        ctx.f32_axpy(tb, hb, alpha, n)
+        ctx.rmsnorm(hb, wb, yb, rows, cols, eps)
+        if grouped:
+            ctx.end_group()
+        ctx.fence()
+        return (hb.download_f32(0, n).copy(), yb.download_f32(0, n).copy(),
+                ctx.kernel_launches() - before)
+
+    h_apart, y_apart, n_apart = run(False)
+    assert n_apart == 2
+    if not in_place:
+        assert np.array_equal(bits(h_apart), bits(h0 + np.float32(alpha) * t))
+        for r in range(0, rows, max(1, rows // 7)):
+            want = O.rmsnorm(h_apart[r * cols:(r + 1) * cols], w, eps)
+            assert close(y_apart[r * cols:(r + 1) * cols], want), f"row {r}"
+    for attempt in range(2):
+        h_fused, y_fused, n_fused = run(True)
+        assert n_fused == 1
+        assert np.array_equal(bits(h_fused), bits(h_apart)), f"attempt {attempt}"
+        assert np.array_equal(bits(y_fused), bits(y_apart)), f"attempt {attempt}"
+
+    # an update of only part of the norm's input, or of another buffer, stays a launch of its own
+    hb.upload(0, h0)
+    before = ctx.kernel_launches()
+    ctx.begin_group()
+    ctx.f32_axpy(tb, hb, alpha, n - 1 if n > 1 else 1)
+    ctx.rmsnorm(hb, wb, yb, rows, cols, eps)
+    ctx.end_group()
+    ctx.fence()
+    assert ctx.kernel_launches() - before == (2 if n > 1 else 1)
+    for b in {hb, tb, wb, yb}:
+        b.free()

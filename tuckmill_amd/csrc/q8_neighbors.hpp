@@ -82,41 +82,144 @@ __global__ __launch_bounds__(256) void gelu_tanh_mul_kernel(const float *gate, c
 // bits. In place (x == y) is safe: a lane rereads only what it writes itself.
 constexpr uint32_t RMSNORM_ROWS = 1;
 
-__global__ __launch_bounds__(64 * RMSNORM_ROWS) void rmsnorm_kernel(const float *x, const float *weight,
+// `add` non-null: the residual update x += alpha * add of the same rows comes
+// first (axpy_kernel's operations: multiply, then add; x is written back), for
+// the pair "h += alpha * t; xn = rmsnorm(h)" between two layers' products. Every
+// lane then updates, squares and normalises its own elements only (row_sumsq's
+// runs of 16), so the row never passes from one lane to another through memory.
+__global__ __launch_bounds__(64 * RMSNORM_ROWS) void rmsnorm_kernel(float *x, const float *weight,
                                                                     float *y, uint32_t rows,
                                                                     uint32_t cols, float eps,
-                                                                    uint16_t *xs) {
+                                                                    uint16_t *xs, const float *add,
+                                                                    float alpha) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t row = blockIdx.x * RMSNORM_ROWS + (threadIdx.x >> 6);
     if (row >= rows) {
         return;
     }
-    const float *xr = x + (size_t)row * cols;
+    float *xr = x + (size_t)row * cols;
     float *yr = y + (size_t)row * cols;
+    const bool vec = (cols & 3u) == 0u && ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)weight) |
+                                            ((uintptr_t)add)) & 15u) == 0u;
+    if (add != nullptr && vec && cols <= 1024u) {
+        // One run of 16 per lane: the updated values stay in registers for the sum
+        // of squares (row_sumsq's order: the lane's elements in turn, then
+        // q8::wave_sum) and for the normalisation.
+        const float *ar = add + (size_t)row * cols;
+        const uint32_t e0 = lane * 16u;
+        const uint32_t mine = e0 >= cols ? 0u : (cols - e0 < 16u ? cols - e0 : 16u); // a multiple of 4
+        float hv[16];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if ((uint32_t)(4 * q) < mine) {
+                const float4 h = *(const float4 *)(xr + e0 + 4 * q);
+                const float4 t = *(const float4 *)(ar + e0 + 4 * q);
+                hv[4 * q] = __fadd_rn(h.x, __fmul_rn(alpha, t.x));
+                hv[4 * q + 1] = __fadd_rn(h.y, __fmul_rn(alpha, t.y));
+                hv[4 * q + 2] = __fadd_rn(h.z, __fmul_rn(alpha, t.z));
+                hv[4 * q + 3] = __fadd_rn(h.w, __fmul_rn(alpha, t.w));
+                *(float4 *)(xr + e0 + 4 * q) = make_float4(hv[4 * q], hv[4 * q + 1], hv[4 * q + 2], hv[4 * q + 3]);
+            } else {
+                hv[4 * q] = hv[4 * q + 1] = hv[4 * q + 2] = hv[4 * q + 3] = 0.0f;
+            }
+        }
+        float acc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            if ((uint32_t)i < mine) {
+                acc += hv[i] * hv[i];
+            }
+        }
+        const float inv = 1.0f / sqrtf(wave_sum(acc) / (float)cols + eps);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if ((uint32_t)(4 * q) < mine) {
+                const uint32_t e = e0 + 4u * q;
+                const float4 wv = *(const float4 *)(weight + e);
+                const float4 v = make_float4(hv[4 * q] * inv * wv.x, hv[4 * q + 1] * inv * wv.y,
+                                             hv[4 * q + 2] * inv * wv.z, hv[4 * q + 3] * inv * wv.w);
+                *(float4 *)(yr + e) = v;
+                if (xs != nullptr) {
+                    const float in[4] = {v.x, v.y, v.z, v.w};
+                    uint32_t h[4], m[4], l[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        split3_bf16(in[i], h[i], m[i], l[i]);
+                    }
+                    uint16_t *dst = xs + split_index(rows, row, e);
+                    const size_t piece = (size_t)rows * 32u;
+                    *(uint2 *)dst = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+                    *(uint2 *)(dst + piece) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
+                    *(uint2 *)(dst + 2u * piece) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
+                }
+            }
+        }
+        return;
+    }
+    if (add != nullptr) {
+        const float *ar = add + (size_t)row * cols;
+        for (uint32_t e0 = lane * 16u; e0 < cols; e0 += 1024u) {
+            const uint32_t e1 = e0 + 16u < cols ? e0 + 16u : cols;
+            if (vec) {
+                for (uint32_t e = e0; e < e1; e += 4u) {
+                    const float4 h = *(const float4 *)(xr + e);
+                    const float4 t = *(const float4 *)(ar + e);
+                    *(float4 *)(xr + e) = make_float4(
+                        __fadd_rn(h.x, __fmul_rn(alpha, t.x)), __fadd_rn(h.y, __fmul_rn(alpha, t.y)),
+                        __fadd_rn(h.z, __fmul_rn(alpha, t.z)), __fadd_rn(h.w, __fmul_rn(alpha, t.w)));
+                }
+            } else {
+                for (uint32_t e = e0; e < e1; ++e) {
+                    xr[e] = __fadd_rn(xr[e], __fmul_rn(alpha, ar[e]));
+                }
+            }
+        }
+    }
     const float sumsq = row_sumsq(xr, cols, lane);
     const float inv = 1.0f / sqrtf(sumsq / (float)cols + eps);
-    const bool vec = (cols & 3u) == 0u && ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)weight)) & 15u) == 0u;
+    auto four = [&](uint32_t e) { // elements e .. e+3 of the row: normalise, store, split
+        const float4 xv = *(const float4 *)(xr + e);
+        const float4 wv = *(const float4 *)(weight + e);
+        const float4 v = make_float4(xv.x * inv * wv.x, xv.y * inv * wv.y, xv.z * inv * wv.z,
+                                     xv.w * inv * wv.w);
+        *(float4 *)(yr + e) = v;
+        if (xs != nullptr) {
+            const float in[4] = {v.x, v.y, v.z, v.w};
+            uint32_t h[4], m[4], l[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                split3_bf16(in[i], h[i], m[i], l[i]);
+            }
+            uint16_t *dst = xs + split_index(rows, row, e); // the four share a block of 32
+            const size_t piece = (size_t)rows * 32u;
+            *(uint2 *)dst = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+            *(uint2 *)(dst + piece) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
+            *(uint2 *)(dst + 2u * piece) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
+        }
+    };
+    if (add != nullptr) {
+        for (uint32_t e0 = lane * 16u; e0 < cols; e0 += 1024u) {
+            const uint32_t e1 = e0 + 16u < cols ? e0 + 16u : cols;
+            if (vec) {
+                for (uint32_t e = e0; e < e1; e += 4u) {
+                    four(e);
+                }
+            } else {
+                for (uint32_t e = e0; e < e1; ++e) {
+                    const float v = xr[e] * inv * weight[e];
+                    yr[e] = v;
+                    if (xs != nullptr) {
+                        split_store(xs, rows, row, e, v);
+                    }
+                }
+            }
+        }
+        return;
+    }
     if (vec) {
         // four consecutive elements per lane, a wave's 1 KiB in one piece
         for (uint32_t e = lane * 4u; e < cols; e += 256u) {
-            const float4 xv = *(const float4 *)(xr + e);
-            const float4 wv = *(const float4 *)(weight + e);
-            const float4 v = make_float4(xv.x * inv * wv.x, xv.y * inv * wv.y, xv.z * inv * wv.z,
-                                         xv.w * inv * wv.w);
-            *(float4 *)(yr + e) = v;
-            if (xs != nullptr) {
-                const float in[4] = {v.x, v.y, v.z, v.w};
-                uint32_t h[4], m[4], l[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    split3_bf16(in[i], h[i], m[i], l[i]);
-                }
-                uint16_t *dst = xs + split_index(rows, row, e); // the four share a block of 32
-                const size_t piece = (size_t)rows * 32u;
-                *(uint2 *)dst = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-                *(uint2 *)(dst + piece) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
-                *(uint2 *)(dst + 2u * piece) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
-            }
+            four(e);
         }
         return;
     }

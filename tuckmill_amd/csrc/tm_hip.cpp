@@ -686,6 +686,8 @@ struct Launch {
     // split form as well, or -1.
     int64_t split_xs_off = -1;
     uint32_t split_cols = 0; // the row length that result is cut by
+    // An RMSNorm on its own: the residual update of its input that it does first.
+    const Op *update = nullptr;
 };
 
 // Two products read the same activations (and can share their split form).
@@ -984,8 +986,11 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
 
 // `split_to`: where an RMSNorm or gated activation writes the split form of its
 // result as well (the planner's fuse_split_passes), or null.
+// `update`: a residual update h += alpha * t that an RMSNorm of h takes in
+// front of itself (plan_launches), or null.
 hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op,
-                         uint16_t *split_to = nullptr, uint32_t split_cols = 0) {
+                         uint16_t *split_to = nullptr, uint32_t split_cols = 0,
+                         const Op *update = nullptr) {
     const uint8_t *w = op.a[0] ? (const uint8_t *)op.a[0]->ptr : nullptr;
     hipStream_t st = ctx->stream;
     switch (op.kind) {
@@ -1042,8 +1047,10 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op,
     case OP_RMSNORM:
         Q8_LAUNCH(q8::rmsnorm_kernel, dim3((op.rows + q8::RMSNORM_ROWS - 1u) / q8::RMSNORM_ROWS),
                   dim3(64u * q8::RMSNORM_ROWS), 0, st, stop,
-                  (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
-                  op.rows, op.cols, op.scalar, split_to);
+                  (float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
+                  op.rows, op.cols, op.scalar, split_to,
+                  update != nullptr ? (const float *)update->a[0]->ptr : (const float *)nullptr,
+                  update != nullptr ? update->scalar : 0.0f);
         break;
     case OP_ARGMAX: {
         float *part_v = (float *)op.a[1]->ptr;
@@ -1404,6 +1411,20 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 }
             }
             flush();
+            // h += alpha * t, then the norm of h (the end of one block of a layer
+            // and the start of the next, at prefill sizes): the norm does the
+            // update on its way, one launch instead of two. The update must be
+            // the launch right before, over exactly the norm's input.
+            if (op.kind == OP_RMSNORM && !plan.empty() && plan.back().single != nullptr &&
+                plan.back().single->kind == OP_AXPY && plan.back().update == nullptr) {
+                const Op &up = *plan.back().single;
+                if (up.a[1] == op.a[0] && (uint64_t)op.rows * op.cols == up.extra &&
+                    up.a[0] != op.a[0] && up.a[0] != op.a[2] && op.a[1] != op.a[0]) {
+                    plan.back().single = &op;
+                    plan.back().update = &up;
+                    continue;
+                }
+            }
             Launch one;
             one.single = &op;
             plan.push_back(std::move(one));
@@ -1421,9 +1442,9 @@ hipError_t issue_launch(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &l) {
     }
     if (l.split_xs_off >= 0) {
         return launch_single(ctx, stop, *l.single, (uint16_t *)(ctx->ws.xs + l.split_xs_off),
-                             l.split_cols);
+                             l.split_cols, l.update);
     }
-    return launch_single(ctx, stop, *l.single);
+    return launch_single(ctx, stop, *l.single, nullptr, 0, l.update);
 }
 
 // Issue the launches; the last one carries the commit's stop event.
