@@ -239,6 +239,73 @@ def _gemm_point(flops, t, steps, shapes):
     return out
 
 
+def _layer_matrices(ctx, M):
+    """The seven projection matrices of a Qwen3-0.6B layer, sealed, each with an X
+    [M, K] and a Y [M, N] of its own: (products, buffers to free, by name)."""
+    products, keep, mats = [], [], {}
+    for name, rows, cols in S.QWEN3_0_6B_LAYER:
+        raw = S.make_weights(rows, cols, S.tensor_seed(2, 0, name))
+        m = H.Matrix.load(ctx, raw, cols, rows)
+        xb = ctx.buffer(M * cols * 4)
+        xb.upload(0, S.make_activations(M * cols, rows))
+        yb = ctx.buffer(M * rows * 4)
+        keep += [m.buf, xb, yb]
+        mats[name] = (m, xb, yb, rows, cols)
+        products.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA))
+    return products, keep, mats
+
+
+def _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, out, keep):
+    """The layer as an executor encodes it, with the operators between the
+    products (attention itself stands outside this path: o reads q's output):
+    norm -> q,k,v -> o -> residual -> norm -> gate,up -> gated activation ->
+    down -> residual, at M tokens and at the engine's prefill chunk of 128. The
+    norms and the activation write the split form of their result themselves,
+    the second norm takes the residual update in front of it."""
+    hid, ffn = mats["q"][4], mats["gate"][3]
+    bufs = {n: ctx.buffer(M * c * 4) for n, c in (("h", hid), ("xn", hid), ("xn2", hid), ("act", ffn))}
+    wn = ctx.buffer(hid * 4)
+    wn.upload(0, (1.0 + 0.1 * S.make_activations(hid, 11)).astype(np.float32))
+    bufs["h"].upload(0, S.make_activations(M * hid, 12))
+    def layer(tokens):
+        def prod(name, x):
+            m, _, yb, rows, cols = mats[name]
+            return tmh_product(m.buf.raw, x.raw, yb.raw, rows, cols, tokens, TMH_GEMM_MMA)
+        return [tmh_product(wn.raw, bufs["h"].raw, bufs["xn"].raw, tokens, hid, tokens, TMH_RMSNORM),
+                prod("q", bufs["xn"]), prod("k", bufs["xn"]), prod("v", bufs["xn"]),
+                prod("o", mats["q"][2]),
+                tmh_product(bufs["h"].raw, mats["o"][2].raw, bufs["h"].raw, 1, tokens * hid, 1, TMH_AXPY),
+                tmh_product(wn.raw, bufs["h"].raw, bufs["xn2"].raw, tokens, hid, tokens, TMH_RMSNORM),
+                prod("gate", bufs["xn2"]), prod("up", bufs["xn2"]),
+                tmh_product(mats["gate"][2].raw, mats["up"][2].raw, bufs["act"].raw, 1, tokens * ffn, 1,
+                            TMH_SILU_MUL),
+                prod("down", bufs["act"]),
+                tmh_product(bufs["h"].raw, mats["down"][2].raw, bufs["h"].raw, 1, tokens * hid, 1,
+                            TMH_AXPY)]
+    for key, tokens in (("layer_with_operators", M), ("layer_with_operators_m128", 128)):
+        t = run_steps(host, ctx, layer(tokens), warmup, steps, grouped=True)
+        stats = step_stats(t, steps)
+        us = stats.get("median_us") or stats["mean_us"]
+        out[key] = {
+            "M": tokens, "us": us, "step_us": stats, "launches_per_step": t.launches / steps,
+            "tflops": flops_total * tokens / M / us / 1e6,
+            "order": "rmsnorm -> q,k,v -> o(q) -> axpy -> rmsnorm -> gate,up -> silu_mul -> down -> axpy; "
+                     "no attention"}
+    keep += list(bufs.values()) + [wn]
+
+
+def bench_layer(host, ctx, steps, warmup):
+    """Only the layer with its operators (for a kernel trace of just these launches)."""
+    M = 512
+    out = {"workload": "Qwen3-0.6B layer with its operators, 512 and 128 tokens (no attention)", "M": M}
+    products, keep, mats = _layer_matrices(ctx, M)
+    flops_total = sum(2.0 * M * p.rows * p.cols for p in products)
+    _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, out, keep)
+    for b in keep:
+        b.free()
+    return out
+
+
 def bench_gemm(host, ctx, steps, warmup):
     """BASELINE config 2: M = 512 tokens against the seven projection matrices
     of a Qwen3-0.6B layer, each with its own X [512, K]. Timed as one dispatch
@@ -250,16 +317,7 @@ def bench_gemm(host, ctx, steps, warmup):
     apart, means otherwise."""
     M = 512
     out = {"M": M, "shapes": []}
-    products, keep, mats = [], [], {}
-    for name, rows, cols in S.QWEN3_0_6B_LAYER:
-        raw = S.make_weights(rows, cols, S.tensor_seed(2, 0, name))
-        m = H.Matrix.load(ctx, raw, cols, rows)
-        xb = ctx.buffer(M * cols * 4)
-        xb.upload(0, S.make_activations(M * cols, rows))
-        yb = ctx.buffer(M * rows * 4)
-        keep += [m.buf, xb, yb]
-        mats[name] = (m, xb, yb, rows, cols)
-        products.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA))
+    products, keep, mats = _layer_matrices(ctx, M)
     flops_total = sum(2.0 * M * p.rows * p.cols for p in products)
     us_sum = 0.0
     for (name, rows, cols), p in zip(S.QWEN3_0_6B_LAYER, products):
@@ -292,41 +350,7 @@ def bench_gemm(host, ctx, steps, warmup):
     out["dependent_layer"] = {"us": us, "step_us": stats, "launches_per_step": t.launches / steps,
                               "tflops": flops_total / us / 1e6,
                               "order": "q,k,v -> o(q) -> gate,up -> down(gate); no attention"}
-    # The layer as an executor encodes it, with the operators between the
-    # products (attention itself stands outside this path: o reads q's output):
-    # norm -> q,k,v -> o -> residual -> norm -> gate,up -> gated activation ->
-    # down -> residual. The norms and the activation write the split form of
-    # their result themselves, so only o's launch keeps a split pass.
-    hid, ffn = mats["q"][4], mats["gate"][3]
-    bufs = {n: ctx.buffer(M * c * 4) for n, c in (("h", hid), ("xn", hid), ("xn2", hid), ("act", ffn))}
-    wn = ctx.buffer(hid * 4)
-    wn.upload(0, (1.0 + 0.1 * S.make_activations(hid, 11)).astype(np.float32))
-    bufs["h"].upload(0, S.make_activations(M * hid, 12))
-    def layer(tokens):
-        def prod(name, x):
-            m, _, yb, rows, cols = mats[name]
-            return tmh_product(m.buf.raw, x.raw, yb.raw, rows, cols, tokens, TMH_GEMM_MMA)
-        return [tmh_product(wn.raw, bufs["h"].raw, bufs["xn"].raw, tokens, hid, tokens, TMH_RMSNORM),
-                prod("q", bufs["xn"]), prod("k", bufs["xn"]), prod("v", bufs["xn"]),
-                prod("o", mats["q"][2]),
-                tmh_product(bufs["h"].raw, mats["o"][2].raw, bufs["h"].raw, 1, tokens * hid, 1, TMH_AXPY),
-                tmh_product(wn.raw, bufs["h"].raw, bufs["xn2"].raw, tokens, hid, tokens, TMH_RMSNORM),
-                prod("gate", bufs["xn2"]), prod("up", bufs["xn2"]),
-                tmh_product(mats["gate"][2].raw, mats["up"][2].raw, bufs["act"].raw, 1, tokens * ffn, 1,
-                            TMH_SILU_MUL),
-                prod("down", bufs["act"]),
-                tmh_product(bufs["h"].raw, mats["down"][2].raw, bufs["h"].raw, 1, tokens * hid, 1,
-                            TMH_AXPY)]
-    for key, tokens in (("layer_with_operators", M), ("layer_with_operators_m128", 128)):
-        t = run_steps(host, ctx, layer(tokens), warmup, steps, grouped=True)
-        stats = step_stats(t, steps)
-        us = stats.get("median_us") or stats["mean_us"]
-        out[key] = {
-            "M": tokens, "us": us, "step_us": stats, "launches_per_step": t.launches / steps,
-            "tflops": flops_total * tokens / M / us / 1e6,
-            "order": "rmsnorm -> q,k,v -> o(q) -> axpy -> rmsnorm -> gate,up -> silu_mul -> down -> axpy; "
-                     "no attention"}
-    keep += list(bufs.values()) + [wn]
+    _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, out, keep)
     # the engine's prefill chunk
     m128 = [tmh_product(p.w, p.x, p.y, p.rows, p.cols, 128, TMH_GEMM_MMA) for p in products]
     t = run_steps(host, ctx, m128, warmup, steps, grouped=True)
@@ -725,7 +749,8 @@ def main():
                          "crashed on stream capture here)")
     ap.add_argument("--ungrouped", action="store_true",
                     help="one commit per GEMV instead of one group per step")
-    ap.add_argument("--workload", choices=["decode", "gemma", "sweep", "chain", "f16", "traffic"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "gemma", "sweep", "chain", "f16", "layer", "traffic"],
+                    default="decode",
                     help="decode (default, the headline line); gemma / sweep print the "
                          "BASELINE config 3 / 4 measurements as one JSON object")
     args = ap.parse_args()
@@ -743,7 +768,7 @@ def main():
         return
     if args.workload != "decode":
         fn = {"gemma": bench_gemma, "sweep": bench_sweep, "chain": bench_chain,
-              "f16": bench_f16}[args.workload]
+              "f16": bench_f16, "layer": bench_layer}[args.workload]
         extra = {"recorded": not args.no_recorded} if args.workload == "chain" else {}
         print(json.dumps(fn(host, ctx, args.steps, args.warmup, **extra)), flush=True)
         ctx.close()
