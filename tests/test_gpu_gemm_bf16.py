@@ -293,6 +293,62 @@ def test_the_operator_in_front_writes_the_split_form_itself(ctx, kind, batch):
         m[4].free()
 
 
+@pytest.mark.parametrize("batch", [512, 128, 40])
+def test_update_norm_and_products_in_one_group(ctx, batch):
+    # The seam between two blocks of a layer: h += t, xn = rmsnorm(h), then the
+    # products that read xn. In one group that is two launches (the norm does the
+    # update in front of itself and writes xn's split form for the products
+    # behind it); h, xn and the products come out bit for bit as with the
+    # update, the norm and the products' group issued one after the other.
+    cols = 1024
+    shapes = [(6144, cols), (6144, cols), (6144, cols)]
+    assert H.gemm_mma_launch_tile([(r, c, batch) for r, c in shapes]) != 0
+    h0 = S.make_activations(batch * cols, 91)
+    t = S.make_activations(batch * cols, 92)
+    wn = upload_new(ctx, (1.0 + 0.1 * S.make_activations(cols, 9)).astype(np.float32))
+    hb, tb = upload_new(ctx, h0), upload_new(ctx, t)
+    xb = ctx.buffer(batch * cols * 4)
+    mats = []
+    for i, (rows, c) in enumerate(shapes):
+        w = S.make_weights(rows, c, 800 + i)
+        mats.append((rows, weights_buffer(ctx, w, rows, c, True), ctx.buffer(batch * rows * 4)))
+
+    def products():
+        for rows, wb, yb in mats:
+            ctx.q8_0_gemm_mma(wb, xb, yb, rows, cols, batch, 0, 0)
+
+    def state():
+        ctx.fence()
+        return [hb.download_f32(0, batch * cols).copy(), xb.download_f32(0, batch * cols).copy()] + \
+               [yb.download_f32(0, batch * rows).copy() for rows, _, yb in mats]
+
+    ctx.f32_axpy(tb, hb, 1.0, batch * cols)
+    ctx.rmsnorm(hb, wn, xb, batch, cols, 1e-6)
+    ctx.begin_group()
+    products()
+    ctx.end_group()
+    apart = state()
+    assert np.array_equal(bits(apart[0]), bits(h0 + t))
+
+    for attempt in range(2):
+        hb.upload(0, h0)
+        xb.zero(0, batch * cols * 4)
+        for _, _, yb in mats:
+            yb.zero(0, yb.len())
+        before = ctx.kernel_launches()
+        ctx.begin_group()
+        ctx.f32_axpy(tb, hb, 1.0, batch * cols)
+        ctx.rmsnorm(hb, wn, xb, batch, cols, 1e-6)
+        products()
+        ctx.end_group()
+        fused = state()
+        assert ctx.kernel_launches() == before + 2
+        for i, (a, b) in enumerate(zip(apart, fused)):
+            assert np.array_equal(bits(a), bits(b)), f"attempt {attempt}, buffer {i}"
+    for b in [wn, hb, tb, xb] + [m[1] for m in mats] + [m[2] for m in mats]:
+        b.free()
+
+
 @pytest.mark.parametrize("rows,cols,batch", [(8192, 1024, 512), (8191, 1024, 512), (7936, 1024, 512),
                                              (32768, 1024, 65), (32768, 1024, 64), (32513, 1024, 65),
                                              (4096, 4096, 128), (4096, 4096, 129), (6144, 2048, 512),
