@@ -125,6 +125,16 @@ int tm_hip_copy_f32(tm_hip_ctx *ctx, tm_hip_buffer *src, uint32_t src_off, tm_hi
 int tm_hip_f32_scale(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *y, float factor, uint32_t n,
                      char *err, size_t err_cap);
 
+/* y[i] = (float)x[i], i < n, x in IEEE binary16 (n * 2 bytes), exact
+ * (native/metal/tm_metal.h:118-120). */
+int tm_hip_cast_f16_f32(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *y, uint32_t n, char *err,
+                        size_t err_cap);
+
+/* y[i] = (half)x[i], i < n, y in IEEE binary16 (n * 2 bytes): round to nearest
+ * even, overflow to infinity, a NaN stays a NaN (native/metal/tm_metal.h:122-124). */
+int tm_hip_cast_f32_f16(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *y, uint32_t n, char *err,
+                        size_t err_cap);
+
 /* y[i] = y[i] + alpha * a[i], i < n: multiply, then add, unfused
  * (native/metal/tm_metal.h:115-116). */
 int tm_hip_f32_axpy(tm_hip_ctx *ctx, tm_hip_buffer *a, tm_hip_buffer *y, float alpha, uint32_t n,

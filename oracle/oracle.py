@@ -18,7 +18,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libq8_oracle.so")
 
 __all__ = [
-    "OracleError", "build", "lib", "f16_to_f32", "f32_to_f16_bits", "dequant_q8_0",
+    "OracleError", "build", "lib", "f16_to_f32", "f32_to_f16_bits", "f16_to_f32_array",
+    "f32_to_f16_bits_array", "dequant_q8_0",
     "quantize_row_q8_0", "dot_q8_0_x_f32", "dot_q8_0_q8_0", "gemv_q8_0_f32",
     "gemv_q8_0_q8_0", "gemm_q8_0_f32", "gemm_q8_0_q8_0", "gemv_q8_0_f32_dequant_first",
     "gemv_q8_0_f64", "Rng", "boundary_weights", "boundary_input", "KRng",
@@ -57,6 +58,10 @@ def lib() -> ctypes.CDLL:
         L.q8o_f16_to_f32.argtypes = [c.c_uint16]
         L.q8o_f32_to_f16_bits.restype = c.c_uint16
         L.q8o_f32_to_f16_bits.argtypes = [c.c_float]
+        L.q8o_f16_to_f32_n.restype = None
+        L.q8o_f16_to_f32_n.argtypes = [c.c_void_p, c.c_size_t, f32p]
+        L.q8o_f32_to_f16_bits_n.restype = None
+        L.q8o_f32_to_f16_bits_n.argtypes = [f32p, c.c_size_t, c.c_void_p]
         L.q8o_dequant_q8_0.argtypes = [u8p, c.c_size_t, f32p]
         L.q8o_quantize_row_q8_0.argtypes = [f32p, c.c_size_t, i8p, f32p]
         L.q8o_validate_q8_0_row.argtypes = [c.c_size_t, c.c_size_t]
@@ -118,6 +123,20 @@ def f16_to_f32(bits: int) -> np.float32:
 
 def f32_to_f16_bits(value) -> int:
     return int(lib().q8o_f32_to_f16_bits(float(np.float32(value))))
+
+
+def f16_to_f32_array(bits) -> np.ndarray:
+    b = np.ascontiguousarray(bits, dtype=np.uint16).ravel()
+    out = np.empty(b.size, dtype=np.float32)
+    lib().q8o_f16_to_f32_n(_ptr(b), b.size, _ptr(out))
+    return out
+
+
+def f32_to_f16_bits_array(values) -> np.ndarray:
+    v = _f32(values).ravel()
+    out = np.empty(v.size, dtype=np.uint16)
+    lib().q8o_f32_to_f16_bits_n(_ptr(v), v.size, _ptr(out))
+    return out
 
 
 def dequant_q8_0(raw) -> np.ndarray:

@@ -77,6 +77,22 @@ uint16_t q8o_f32_to_f16_bits(float value) {
     return (uint16_t)(sign | (uint16_t)((uint32_t)exp << 10) | (uint16_t)(rounded >> 13));
 }
 
+/* The two conversions over arrays (the checker of the device cast operators,
+ * crates/metal/src/tests.rs:257-305): element by element through the functions above. */
+void q8o_f16_to_f32_n(const uint16_t *bits, size_t n, float *out) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) {
+        out[i] = q8o_f16_to_f32(bits[i]);
+    }
+}
+
+void q8o_f32_to_f16_bits_n(const float *values, size_t n, uint16_t *out) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) {
+        out[i] = q8o_f32_to_f16_bits(values[i]);
+    }
+}
+
 static inline uint16_t read_u16_le(const uint8_t *p) {
     return (uint16_t)((uint16_t)p[0] | ((uint16_t)p[1] << 8));
 }

@@ -29,6 +29,11 @@ float q8o_f16_to_f32(uint16_t bits);
  * `exp >= 0x1f` branch at :150-153 does not keep the NaN payload). */
 uint16_t q8o_f32_to_f16_bits(float value);
 
+/* The two functions above over n elements (crates/metal/src/tests.rs:257-305 checks the
+ * device casts against them element by element). */
+void q8o_f16_to_f32_n(const uint16_t *bits, size_t n, float *out);
+void q8o_f32_to_f16_bits_n(const float *values, size_t n, uint16_t *out);
+
 /* crates/tuckcore/src/tensor.rs:94-104: out[i] = d * q for `blocks` blocks. */
 void q8o_dequant_q8_0(const uint8_t *bytes, size_t blocks, float *out);
 

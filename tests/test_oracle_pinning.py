@@ -115,6 +115,20 @@ def test_f32_to_f16_nan_becomes_infinity():
     assert O.f32_to_f16_bits(np.float32(-np.inf)) == 0xFC00
 
 
+def test_array_forms_are_the_scalar_functions_element_by_element():
+    enc = np.arange(1 << 16, dtype=np.uint16)
+    want = np.array([O.f16_to_f32(int(b)) for b in enc], dtype=np.float32)
+    assert np.array_equal(O.f16_to_f32_array(enc).view(np.uint32), want.view(np.uint32))
+    # a wide sample of f32, with all finite ones against numpy's IEEE rounding too
+    rng = np.random.default_rng(77)
+    vals = rng.integers(0, 1 << 32, size=2_000_000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    got = O.f32_to_f16_bits_array(vals)
+    some = np.array([O.f32_to_f16_bits(v) for v in vals[:50_000]], dtype=np.uint16)
+    assert np.array_equal(got[:50_000], some)
+    finite = np.isfinite(vals)
+    assert np.array_equal(got[finite], _np_f16_bits(vals[finite]))
+
+
 # ---------------------------------------------------------------- dequant --
 
 def test_q8_0_layout_and_scaling():

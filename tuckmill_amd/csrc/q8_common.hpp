@@ -123,6 +123,7 @@ __device__ __forceinline__ float sbyte_to_float(uint32_t w, int i) {
 // over the same 633 MB).
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 template <bool NT, class T> __device__ __forceinline__ T load_maybe_nt(const T *p) {
     if constexpr (NT) {

@@ -34,6 +34,63 @@ __global__ __launch_bounds__(256) void axpy_kernel(const float *a, float *y, flo
     }
 }
 
+// y[i] = (float)x[i], x in IEEE binary16: exact for every encoding (a NaN stays a
+// NaN of the same sign). Eight elements per lane while eight are left (16 bytes in,
+// 32 out), single elements behind them.
+__global__ __launch_bounds__(256) void cast_f16_f32_kernel(const uint16_t *x, float *y, uint32_t n) {
+    const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * 8u;
+    if (i + 8u <= n) {
+        const u32x4 v = *(const u32x4 *)(x + i);
+        f32x4 lo, hi;
+        lo[0] = f16_bits_to_f32(v[0] & 0xffffu);
+        lo[1] = f16_bits_to_f32(v[0] >> 16);
+        lo[2] = f16_bits_to_f32(v[1] & 0xffffu);
+        lo[3] = f16_bits_to_f32(v[1] >> 16);
+        hi[0] = f16_bits_to_f32(v[2] & 0xffffu);
+        hi[1] = f16_bits_to_f32(v[2] >> 16);
+        hi[2] = f16_bits_to_f32(v[3] & 0xffffu);
+        hi[3] = f16_bits_to_f32(v[3] >> 16);
+        *(f32x4 *)(y + i) = lo;
+        *(f32x4 *)(y + i + 4u) = hi;
+    } else {
+        for (uint32_t k = i; k < n; ++k) {
+            y[k] = f16_bits_to_f32(x[k]);
+        }
+    }
+}
+
+// binary32 -> binary16 for the cast operator: round to nearest even, overflow to
+// infinity, magnitudes below 2^-25 to a signed zero - the rounding of
+// crates/tuckcore/src/tensor.rs:145-178 on every number - and a NaN to the quiet
+// NaN of its sign, as a conversion in hardware gives (native/metal/kernels.metal:50-58;
+// tensor.rs:150-153 would make it an infinity).
+__device__ __forceinline__ uint32_t cast_to_f16_bits(float v) {
+    const uint32_t bits = __float_as_uint(v);
+    if ((bits & 0x7fffffffu) > 0x7f800000u) {
+        return ((bits >> 16) & 0x8000u) | 0x7e00u;
+    }
+    return f32_to_f16_bits(v);
+}
+
+// y[i] = (half)x[i]. Eight elements per lane while eight are left.
+__global__ __launch_bounds__(256) void cast_f32_f16_kernel(const float *x, uint16_t *y, uint32_t n) {
+    const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * 8u;
+    if (i + 8u <= n) {
+        const f32x4 lo = *(const f32x4 *)(x + i);
+        const f32x4 hi = *(const f32x4 *)(x + i + 4u);
+        u32x4 v;
+        v[0] = cast_to_f16_bits(lo[0]) | (cast_to_f16_bits(lo[1]) << 16);
+        v[1] = cast_to_f16_bits(lo[2]) | (cast_to_f16_bits(lo[3]) << 16);
+        v[2] = cast_to_f16_bits(hi[0]) | (cast_to_f16_bits(hi[1]) << 16);
+        v[3] = cast_to_f16_bits(hi[2]) | (cast_to_f16_bits(hi[3]) << 16);
+        *(u32x4 *)(y + i) = v;
+    } else {
+        for (uint32_t k = i; k < n; ++k) {
+            y[k] = (uint16_t)cast_to_f16_bits(x[k]);
+        }
+    }
+}
+
 // The three operators below can write, next to their f32 result, its split form
 // for the bf16 matrix cores (q8_gemm_bf16x3.hpp) when the product that reads
 // the result follows directly: `xs` non-null, the result taken as a

@@ -116,7 +116,7 @@ void alloc_release(Alloc *a) {
 enum OpKind {
     OP_GEMV_LIST, OP_MMA, OP_ROW, OP_ROW_INDIRECT, OP_COPY, OP_PACK, OP_QUANT, OP_I8,
     OP_SCALE, OP_AXPY, OP_SILU_MUL, OP_GELU_MUL, OP_RMSNORM, OP_ARGMAX,
-    OP_F16_GEMM, OP_F16_ROW, OP_F16_ROW_INDIRECT
+    OP_F16_GEMM, OP_F16_ROW, OP_F16_ROW_INDIRECT, OP_CAST_F16_F32, OP_CAST_F32_F16
 };
 
 struct Op {
@@ -1029,6 +1029,14 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op,
     case OP_SCALE:
         Q8_LAUNCH(q8::scale_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
                   (const float *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.scalar, op.extra);
+        break;
+    case OP_CAST_F16_F32:
+        Q8_LAUNCH(q8::cast_f16_f32_kernel, dim3((op.extra + 2047u) / 2048u), dim3(256), 0, st, stop,
+                  (const uint16_t *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.extra);
+        break;
+    case OP_CAST_F32_F16:
+        Q8_LAUNCH(q8::cast_f32_f16_kernel, dim3((op.extra + 2047u) / 2048u), dim3(256), 0, st, stop,
+                  (const float *)op.a[0]->ptr, (uint16_t *)op.a[1]->ptr, op.extra);
         break;
     case OP_AXPY:
         Q8_LAUNCH(q8::axpy_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
@@ -2059,9 +2067,12 @@ int tm_hip_copy_f32(tm_hip_ctx *ctx, tm_hip_buffer *src, uint32_t src_off, tm_hi
 
 namespace {
 
-// x -> y over n f32 elements with one scalar (native/metal/tm_metal.m:770-810).
+// x -> y over n elements (f32, or binary16 on the side a cast names) with one scalar
+// (native/metal/tm_metal.m:770-810).
 int submit_1d(tm_hip_ctx *ctx, OpKind kind, tm_hip_buffer *a, tm_hip_buffer *b, float scalar,
               uint32_t n, char *err, size_t cap, const char *what) {
+    const size_t a_elem = kind == OP_CAST_F16_F32 ? 2u : 4u;
+    const size_t b_elem = kind == OP_CAST_F32_F16 ? 2u : 4u;
     if (check_ctx(ctx, err, cap, what) != TM_HIP_OK) {
         return TM_HIP_ERR_UNSUPPORTED;
     }
@@ -2069,8 +2080,8 @@ int submit_1d(tm_hip_ctx *ctx, OpKind kind, tm_hip_buffer *a, tm_hip_buffer *b, 
         return fail(err, cap, TM_HIP_ERR_BOUNDS, "%s: zero length", what);
     }
     int rc;
-    if ((rc = check_buffer(ctx, a, (size_t)n * 4u, err, cap, what)) != TM_HIP_OK ||
-        (rc = check_buffer(ctx, b, (size_t)n * 4u, err, cap, what)) != TM_HIP_OK) {
+    if ((rc = check_buffer(ctx, a, (size_t)n * a_elem, err, cap, what)) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, b, (size_t)n * b_elem, err, cap, what)) != TM_HIP_OK) {
         return rc;
     }
     if (a->alloc->packed || b->alloc->packed) {
@@ -2130,6 +2141,16 @@ int tm_hip_f32_scale(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *y, float 
 int tm_hip_f32_axpy(tm_hip_ctx *ctx, tm_hip_buffer *a, tm_hip_buffer *y, float alpha, uint32_t n,
                     char *err, size_t err_cap) {
     return submit_1d(ctx, OP_AXPY, a, y, alpha, n, err, err_cap, "f32_axpy");
+}
+
+int tm_hip_cast_f16_f32(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *y, uint32_t n, char *err,
+                        size_t err_cap) {
+    return submit_1d(ctx, OP_CAST_F16_F32, x, y, 0.0f, n, err, err_cap, "cast_f16_f32");
+}
+
+int tm_hip_cast_f32_f16(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *y, uint32_t n, char *err,
+                        size_t err_cap) {
+    return submit_1d(ctx, OP_CAST_F32_F16, x, y, 0.0f, n, err, err_cap, "cast_f32_f16");
 }
 
 int tm_hip_silu_mul_f32(tm_hip_ctx *ctx, tm_hip_buffer *gate, tm_hip_buffer *up, tm_hip_buffer *out,

@@ -241,6 +241,10 @@ _SIGS = {
     "tm_hip_f32_scale": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                          ctypes.c_float, ctypes.c_uint32, ctypes.c_char_p,
                                          ctypes.c_size_t]),
+    "tm_hip_cast_f16_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                            ctypes.c_uint32, ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_cast_f32_f16": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                            ctypes.c_uint32, ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_f32_axpy": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                         ctypes.c_float, ctypes.c_uint32, ctypes.c_char_p,
                                         ctypes.c_size_t]),
@@ -491,6 +495,17 @@ class HipContext:
     #    :2244-2319) --
     def f32_scale(self, x, y, factor, n):
         self._operate("f32_scale", self._lib.tm_hip_f32_scale, x.raw, y.raw, float(factor), n)
+
+    def cast_f16_to_f32(self, x, y, n):
+        """y = (f32) x over n binary16 elements (crates/metal/src/lib.rs:1636-1648)."""
+        self._check_owned(x, y)
+        self._operate("cast_f16_f32", self._lib.tm_hip_cast_f16_f32, x.raw, y.raw, n)
+
+    def cast_f32_to_f16(self, x, y, n):
+        """y = (half) x over n f32 elements, round to nearest even
+        (crates/metal/src/lib.rs:1650-1662)."""
+        self._check_owned(x, y)
+        self._operate("cast_f32_f16", self._lib.tm_hip_cast_f32_f16, x.raw, y.raw, n)
 
     def f32_axpy(self, a, y, alpha, n):
         self._operate("f32_axpy", self._lib.tm_hip_f32_axpy, a.raw, y.raw, float(alpha), n)

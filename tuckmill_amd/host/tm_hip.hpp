@@ -451,6 +451,18 @@ class HipContext {
             return tm_hip_f32_scale(raw(), x.raw(), y.raw(), factor, n, e, ERR_CAP);
         });
     }
+    // y = (f32) x over n binary16 elements / y = (half) x over n f32 elements
+    // (crates/metal/src/lib.rs:1636-1662).
+    void cast_f16_to_f32(const HipBuffer &x, const HipBuffer &y, uint32_t n) const {
+        operate("cast_f16_f32", [&](char *e) {
+            return tm_hip_cast_f16_f32(raw(), x.raw(), y.raw(), n, e, ERR_CAP);
+        });
+    }
+    void cast_f32_to_f16(const HipBuffer &x, const HipBuffer &y, uint32_t n) const {
+        operate("cast_f32_f16", [&](char *e) {
+            return tm_hip_cast_f32_f16(raw(), x.raw(), y.raw(), n, e, ERR_CAP);
+        });
+    }
     void f32_axpy(const HipBuffer &a, const HipBuffer &y, float alpha, uint32_t n) const {
         operate("f32_axpy", [&](char *e) {
             return tm_hip_f32_axpy(raw(), a.raw(), y.raw(), alpha, n, e, ERR_CAP);
