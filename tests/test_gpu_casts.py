@@ -156,3 +156,41 @@ def test_cast_refusals(ctx):
     ctx.fence()
     f32.free()
     f16.free()
+
+
+def test_lengths_just_below_two_to_the_32(ctx):
+    """n = 2^32 - 5 elements: the last workgroup is partly beyond the end and
+    `n + (elements per workgroup) - 1` does not fit 32 bits. Only the ends are
+    looked at (16 GiB of input stay zero)."""
+    n = (1 << 32) - 5
+    tail = np.array([1.0, -2.5, 65504.0, 1e-7, 3.0, -0.0, 70000.0, 0.5, 0.1, -1.0, 2.0],
+                    dtype=np.float32)
+    xb = ctx.buffer(n * 4)
+    xb.zero(0, n * 4)
+    xb.upload((n - tail.size) * 4, tail)
+    xb.upload(0, np.array([4.0, -8.0], np.float32))
+    hb = ctx.buffer(n * 2 + 32)
+    hb.upload(n * 2, np.full(16, 0xABCD, np.uint16))
+    ctx.cast_f32_to_f16(xb, hb, n)
+    ctx.fence()
+    assert list(hb.download(0, 8).view(np.uint16)) == [0x4400, 0xC800, 0, 0]
+    got = hb.download((n - tail.size) * 2, tail.size * 2 + 32).view(np.uint16)
+    assert np.array_equal(got[:tail.size], O.f32_to_f16_bits_array(tail))
+    assert np.all(got[tail.size:] == 0xABCD)
+    # the way back over the same length, and an f32 operator with one element per lane
+    yb = ctx.buffer(n * 4 + 64)
+    yb.upload(n * 4, np.full(16, 7.0, np.float32))
+    ctx.cast_f16_to_f32(hb, yb, n)
+    ctx.fence()
+    back = yb.download_f32(n - tail.size, tail.size + 16)
+    assert np.array_equal(bits(back[:tail.size]),
+                          bits(O.f16_to_f32_array(O.f32_to_f16_bits_array(tail))))
+    assert np.all(back[tail.size:] == 7.0)
+    ctx.f32_scale(xb, yb, 2.0, n)
+    ctx.fence()
+    doubled = yb.download_f32(n - tail.size, tail.size + 16)
+    assert np.array_equal(bits(doubled[:tail.size]), bits(tail * np.float32(2.0)))
+    assert np.all(doubled[tail.size:] == 7.0)
+    assert list(yb.download_f32(0, 3)) == [8.0, -16.0, 0.0]
+    for b in (xb, hb, yb):
+        b.free()

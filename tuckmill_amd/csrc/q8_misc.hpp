@@ -69,8 +69,8 @@ __global__ __launch_bounds__(256) void row_indirect_kernel(const uint8_t *__rest
 
 __global__ __launch_bounds__(256) void copy_f32_kernel(const float *src, float *dst,
                                                        uint32_t n) {
-    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) {
+    for (uint64_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (uint64_t)gridDim.x * blockDim.x) {
         dst[i] = src[i];
     }
 }

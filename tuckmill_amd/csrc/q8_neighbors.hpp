@@ -15,11 +15,14 @@
 
 namespace q8 {
 
+// The element-wise kernels walk n elements in strides of the whole grid: one
+// step for every size in practice, and no limit from the 2^32 threads a launch
+// may hold (the host caps the grid, tm_hip.cpp::strided_blocks_of).
+
 // y[i] = x[i] * factor
 __global__ __launch_bounds__(256) void scale_kernel(const float *x, float *y, float factor,
                                                     uint32_t n) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i < n) {
+    for (uint64_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256u) {
         y[i] = x[i] * factor;
     }
 }
@@ -27,8 +30,7 @@ __global__ __launch_bounds__(256) void scale_kernel(const float *x, float *y, fl
 // y[i] = y[i] + alpha * a[i]   (multiply, then add: no contraction)
 __global__ __launch_bounds__(256) void axpy_kernel(const float *a, float *y, float alpha,
                                                    uint32_t n) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i < n) {
+    for (uint64_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256u) {
         const float p = __fmul_rn(alpha, a[i]);
         y[i] = __fadd_rn(y[i], p);
     }
@@ -39,7 +41,7 @@ __global__ __launch_bounds__(256) void axpy_kernel(const float *a, float *y, flo
 // 32 out), single elements behind them.
 __global__ __launch_bounds__(256) void cast_f16_f32_kernel(const uint16_t *x, float *y, uint32_t n) {
     const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * 8u;
-    if (i + 8u <= n) {
+    if (i < n && n - i >= 8u) {
         const u32x4 v = *(const u32x4 *)(x + i);
         f32x4 lo, hi;
         lo[0] = f16_bits_to_f32(v[0] & 0xffffu);
@@ -75,7 +77,7 @@ __device__ __forceinline__ uint32_t cast_to_f16_bits(float v) {
 // y[i] = (half)x[i]. Eight elements per lane while eight are left.
 __global__ __launch_bounds__(256) void cast_f32_f16_kernel(const float *x, uint16_t *y, uint32_t n) {
     const uint32_t i = (blockIdx.x * 256u + threadIdx.x) * 8u;
-    if (i + 8u <= n) {
+    if (i < n && n - i >= 8u) {
         const f32x4 lo = *(const f32x4 *)(x + i);
         const f32x4 hi = *(const f32x4 *)(x + i + 4u);
         u32x4 v;
@@ -101,8 +103,8 @@ __global__ __launch_bounds__(256) void cast_f32_f16_kernel(const float *x, uint1
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float *gate, const float *up,
                                                        float *out, uint32_t n, uint16_t *xs,
                                                        uint32_t cols) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i < n) {
+    for (uint64_t e = blockIdx.x * 256u + threadIdx.x; e < n; e += (uint64_t)gridDim.x * 256u) {
+        const uint32_t i = (uint32_t)e;
         const float g = gate[i];
         const float s = g / (1.0f + expf(-g));
         const float v = s * up[i];
@@ -119,8 +121,8 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float *gate, const 
 __global__ __launch_bounds__(256) void gelu_tanh_mul_kernel(const float *gate, const float *up,
                                                             float *out, uint32_t n, uint16_t *xs,
                                                             uint32_t cols) {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i < n) {
+    for (uint64_t e = blockIdx.x * 256u + threadIdx.x; e < n; e += (uint64_t)gridDim.x * 256u) {
+        const uint32_t i = (uint32_t)e;
         const float x = gate[i];
         const float inner = 0.7978845608028654f * x * (1.0f + 0.044715f * x * x);
         const float v = 0.5f * x * (1.0f + tanhf(inner)) * up[i];

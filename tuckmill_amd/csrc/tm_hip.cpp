@@ -571,7 +571,9 @@ GemvKey gemv_key(const Op &op) {
     k.flag = x_aligned_of(op);
     if (op.batch == 1) {
         k.variant = V_DECODE;
-    } else if (op.packed && op.cols >= 1024u) {
+    } else if (op.packed && op.cols >= 1024u && op.cols < (1u << 27)) {
+        // (the kernel indexes a token group's activations and a tile's quants in
+        // 32 bits: rows of 2^27 columns and more take the general form)
         // waves x tokens per wave, measured on 2B-class shapes (the
         // alternatives were within 5 %)
         k.variant = V_SPLIT;
@@ -605,6 +607,18 @@ uint32_t pick_rows_per_tile(uint32_t rows, uint32_t cols, uint32_t tile_bytes, i
         rpt -= (uint32_t)R;
     }
     return rpt;
+}
+
+// Workgroups of `per` elements that cover n (n + per - 1 may not fit 32 bits).
+inline unsigned blocks_of(uint32_t n, uint32_t per) {
+    return (unsigned)(((uint64_t)n + per - 1u) / per);
+}
+
+// The same for the element-wise kernels that stride over what one pass of the
+// grid leaves: at most 2^22 workgroups (a launch holds fewer than 2^32 threads).
+inline unsigned strided_blocks_of(uint32_t n, uint32_t per) {
+    const unsigned blocks = blocks_of(n, per);
+    return blocks < (1u << 22) ? blocks : (1u << 22);
 }
 
 template <int L, int R, int TB, bool XA>
@@ -996,7 +1010,7 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op,
     switch (op.kind) {
     case OP_ROW: {
         float *out = (float *)op.a[1]->ptr;
-        dim3 grid((op.cols + 255u) / 256u);
+        dim3 grid(blocks_of(op.cols, 256u));
         if (op.packed) {
             Q8_LAUNCH(q8::row_kernel<q8::PACKED>, grid, dim3(256), 0, st, stop, w, out, op.rows,
                       op.cols, op.extra, op.y_off);
@@ -1009,7 +1023,7 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op,
     case OP_ROW_INDIRECT: {
         float *out = (float *)op.a[1]->ptr;
         const uint32_t *ids = (const uint32_t *)op.a[2]->ptr;
-        dim3 grid((op.cols + 255u) / 256u);
+        dim3 grid(blocks_of(op.cols, 256u));
         if (op.packed) {
             Q8_LAUNCH(q8::row_indirect_kernel<q8::PACKED>, grid, dim3(256), 0, st, stop, w, out, ids,
                       op.extra, op.rows, op.cols);
@@ -1022,34 +1036,34 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op,
     case OP_COPY: {
         const float *src = (const float *)op.a[0]->ptr + op.x_off;
         float *dst = (float *)op.a[1]->ptr + op.y_off;
-        Q8_LAUNCH(q8::copy_f32_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop, src,
-                  dst, op.extra);
+        Q8_LAUNCH(q8::copy_f32_kernel, dim3(strided_blocks_of(op.extra, 256u)), dim3(256), 0, st,
+                  stop, src, dst, op.extra);
         break;
     }
     case OP_SCALE:
-        Q8_LAUNCH(q8::scale_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
-                  (const float *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.scalar, op.extra);
+        Q8_LAUNCH(q8::scale_kernel, dim3(strided_blocks_of(op.extra, 256u)), dim3(256), 0, st,
+                  stop, (const float *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.scalar, op.extra);
         break;
     case OP_CAST_F16_F32:
-        Q8_LAUNCH(q8::cast_f16_f32_kernel, dim3((op.extra + 2047u) / 2048u), dim3(256), 0, st, stop,
+        Q8_LAUNCH(q8::cast_f16_f32_kernel, dim3(blocks_of(op.extra, 2048u)), dim3(256), 0, st, stop,
                   (const uint16_t *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.extra);
         break;
     case OP_CAST_F32_F16:
-        Q8_LAUNCH(q8::cast_f32_f16_kernel, dim3((op.extra + 2047u) / 2048u), dim3(256), 0, st, stop,
+        Q8_LAUNCH(q8::cast_f32_f16_kernel, dim3(blocks_of(op.extra, 2048u)), dim3(256), 0, st, stop,
                   (const float *)op.a[0]->ptr, (uint16_t *)op.a[1]->ptr, op.extra);
         break;
     case OP_AXPY:
-        Q8_LAUNCH(q8::axpy_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
-                  (const float *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.scalar, op.extra);
+        Q8_LAUNCH(q8::axpy_kernel, dim3(strided_blocks_of(op.extra, 256u)), dim3(256), 0, st,
+                  stop, (const float *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.scalar, op.extra);
         break;
     case OP_SILU_MUL:
-        Q8_LAUNCH(q8::silu_mul_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
-                  (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
+        Q8_LAUNCH(q8::silu_mul_kernel, dim3(strided_blocks_of(op.extra, 256u)), dim3(256), 0, st,
+                  stop, (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
                   op.extra, split_to, split_cols);
         break;
     case OP_GELU_MUL:
-        Q8_LAUNCH(q8::gelu_tanh_mul_kernel, dim3((op.extra + 255u) / 256u), dim3(256), 0, st, stop,
-                  (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
+        Q8_LAUNCH(q8::gelu_tanh_mul_kernel, dim3(strided_blocks_of(op.extra, 256u)), dim3(256), 0,
+                  st, stop, (const float *)op.a[0]->ptr, (const float *)op.a[1]->ptr, (float *)op.a[2]->ptr,
                   op.extra, split_to, split_cols);
         break;
     case OP_RMSNORM:
@@ -1074,12 +1088,12 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op,
         break;
     }
     case OP_F16_ROW:
-        Q8_LAUNCH(q8::f16_row_kernel, dim3((op.cols + 255u) / 256u), dim3(256), 0, st, stop,
+        Q8_LAUNCH(q8::f16_row_kernel, dim3(blocks_of(op.cols, 256u)), dim3(256), 0, st, stop,
                   (const uint16_t *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.cols, op.extra,
                   op.y_off);
         break;
     case OP_F16_ROW_INDIRECT:
-        Q8_LAUNCH(q8::f16_row_indirect_kernel, dim3((op.cols + 255u) / 256u), dim3(256), 0, st, stop,
+        Q8_LAUNCH(q8::f16_row_indirect_kernel, dim3(blocks_of(op.cols, 256u)), dim3(256), 0, st, stop,
                   (const uint16_t *)op.a[0]->ptr, (float *)op.a[1]->ptr,
                   (const uint32_t *)op.a[2]->ptr, op.extra, op.rows, op.cols);
         break;
