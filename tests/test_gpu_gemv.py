@@ -55,8 +55,11 @@ def test_gemv_matches_the_scalar_reference_across_real_shapes(ctx, rows, cols, s
 
 
 def test_raw_and_packed_layouts_give_identical_bits(ctx):
+    # (rows of whole 1024-column chunks stream through LDS in the raw layout: tiles whose
+    # last pass is short, one to six chunks per row)
     for rows, cols, seed in [(17, 64, 3), (1024, 1024, 4), (300, 1152, 9), (77, 6912, 10),
-                             (64, 2016, 11)]:
+                             (64, 2016, 11), (259, 1024, 12), (1021, 2048, 13), (13, 3072, 14),
+                             (4100, 1024, 15), (530, 6144, 16)]:
         w = O.boundary_weights(rows, cols, seed)
         x = O.boundary_input(cols, seed + 100)
         a = gemv(ctx, weights_buffer(ctx, w, rows, cols, False), x, rows, cols)

@@ -50,6 +50,23 @@ def test_decode_kernel_keeps_four_waves_per_simd(resource_remarks):
         assert vgprs <= 128 and occupancy >= 4, f"{vgprs} VGPRs, {occupancy} waves/SIMD"
 
 
+# gemv_list_kernel<RAW, 8 rows, 1 token, ...>: one token over weights as uploaded
+RAW_DECODE_KERNEL = re.compile(r"Function Name: _ZN2q816gemv_list_kernelILi0ELi8ELi1ELb[01]ELi0ELi\d+ELb0EEE")
+
+
+def test_raw_decode_kernel_keeps_four_waves_per_simd(resource_remarks):
+    """It stages a wave's 8 x 1088 bytes per step in LDS: four workgroups of
+    four waves must fit a CU's 160 KiB, and the registers four waves per SIMD."""
+    blocks = _blocks(resource_remarks, RAW_DECODE_KERNEL)
+    assert blocks, "raw decode kernel not found in the resource remarks"
+    for block in blocks:
+        vgprs = int(re.search(r" VGPRs: (\d+)", block).group(1))
+        spill = int(re.search(r"VGPRs Spill: (\d+)", block).group(1))
+        lds = int(re.search(r"LDS Size \[bytes/block\]: (\d+)", block).group(1))
+        assert spill == 0 and vgprs <= 128, f"{vgprs} VGPRs, {spill} spilled"
+        assert lds == 4 * 8 * 1088 and 4 * lds <= 160 * 1024
+
+
 # gemm_bf16x3_kernel<WM, 4, 2, NS>: the 128-token and the 64-token tile
 BF16_KERNEL = re.compile(r"Function Name: _ZN2q818gemm_bf16x3_kernelILi[12]ELi4ELi2ELi[34]EEE")
 

@@ -419,6 +419,122 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs
                                     });
 }
 
+// One token over weights in the raw layout (34-byte blocks: f16 scale, 32
+// quants), rows of whole 1024-column chunks. A lane's 16 quants start 2 or 18
+// bytes into a block, at an even address: loaded from memory in that shape, a
+// wave's 16-byte pieces straddle the aligned ones and the step runs at half the
+// sealed layout's rate. Instead the wave streams the R x 1088 bytes of a step
+// (R rows of one chunk; 1088 = 68 aligned 16-byte pieces) exactly like sealed
+// quants - aligned, contiguous, non-temporal - parks them in its own piece of
+// LDS, and every lane reads back the five aligned dwords that hold its quants
+// and moves the bytes into place (even lanes find the block's scale in front of
+// them; odd lanes take it from their neighbour). From there on the registers
+// and the arithmetic are those of stream_rows. The loads of step s+1 are in
+// flight while step s is multiplied.
+constexpr uint32_t RAW_CHUNK_BYTES = 1088u; // 32 blocks of 34 bytes
+template <int R> constexpr uint32_t raw_stage_bytes() { return (uint32_t)R * RAW_CHUNK_BYTES; }
+
+template <int R, bool XA>
+__device__ __forceinline__ void stream_rows_raw(const WView<RAW> &wv, const float *x, float *y,
+                                                uint32_t cols, uint32_t row_first,
+                                                uint32_t row_end, uint32_t lane, uint8_t *stage,
+                                                float *res, float alpha) {
+    constexpr uint32_t PIECES = (uint32_t)R * 68u;      // 16-byte pieces of a step
+    constexpr int NL = (int)((PIECES + 63u) / 64u);     // loads per lane and step
+    const uint32_t full = cols >> 10;
+    // Piece g = i * 64 + lane of a step is piece g % 68 of row g / 68 and is
+    // staged at byte 16 g; a last, partly filled round of pieces is left to the
+    // lanes below PIECES % 64.
+    const uint32_t row_bytes = (uint32_t)wv.row_bytes;
+    auto piece_offset = [&](int i, uint32_t last) { // from the step's first byte
+        const uint32_t g = (uint32_t)i * 64u + lane;
+        const uint32_t row = g / 68u;
+        return (row < last ? row : last) * row_bytes + (g % 68u) * 16u;
+    };
+    uint32_t poff[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        poff[i] = piece_offset(i, (uint32_t)R - 1u);
+    }
+    const bool tail_lane = lane < PIECES % 64u || PIECES % 64u == 0u;
+    auto fetch = [&](uint32_t r0, uint32_t c, u32x4 (&p)[NL]) {
+        const uint32_t last = row_end - 1u - r0; // rows past the tile's end repeat its last row
+        const uint8_t *base = wv.base + (size_t)r0 * wv.row_bytes + (size_t)c * RAW_CHUNK_BYTES;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const uint32_t o = last >= (uint32_t)R - 1u ? poff[i] : piece_offset(i, last);
+            if (i < NL - 1 || tail_lane) {
+                p[i] = __builtin_nontemporal_load((const u32x4 *)(base + o));
+            }
+        }
+    };
+    // this lane's window in a staged row: the aligned dword at or below the
+    // block's first byte (even lanes) or its 17th (odd lanes)
+    const uint32_t off = (lane >> 1) * 34u + (lane & 1u) * 16u;
+    const bool high = (off & 2u) != 0u; // quants from dword 1 on, the scale in dword 0's upper half
+    const uint32_t sel = high ? 0x07060504u : 0x05040302u;
+    const uint8_t *window = stage + (off & ~3u);
+
+    float xv[16];
+    if (full == 1u) {
+        load_x<16, XA>(x + lane * 16u, xv);
+    }
+    const uint32_t nsteps = ((row_end - row_first + R - 1) / R) * full;
+    uint32_t r0 = row_first, c = 0;
+    u32x4 p[NL];
+    fetch(r0, 0, p);
+    float acc[R];
+    for (uint32_t step = 0; step < nsteps; ++step) {
+        __builtin_amdgcn_wave_barrier(); // the previous step's reads come first
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            if (i < NL - 1 || tail_lane) {
+                *(u32x4 *)(stage + (uint32_t)i * 1024u + lane * 16u) = p[i];
+            }
+        }
+        uint32_t cn = c + 1u, rn = r0;
+        if (cn == full) {
+            cn = 0;
+            rn = r0 + (uint32_t)R;
+        }
+        if (step + 1u < nsteps) {
+            fetch(rn, cn, p);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (c == 0u) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                acc[r] = 0.0f;
+            }
+        }
+        if (full > 1u) {
+            load_x<16, XA>(x + (c << 10) + lane * 16u, xv);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t *w = (const uint32_t *)(window + (uint32_t)r * RAW_CHUNK_BYTES);
+            const uint32_t d0 = w[0], d1 = w[1], d2 = w[2], d3 = w[3], d4 = w[4];
+            uint32_t q[4];
+            q[0] = __builtin_amdgcn_perm(d1, d0, sel);
+            q[1] = __builtin_amdgcn_perm(d2, d1, sel);
+            q[2] = __builtin_amdgcn_perm(d3, d2, sel);
+            q[3] = __builtin_amdgcn_perm(d4, d3, sel);
+            const uint32_t own = high ? d0 >> 16 : d0;
+            // quad_perm [0, 0, 2, 2]: odd lanes take their even neighbour's scale
+            const uint32_t sb =
+                (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own, 0xA0, 0xf, 0xf, false) & 0xffffu;
+            acc[r] = __builtin_fmaf(f16_bits_to_f32(sb), piece_dot<16>(q, xv), acc[r]);
+        }
+        if (cn == 0u) {
+            reduce_store<R>(acc, y, r0, row_end, lane, true, res, alpha);
+        }
+        c = cn;
+        r0 = rn;
+    }
+}
+
 // Gate and up projection of the same activations with the gated activation on
 // top: out[r] = act(gate[r]) * up[r], act = silu (kind 0) or ggml's tanh GELU
 // (kind 1), the expressions of silu_mul_kernel / gelu_tanh_mul_kernel. After
@@ -594,6 +710,17 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
                     return;
                 }
             }
+        }
+    }
+
+    if constexpr (TB == 1 && L == RAW) {
+        // One token over weights as uploaded: rows of whole 1024-column chunks
+        // stream through LDS (stream_rows_raw); other shapes take the general path.
+        if (full >= 1u && (cols & 1023u) == 0u) {
+            __shared__ __attribute__((aligned(16))) uint8_t raw_stage[4][raw_stage_bytes<R>()];
+            stream_rows_raw<R, XA>(wv, x, y, cols, row_first, row_end, lane, raw_stage[wave], d.res,
+                                   d.alpha);
+            return;
         }
     }
 

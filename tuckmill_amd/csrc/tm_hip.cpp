@@ -886,8 +886,12 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     bool norm_written = false;
     bool fused = launch.norm != nullptr; // the launch needs the kernel variant with fused forms
     const int R = key.variant == V_GENERAL ? kGemvR4 : kGemvR1;
-    // a workgroup's tile in the token-split kernel, a wave's tile otherwise
-    const uint32_t tile_bytes = key.variant == V_SPLIT ? 32768u : 8192u;
+    // a workgroup's tile in the token-split kernel, a wave's tile otherwise (one
+    // token over raw weights: two passes per wave, so that the second pass's
+    // loads fly while the first goes through LDS)
+    const uint32_t tile_bytes = key.variant == V_SPLIT ? 32768u
+                                : (!key.packed && key.variant == V_DECODE) ? 16384u
+                                                                           : 8192u;
     uint32_t tiles = 0;
     uint64_t launch_bytes = 0;
     for (const Op *op : ops) {
