@@ -70,6 +70,20 @@ def test_buffers_are_context_scoped_and_accounted(ctx):
     other.close()
 
 
+def test_an_allocation_the_device_cannot_hold_is_refused_and_leaves_the_context_usable(ctx):
+    # crates/metal/src/lib.rs:732-745: an allocation failure is "Unavailable", not a crash
+    before = ctx.allocated_bytes()
+    with pytest.raises(H.TuckmillError) as e:
+        ctx.buffer(1 << 40)  # 1 TiB: more than the device has
+    assert e.value.abi_code == H.TM_HIP_ERR_ALLOC and e.value.code == "Unavailable"
+    assert ctx.allocated_bytes() == before
+    b = ctx.buffer(64)
+    b.upload(0, np.arange(16, dtype=np.float32))
+    assert np.array_equal(b.download_f32(0, 16), np.arange(16, dtype=np.float32))
+    b.free()
+    assert ctx.allocated_bytes() == before
+
+
 def test_dispatch_completion_accounting_is_exact(ctx):
     wb, xb, yb = ones_problem(ctx, xval=2.0)
     base = ctx.committed_dispatches()
