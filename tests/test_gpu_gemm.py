@@ -93,6 +93,29 @@ def test_every_token_of_the_small_gemm_equals_its_own_gemv(ctx, rows, cols, batc
         assert np.array_equal(bits(single), bits(got[b])), f"token {b}"
 
 
+@pytest.mark.parametrize("x_off", [0, 3])
+@pytest.mark.parametrize("rows,cols,batch", [(64, 1024, 32), (513, 2048, 13), (100, 3072, 2),
+                                             (33, 1024, 4), (4099, 6144, 16), (8, 1024, 17),
+                                             (9, 4096, 31), (520, 2048, 8), (77, 1024, 5)])
+def test_the_small_gemm_over_weights_as_uploaded_gives_the_sealed_bits(ctx, rows, cols, batch, x_off):
+    # Weights in the raw layout (never sealed), rows of whole 1024-column chunks:
+    # the token-split kernel reads them through LDS. Every token equals its own
+    # GEMV over the same raw buffer and the sealed kernel's result, bit for bit.
+    w = S.make_weights(rows, cols, 57 + rows)
+    x = S.make_activations(cols * batch, 91)
+    raw_b = weights_buffer(ctx, w, rows, cols, False)
+    sealed_b = weights_buffer(ctx, w, rows, cols, True)
+    got = run_gemm(ctx, ctx.q8_0_gemm, raw_b, x, rows, cols, batch, x_off, 5)[5:].reshape(batch, rows)
+    sealed = run_gemm(ctx, ctx.q8_0_gemm, sealed_b, x, rows, cols, batch, x_off, 5)[5:]
+    assert norm_err(got, O.gemm_q8_0_f32(w, rows, cols, x, batch)) <= 1e-5
+    assert np.array_equal(bits(got), bits(sealed.reshape(batch, rows)))
+    for b in (0, batch // 2, batch - 1):
+        single = gemv(ctx, raw_b, x[b * cols:(b + 1) * cols], rows, cols)
+        assert np.array_equal(bits(single), bits(got[b])), f"token {b}"
+    raw_b.free()
+    sealed_b.free()
+
+
 def test_products_that_go_as_two_token_groups_share_launches_by_descriptor_count(ctx):
     # 17 to 32 tokens over a matrix with a column tail go as two descriptors of up
     # to 16 tokens each (the 8-tokens-per-wave form has no tail variant). A

@@ -1,5 +1,5 @@
 // Small-batch Q8_0 product with the GEMV's arithmetic (2 <= batch <= 32,
-// sealed weights, cols >= 1024): the exact / speculative-verify
+// cols >= 1024; sealed weights, or raw ones with cols a multiple of 1024): the exact / speculative-verify
 // path (contract: native/metal/tm_metal.h:161-164,
 // crates/tuckcore/src/engine/metal.rs:81-83).
 //
@@ -33,14 +33,24 @@ constexpr int SMALL_R = 8; // rows per step
 // registers, one wave per SIMD); held to 256 it keeps 72 dwords per lane in
 // scratch memory instead and is still 22 % faster on the Gemma FFN shapes at
 // 17-32 tokens, because the second wave hides the first one's waits.
-template <int NW, int TW, bool XA, bool TAIL>
+//
+// L == RAW: weights as uploaded (34-byte blocks), rows of whole 1024-column
+// chunks only (no TAIL form). A row's chunk is then 1088 bytes, fetched into LDS
+// as 68 aligned 16-byte pieces (a second, four-lane fetch per row brings the
+// last 64 bytes); a lane reads back the five aligned dwords that hold its 16
+// quants and moves the bytes into place, and the block's scale comes out of the
+// same bytes (q8_gemv.hpp's stream_rows_raw has the details). The arithmetic is
+// the sealed form's.
+template <int L, int NW, int TW, bool XA, bool TAIL>
 __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvArgs args) {
+    static_assert(L == PACKED || !TAIL, "raw weights with a column tail take the general kernel");
     constexpr int R = SMALL_R;
+    constexpr uint32_t ROWB = L == PACKED ? 1024u : RAW_CHUNK_BYTES; // a staged row
     // Two separate objects (not one array indexed by parity): the compiler then
     // sees that reads of one buffer cannot alias the fetch into the other and
     // does not wait for the prefetch before reading.
-    __shared__ __attribute__((aligned(16))) uint8_t stage_a[R * 1024];
-    __shared__ __attribute__((aligned(16))) uint8_t stage_b[R * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t stage_a[R * ROWB];
+    __shared__ __attribute__((aligned(16))) uint8_t stage_b[R * ROWB];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t tile = blockIdx.x; // one tile per workgroup; the grid is exactly total_tiles
@@ -55,7 +65,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
     }
     const GemvDesc &d = args.d[lo];
     const uint32_t rows = d.rows, cols = d.cols, batch = d.batch;
-    const WView<PACKED> wv(d.w, rows, cols);
+    const WView<L> wv(d.w, rows, cols);
     const float *x = d.x;
     float *y = d.y;
     const uint32_t row_first = (tile - d.tile_begin) * d.rows_per_tile;
@@ -82,8 +92,14 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
     // a global one): the compiler's wait-count bookkeeping treats a global
     // load into LDS as a flat access and would make every later wait drain
     // the prefetch too. The descriptor covers the tile's quants only.
-    const uint8_t *tile_q = wv.q + (size_t)row_first * cols;
-    const size_t tile_len = (size_t)(row_end - row_first) * cols;
+    const uint32_t row_stride = L == PACKED ? cols : full * RAW_CHUNK_BYTES; // bytes from row to row
+    const uint8_t *tile_q;
+    if constexpr (L == PACKED) {
+        tile_q = wv.q + (size_t)row_first * row_stride;
+    } else {
+        tile_q = wv.base + (size_t)row_first * row_stride;
+    }
+    const size_t tile_len = (size_t)(row_end - row_first) * row_stride;
     const __amdgpu_buffer_rsrc_t tile_rs = __builtin_amdgcn_make_buffer_rsrc(
         (void *)tile_q, 0, tile_len > 0xffffffffull ? 0xffffffffu : (uint32_t)tile_len, 0x00020000);
     auto fetch = [&](uint32_t r0, uint32_t c, uint8_t *stage) {
@@ -91,19 +107,34 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
         for (int i = 0; i < R / NW; ++i) {
             const uint32_t r = wave * (R / NW) + i;
             const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
-            const uint32_t base = __builtin_amdgcn_readfirstlane((row - row_first) * cols + (c << 10));
+            const uint32_t base =
+                __builtin_amdgcn_readfirstlane((row - row_first) * row_stride + c * ROWB);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                tile_rs, (__attribute__((address_space(3))) void *)(stage + r * 1024), 16,
+                tile_rs, (__attribute__((address_space(3))) void *)(stage + r * ROWB), 16,
                 lane * 16u, base, 0, 0);
+            if constexpr (L == RAW) {
+                if (lane < 4u) { // bytes 1024..1087 of the row's chunk
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                        tile_rs,
+                        (__attribute__((address_space(3))) void *)(stage + r * ROWB + 1024u), 16,
+                        lane * 16u + 1024u, base, 0, 0);
+                }
+            }
         }
     };
     auto load_scales = [&](uint32_t r0, uint32_t c, uint32_t (&ss)[R]) {
+        if constexpr (L == PACKED) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
-            ss[r] = wv.scale_bits(row, (c << 5) + (lane >> 1));
+            for (int r = 0; r < R; ++r) {
+                const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+                ss[r] = wv.scale_bits(row, (c << 5) + (lane >> 1));
+            }
         }
     };
+    // raw layout: this lane's window in a staged row (see stream_rows_raw)
+    const uint32_t raw_off = (lane >> 1) * 34u + (lane & 1u) * 16u;
+    const bool raw_high = (raw_off & 2u) != 0u;
+    const uint32_t raw_sel = raw_high ? 0x07060504u : 0x05040302u;
 
     uint32_t sb[R], sn[R];
     fetch(row_first, 0, stage_a);
@@ -153,7 +184,8 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
                 }
                 // Column tail first, as in the decode kernel; these few pieces
                 // come straight from global memory.
-                if (TAIL && (cols & 1023u)) {
+                if constexpr (TAIL) {
+                  if (cols & 1023u) {
                     uint32_t row[R];
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
@@ -180,12 +212,30 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
                         chunk<PACKED, R, TW, 1, XA, false>(wv, x, cols, row, tok, col0, lane,
                                                            lane < 32u, acc);
                     }
+                  }
                 }
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const uint4 qv = *(const uint4 *)(cur + r * 1024 + lane * 16u);
-                const uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
+                uint32_t q[4];
+                if constexpr (L == PACKED) {
+                    const uint4 qv = *(const uint4 *)(cur + r * ROWB + lane * 16u);
+                    q[0] = qv.x;
+                    q[1] = qv.y;
+                    q[2] = qv.z;
+                    q[3] = qv.w;
+                } else {
+                    const uint32_t *w = (const uint32_t *)(cur + r * ROWB + (raw_off & ~3u));
+                    const uint32_t d0 = w[0], d1 = w[1], d2 = w[2], d3 = w[3], d4 = w[4];
+                    q[0] = __builtin_amdgcn_perm(d1, d0, raw_sel);
+                    q[1] = __builtin_amdgcn_perm(d2, d1, raw_sel);
+                    q[2] = __builtin_amdgcn_perm(d3, d2, raw_sel);
+                    q[3] = __builtin_amdgcn_perm(d4, d3, raw_sel);
+                    const uint32_t own = raw_high ? d0 >> 16 : d0;
+                    // quad_perm [0, 0, 2, 2]: odd lanes take their even neighbour's scale
+                    sb[r] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own, 0xA0, 0xf, 0xf, false) &
+                            0xffffu;
+                }
                 float qf[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
@@ -215,9 +265,11 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
                 }
             }
         }
+        if constexpr (L == PACKED) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            sb[r] = sn[r];
+            for (int r = 0; r < R; ++r) {
+                sb[r] = sn[r];
+            }
         }
         c = cn;
         r0 = rn;

@@ -571,7 +571,7 @@ GemvKey gemv_key(const Op &op) {
     k.flag = x_aligned_of(op);
     if (op.batch == 1) {
         k.variant = V_DECODE;
-    } else if (op.packed && op.cols >= 1024u && op.cols < (1u << 27)) {
+    } else if ((op.packed || (op.cols & 1023u) == 0u) && op.cols >= 1024u && op.cols < (1u << 27)) {
         // (the kernel indexes a token group's activations and a tile's quants in
         // 32 bits: rows of 2^27 columns and more take the general form)
         // waves x tokens per wave, measured on 2B-class shapes (the
@@ -963,25 +963,30 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         ++at;
     }
     args.total_tiles = tiles;
-#define TM_SPLIT_CASE(W, T, A, TL)                                                           \
-    if (key.variant == V_SPLIT && key.p0 == (W) && key.p1 == (T) && key.p2 == ((TL) ? 1 : 0) && \
-        key.flag == (A)) {                                                                   \
-        Q8_LAUNCH((q8::gemm_split_list_kernel<W, T, A, TL>), dim3(tiles), dim3((W) * 64), 0, \
-                  ctx->stream, stop, args);                                                  \
+#define TM_SPLIT_CASE(P, W, T, A, TL)                                                        \
+    if (key.variant == V_SPLIT && key.packed == (P) && key.p0 == (W) && key.p1 == (T) &&     \
+        key.p2 == ((TL) ? 1 : 0) && key.flag == (A)) {                                       \
+        Q8_LAUNCH((q8::gemm_split_list_kernel<(P) ? q8::PACKED : q8::RAW, W, T, A, TL>),     \
+                  dim3(tiles), dim3((W) * 64), 0, ctx->stream, stop, args);                  \
         return hipGetLastError();                                                            \
     }
+    // (raw weights: rows of whole chunks only, so no column-tail form)
 #define TM_SPLIT_ALL(W, T)                                                                   \
-    TM_SPLIT_CASE(W, T, true, false)                                                         \
-    TM_SPLIT_CASE(W, T, false, false)                                                        \
-    TM_SPLIT_CASE(W, T, true, true)                                                          \
-    TM_SPLIT_CASE(W, T, false, true)
+    TM_SPLIT_CASE(true, W, T, true, false)                                                   \
+    TM_SPLIT_CASE(true, W, T, false, false)                                                  \
+    TM_SPLIT_CASE(true, W, T, true, true)                                                    \
+    TM_SPLIT_CASE(true, W, T, false, true)                                                   \
+    TM_SPLIT_CASE(false, W, T, true, false)                                                  \
+    TM_SPLIT_CASE(false, W, T, false, false)
     TM_SPLIT_ALL(1, 2)
     TM_SPLIT_ALL(1, 4)
     TM_SPLIT_ALL(2, 4)
     TM_SPLIT_ALL(4, 4)
     // (eight tokens per wave: no column-tail form, see gemv_key)
-    TM_SPLIT_CASE(4, 8, true, false)
-    TM_SPLIT_CASE(4, 8, false, false)
+    TM_SPLIT_CASE(true, 4, 8, true, false)
+    TM_SPLIT_CASE(true, 4, 8, false, false)
+    TM_SPLIT_CASE(false, 4, 8, true, false)
+    TM_SPLIT_CASE(false, 4, 8, false, false)
 #undef TM_SPLIT_ALL
 #undef TM_SPLIT_CASE
 #define TM_GEMV_CASE(P, T, A)                                                                \
