@@ -59,7 +59,13 @@ def test_raw_and_packed_layouts_give_identical_bits(ctx):
     # last pass is short, one to six chunks per row)
     for rows, cols, seed in [(17, 64, 3), (1024, 1024, 4), (300, 1152, 9), (77, 6912, 10),
                              (64, 2016, 11), (259, 1024, 12), (1021, 2048, 13), (13, 3072, 14),
-                             (4100, 1024, 15), (530, 6144, 16)]:
+                             (4100, 1024, 15), (530, 6144, 16),
+                             # 1152 and 6912 columns: tails that stream too (rows of 1224 bytes
+                             # staged whole, odd and even numbers of rows in the last pass)
+                             (1, 1152, 17), (7, 1152, 18), (301, 1152, 19), (1030, 1152, 20),
+                             (13, 6912, 21), (260, 6912, 22),
+                             # other tails (general form)
+                             (40, 2176, 23), (24, 1792, 24)]:
         w = O.boundary_weights(rows, cols, seed)
         x = O.boundary_input(cols, seed + 100)
         a = gemv(ctx, weights_buffer(ctx, w, rows, cols, False), x, rows, cols)

@@ -67,6 +67,22 @@ def test_raw_decode_kernel_keeps_four_waves_per_simd(resource_remarks):
         assert lds == 4 * 8 * 1088 and 4 * lds <= 160 * 1024
 
 
+# the same with the Gemma column tails: a pass of eight 1152-column rows is staged whole
+RAW_DECODE_TAILS_KERNEL = re.compile(
+    r"Function Name: _ZN2q816gemv_list_kernelILi0ELi8ELi1ELb[01]ELi1ELi\d+ELb0EEE")
+
+
+def test_raw_decode_kernel_with_column_tails_fits_three_workgroups_per_cu(resource_remarks):
+    blocks = _blocks(resource_remarks, RAW_DECODE_TAILS_KERNEL)
+    assert blocks, "raw decode kernel with tails not found in the resource remarks"
+    for block in blocks:
+        vgprs = int(re.search(r" VGPRs: (\d+)", block).group(1))
+        spill = int(re.search(r"VGPRs Spill: (\d+)", block).group(1))
+        lds = int(re.search(r"LDS Size \[bytes/block\]: (\d+)", block).group(1))
+        assert spill == 0 and vgprs <= 168, f"{vgprs} VGPRs, {spill} spilled"  # three waves per SIMD
+        assert lds == 4 * 8 * 1224 and 3 * lds <= 160 * 1024
+
+
 # gemm_bf16x3_kernel<WM, 4, 2, NS>: the 128-token and the 64-token tile
 BF16_KERNEL = re.compile(r"Function Name: _ZN2q818gemm_bf16x3_kernelILi[12]ELi4ELi2ELi[34]EEE")
 

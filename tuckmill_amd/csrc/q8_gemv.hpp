@@ -432,105 +432,229 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs
 // and the arithmetic are those of stream_rows. The loads of step s+1 are in
 // flight while step s is multiplied.
 constexpr uint32_t RAW_CHUNK_BYTES = 1088u; // 32 blocks of 34 bytes
-template <int R> constexpr uint32_t raw_stage_bytes() { return (uint32_t)R * RAW_CHUNK_BYTES; }
+typedef unsigned int u32x4_a8 __attribute__((ext_vector_type(4), aligned(8)));
+// LDS a wave needs for it: R staged rows of a chunk, or (TAILS >= 1) of a whole
+// 1152-column row.
+template <int R, int TAILS> constexpr uint32_t raw_stage_bytes() {
+    return (uint32_t)R * (TAILS >= 1 ? RAW_CHUNK_BYTES + 136u : RAW_CHUNK_BYTES);
+}
 
-template <int R, bool XA>
+// A lane's 2, 4 or 8 quants of a tail piece out of staged raw bytes: they start
+// at the even byte `at`; the aligned dwords that hold them, bytes moved into place.
+__device__ __forceinline__ uint32_t raw_sel(uint32_t at) {
+    return (at & 2u) ? 0x05040302u : 0x03020100u;
+}
+
+// TAILMASK = cols % 1024: 0, or one of the two column tails with a path of their
+// own. 768 (rows of 6912 columns: 16-byte aligned like rows of whole chunks): the
+// tail's 24 blocks of each row are a step of their own in front of the chunks, as
+// the arithmetic has the tail pieces first. 128 with a single chunk (rows of 1152
+// columns, 1224 bytes: only 8-byte aligned, but R of them are contiguous and
+// start aligned): a pass is staged whole, chunk and tail in one step.
+template <int R, bool XA, int TAILMASK>
 __device__ __forceinline__ void stream_rows_raw(const WView<RAW> &wv, const float *x, float *y,
                                                 uint32_t cols, uint32_t row_first,
                                                 uint32_t row_end, uint32_t lane, uint8_t *stage,
                                                 float *res, float alpha) {
-    constexpr uint32_t PIECES = (uint32_t)R * 68u;      // 16-byte pieces of a step
-    constexpr int NL = (int)((PIECES + 63u) / 64u);     // loads per lane and step
+    static_assert(TAILMASK == 0 || TAILMASK == 128 || TAILMASK == 768, "column tails with a path");
+    constexpr bool WHOLE = TAILMASK == 128; // a pass is one step over R whole rows
+    constexpr bool TSEG = TAILMASK == 768;  // the tail blocks are a step of their own
+    constexpr uint32_t TAILB = (uint32_t)TAILMASK / 32u * 34u;          // a row's tail bytes
+    constexpr uint32_t ROWB = WHOLE ? RAW_CHUNK_BYTES + TAILB : RAW_CHUNK_BYTES; // a staged row
+    constexpr uint32_t PIECES = (uint32_t)R * ROWB / 16u;               // 16-byte pieces of a step
+    constexpr int NL = (int)((PIECES + 63u) / 64u);                     // loads per lane and step
+    constexpr uint32_t ROW_PIECES = ROWB / 16u;
+    constexpr uint32_t TROW_PIECES = TAILB / 16u;                       // (TSEG) 51
+    constexpr uint32_t TPIECES = (uint32_t)R * TROW_PIECES;
+    constexpr int NLT = TSEG ? (int)((TPIECES + 63u) / 64u) : 0;
+    static_assert(!TSEG || TAILB % 16u == 0u, "tail rows are whole pieces");
     const uint32_t full = cols >> 10;
-    // Piece g = i * 64 + lane of a step is piece g % 68 of row g / 68 and is
-    // staged at byte 16 g; a last, partly filled round of pieces is left to the
-    // lanes below PIECES % 64.
     const uint32_t row_bytes = (uint32_t)wv.row_bytes;
+    // Piece g = i * 64 + lane of a step is piece g % ROW_PIECES of row
+    // g / ROW_PIECES and is staged at byte 16 g; a last, partly filled round
+    // of pieces is left to the lanes below PIECES % 64. Rows past the tile's
+    // end repeat its last row. With rows staged whole a piece's place in the
+    // stage is its offset in memory, and pieces that would reach past the last
+    // row of the tile are its last 16 bytes instead (an odd number of 1224-byte
+    // rows ends on an 8-byte boundary: such a piece is 8-byte aligned, in
+    // memory and in the stage).
     auto piece_offset = [&](int i, uint32_t last) { // from the step's first byte
         const uint32_t g = (uint32_t)i * 64u + lane;
-        const uint32_t row = g / 68u;
-        return (row < last ? row : last) * row_bytes + (g % 68u) * 16u;
+        if constexpr (WHOLE) {
+            const uint32_t end = (last + 1u) * ROWB - 16u;
+            return g * 16u < end ? g * 16u : end;
+        } else {
+            const uint32_t row = g / ROW_PIECES;
+            return (row < last ? row : last) * row_bytes + (g % ROW_PIECES) * 16u;
+        }
     };
     uint32_t poff[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         poff[i] = piece_offset(i, (uint32_t)R - 1u);
     }
-    const bool tail_lane = lane < PIECES % 64u || PIECES % 64u == 0u;
-    auto fetch = [&](uint32_t r0, uint32_t c, u32x4 (&p)[NL]) {
-        const uint32_t last = row_end - 1u - r0; // rows past the tile's end repeat its last row
-        const uint8_t *base = wv.base + (size_t)r0 * wv.row_bytes + (size_t)c * RAW_CHUNK_BYTES;
+    // seg -1: the tail step (TSEG only); 0 .. full-1: the chunks
+    auto fetch = [&](uint32_t r0, int32_t seg, u32x4 (&p)[NL]) {
+        const uint32_t last = row_end - 1u - r0;
+        const uint8_t *row0 = wv.base + (size_t)r0 * wv.row_bytes;
+        if constexpr (TSEG) {
+            if (seg < 0) {
+                const uint8_t *base = row0 + (size_t)full * RAW_CHUNK_BYTES;
+#pragma unroll
+                for (int i = 0; i < NLT; ++i) {
+                    const uint32_t g = (uint32_t)i * 64u + lane;
+                    const uint32_t row = g / TROW_PIECES;
+                    const uint32_t o =
+                        (row < last ? row : last) * row_bytes + (g % TROW_PIECES) * 16u;
+                    if (i < NLT - 1 || lane < TPIECES % 64u || TPIECES % 64u == 0u) {
+                        p[i] = __builtin_nontemporal_load((const u32x4 *)(base + o));
+                    }
+                }
+                return;
+            }
+        }
+        const uint8_t *base = row0 + (size_t)seg * RAW_CHUNK_BYTES;
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
             const uint32_t o = last >= (uint32_t)R - 1u ? poff[i] : piece_offset(i, last);
-            if (i < NL - 1 || tail_lane) {
-                p[i] = __builtin_nontemporal_load((const u32x4 *)(base + o));
+            if (i < NL - 1 || lane < PIECES % 64u || PIECES % 64u == 0u) {
+                if constexpr (WHOLE) {
+                    p[i] = __builtin_nontemporal_load((const u32x4_a8 *)(base + o));
+                } else {
+                    p[i] = __builtin_nontemporal_load((const u32x4 *)(base + o));
+                }
             }
         }
     };
-    // this lane's window in a staged row: the aligned dword at or below the
+    // where the pieces of a chunk step go in the stage
+    auto stage_at = [&](int i, uint32_t last) {
+        if constexpr (WHOLE) {
+            return last >= (uint32_t)R - 1u ? poff[i] : piece_offset(i, last);
+        } else {
+            return (uint32_t)i * 1024u + lane * 16u;
+        }
+    };
+    // this lane's window in a staged chunk: the aligned dword at or below the
     // block's first byte (even lanes) or its 17th (odd lanes)
     const uint32_t off = (lane >> 1) * 34u + (lane & 1u) * 16u;
     const bool high = (off & 2u) != 0u; // quants from dword 1 on, the scale in dword 0's upper half
     const uint32_t sel = high ? 0x07060504u : 0x05040302u;
     const uint8_t *window = stage + (off & ~3u);
 
+    // the tail pieces' activations and places in a staged row (loop invariant)
+    float x8[8], x4[4], x2[2];
+    uint32_t s8_at = 0, q8_at = 0, s4_at = 0, q4_at = 0, s2_at = 0, q2_at = 0;
+    if constexpr (TSEG) { // 512 columns as 8 quants per lane, then 256 as 4
+        load_x<8, XA>(x + (full << 10) + lane * 8u, x8);
+        load_x<4, XA>(x + (full << 10) + 512u + lane * 4u, x4);
+        s8_at = (lane >> 2) * 34u;
+        q8_at = s8_at + 2u + 8u * (lane & 3u);
+        s4_at = (16u + (lane >> 3)) * 34u;
+        q4_at = s4_at + 2u + 4u * (lane & 7u);
+    }
+    if constexpr (WHOLE) { // 128 columns as 2 quants per lane
+        load_x<2, XA>(x + 1024u + lane * 2u, x2);
+        s2_at = RAW_CHUNK_BYTES + (lane >> 4) * 34u;
+        q2_at = s2_at + 2u + 2u * (lane & 15u);
+    }
+
     float xv[16];
     if (full == 1u) {
         load_x<16, XA>(x + lane * 16u, xv);
     }
-    const uint32_t nsteps = ((row_end - row_first + R - 1) / R) * full;
-    uint32_t r0 = row_first, c = 0;
+    constexpr int32_t SEG0 = TSEG ? -1 : 0;
+    const uint32_t nsteps = ((row_end - row_first + R - 1) / R) * (full + (TSEG ? 1u : 0u));
+    uint32_t r0 = row_first;
+    int32_t seg = SEG0;
     u32x4 p[NL];
-    fetch(r0, 0, p);
+    fetch(r0, seg, p);
     float acc[R];
     for (uint32_t step = 0; step < nsteps; ++step) {
         __builtin_amdgcn_wave_barrier(); // the previous step's reads come first
+        if (TSEG && seg < 0) {
 #pragma unroll
-        for (int i = 0; i < NL; ++i) {
-            if (i < NL - 1 || tail_lane) {
-                *(u32x4 *)(stage + (uint32_t)i * 1024u + lane * 16u) = p[i];
+            for (int i = 0; i < NLT; ++i) {
+                if (i < NLT - 1 || lane < TPIECES % 64u || TPIECES % 64u == 0u) {
+                    *(u32x4 *)(stage + (uint32_t)i * 1024u + lane * 16u) = p[i];
+                }
+            }
+        } else {
+            const uint32_t last = row_end - 1u - r0;
+#pragma unroll
+            for (int i = 0; i < NL; ++i) {
+                if (i < NL - 1 || lane < PIECES % 64u || PIECES % 64u == 0u) {
+                    if constexpr (WHOLE) {
+                        *(u32x4_a8 *)(stage + stage_at(i, last)) = p[i];
+                    } else {
+                        *(u32x4 *)(stage + stage_at(i, last)) = p[i];
+                    }
+                }
             }
         }
-        uint32_t cn = c + 1u, rn = r0;
-        if (cn == full) {
-            cn = 0;
+        int32_t segn = seg + 1;
+        uint32_t rn = r0;
+        if (segn == (int32_t)full) {
+            segn = SEG0;
             rn = r0 + (uint32_t)R;
         }
         if (step + 1u < nsteps) {
-            fetch(rn, cn, p);
+            fetch(rn, segn, p);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        if (c == 0u) {
+        if (TSEG && seg < 0) {
+            // the pass starts with its tail pieces, widest first
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                acc[r] = 0.0f;
+                const uint8_t *row = stage + (uint32_t)r * TAILB;
+                const uint32_t *w8 = (const uint32_t *)(row + (q8_at & ~3u));
+                const uint32_t *w4 = (const uint32_t *)(row + (q4_at & ~3u));
+                const uint32_t e0 = w8[0], e1 = w8[1], e2 = w8[2], f0 = w4[0], f1 = w4[1];
+                const uint32_t q8[2] = {__builtin_amdgcn_perm(e1, e0, raw_sel(q8_at)),
+                                        __builtin_amdgcn_perm(e2, e1, raw_sel(q8_at))};
+                const uint32_t q4[1] = {__builtin_amdgcn_perm(f1, f0, raw_sel(q4_at))};
+                const uint32_t s8 = *(const uint16_t *)(row + s8_at);
+                const uint32_t s4 = *(const uint16_t *)(row + s4_at);
+                float a = __builtin_fmaf(f16_bits_to_f32(s8), piece_dot<8>(q8, x8), 0.0f);
+                a = __builtin_fmaf(f16_bits_to_f32(s4), piece_dot<4>(q4, x4), a);
+                acc[r] = a;
+            }
+        } else {
+            if (full > 1u) {
+                load_x<16, XA>(x + ((uint32_t)seg << 10) + lane * 16u, xv);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float a = acc[r];
+                if (!TSEG && seg == 0) {
+                    a = 0.0f;
+                    if constexpr (WHOLE) {
+                        const uint8_t *row = stage + (uint32_t)r * ROWB;
+                        const uint32_t q2[1] = {*(const uint16_t *)(row + q2_at)};
+                        const uint32_t s2 = *(const uint16_t *)(row + s2_at);
+                        a = __builtin_fmaf(f16_bits_to_f32(s2), piece_dot<2>(q2, x2), a);
+                    }
+                }
+                const uint32_t *w = (const uint32_t *)(window + (uint32_t)r * ROWB);
+                const uint32_t d0 = w[0], d1 = w[1], d2 = w[2], d3 = w[3], d4 = w[4];
+                uint32_t q[4];
+                q[0] = __builtin_amdgcn_perm(d1, d0, sel);
+                q[1] = __builtin_amdgcn_perm(d2, d1, sel);
+                q[2] = __builtin_amdgcn_perm(d3, d2, sel);
+                q[3] = __builtin_amdgcn_perm(d4, d3, sel);
+                const uint32_t own = high ? d0 >> 16 : d0;
+                // quad_perm [0, 0, 2, 2]: odd lanes take their even neighbour's scale
+                const uint32_t sb =
+                    (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own, 0xA0, 0xf, 0xf, false) &
+                    0xffffu;
+                acc[r] = __builtin_fmaf(f16_bits_to_f32(sb), piece_dot<16>(q, xv), a);
             }
         }
-        if (full > 1u) {
-            load_x<16, XA>(x + (c << 10) + lane * 16u, xv);
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const uint32_t *w = (const uint32_t *)(window + (uint32_t)r * RAW_CHUNK_BYTES);
-            const uint32_t d0 = w[0], d1 = w[1], d2 = w[2], d3 = w[3], d4 = w[4];
-            uint32_t q[4];
-            q[0] = __builtin_amdgcn_perm(d1, d0, sel);
-            q[1] = __builtin_amdgcn_perm(d2, d1, sel);
-            q[2] = __builtin_amdgcn_perm(d3, d2, sel);
-            q[3] = __builtin_amdgcn_perm(d4, d3, sel);
-            const uint32_t own = high ? d0 >> 16 : d0;
-            // quad_perm [0, 0, 2, 2]: odd lanes take their even neighbour's scale
-            const uint32_t sb =
-                (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own, 0xA0, 0xf, 0xf, false) & 0xffffu;
-            acc[r] = __builtin_fmaf(f16_bits_to_f32(sb), piece_dot<16>(q, xv), acc[r]);
-        }
-        if (cn == 0u) {
+        if (segn == SEG0) {
             reduce_store<R>(acc, y, r0, row_end, lane, true, res, alpha);
         }
-        c = cn;
+        seg = segn;
         r0 = rn;
     }
 }
@@ -714,13 +838,29 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
     }
 
     if constexpr (TB == 1 && L == RAW) {
-        // One token over weights as uploaded: rows of whole 1024-column chunks
-        // stream through LDS (stream_rows_raw); other shapes take the general path.
-        if (full >= 1u && (cols & 1023u) == 0u) {
-            __shared__ __attribute__((aligned(16))) uint8_t raw_stage[4][raw_stage_bytes<R>()];
-            stream_rows_raw<R, XA>(wv, x, y, cols, row_first, row_end, lane, raw_stage[wave], d.res,
-                                   d.alpha);
-            return;
+        // One token over weights as uploaded: rows of whole 1024-column chunks,
+        // and the column tails that have a decode path of their own, stream
+        // through LDS (stream_rows_raw); other shapes take the general path.
+        if (full >= 1u) {
+            __shared__ __attribute__((aligned(16))) uint8_t raw_stage[4][raw_stage_bytes<R, TAILS>()];
+            const uint32_t tail = cols & 1023u;
+            if (tail == 0u) {
+                stream_rows_raw<R, XA, 0>(wv, x, y, cols, row_first, row_end, lane, raw_stage[wave],
+                                          d.res, d.alpha);
+                return;
+            }
+            if constexpr (TAILS >= 1) {
+                if (tail == 128u && full == 1u) { // hidden 1152 (Gemma-3-1B)
+                    stream_rows_raw<R, XA, 128>(wv, x, y, cols, row_first, row_end, lane,
+                                                raw_stage[wave], d.res, d.alpha);
+                    return;
+                }
+                if (tail == 768u) { // FFN 6912 (Gemma-3-1B)
+                    stream_rows_raw<R, XA, 768>(wv, x, y, cols, row_first, row_end, lane,
+                                                raw_stage[wave], d.res, d.alpha);
+                    return;
+                }
+            }
         }
     }
 

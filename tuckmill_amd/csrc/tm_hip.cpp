@@ -670,6 +670,13 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &arg
             return hipGetLastError();
         }
     }
+    if constexpr (L == q8::RAW && TB == 1) {
+        if (tails) { // weights as uploaded with the column tails that stream
+            Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1>), dim3(groups), dim3(256), 0,
+                      ctx->stream, stop, args);
+            return hipGetLastError();
+        }
+    }
     Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 0>), dim3(groups), dim3(256), 0, ctx->stream,
               stop, args);
     return hipGetLastError();
