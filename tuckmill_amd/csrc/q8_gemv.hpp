@@ -840,8 +840,9 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
     if constexpr (TB == 1 && L == RAW) {
         // One token over weights as uploaded: rows of whole 1024-column chunks,
         // and the column tails that have a decode path of their own, stream
-        // through LDS (stream_rows_raw); other shapes take the general path.
-        if (full >= 1u) {
+        // through LDS (stream_rows_raw); other shapes take the general path
+        // (rows of 2^27 columns and more too: the staging indexes a pass in 32 bits).
+        if (full >= 1u && cols < (1u << 27)) {
             __shared__ __attribute__((aligned(16))) uint8_t raw_stage[4][raw_stage_bytes<R, TAILS>()];
             const uint32_t tail = cols & 1023u;
             if (tail == 0u) {
