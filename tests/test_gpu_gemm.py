@@ -96,11 +96,17 @@ def test_every_token_of_the_small_gemm_equals_its_own_gemv(ctx, rows, cols, batc
 @pytest.mark.parametrize("x_off", [0, 3])
 @pytest.mark.parametrize("rows,cols,batch", [(64, 1024, 32), (513, 2048, 13), (100, 3072, 2),
                                              (33, 1024, 4), (4099, 6144, 16), (8, 1024, 17),
-                                             (9, 4096, 31), (520, 2048, 8), (77, 1024, 5)])
+                                             (9, 4096, 31), (520, 2048, 8), (77, 1024, 5),
+                                             # column tails (cols a multiple of 64): rows that are
+                                             # only 8- or 4-byte aligned, two token groups at 17+
+                                             (100, 1152, 7), (40, 6912, 3), (41, 6912, 32),
+                                             (70, 1152, 20), (64, 1088, 3), (50, 2112, 5),
+                                             # cols not a multiple of 64: the general form
+                                             (33, 2016, 6)])
 def test_the_small_gemm_over_weights_as_uploaded_gives_the_sealed_bits(ctx, rows, cols, batch, x_off):
-    # Weights in the raw layout (never sealed), rows of whole 1024-column chunks:
-    # the token-split kernel reads them through LDS. Every token equals its own
-    # GEMV over the same raw buffer and the sealed kernel's result, bit for bit.
+    # Weights in the raw layout (never sealed): the token-split kernel reads their
+    # whole 1024-column chunks through LDS. Every token equals its own GEMV over
+    # the same raw buffer and the sealed kernel's result, bit for bit.
     w = S.make_weights(rows, cols, 57 + rows)
     x = S.make_activations(cols * batch, 91)
     raw_b = weights_buffer(ctx, w, rows, cols, False)

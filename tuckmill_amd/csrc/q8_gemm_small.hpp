@@ -34,16 +34,15 @@ constexpr int SMALL_R = 8; // rows per step
 // scratch memory instead and is still 22 % faster on the Gemma FFN shapes at
 // 17-32 tokens, because the second wave hides the first one's waits.
 //
-// L == RAW: weights as uploaded (34-byte blocks), rows of whole 1024-column
-// chunks only (no TAIL form). A row's chunk is then 1088 bytes, fetched into LDS
-// as 68 aligned 16-byte pieces (a second, four-lane fetch per row brings the
-// last 64 bytes); a lane reads back the five aligned dwords that hold its 16
-// quants and moves the bytes into place, and the block's scale comes out of the
-// same bytes (q8_gemv.hpp's stream_rows_raw has the details). The arithmetic is
-// the sealed form's.
+// L == RAW: weights as uploaded (34-byte blocks), cols a multiple of 64 (rows
+// start dword aligned). A row's chunk is then 1088 bytes, fetched into LDS as 68
+// 16-byte pieces (a second, four-lane fetch per row brings the last 64 bytes);
+// a lane reads back the five aligned dwords that hold its 16 quants and moves
+// the bytes into place, and the block's scale comes out of the same bytes
+// (q8_gemv.hpp's stream_rows_raw has the details). The arithmetic is the sealed
+// form's.
 template <int L, int NW, int TW, bool XA, bool TAIL>
 __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvArgs args) {
-    static_assert(L == PACKED || !TAIL, "raw weights with a column tail take the general kernel");
     constexpr int R = SMALL_R;
     constexpr uint32_t ROWB = L == PACKED ? 1024u : RAW_CHUNK_BYTES; // a staged row
     // Two separate objects (not one array indexed by parity): the compiler then
@@ -92,7 +91,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
     // a global one): the compiler's wait-count bookkeeping treats a global
     // load into LDS as a flat access and would make every later wait drain
     // the prefetch too. The descriptor covers the tile's quants only.
-    const uint32_t row_stride = L == PACKED ? cols : full * RAW_CHUNK_BYTES; // bytes from row to row
+    const uint32_t row_stride = L == PACKED ? cols : (cols >> 5) * 34u; // bytes from row to row
     const uint8_t *tile_q;
     if constexpr (L == PACKED) {
         tile_q = wv.q + (size_t)row_first * row_stride;
@@ -193,23 +192,23 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
                     }
                     uint32_t col0 = full << 10;
                     if (cols & 512u) {
-                        chunk<PACKED, R, TW, 8, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
+                        chunk<L, R, TW, 8, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
                         col0 += 512u;
                     }
                     if (cols & 256u) {
-                        chunk<PACKED, R, TW, 4, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
+                        chunk<L, R, TW, 4, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
                         col0 += 256u;
                     }
                     if (cols & 128u) {
-                        chunk<PACKED, R, TW, 2, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
+                        chunk<L, R, TW, 2, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
                         col0 += 128u;
                     }
                     if (cols & 64u) {
-                        chunk<PACKED, R, TW, 1, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
+                        chunk<L, R, TW, 1, XA, false>(wv, x, cols, row, tok, col0, lane, true, acc);
                         col0 += 64u;
                     }
                     if (cols & 32u) {
-                        chunk<PACKED, R, TW, 1, XA, false>(wv, x, cols, row, tok, col0, lane,
+                        chunk<L, R, TW, 1, XA, false>(wv, x, cols, row, tok, col0, lane,
                                                            lane < 32u, acc);
                     }
                   }

@@ -571,7 +571,7 @@ GemvKey gemv_key(const Op &op) {
     k.flag = x_aligned_of(op);
     if (op.batch == 1) {
         k.variant = V_DECODE;
-    } else if ((op.packed || (op.cols & 1023u) == 0u) && op.cols >= 1024u && op.cols < (1u << 27)) {
+    } else if ((op.packed || (op.cols & 63u) == 0u) && op.cols >= 1024u && op.cols < (1u << 27)) {
         // (the kernel indexes a token group's activations and a tile's quants in
         // 32 bits: rows of 2^27 columns and more take the general form)
         // waves x tokens per wave, measured on 2B-class shapes (the
@@ -977,14 +977,15 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
                   dim3(tiles), dim3((W) * 64), 0, ctx->stream, stop, args);                  \
         return hipGetLastError();                                                            \
     }
-    // (raw weights: rows of whole chunks only, so no column-tail form)
 #define TM_SPLIT_ALL(W, T)                                                                   \
     TM_SPLIT_CASE(true, W, T, true, false)                                                   \
     TM_SPLIT_CASE(true, W, T, false, false)                                                  \
     TM_SPLIT_CASE(true, W, T, true, true)                                                    \
     TM_SPLIT_CASE(true, W, T, false, true)                                                   \
     TM_SPLIT_CASE(false, W, T, true, false)                                                  \
-    TM_SPLIT_CASE(false, W, T, false, false)
+    TM_SPLIT_CASE(false, W, T, false, false)                                                 \
+    TM_SPLIT_CASE(false, W, T, true, true)                                                   \
+    TM_SPLIT_CASE(false, W, T, false, true)
     TM_SPLIT_ALL(1, 2)
     TM_SPLIT_ALL(1, 4)
     TM_SPLIT_ALL(2, 4)
