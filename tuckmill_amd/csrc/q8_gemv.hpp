@@ -433,10 +433,10 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs
 // flight while step s is multiplied.
 constexpr uint32_t RAW_CHUNK_BYTES = 1088u; // 32 blocks of 34 bytes
 typedef unsigned int u32x4_a8 __attribute__((ext_vector_type(4), aligned(8)));
-// LDS a wave needs for it: R staged rows of a chunk, or (TAILS >= 1) of a whole
+// LDS a wave needs for it: R staged rows of a chunk, or (TAILS == 1) of a whole
 // 1152-column row.
 template <int R, int TAILS> constexpr uint32_t raw_stage_bytes() {
-    return (uint32_t)R * (TAILS >= 1 ? RAW_CHUNK_BYTES + 136u : RAW_CHUNK_BYTES);
+    return (uint32_t)R * (TAILS == 1 ? RAW_CHUNK_BYTES + 136u : RAW_CHUNK_BYTES);
 }
 
 // A lane's 2, 4 or 8 quants of a tail piece out of staged raw bytes: they start
@@ -723,8 +723,10 @@ __device__ __forceinline__ void stream_rows_glu(const WView<PACKED> &wg, const W
 
 // TAILS selects which column tails get the streaming decode path: 0 = none
 // (cols a multiple of 1024 only; fewest registers, the Qwen3 shapes), 1 = also
-// cols % 1024 == 128 and == 768 (the Gemma-3-1B shapes). The host picks the
-// smallest set that covers the products of a launch.
+// cols % 1024 == 128 and == 768 (the Gemma-3-1B shapes), 2 = also == 768 but
+// not 128 (a launch of Gemma's down projections only: the 128-column tail is
+// what costs the registers, without it four waves fit a SIMD). The host picks
+// the cheapest set that covers the products of a launch.
 // NORM: the launch carries fused forms, an RMSNorm in front of its products
 // and/or gate-up pairs with their activation (a separate instantiation, so that
 // the plain decode kernel keeps its register budget).
@@ -824,13 +826,31 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
                 }
                 return;
             }
-            if constexpr (TAILS >= 1) {
+            // (as above, a small product may be cut into shorter tiles)
+            if constexpr (TAILS == 1) {
                 if (tail == 128u) { // hidden 1152 (Gemma-3-1B)
-                    stream_rows<R, XA, 128>(wv, PlainX{x}, y, cols, row_first, row_end, lane, d.res, d.alpha);
+                    if (d.rows_per_tile % (R / 2) != 0u) {
+                        stream_rows<R / 4, XA, 128>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
+                                                    d.res, d.alpha);
+                    } else if (d.rows_per_tile % R != 0u) {
+                        stream_rows<R / 2, XA, 128>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
+                                                    d.res, d.alpha);
+                    } else {
+                        stream_rows<R, XA, 128>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
+                                                d.res, d.alpha);
+                    }
                     return;
                 }
+            }
+            if constexpr (TAILS >= 1) {
                 if (tail == 768u) { // FFN 6912 (Gemma-3-1B); half the rows per pass
-                    stream_rows<R / 2, XA, 768>(wv, PlainX{x}, y, cols, row_first, row_end, lane, d.res, d.alpha);
+                    if (d.rows_per_tile % (R / 2) != 0u) {
+                        stream_rows<R / 4, XA, 768>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
+                                                    d.res, d.alpha);
+                    } else {
+                        stream_rows<R / 2, XA, 768>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
+                                                    d.res, d.alpha);
+                    }
                     return;
                 }
             }
@@ -850,12 +870,14 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
                                           d.res, d.alpha);
                 return;
             }
-            if constexpr (TAILS >= 1) {
+            if constexpr (TAILS == 1) {
                 if (tail == 128u && full == 1u) { // hidden 1152 (Gemma-3-1B)
                     stream_rows_raw<R, XA, 128>(wv, x, y, cols, row_first, row_end, lane,
                                                 raw_stage[wave], d.res, d.alpha);
                     return;
                 }
+            }
+            if constexpr (TAILS >= 1) {
                 if (tail == 768u) { // FFN 6912 (Gemma-3-1B)
                     stream_rows_raw<R, XA, 768>(wv, x, y, cols, row_first, row_end, lane,
                                                 raw_stage[wave], d.res, d.alpha);

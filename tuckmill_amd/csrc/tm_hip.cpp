@@ -622,7 +622,7 @@ inline unsigned strided_blocks_of(uint32_t n, uint32_t per) {
 }
 
 template <int L, int R, int TB, bool XA>
-hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args, bool tails,
+hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args, int tails,
                        bool fused) {
     const uint32_t groups = (args.total_tiles + 3u) / 4u;
     if constexpr (L == q8::PACKED && TB == 1) {
@@ -647,8 +647,11 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &arg
                 }
                 return hipErrorInvalidValue;
             }
-            if (tails) {
+            if (tails == 1) {
                 Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1, q8::GEMV_FEW_DESCS>), dim3(groups),
+                          dim3(256), 0, ctx->stream, stop, few);
+            } else if (tails == 2) {
+                Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 2, q8::GEMV_FEW_DESCS>), dim3(groups),
                           dim3(256), 0, ctx->stream, stop, few);
             } else {
                 Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 0, q8::GEMV_FEW_DESCS>), dim3(groups),
@@ -664,15 +667,15 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &arg
             }
             return hipErrorInvalidValue;
         }
-        if (tails) {
+    }
+    if constexpr (TB == 1) { // (either layout: the column tails that stream)
+        if (tails == 1) {
             Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1>), dim3(groups), dim3(256), 0,
                       ctx->stream, stop, args);
             return hipGetLastError();
         }
-    }
-    if constexpr (L == q8::RAW && TB == 1) {
-        if (tails) { // weights as uploaded with the column tails that stream
-            Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1>), dim3(groups), dim3(256), 0,
+        if (tails == 2) {
+            Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 2>), dim3(groups), dim3(256), 0,
                       ctx->stream, stop, args);
             return hipGetLastError();
         }
@@ -905,11 +908,17 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         launch_bytes += (uint64_t)op->rows * (op->cols / 32u) * 34u;
     }
     const bool small_launch = launch_bytes < (16u << 20);
-    bool tails = false; // some product has a column tail with a streaming path of its own
+    // which column tails with a streaming path of their own the products have:
+    // 0 none, 1 128 columns (and maybe 768), 2 768 columns only
+    int tails = 0;
     size_t at = 0; // the product's place in the launch's list (the fusions are recorded per product)
     for (const Op *op : ops) {
         const uint32_t tail = op->cols & 1023u;
-        tails = tails || (op->cols >= 1024u && (tail == 128u || tail == 768u));
+        if (op->cols >= 1024u && tail == 128u) {
+            tails = 1;
+        } else if (op->cols >= 1024u && tail == 768u && tails == 0) {
+            tails = 2;
+        }
         // The token-split kernel covers waves x tokens-per-wave tokens per
         // descriptor: a larger batch goes as several descriptors over the same
         // weights, each with its own rows of X and Y.
@@ -931,8 +940,9 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
                                       : group_tokens);
         d.tile_begin = tiles;
         d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
-        if (small_launch && key.decode() && d.rows_per_tile == (uint32_t)R &&
-            (op->cols & 1023u) == 0u && (op->rows + R - 1) / R < 256u) {
+        const bool streams = tail == 0u || (op->cols >= 1024u && (tail == 128u || tail == 768u));
+        if (small_launch && key.decode() && d.rows_per_tile == (uint32_t)R && streams &&
+            (op->rows + R - 1) / R < 256u) {
             // Fewer than 256 tiles even at one pass per wave, in a launch that
             // is all latency (a projection of a few MB between two dependent
             // operators): half-height tiles put twice as many waves on it.
