@@ -865,25 +865,33 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
         if (full >= 1u && cols < (1u << 27)) {
             __shared__ __attribute__((aligned(16))) uint8_t raw_stage[4][raw_stage_bytes<R, TAILS>()];
             const uint32_t tail = cols & 1023u;
+            // (a small product may be cut into shorter tiles, as in the sealed layout)
+#define Q8_RAW_STREAM(TAILMASK)                                                                  \
+    if (d.rows_per_tile % (R / 2) != 0u) {                                                       \
+        stream_rows_raw<R / 4, XA, TAILMASK>(wv, x, y, cols, row_first, row_end, lane,           \
+                                             raw_stage[wave], d.res, d.alpha);                   \
+    } else if (d.rows_per_tile % R != 0u) {                                                      \
+        stream_rows_raw<R / 2, XA, TAILMASK>(wv, x, y, cols, row_first, row_end, lane,           \
+                                             raw_stage[wave], d.res, d.alpha);                   \
+    } else {                                                                                     \
+        stream_rows_raw<R, XA, TAILMASK>(wv, x, y, cols, row_first, row_end, lane,               \
+                                         raw_stage[wave], d.res, d.alpha);                       \
+    }                                                                                            \
+    return;
             if (tail == 0u) {
-                stream_rows_raw<R, XA, 0>(wv, x, y, cols, row_first, row_end, lane, raw_stage[wave],
-                                          d.res, d.alpha);
-                return;
+                Q8_RAW_STREAM(0)
             }
             if constexpr (TAILS == 1) {
                 if (tail == 128u && full == 1u) { // hidden 1152 (Gemma-3-1B)
-                    stream_rows_raw<R, XA, 128>(wv, x, y, cols, row_first, row_end, lane,
-                                                raw_stage[wave], d.res, d.alpha);
-                    return;
+                    Q8_RAW_STREAM(128)
                 }
             }
             if constexpr (TAILS >= 1) {
                 if (tail == 768u) { // FFN 6912 (Gemma-3-1B)
-                    stream_rows_raw<R, XA, 768>(wv, x, y, cols, row_first, row_end, lane,
-                                                raw_stage[wave], d.res, d.alpha);
-                    return;
+                    Q8_RAW_STREAM(768)
                 }
             }
+#undef Q8_RAW_STREAM
         }
     }
 

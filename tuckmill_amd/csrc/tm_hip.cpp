@@ -941,7 +941,8 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         d.tile_begin = tiles;
         d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
         const bool streams = tail == 0u || (op->cols >= 1024u && (tail == 128u || tail == 768u));
-        if (small_launch && key.decode() && d.rows_per_tile == (uint32_t)R && streams &&
+        const bool one_token = key.kind == OP_GEMV_LIST && key.variant == V_DECODE;
+        if (small_launch && one_token && d.rows_per_tile == (uint32_t)R && streams &&
             (op->rows + R - 1) / R < 256u) {
             // Fewer than 256 tiles even at one pass per wave, in a launch that
             // is all latency (a projection of a few MB between two dependent
