@@ -864,7 +864,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
                             const Workspace &ws) {
     const std::vector<const Op *> &ops = launch.list;
     const std::vector<const Op *> &residual = launch.residual;
-    const GemvKey key = launch.key;
+    GemvKey key = launch.key;
     if (key.variant == V_BF16X3) {
         return launch_bx3_list(ctx, stop, launch, ws);
     }
@@ -896,18 +896,27 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     bool norm_written = false;
     bool fused = launch.norm != nullptr; // the launch needs the kernel variant with fused forms
     const int R = key.variant == V_GENERAL ? kGemvR4 : kGemvR1;
-    // a workgroup's tile in the token-split kernel, a wave's tile otherwise (one
-    // token over raw weights: two passes per wave, so that the second pass's
-    // loads fly while the first goes through LDS)
-    const uint32_t tile_bytes = key.variant == V_SPLIT ? 32768u
-                                : (!key.packed && key.variant == V_DECODE) ? 16384u
-                                                                           : 8192u;
     uint32_t tiles = 0;
     uint64_t launch_bytes = 0;
     for (const Op *op : ops) {
         launch_bytes += (uint64_t)op->rows * (op->cols / 32u) * 34u;
     }
     const bool small_launch = launch_bytes < (16u << 20);
+    // The token-split kernel in a launch that is all latency (the projections
+    // of one layer between two dependent operators, a few tokens of a
+    // speculative step): one pass of rows per workgroup, and the same tokens
+    // over twice the waves. A token's result does not depend on either.
+    const bool small_split = key.variant == V_SPLIT && launch_bytes < (32u << 20);
+    if (small_split && key.p1 == 4 && key.p0 <= 2) {
+        key.p0 = (uint8_t)(key.p0 * 2);
+        key.p1 = 2;
+    }
+    // a workgroup's tile in the token-split kernel, a wave's tile otherwise (one
+    // token over raw weights: two passes per wave, so that the second pass's
+    // loads fly while the first goes through LDS)
+    const uint32_t tile_bytes = key.variant == V_SPLIT ? (small_split ? 8192u : 32768u)
+                                : (!key.packed && key.variant == V_DECODE) ? 16384u
+                                                                           : 8192u;
     // which column tails with a streaming path of their own the products have:
     // 0 none, 1 128 columns (and maybe 768), 2 768 columns only
     int tails = 0;
@@ -998,6 +1007,8 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     TM_SPLIT_CASE(false, W, T, true, true)                                                   \
     TM_SPLIT_CASE(false, W, T, false, true)
     TM_SPLIT_ALL(1, 2)
+    TM_SPLIT_ALL(2, 2)
+    TM_SPLIT_ALL(4, 2)
     TM_SPLIT_ALL(1, 4)
     TM_SPLIT_ALL(2, 4)
     TM_SPLIT_ALL(4, 4)
