@@ -67,10 +67,15 @@ def test_products_that_share_a_launch_decide_together():
     assert tile([layer["o"]]) == 0 and tile([layer["down"]]) == 64
     # the engine's prefill chunk of 128 tokens: all seven on the small tile
     assert tile([(r, c, 128) for _, r, c in S.QWEN3_0_6B_LAYER]) == 64
-    # ... and alone there: few tiles under a deep K take the small tile from 3072 columns
-    assert tile([(1024, 3072, 128)]) == 64 and tile([(1152, 6912, 128)]) == 64
+    # ... and alone there: few tiles under a deep K (3072 columns and more) take the small
+    # tile where the f32 kernel is estimated slower. It is not where it can share its output
+    # tiles between workgroups (up to 128 tiles) or still fills the chip in one round ...
+    assert tile([(1024, 3072, 128)]) == 0 and tile([(1152, 6912, 96)]) == 0
+    assert tile([(1024, 4096, 192)]) == 0 and tile([(1024, 4096, 256)]) == 0
+    # ... and is with more tiles than that under a deeper K
+    assert tile([(1152, 6912, 128)]) == 64 and tile([(2048, 6144, 65)]) == 64
+    assert tile([(2048, 8192, 96)]) == 64 and tile([(1030, 4096, 256)]) == 64
     assert tile([(1024, 2048, 128)]) == 0 and tile([(4096, 1024, 128)]) == 0
-    assert tile([(1024, 4096, 256)]) == 64
     # up to 64 tokens: 16 M weights between them
     assert tile([(6144, 2048, 64)]) == 0 and tile([(6144, 2048, 64), (6144, 2048, 64)]) == 64
     assert tile([]) == 0

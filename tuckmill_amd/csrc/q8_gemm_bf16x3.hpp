@@ -30,6 +30,7 @@
 #pragma once
 
 #include "q8_common.hpp"
+#include "q8_gemm_mma.hpp"
 
 namespace q8 {
 
@@ -722,11 +723,37 @@ inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
     if (large >= 128u) {
         return 128u;
     }
-    // Few output tiles under a deep K: the f32 kernels walk K in one piece per
-    // workgroup (4.6 + 9.8 us per 1024 columns at 128 tokens and up to 4096 rows),
-    // this kernel cuts it into chunks (22.5 + 2.3 us per 1024 columns, its split
-    // pass included).
-    return least_cols >= 3072u && small >= 32u ? 64u : 0u;
+    // Few output tiles under a deep K: this kernel cuts K into chunks and takes
+    // 22.5 + 2.3 us per 1024 columns, its split pass included. A wave of the f32
+    // kernel takes 0.72 us per block of a 32-token tile (twice that for 64
+    // tokens) after 4.5 us, over K divided by its 4 waves and by the workgroups
+    // that share a tile (q8::mma_shared_parts), once per round of 256
+    // workgroups: 1024 x 3072 at 128 tokens 14.8 us against 29.1 here, 1024 x 4096
+    // at 192 tokens 26.4 against 33.1, but 1152 x 6912 at 128 tokens 42.0 against
+    // 37.9 and 2048 x 8192 at 96 tokens 49.0 against 41.3. The cheaper estimate wins.
+    if (least_cols < 3072u || small < 32u) {
+        return 0u;
+    }
+    MmaProduct prods[MMA_MAX_DESCS];
+    const int m = n < MMA_MAX_DESCS ? n : MMA_MAX_DESCS;
+    uint32_t min_blocks = 0xffffffffu, max_blocks = 0;
+    for (int i = 0; i < m; ++i) {
+        prods[i] = MmaProduct{nullptr, nullptr, nullptr, shapes[i].rows, shapes[i].cols, shapes[i].batch};
+        const uint32_t blocks = shapes[i].cols / 32u;
+        min_blocks = blocks < min_blocks ? blocks : min_blocks;
+        max_blocks = blocks > max_blocks ? blocks : max_blocks;
+    }
+    const MmaConfig c = pick_mma_config(prods, m);
+    uint64_t tiles = 0;
+    for (int i = 0; i < m; ++i) {
+        tiles += mma_tiles(prods[i], c);
+    }
+    const uint32_t z = c.s == 4 ? mma_shared_parts(tiles, min_blocks) : 1u;
+    const uint64_t rounds = (tiles * z + 255u) / 256u;
+    const uint64_t per_wave = (max_blocks + 4u * z - 1u) / (4u * z);
+    const uint64_t f32_us_x100 = 450u + 72u * (uint64_t)c.tmw * per_wave * rounds;
+    const uint64_t here_us_x100 = 2250u + 230u * (uint64_t)(max_blocks * 32u) / 1024u;
+    return here_us_x100 < f32_us_x100 ? 64u : 0u;
 }
 
 // A product on its own: its plan, and whether the kernel pays for it (`worth`).

@@ -60,9 +60,28 @@ struct MmaArgs {
     uint32_t n;
     uint32_t total_tiles;
     uint32_t chunk_wgs; // workgroups that share one weight row-tile (see the XCD mapping)
-    uint32_t pad;
+    uint32_t z;         // workgroups that share one output tile, each with a part of K (1: none)
+    float *partials;    // z > 1: total_tiles x z partial tiles
+    uint32_t *arrivals; // z > 1: one counter per output tile, zero between launches
     MmaDesc d[MMA_MAX_DESCS];
 };
+
+// How many workgroups share each output tile of a launch, each with its own
+// part of K: a launch with few output tiles and a long K otherwise leaves most
+// of the chip idle (1024 x 2048 at 32 tokens is 32 tiles of 64 blocks each).
+// Doubled while the launch's tiles, times it, stay within 256 workgroups and
+// every wave keeps at least 4 blocks of the shortest K. It depends on what
+// shares the launch, and with it the order of a product's f32 sums (the same
+// launch gives the same bits every time).
+constexpr uint32_t MMA_SHARED_MAX_TILES = 128;  // tiles x parts <= 256, parts >= 2
+constexpr size_t MMA_SHARED_PARTIAL_FLOATS = 256u * 2u * 16u * 64u; // 256 partial tiles of 64 x 32
+inline uint32_t mma_shared_parts(uint64_t tiles, uint32_t min_blocks) {
+    uint32_t z = 1;
+    while (z < 8u && tiles * (z * 2u) <= 256u && min_blocks / (4u * z * 2u) >= 4u) {
+        z *= 2u;
+    }
+    return z;
+}
 
 // Operands of one Q8_0 block for a wave's TMW x TNW tiles, as loaded.
 template <int TMW, int TNW> struct MmaRaw {
@@ -95,8 +114,15 @@ __device__ __forceinline__ void mma_load_block(const WView<L> &wv, const float *
 // of the Q8_0 blocks and wave s = 0 adds the partial tiles of s = 1..S-1 in
 // that order. The k loop is software-pipelined: the operands of block kb+1
 // are requested before the 16*TMW*TNW MFMAs of block kb are issued.
-template <int L, int TMW, int TNW, int S, bool XA>
+// ZS: args.z workgroups share an output tile (S == 4 only: one tile per
+// workgroup). Workgroup g takes part g % z of the K range of tile g / z; what its
+// four waves add up goes to args.partials, and the workgroup that arrives last
+// at the tile's counter adds the z partial tiles in part order (whoever it is:
+// the result does not depend on the order of arrival), stores the sum and puts
+// the counter back to zero.
+template <int L, int TMW, int TNW, int S, bool XA, bool ZS = false>
 __global__ __launch_bounds__(256) void gemm_mma_kernel(const MmaArgs args) {
+    static_assert(!ZS || S == 4, "shared tiles: one tile per workgroup");
     constexpr int P = 4 / S;
     constexpr int TILE_FLOATS = TMW * TNW * 16 * WAVE;
     extern __shared__ float red[]; // [P][S-1][TILE_FLOATS]
@@ -113,7 +139,11 @@ __global__ __launch_bounds__(256) void gemm_mma_kernel(const MmaArgs args) {
     // heavy products (large K) are spread over all XCDs instead of landing on
     // the one that owns their index range.
     uint32_t g = blockIdx.x;
-    {
+    uint32_t zpart = 0;
+    if constexpr (ZS) {
+        zpart = g % args.z;
+        g = g / args.z;
+    } else {
         const uint32_t cw = args.chunk_wgs;
         const uint32_t span = 8u * cw;
         const uint32_t g_full = (gridDim.x / span) * span;
@@ -143,8 +173,11 @@ __global__ __launch_bounds__(256) void gemm_mma_kernel(const MmaArgs args) {
 
     const WView<L> wv(d.w, rows, cols);
     const uint32_t blocks = cols >> 5;
-    const uint32_t kb_begin = (uint32_t)(((uint64_t)blocks * s) / S);
-    const uint32_t kb_end = (uint32_t)(((uint64_t)blocks * (s + 1u)) / S);
+    // this wave's part of K: one of S, or with shared tiles one of z x S
+    const uint32_t kparts = ZS ? args.z * (uint32_t)S : (uint32_t)S;
+    const uint32_t kpart = ZS ? zpart * (uint32_t)S + s : s;
+    const uint32_t kb_begin = (uint32_t)(((uint64_t)blocks * kpart) / kparts);
+    const uint32_t kb_end = (uint32_t)(((uint64_t)blocks * (kpart + 1u)) / kparts);
 
     uint32_t wrow[TNW], tok[TMW];
 #pragma unroll
@@ -242,6 +275,54 @@ __global__ __launch_bounds__(256) void gemm_mma_kernel(const MmaArgs args) {
     }
     if (!valid) {
         return;
+    }
+    if constexpr (ZS) {
+        // (one wave is left: the partial tiles go to memory and come back from it
+        // with device-scope accesses that bypass this XCD's L2, so all it takes to
+        // publish them is to wait for the stores before the arrival is counted)
+        const uint32_t z = args.z;
+        float *mine = args.partials + ((size_t)tile * z + zpart) * TILE_FLOATS + lane;
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+            for (int j = 0; j < TNW; ++j) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    __hip_atomic_store(mine + ((i * TNW + j) * 16 + v) * WAVE, acc[i][j][v],
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); // vmcnt(0)
+        asm volatile("" ::: "memory");
+        uint32_t arrived = 0;
+        if (lane == 0u) {
+            arrived = __hip_atomic_fetch_add(&args.arrivals[tile], 1u, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+        }
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        if (arrived != z - 1u) {
+            return;
+        }
+        if (lane == 0u) {
+            __hip_atomic_store(&args.arrivals[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        const float *first = args.partials + (size_t)tile * z * TILE_FLOATS + lane;
+        for (uint32_t c = 0; c < z; ++c) {
+            const float *part = first + (size_t)c * TILE_FLOATS;
+#pragma unroll
+            for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+                for (int j = 0; j < TNW; ++j) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const float pv = __hip_atomic_load(part + ((i * TNW + j) * 16 + v) * WAVE,
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        acc[i][j][v] = c == 0u ? pv : acc[i][j][v] + pv;
+                    }
+                }
+            }
+        }
     }
     // acc[v] of a 32x32 tile is (token 8*(v/4) + 4*half + v%4, row idx).
 #pragma unroll
@@ -691,12 +772,26 @@ template <class K> inline uint32_t mma_resident_wgs(K kernel) {
 // Launches with at least this many wave tiles per resident wave use the work-queue kernel.
 constexpr uint32_t MMA_QUEUE_MIN_TILES_PER_WAVE = 8;
 
+// What a launch whose output tiles are shared between workgroups needs beside
+// the products: MMA_SHARED_PARTIAL_FLOATS floats for the partial tiles and
+// MMA_SHARED_MAX_TILES zeroed counters (null: no such launches).
+struct MmaShared {
+    float *partials = nullptr;
+    uint32_t *arrivals = nullptr;
+};
+
+// Floats of one partial tile.
+constexpr uint32_t mma_tile_floats(int tmw) { return (uint32_t)tmw * 16u * WAVE; }
+
 template <int L, int TMW, int TNW, int S, bool XA>
 inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods_in,
-                                 int n, uint32_t *queue) {
+                                 int n, uint32_t *queue, const MmaShared &shared) {
     constexpr int P = 4 / S;
     MmaArgs args;
     args.n = (uint32_t)n;
+    args.z = 1;
+    args.partials = nullptr;
+    args.arrivals = nullptr;
     const MmaConfig c{TMW, TNW, S};
     uint64_t tiles = 0;
     uint32_t min_batch = 0xffffffffu;
@@ -712,14 +807,24 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
     bool use_queue = false, use_persistent = false;
     uint32_t launch_wgs = 0;
     const uint32_t groups = (uint32_t)((tiles + P - 1) / P);
-    if constexpr (S == 4 && TNW == 1 && TMW == 2) if (queue != nullptr) {
+    uint32_t z = 1;
+    if constexpr (S == 4 && TNW == 1) if (shared.partials != nullptr && shared.arrivals != nullptr) {
+        uint32_t min_blocks = 0xffffffffu;
+        for (int i = 0; i < n; ++i) {
+            const uint32_t blocks = prods_in[i].cols / 32u;
+            min_blocks = blocks < min_blocks ? blocks : min_blocks;
+        }
+        z = mma_shared_parts(tiles, min_blocks);
+    }
+    const bool shared_tiles = z > 1u;
+    if constexpr (S == 4 && TNW == 1 && TMW == 2) if (queue != nullptr && !shared_tiles) {
         static const uint32_t resident = mma_resident_wgs(gemm_mma_queue_kernel<L, TMW, XA>);
         if (tiles >= (uint64_t)resident * 4u * MMA_QUEUE_MIN_TILES_PER_WAVE) {
             use_queue = true;
             launch_wgs = resident;
         }
     }
-    if constexpr (S == 4 && TNW == 1) if (!use_queue && min_batch >= 256u) {
+    if constexpr (S == 4 && TNW == 1) if (!use_queue && !shared_tiles && min_batch >= 256u) {
         static const uint32_t resident = mma_resident_wgs(gemm_mma_persistent_kernel<L, TMW, XA>);
         const uint32_t wgs = groups < resident ? groups : resident;
         if (wgs == groups || wgs % 8u == 0u) {
@@ -757,7 +862,16 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
     }
     args.total_tiles = (uint32_t)tiles;
     args.chunk_wgs = args.d[0].tiles_t >= (uint32_t)P ? args.d[0].tiles_t / P : 1u;
-    args.pad = 0;
+    if constexpr (S == 4 && TNW == 1) if (shared_tiles) {
+        static_assert(256u * mma_tile_floats(2) <= MMA_SHARED_PARTIAL_FLOATS, "partial tiles");
+        args.z = z;
+        args.partials = shared.partials;
+        args.arrivals = shared.arrivals;
+        const size_t lds = (size_t)(S - 1) * TMW * TNW * 16 * WAVE * sizeof(float);
+        Q8_LAUNCH((gemm_mma_kernel<L, TMW, TNW, S, XA, true>), dim3(groups * z), dim3(256), lds,
+                  stream, stop, args);
+        return hipGetLastError();
+    }
     if constexpr (S == 4 && TNW == 1 && TMW == 2) if (use_queue) {
         Q8_LAUNCH((gemm_mma_queue_kernel<L, TMW, XA>), dim3(launch_wgs), dim3(256), 0, stream, stop,
                   args, queue);
@@ -776,11 +890,12 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
 
 template <int L, bool XA>
 inline hipError_t launch_mma_layout(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods,
-                                    int n, const MmaConfig *forced, uint32_t *queue) {
+                                    int n, const MmaConfig *forced, uint32_t *queue,
+                                    const MmaShared &shared) {
     const MmaConfig c = forced != nullptr ? *forced : pick_mma_config(prods, n);
-#define TM_MMA_CASE(A, B, C)                                                  \
-    if (c.tmw == A && c.tnw == B && c.s == C) {                               \
-        return launch_mma_cfg<L, A, B, C, XA>(stream, stop, prods, n, queue);       \
+#define TM_MMA_CASE(A, B, C)                                                          \
+    if (c.tmw == A && c.tnw == B && c.s == C) {                                       \
+        return launch_mma_cfg<L, A, B, C, XA>(stream, stop, prods, n, queue, shared); \
     }
     TM_MMA_CASE(2, 1, 1)
     TM_MMA_CASE(1, 1, 1)
@@ -799,16 +914,18 @@ inline hipError_t launch_mma_layout(hipStream_t stream, hipEvent_t stop, const M
 inline hipError_t launch_gemm_mma_list(hipStream_t stream, hipEvent_t stop, bool packed,
                                        bool xaligned, const MmaProduct *prods, int n,
                                        const MmaConfig *forced = nullptr,
-                                       uint32_t *queue = nullptr) {
+                                       uint32_t *queue = nullptr,
+                                       const MmaShared &shared = MmaShared()) {
     if (n <= 0 || n > MMA_MAX_DESCS) {
         return hipErrorInvalidValue;
     }
     if (packed) {
-        return xaligned ? launch_mma_layout<PACKED, true>(stream, stop, prods, n, forced, queue)
-                        : launch_mma_layout<PACKED, false>(stream, stop, prods, n, forced, queue);
+        return xaligned
+                   ? launch_mma_layout<PACKED, true>(stream, stop, prods, n, forced, queue, shared)
+                   : launch_mma_layout<PACKED, false>(stream, stop, prods, n, forced, queue, shared);
     }
-    return xaligned ? launch_mma_layout<RAW, true>(stream, stop, prods, n, forced, queue)
-                    : launch_mma_layout<RAW, false>(stream, stop, prods, n, forced, queue);
+    return xaligned ? launch_mma_layout<RAW, true>(stream, stop, prods, n, forced, queue, shared)
+                    : launch_mma_layout<RAW, false>(stream, stop, prods, n, forced, queue, shared);
 }
 
 } // namespace q8

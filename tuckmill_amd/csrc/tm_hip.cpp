@@ -49,6 +49,8 @@ constexpr size_t kScratchXsBytes = TM_HIP_NOALLOC_XS_BYTES;
 constexpr size_t kScratchPartialOff = kScratchXsOff + kScratchXsBytes;
 constexpr size_t kScratchPartialBytes = kScratchBytes - kScratchPartialOff;
 static_assert(kScratchArrivalsOff + q8::BX3_MAX_SPLIT_TILES * 4u <= kScratchXsOff, "counters");
+static_assert(q8::MMA_SHARED_PARTIAL_FLOATS * 4u <= kScratchPartialBytes, "f32 partial tiles");
+static_assert(q8::MMA_SHARED_MAX_TILES <= q8::BX3_MAX_SPLIT_TILES, "f32 arrival counters");
 static __device__ __align__(256) uint8_t scratch[kScratchBytes];
 
 namespace {
@@ -83,6 +85,10 @@ hipError_t scratch_on_current_device(int device, uint8_t **out) {
 // Device memory the kernels use beyond a product's own buffers.
 struct Workspace {
     uint32_t *mma_queue = nullptr; // two counters of the work-queue MFMA kernel, zero between launches
+    // An f32 MFMA launch with few output tiles shares each tile between
+    // workgroups (q8::mma_shared_parts): room for their partial tiles; the
+    // arrival counters are the first of `arrivals` below.
+    float *mma_partials = nullptr;
     // The bf16 split-float GEMM: split activations, partial tiles of products
     // whose K is cut into chunks, their arrival counters (zero between launches).
     uint8_t *xs = nullptr;
@@ -731,8 +737,9 @@ hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<c
                                     op->batch};
     }
     const q8::MmaConfig c{key.p0, key.p1, key.p2};
+    const q8::MmaShared shared{ws.mma_partials, ws.arrivals};
     return q8::launch_gemm_mma_list(ctx->stream, stop, key.packed, key.flag, prods, n, &c,
-                                    ws.mma_queue);
+                                    ws.mma_queue, shared);
 }
 
 // The split-float GEMM: one launch that splits every distinct input of the list
@@ -1796,6 +1803,9 @@ tm_hip_ctx *tm_hip_create(char *err, size_t err_cap) {
         e = hipMemset(ctx->ws.mma_queue, 0, 256);
     }
     if (e == hipSuccess) {
+        e = hipMalloc((void **)&ctx->ws.mma_partials, q8::MMA_SHARED_PARTIAL_FLOATS * sizeof(float));
+    }
+    if (e == hipSuccess) {
         e = hipMalloc((void **)&ctx->ws.arrivals, q8::BX3_MAX_SPLIT_TILES * sizeof(uint32_t));
     }
     if (e == hipSuccess) {
@@ -1822,6 +1832,7 @@ tm_hip_ctx *tm_hip_create(char *err, size_t err_cap) {
     ctx->fixed.xs_bytes = kScratchXsBytes;
     ctx->fixed.partials = (float *)(fixed + kScratchPartialOff);
     ctx->fixed.partial_bytes = kScratchPartialBytes;
+    ctx->fixed.mma_partials = ctx->fixed.partials; // (a call runs one kernel family or the other)
     ctx->noalloc_keep.reserve(kNoallocKeepCap);
     // Fail at creation, not at first use, when the device code is missing.
     hipFuncAttributes attr;
@@ -1870,8 +1881,8 @@ void tm_hip_destroy(tm_hip_ctx *ctx) {
         ctx->event_pool.clear();
     }
     noalloc_release(ctx);
-    for (void *p : {(void *)ctx->ws.mma_queue, (void *)ctx->ws.arrivals, (void *)ctx->ws.xs,
-                    (void *)ctx->ws.partials}) {
+    for (void *p : {(void *)ctx->ws.mma_queue, (void *)ctx->ws.mma_partials,
+                    (void *)ctx->ws.arrivals, (void *)ctx->ws.xs, (void *)ctx->ws.partials}) {
         if (p != nullptr) {
             (void)hipFree(p);
         }

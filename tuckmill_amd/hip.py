@@ -51,7 +51,7 @@ def gemm_mma_launch_tile(shapes) -> int:
     from 33 to 64, or all above. Up to 64 tokens: 16 M weights (32 M up to 32 tokens) and 128 units of
     the small tile between them. Above, in order of preference: 192 units or more of the large tile; 192 or
     more of the small tile; 128 or more of the large tile; the small tile for products of 3072
-    columns and more with 32 units or more."""
+    columns and more with 32 units or more where the f32 kernel is estimated slower."""
     shapes = list(shapes)
     if not shapes:
         return 0
@@ -67,8 +67,32 @@ def gemm_mma_launch_tile(shapes) -> int:
         return 64
     if large >= 128:
         return 128
-    # few output tiles under a deep K
-    return 64 if min(c for _, c, _ in shapes) >= 3072 and small >= 32 else 0
+    # few output tiles under a deep K: the cheaper of two estimates (hundredths of a microsecond)
+    if min(c for _, c, _ in shapes) < 3072 or small < 32:
+        return 0
+    shapes = shapes[:64]
+    tmw, tiles, z = _f32_launch_shape(shapes)
+    max_blocks = max(c // 32 for _, c, _ in shapes)
+    per_wave = -(-max_blocks // (4 * z))
+    f32_us = 450 + 72 * tmw * per_wave * (-(-(tiles * z) // 256))
+    here_us = 2250 + 230 * (max_blocks * 32) // 1024
+    return 64 if here_us < f32_us else 0
+
+
+def _f32_launch_shape(shapes):
+    """(tokens per wave tile / 32, output tiles, workgroups per tile) of a launch of
+    `shapes` on the f32 matrix cores (mirror of q8::pick_mma_config, q8::mma_tiles and
+    q8::mma_shared_parts)."""
+    tiles64 = sum(-(-b // 64) * -(-r // 32) for r, _, b in shapes)
+    short_last_round = tiles64 <= 128 or 256 < tiles64 <= 384
+    tmw = 2 if max(b for _, _, b in shapes) > 32 and not short_last_round else 1
+    tiles = sum(-(-b // (32 * tmw)) * -(-r // 32) for r, _, b in shapes)
+    min_blocks = min(c // 32 for _, c, _ in shapes)
+    z = 1
+    if min_blocks >= 4:  # K split over the four waves of a workgroup
+        while z < 8 and tiles * z * 2 <= 256 and min_blocks // (4 * z * 2) >= 4:
+            z *= 2
+    return tmw, tiles, z
 
 
 def gemm_mma_bf16_plan(rows: int, cols: int, batch: int):
