@@ -918,6 +918,28 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         key.p0 = (uint8_t)(key.p0 * 2);
         key.p1 = 2;
     }
+    // Such a launch with few rows (fewer than 160 of the token-split kernel's
+    // workgroups of 8 rows: the o and down projections) and up to 4 tokens goes
+    // to the one-token kernel instead, one descriptor per token: every token is
+    // its own GEMV anyway, and that kernel cuts a small product into tiles of 2
+    // rows (lone 1024 x 3072: 2 tokens 6.0 -> 4.2 us, 4 tokens 5.9 -> 5.0; 1152 x 6912:
+    // 10.3 -> 6.6 and 10.2 -> 9.0). With more rows the weights read once per
+    // token cost more than the waves bring (q,k,v at 4 tokens 4.8 -> 6.1 us; Gemma's,
+    // 192 such workgroups, at 3 tokens 4.4 -> 7.4).
+    bool per_token = false;
+    if (small_split) {
+        uint32_t max_batch = 0, descs = 0;
+        uint64_t row_groups = 0;
+        for (const Op *op : ops) {
+            max_batch = op->batch > max_batch ? op->batch : max_batch;
+            descs += op->batch;
+            row_groups += (op->rows + 7u) / 8u;
+        }
+        if (max_batch <= 4u && row_groups < 160u && descs <= (uint32_t)q8::GEMV_MAX_DESCS) {
+            per_token = true;
+            key.variant = V_DECODE;
+        }
+    }
     // a workgroup's tile in the token-split kernel, a wave's tile otherwise (one
     // token over raw weights: two passes per wave, so that the second pass's
     // loads fly while the first goes through LDS)
@@ -938,8 +960,10 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         // The token-split kernel covers waves x tokens-per-wave tokens per
         // descriptor: a larger batch goes as several descriptors over the same
         // weights, each with its own rows of X and Y.
-        const uint32_t group_tokens = key.variant == V_SPLIT ? (uint32_t)key.p0 * key.p1 : op->batch;
-        const uint32_t groups = split_token_groups(key, op->batch);
+        const uint32_t group_tokens = per_token                  ? 1u
+                                      : key.variant == V_SPLIT ? (uint32_t)key.p0 * key.p1
+                                                               : op->batch;
+        const uint32_t groups = per_token ? op->batch : split_token_groups(key, op->batch);
         if (args.n + groups > (uint32_t)q8::GEMV_MAX_DESCS) {
             return hipErrorInvalidValue;
         }
