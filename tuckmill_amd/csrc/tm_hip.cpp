@@ -519,8 +519,10 @@ GemvKey bx3_key(uint32_t tile_tokens) {
     return k;
 }
 
-// The f32 matrix-core kernel's key: tile shape and K split are chosen per
-// product, so its result does not depend on what else shares the launch.
+// The f32 matrix-core kernel's key: tile shape and the K split over a
+// workgroup's waves are chosen per product. (What else shares the launch still
+// shows in a product's last bits when the launch has few output tiles: each
+// tile is then shared between workgroups, q8::mma_shared_parts.)
 GemvKey mma_f32_key(const Op &op) {
     GemvKey k;
     k.kind = OP_MMA;
