@@ -61,7 +61,7 @@ class tmh_timing(ctypes.Structure):
 
 
 TMH_GEMV, TMH_GEMM, TMH_GEMM_MMA, TMH_GEMM_I8, TMH_QUANT = range(5)
-TMH_RMSNORM, TMH_SILU_MUL, TMH_AXPY, TMH_ARGMAX, TMH_F16_GEMM = range(5, 10)
+TMH_RMSNORM, TMH_SILU_MUL, TMH_AXPY, TMH_ARGMAX, TMH_F16_GEMM, TMH_GELU_MUL = range(5, 11)
 
 
 def load_host():
@@ -577,16 +577,23 @@ def bench_f16(host, ctx, steps, warmup):
     return out
 
 
-def bench_chain(host, ctx, steps, warmup, recorded=True):
+# (hidden, q width, k/v width, FFN width, vocabulary, layers, gated activation)
+CHAIN_MODELS = {
+    "qwen": ("Qwen3-0.6B", 1024, 2048, 1024, 3072, 151_936, S.QWEN3_0_6B_LAYERS, "silu"),
+    "gemma": ("Gemma-3-1B", 1152, 1024, 256, 6912, 262_144, 26, "gelu_tanh"),
+}
+
+
+def bench_chain(host, ctx, steps, warmup, recorded=True, model="qwen"):
     """The decode step with its data dependencies: per layer rmsnorm -> q,k,v -> o ->
     residual -> rmsnorm -> gate,up -> silu_mul -> down -> residual, then final norm,
-    lm_head and greedy argmax, Qwen3-0.6B shapes, one dispatch group per token
+    lm_head and greedy argmax, Qwen3-0.6B shapes (or Gemma-3-1B's), one dispatch group per token
     (attention, RoPE and the KV cache are not part of this path: o reads q in place of
     the attention output, which has the same length and the same dependence). Products that do not depend on each other still share a launch (q,k,v and
     gate,up), everything else is ordered, so the step is bound by launch latency, not by
     HBM: this is the figure a graph replay or wider fusion would have to beat."""
-    hidden, qdim, kvdim, ffn, vocab = 1024, 2048, 1024, 3072, 151_936
-    layers = S.QWEN3_0_6B_LAYERS
+    model_name, hidden, qdim, kvdim, ffn, vocab, layers, act = CHAIN_MODELS[model]
+    act_kind = TMH_SILU_MUL if act == "silu" else TMH_GELU_MUL
     keep, prods = [], []
 
     def fbuf(n, seed=None):
@@ -624,7 +631,7 @@ def bench_chain(host, ctx, steps, warmup, recorded=True):
         prods.append(tmh_product(g2.raw, h.raw, n.raw, 1, hidden, 1, TMH_RMSNORM))
         product(mat(ffn, hidden, 5004 + 7 * layer), n, gate, ffn, hidden)
         product(mat(ffn, hidden, 5005 + 7 * layer), n, up, ffn, hidden)
-        prods.append(tmh_product(gate.raw, up.raw, gate.raw, 1, ffn, 1, TMH_SILU_MUL))
+        prods.append(tmh_product(gate.raw, up.raw, gate.raw, 1, ffn, 1, act_kind))
         product(mat(hidden, ffn, 5006 + 7 * layer), gate, t, hidden, ffn)
         prods.append(tmh_product(h.raw, t.raw, h.raw, 1, hidden, 1, TMH_AXPY))
     gf = fbuf(hidden, 999)
@@ -633,7 +640,7 @@ def bench_chain(host, ctx, steps, warmup, recorded=True):
     prods.append(tmh_product(partial.raw, logits.raw, token.raw, 1, vocab, 1, TMH_ARGMAX))
     ctx.fence()
     tg = run_steps(host, ctx, prods, warmup, steps, grouped=True)
-    out = {"workload": "Qwen3-0.6B decode step with data dependencies (no attention)",
+    out = {"workload": f"{model_name} decode step with data dependencies (no attention)",
            "operators_per_step": len(prods), "algorithmic_bytes": wbytes,
            "grouped": {"us": tg.wall_ms / steps * 1e3, "gpu_us": tg.gpu_ms / steps * 1e3,
                        "launches_per_step": tg.launches / steps,
@@ -749,6 +756,8 @@ def main():
                          "crashed on stream capture here)")
     ap.add_argument("--ungrouped", action="store_true",
                     help="one commit per GEMV instead of one group per step")
+    ap.add_argument("--model", choices=sorted(CHAIN_MODELS), default="qwen",
+                    help="chain workload: whose shapes the dependent decode step has")
     ap.add_argument("--unsealed", action="store_true",
                     help="decode workload: leave the weights in the layout they are uploaded in "
                          "(what a binding that never calls tm_hip_q8_0_pack runs on)")
@@ -772,7 +781,8 @@ def main():
     if args.workload != "decode":
         fn = {"gemma": bench_gemma, "sweep": bench_sweep, "chain": bench_chain,
               "f16": bench_f16, "layer": bench_layer}[args.workload]
-        extra = {"recorded": not args.no_recorded} if args.workload == "chain" else {}
+        extra = ({"recorded": not args.no_recorded, "model": args.model}
+                 if args.workload == "chain" else {})
         print(json.dumps(fn(host, ctx, args.steps, args.warmup, **extra)), flush=True)
         ctx.close()
         return

@@ -220,11 +220,13 @@ def test_residual_update_is_not_fused_when_it_would_reorder_accesses(ctx):
     assert np.array_equal(bits(hb.download_f32(0, rows)), bits(O.axpy(t, 1.0, h0)))
 
 
-def test_rmsnorm_in_front_of_its_products_is_fused_into_their_launch(ctx):
+@pytest.mark.parametrize("hidden,qdim,kvdim,ffn", [(1024, 2048, 1024, 3072),     # Qwen3-0.6B
+                                                   (1152, 1024, 256, 6912)])     # Gemma-3-1B
+def test_rmsnorm_in_front_of_its_products_is_fused_into_their_launch(ctx, hidden, qdim, kvdim, ffn):
     # norm -> q, k, v (one launch) -> o with its residual update -> norm -> gate, up:
     # grouped, the norms ride in the launches of the products that read them and the
     # update in the epilogue of o; every buffer must hold the bits of the separate run.
-    hidden, qdim, kvdim, ffn = 1024, 2048, 1024, 3072
+    # (Gemma's hidden width leaves a column tail of 128 behind the 1024-column chunk.)
     mats = {}
     for i, (name, rows, cols) in enumerate([("q", qdim, hidden), ("k", kvdim, hidden),
                                             ("v", kvdim, hidden), ("o", hidden, qdim),
@@ -289,13 +291,15 @@ def test_a_norm_nobody_reads_still_runs(ctx):
     assert np.max(np.abs(yb.download_f32(0, 64) - want)) <= 1e-5 * np.max(np.abs(want))
 
 
+@pytest.mark.parametrize("hidden", [1024, 1152, 2048 + 128])
 @pytest.mark.parametrize("act,in_place,with_norm", [("silu", True, True), ("silu", False, False),
                                                     ("gelu", True, False), ("gelu", False, True)])
-def test_gated_activation_behind_gate_and_up_is_fused(ctx, act, in_place, with_norm):
+def test_gated_activation_behind_gate_and_up_is_fused(ctx, act, in_place, with_norm, hidden):
     # [norm ->] gate, up -> act(gate) * up -> down with its residual update: grouped,
     # one wave computes a row of gate and of up and applies the activation itself.
-    # Every buffer must hold the bits of the separate operators.
-    hidden, ffn = 1024, 3072 + 8  # a row count that leaves a partial last tile
+    # Every buffer must hold the bits of the separate operators. (Widths with a column
+    # tail of 128 behind the 1024-column chunks too: Gemma-3-1B's 1152.)
+    ffn = 3072 + 8  # a row count that leaves a partial last tile
     wg, wu = S.make_weights(ffn, hidden, 401), S.make_weights(ffn, hidden, 402)
     wd = S.make_weights(hidden, 1024 * 3, 403)
     wgb, wub = weights_buffer(ctx, wg, ffn, hidden, True), weights_buffer(ctx, wu, ffn, hidden, True)

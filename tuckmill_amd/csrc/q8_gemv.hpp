@@ -182,11 +182,16 @@ __device__ __forceinline__ void reduce_store(const float (&acc)[R], float *y, ui
 
 // Where a lane's 16 activations of a chunk come from: memory, or the fused
 // RMSNorm of the launch, (h * inv) * w with the operations of rmsnorm_kernel.
+// (loadn: the N activations of a column-tail piece.)
 struct PlainX {
     const float *x;
     template <bool XA>
     __device__ __forceinline__ void load16(uint32_t col, float (&out)[16]) const {
         load_x<16, XA>(x + col, out);
+    }
+    template <int N, bool XA>
+    __device__ __forceinline__ void loadn(uint32_t col, float (&out)[N]) const {
+        load_x<N, XA>(x + col, out);
     }
 };
 struct NormedX {
@@ -194,11 +199,15 @@ struct NormedX {
     float inv;
     template <bool XA>
     __device__ __forceinline__ void load16(uint32_t col, float (&out)[16]) const {
-        float hv[16], wv[16];
-        load_x<16, true>(h + col, hv);
-        load_x<16, true>(w + col, wv);
+        loadn<16, XA>(col, out);
+    }
+    template <int N, bool XA>
+    __device__ __forceinline__ void loadn(uint32_t col, float (&out)[N]) const {
+        float hv[N], wv[N];
+        load_x<N, true>(h + col, hv);
+        load_x<N, true>(w + col, wv);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < N; ++i) {
             out[i] = hv[i] * inv * wv[i];
         }
     }
@@ -271,20 +280,19 @@ template <int R, bool XA, int TAILMASK, class XS, class ROWS, class SINK>
 __device__ __forceinline__ void stream_rows_to(const ROWS rows_src, const XS xs, uint32_t cols,
                                                uint32_t row_first, uint32_t row_end, uint32_t lane,
                                                SINK sink) {
-    static_assert(TAILMASK == 0 || sizeof(XS) == sizeof(PlainX), "tails read plain activations");
-    static_assert(TAILMASK == 0 || !ROWS::pair, "the paired form has no tail pieces");
     constexpr uint32_t ADV = ROWS::pair ? R / 2 : R; // rows a pass advances by
-    const WView<PACKED> &wv = [&]() -> const WView<PACKED> & {
+    // the matrix row r of a pass comes from (the paired form: gate rows, then up rows)
+    auto view_of = [&](int r) -> const WView<PACKED> & {
         if constexpr (ROWS::pair) {
-            return rows_src.gate;
+            return r < R / 2 ? rows_src.gate : rows_src.up;
         } else {
             return rows_src.wv;
         }
-    }();
-    const float *x = nullptr;
-    if constexpr (TAILMASK != 0) {
-        x = xs.x;
-    }
+    };
+    auto row_of = [&](int r, uint32_t r0) {
+        const uint32_t row = r0 + (ROWS::pair ? (uint32_t)(r % (R / 2)) : (uint32_t)r);
+        return row < row_end ? row : row_end - 1u;
+    };
     constexpr bool T8 = (TAILMASK & 512) != 0, T4 = (TAILMASK & 256) != 0;
     constexpr bool T2 = (TAILMASK & 128) != 0, T1 = (TAILMASK & 64) != 0;
     constexpr bool TH = (TAILMASK & 32) != 0;
@@ -298,22 +306,24 @@ __device__ __forceinline__ void stream_rows_to(const ROWS rows_src, const XS xs,
 
     // activations of the tail pieces: loop invariant, kept in registers
     float x8[8], x4[4], x2[2], x1[1], xh[1];
-    if constexpr (T8) load_x<8, XA>(x + c8 + lane * 8u, x8);
-    if constexpr (T4) load_x<4, XA>(x + c4 + lane * 4u, x4);
-    if constexpr (T2) load_x<2, XA>(x + c2 + lane * 2u, x2);
-    if constexpr (T1) load_x<1, XA>(x + c1 + lane, x1);
-    if constexpr (TH) load_x<1, XA>(x + ch + (low ? lane : 0u), xh);
+    if constexpr (T8) xs.template loadn<8, XA>(c8 + lane * 8u, x8);
+    if constexpr (T4) xs.template loadn<4, XA>(c4 + lane * 4u, x4);
+    if constexpr (T2) xs.template loadn<2, XA>(c2 + lane * 2u, x2);
+    if constexpr (T1) xs.template loadn<1, XA>(c1 + lane, x1);
+    if constexpr (TH) xs.template loadn<1, XA>(ch + (low ? lane : 0u), xh);
     float xv[16];
     if (full == 1u) {
         xs.template load16<XA>(lane * 16u, xv);
     }
+
 
     uint32_t q8[R][2], q4[R][1], q2[R][1], q1[R][1], qh[R][1];
     uint32_t s8[R], s4[R], s2[R], s1[R], sh[R];
     auto load_tails = [&](uint32_t r0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+            const uint32_t row = row_of(r, r0);
+            const WView<PACKED> &wv = view_of(r);
             if constexpr (T8) {
                 wv.template load_quants<8, true>(row, c8 + lane * 8u, q8[r]);
                 s8[r] = wv.scale_bits(row, (c8 + lane * 8u) >> 5);
@@ -675,14 +685,14 @@ __device__ __forceinline__ float glu_act(float g, float u, uint32_t kind) {
     return 0.5f * g * (1.0f + tanhf(inner)) * u;
 }
 
-template <bool XA, class XS>
+template <bool XA, int TAILMASK, class XS>
 __device__ __forceinline__ void stream_rows_glu(const WView<PACKED> &wg, const WView<PACKED> &wu,
                                                 const XS xs, float *gate_out, float *up_out,
                                                 float *out, uint32_t kind, uint32_t cols,
                                                 uint32_t row_first, uint32_t row_end,
                                                 uint32_t lane) {
     constexpr int R = 8;
-    stream_rows_to<R, XA, 0>(
+    stream_rows_to<R, XA, TAILMASK>(
         PairRows{wg, wu}, xs, cols, row_first, row_end, lane,
         [&](const float (&acc)[R], uint32_t r0) {
             // the butterfly of reduce_store<8>: same operands per addition
@@ -776,6 +786,7 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
                 inv = 1.0f / sqrtf(sumsq / (float)cols + args.norm_eps);
             }
             const NormedX xn{args.norm_h, args.norm_w, inv};
+            const uint32_t tail = cols & 1023u; // 0, or (TAILS == 1) 128: the host fuses nothing else
             if ((d.pad & GEMV_WRITES_NORM) && tile == d.tile_begin) {
                 for (uint32_t c = 0; c < full; ++c) {
                     float o[16];
@@ -786,24 +797,47 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
                         dst[i] = make_float4(o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]);
                     }
                 }
-            }
-            if (d.pad & GEMV_PAIR) {
-                // gate (this descriptor) and up (the next one, which owns no
-                // tiles; its `res` is the activation's output, its `alpha` the kind)
-                const GemvDesc &d2 = args.d[lo + 1];
-                const WView<PACKED> wu(d2.w, rows, cols);
-                const uint32_t kind = (uint32_t)d2.alpha;
-                if (d.pad & GEMV_X_NORMED) {
-                    stream_rows_glu<true>(wv, wu, xn, y, d2.y, d2.res, kind, cols, row_first,
-                                          row_end, lane);
-                } else {
-                    stream_rows_glu<true>(wv, wu, PlainX{x}, y, d2.y, d2.res, kind, cols, row_first,
-                                          row_end, lane);
+                if constexpr (TAILS == 1) {
+                    if (tail == 128u) {
+                        float o[2];
+                        xn.template loadn<2, true>(tail0 + lane * 2u, o);
+                        *(float2 *)(args.norm_out + tail0 + lane * 2u) = make_float2(o[0], o[1]);
+                    }
                 }
-            } else {
-                stream_rows<R, true, 0, NormedX>(wv, xn, y, cols, row_first, row_end, lane, d.res,
-                                                 d.alpha);
             }
+            // (a small product may be cut into shorter tiles, as below)
+#define Q8_NORMED_STREAM(TAILMASK)                                                               \
+    if (d.pad & GEMV_PAIR) {                                                                     \
+        /* gate (this descriptor) and up (the next one, which owns no tiles; its                 \
+           `res` is the activation's output, its `alpha` the kind) */                            \
+        const GemvDesc &d2 = args.d[lo + 1];                                                     \
+        const WView<PACKED> wu(d2.w, rows, cols);                                                \
+        const uint32_t kind = (uint32_t)d2.alpha;                                                \
+        if (d.pad & GEMV_X_NORMED) {                                                             \
+            stream_rows_glu<true, TAILMASK>(wv, wu, xn, y, d2.y, d2.res, kind, cols, row_first,  \
+                                            row_end, lane);                                      \
+        } else {                                                                                 \
+            stream_rows_glu<true, TAILMASK>(wv, wu, PlainX{x}, y, d2.y, d2.res, kind, cols,      \
+                                            row_first, row_end, lane);                           \
+        }                                                                                        \
+    } else if (d.rows_per_tile % (R / 2) != 0u) {                                                \
+        stream_rows<R / 4, true, TAILMASK, NormedX>(wv, xn, y, cols, row_first, row_end, lane,   \
+                                                    d.res, d.alpha);                             \
+    } else if (d.rows_per_tile % R != 0u) {                                                      \
+        stream_rows<R / 2, true, TAILMASK, NormedX>(wv, xn, y, cols, row_first, row_end, lane,   \
+                                                    d.res, d.alpha);                             \
+    } else {                                                                                     \
+        stream_rows<R, true, TAILMASK, NormedX>(wv, xn, y, cols, row_first, row_end, lane,       \
+                                                d.res, d.alpha);                                 \
+    }
+            if constexpr (TAILS == 1) {
+                if (tail == 128u) {
+                    Q8_NORMED_STREAM(128)
+                    return;
+                }
+            }
+            Q8_NORMED_STREAM(0)
+#undef Q8_NORMED_STREAM
             return;
         }
     }

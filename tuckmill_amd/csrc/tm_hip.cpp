@@ -649,8 +649,13 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &arg
             }
             if (norm) {
                 if constexpr (XA) {
-                    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, true, 0, q8::GEMV_FEW_DESCS, true>),
-                              dim3(groups), dim3(256), 0, ctx->stream, stop, few);
+                    if (tails == 1) {
+                        Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, true, 1, q8::GEMV_FEW_DESCS, true>),
+                                  dim3(groups), dim3(256), 0, ctx->stream, stop, few);
+                    } else {
+                        Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, true, 0, q8::GEMV_FEW_DESCS, true>),
+                                  dim3(groups), dim3(256), 0, ctx->stream, stop, few);
+                    }
                     return hipGetLastError();
                 }
                 return hipErrorInvalidValue;
@@ -669,8 +674,13 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &arg
         }
         if (norm) {
             if constexpr (XA) {
-                Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, true, 0, q8::GEMV_MAX_DESCS, true>),
-                          dim3(groups), dim3(256), 0, ctx->stream, stop, args);
+                if (tails == 1) {
+                    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, true, 1, q8::GEMV_MAX_DESCS, true>),
+                              dim3(groups), dim3(256), 0, ctx->stream, stop, args);
+                } else {
+                    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, true, 0, q8::GEMV_MAX_DESCS, true>),
+                              dim3(groups), dim3(256), 0, ctx->stream, stop, args);
+                }
                 return hipGetLastError();
             }
             return hipErrorInvalidValue;
@@ -1372,9 +1382,15 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             // whole output as their activations take it in without it going
             // through memory.
             const bool decode_kind = key.decode();
-            const bool normed = cur.norm != nullptr && decode_kind && op.a[1] == cur.norm->a[2] &&
-                                op.x_off == 0 && op.cols == cur.norm->cols;
-            if (cur.norm != nullptr && !decode_kind) {
+            // (Not into a large product: the kernel variant with the fused forms
+            // runs three waves per SIMD where the plain one runs four, which
+            // costs a vocabulary projection three times the launch it saves:
+            // 151936 x 1024 36.8 us with the norm inside against 24.5 + 3.9.)
+            const bool large = (uint64_t)op.rows * op.cols > (16ull << 20);
+            const bool normed = cur.norm != nullptr && decode_kind && !large &&
+                                op.a[1] == cur.norm->a[2] && op.x_off == 0 &&
+                                op.cols == cur.norm->cols;
+            if (cur.norm != nullptr && (!decode_kind || large)) {
                 flush();
             }
             // a[0] = w (read), a[1] = x (read), a[2] = y (written), a[3] =
@@ -1446,7 +1462,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 op.a[3]->write_epoch = epoch;
             }
         } else if (op.kind == OP_RMSNORM && op.rows == 1 && op.cols >= 1024u &&
-                   (op.cols & 1023u) == 0u && op.a[0] != op.a[2]) {
+                   ((op.cols & 1023u) == 0u || (op.cols & 1023u) == 128u) && op.a[0] != op.a[2]) {
             // One row in front of its consumers (the norm before q/k/v, before
             // gate/up, before the vocabulary projection): held back and fused
             // into the launch of the products that read it, if any follow.
@@ -1473,7 +1489,8 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 const bool shapes = pg->batch == 1 && pu->batch == 1 && pg->a[1] == pu->a[1] &&
                                     pg->x_off == pu->x_off && pg->rows == pu->rows &&
                                     pg->cols == pu->cols && pg->cols >= 1024u &&
-                                    (pg->cols & 1023u) == 0u && pg->y_off == 0 && pu->y_off == 0 &&
+                                    ((pg->cols & 1023u) == 0u || (pg->cols & 1023u) == 128u) &&
+                                    pg->y_off == 0 && pu->y_off == 0 &&
                                     op.extra == pg->rows;
                 const bool wiring = pg->a[2] == op.a[0] && pu->a[2] == op.a[1] &&
                                     pg->a[2] != pu->a[2] && out != pu->a[2];

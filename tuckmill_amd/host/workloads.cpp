@@ -25,7 +25,8 @@ enum {
     TMH_SILU_MUL = 6, // w = gate, x = up -> y
     TMH_AXPY = 7,     // y += x (alpha = 1), w unused (pass y)
     TMH_ARGMAX = 8,   // x -> y[0], w = 512 bytes of scratch
-    TMH_F16_GEMM = 9  // w holds rows*cols f16 values
+    TMH_F16_GEMM = 9, // w holds rows*cols f16 values
+    TMH_GELU_MUL = 10 // as TMH_SILU_MUL with ggml's tanh GELU
 };
 
 struct tmh_product {
@@ -62,6 +63,7 @@ static void issue(const HipContext &gpu, const tmh_product *p, const std::vector
         case TMH_QUANT: gpu.q8_0_quantize_act(x, y, q.cols, q.batch, 0); break;
         case TMH_RMSNORM: gpu.rmsnorm(x, w, y, q.rows, q.cols, 1e-6f); break;
         case TMH_SILU_MUL: gpu.silu_mul(w, x, y, q.cols); break;
+        case TMH_GELU_MUL: gpu.gelu_tanh_mul(w, x, y, q.cols); break;
         case TMH_AXPY: gpu.f32_axpy(x, y, 1.0f, q.cols); break;
         case TMH_ARGMAX: gpu.argmax_f32(x, q.cols, w, y, 0); break;
         case TMH_F16_GEMM: gpu.f16_gemm(w, x, y, q.rows, q.cols, q.batch, 0, 0); break;
