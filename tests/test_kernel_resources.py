@@ -14,8 +14,9 @@ import pytest
 
 from tuckmill_amd import build as B
 
-# gemv_list_kernel<PACKED, 8 rows, 1 token, aligned x, no tail set, any list capacity, no fused norm>
-DECODE_KERNEL = re.compile(r"Function Name: _ZN2q816gemv_list_kernelILi1ELi8ELi1ELb1ELi0ELi\d+ELb0EEE")
+# gemv_list_kernel<PACKED, 8 rows, 1 token, aligned x, no tail set, any list capacity, no fused norm,
+# no steps of several chunks>
+DECODE_KERNEL = re.compile(r"Function Name: _ZN2q816gemv_list_kernelILi1ELi8ELi1ELb1ELi0ELi\d+ELb0ELb0EEE")
 
 
 @pytest.fixture(scope="module")
@@ -51,7 +52,7 @@ def test_decode_kernel_keeps_four_waves_per_simd(resource_remarks):
 
 
 # gemv_list_kernel<RAW, 8 rows, 1 token, ...>: one token over weights as uploaded
-RAW_DECODE_KERNEL = re.compile(r"Function Name: _ZN2q816gemv_list_kernelILi0ELi8ELi1ELb[01]ELi0ELi\d+ELb0EEE")
+RAW_DECODE_KERNEL = re.compile(r"Function Name: _ZN2q816gemv_list_kernelILi0ELi8ELi1ELb[01]ELi0ELi\d+ELb0ELb0EEE")
 
 
 def test_raw_decode_kernel_keeps_four_waves_per_simd(resource_remarks):
@@ -69,7 +70,7 @@ def test_raw_decode_kernel_keeps_four_waves_per_simd(resource_remarks):
 
 # the same with the Gemma column tails: a pass of eight 1152-column rows is staged whole
 RAW_DECODE_TAILS_KERNEL = re.compile(
-    r"Function Name: _ZN2q816gemv_list_kernelILi0ELi8ELi1ELb[01]ELi1ELi\d+ELb0EEE")
+    r"Function Name: _ZN2q816gemv_list_kernelILi0ELi8ELi1ELb[01]ELi1ELi\d+ELb0ELb0EEE")
 
 
 def test_raw_decode_kernel_with_column_tails_fits_three_workgroups_per_cu(resource_remarks):

@@ -429,6 +429,135 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs
                                     });
 }
 
+// stream_rows for passes of few rows under a long K (a small product cut into
+// short tiles, so that more waves share it): a step covers C chunks of the R
+// rows instead of one, which keeps R x C kilobytes per wave in flight where the
+// plain form would have R. Same arithmetic: a pass starts with its tail pieces
+// and adds the chunks in ascending order; a last, shorter group of chunks
+// repeats its last chunk's loads and leaves the surplus out of the sums.
+template <int R, int C, bool XA, int TAILMASK, class XS = PlainX>
+__device__ __forceinline__ void stream_rows_wide(const WView<PACKED> &wv, const XS xs, float *y,
+                                                 uint32_t cols, uint32_t row_first,
+                                                 uint32_t row_end, uint32_t lane, float *res,
+                                                 float alpha) {
+    constexpr bool T8 = (TAILMASK & 512) != 0, T4 = (TAILMASK & 256) != 0;
+    constexpr bool T2 = (TAILMASK & 128) != 0;
+    static_assert((TAILMASK & 127) == 0, "the column tails with a streaming path");
+    const uint32_t full = cols >> 10;
+    const uint32_t groups = (full + (uint32_t)C - 1u) / (uint32_t)C;
+    const uint32_t c8 = full << 10;
+    const uint32_t c4 = c8 + (T8 ? 512u : 0u);
+    const uint32_t c2 = c4 + (T4 ? 256u : 0u);
+    auto row_of = [&](int r, uint32_t r0) {
+        return r0 + (uint32_t)r < row_end ? r0 + (uint32_t)r : row_end - 1u;
+    };
+    float x8[8], x4[4], x2[2];
+    if constexpr (T8) xs.template loadn<8, XA>(c8 + lane * 8u, x8);
+    if constexpr (T4) xs.template loadn<4, XA>(c4 + lane * 4u, x4);
+    if constexpr (T2) xs.template loadn<2, XA>(c2 + lane * 2u, x2);
+    uint32_t q8[R][2], q4[R][1], q2[R][1];
+    uint32_t s8[R], s4[R], s2[R];
+    auto load_tails = [&](uint32_t r0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t row = row_of(r, r0);
+            if constexpr (T8) {
+                wv.template load_quants<8, true>(row, c8 + lane * 8u, q8[r]);
+                s8[r] = wv.scale_bits(row, (c8 + lane * 8u) >> 5);
+            }
+            if constexpr (T4) {
+                wv.template load_quants<4, true>(row, c4 + lane * 4u, q4[r]);
+                s4[r] = wv.scale_bits(row, (c4 + lane * 4u) >> 5);
+            }
+            if constexpr (T2) {
+                wv.template load_quants<2, true>(row, c2 + lane * 2u, q2[r]);
+                s2[r] = wv.scale_bits(row, (c2 + lane * 2u) >> 5);
+            }
+        }
+    };
+    auto load_group = [&](uint32_t r0, uint32_t g, uint32_t (&qq)[R][C][4], uint32_t (&ss)[R][C]) {
+#pragma unroll
+        for (int cc = 0; cc < C; ++cc) {
+            const uint32_t want = g * (uint32_t)C + (uint32_t)cc;
+            const uint32_t c = want < full ? want : full - 1u;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const uint32_t row = row_of(r, r0);
+                wv.template load_quants<16, true>(row, (c << 10) + lane * 16u, qq[r][cc]);
+                ss[r][cc] = wv.scale_bits(row, (c << 5) + (lane >> 1));
+            }
+        }
+    };
+    const uint32_t nsteps = ((row_end - row_first + R - 1) / R) * groups;
+    uint32_t r0 = row_first, g = 0;
+    uint32_t q[R][C][4], sb[R][C];
+    if constexpr (TAILMASK != 0) {
+        load_tails(r0);
+    }
+    load_group(r0, 0, q, sb);
+    float acc[R];
+    for (uint32_t step = 0; step < nsteps; ++step) {
+        if (g == 0u) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float a = 0.0f;
+                if constexpr (T8) a = __builtin_fmaf(f16_bits_to_f32(s8[r]), piece_dot<8>(q8[r], x8), a);
+                if constexpr (T4) a = __builtin_fmaf(f16_bits_to_f32(s4[r]), piece_dot<4>(q4[r], x4), a);
+                if constexpr (T2) a = __builtin_fmaf(f16_bits_to_f32(s2[r]), piece_dot<2>(q2[r], x2), a);
+                acc[r] = a;
+            }
+        }
+        // this step's activations are requested before the next step's weights
+        float xv[C][16];
+#pragma unroll
+        for (int cc = 0; cc < C; ++cc) {
+            const uint32_t want = g * (uint32_t)C + (uint32_t)cc;
+            const uint32_t c = want < full ? want : full - 1u;
+            xs.template load16<XA>((c << 10) + lane * 16u, xv[cc]);
+        }
+        uint32_t gn = g + 1u, rn = r0;
+        if (gn == groups) {
+            gn = 0;
+            rn = r0 + (uint32_t)R;
+        }
+        uint32_t qn[R][C][4], sn[R][C];
+        if (step + 1u < nsteps) {
+            if constexpr (TAILMASK != 0) {
+                if (gn == 0u) {
+                    load_tails(rn);
+                }
+            }
+            load_group(rn, gn, qn, sn);
+        }
+#pragma unroll
+        for (int cc = 0; cc < C; ++cc) {
+            if (g * (uint32_t)C + (uint32_t)cc < full) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    acc[r] = __builtin_fmaf(f16_bits_to_f32(sb[r][cc]), piece_dot<16>(q[r][cc], xv[cc]),
+                                            acc[r]);
+                }
+            }
+        }
+        if (gn == 0u) {
+            reduce_store<R>(acc, y, r0, row_end, lane, true, res, alpha);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+            for (int cc = 0; cc < C; ++cc) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    q[r][cc][i] = qn[r][cc][i];
+                }
+                sb[r][cc] = sn[r][cc];
+            }
+        }
+        g = gn;
+        r0 = rn;
+    }
+}
+
 // One token over weights in the raw layout (34-byte blocks: f16 scale, 32
 // quants), rows of whole 1024-column chunks. A lane's 16 quants start 2 or 18
 // bytes into a block, at an even address: loaded from memory in that shape, a
@@ -740,7 +869,10 @@ __device__ __forceinline__ void stream_rows_glu(const WView<PACKED> &wg, const W
 // NORM: the launch carries fused forms, an RMSNorm in front of its products
 // and/or gate-up pairs with their activation (a separate instantiation, so that
 // the plain decode kernel keeps its register budget).
-template <int L, int R, int TB, bool XA, int TAILS = 0, int ND = GEMV_MAX_DESCS, bool NORM = false>
+// WIDE: short tiles under a long K take steps of several chunks
+// (stream_rows_wide; a separate instantiation for the same reason).
+template <int L, int R, int TB, bool XA, int TAILS = 0, int ND = GEMV_MAX_DESCS, bool NORM = false,
+          bool WIDE = false>
 __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -848,10 +980,25 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
         if (full >= 1u) {
             const uint32_t tail = cols & 1023u;
             if (tail == 0u) {
-                if (d.rows_per_tile % (R / 2) != 0u) { // a small product cut into shorter tiles
+                // a small product may be cut into shorter tiles
+                const bool quarter = d.rows_per_tile % (R / 2) != 0u;
+                const bool half = !quarter && d.rows_per_tile % R != 0u;
+                if constexpr (WIDE) {
+                    if (full >= 2u && quarter) {
+                        stream_rows_wide<R / 4, 4, XA, 0>(wv, PlainX{x}, y, cols, row_first, row_end,
+                                                          lane, d.res, d.alpha);
+                        return;
+                    }
+                    if (full >= 2u && half) {
+                        stream_rows_wide<R / 2, 2, XA, 0>(wv, PlainX{x}, y, cols, row_first, row_end,
+                                                          lane, d.res, d.alpha);
+                        return;
+                    }
+                }
+                if (quarter) {
                     stream_rows<R / 4, XA, 0>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
                                               d.res, d.alpha);
-                } else if (d.rows_per_tile % R != 0u) {
+                } else if (half) {
                     stream_rows<R / 2, XA, 0>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
                                               d.res, d.alpha);
                 } else {
@@ -879,8 +1026,13 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
             if constexpr (TAILS >= 1) {
                 if (tail == 768u) { // FFN 6912 (Gemma-3-1B); half the rows per pass
                     if (d.rows_per_tile % (R / 2) != 0u) {
-                        stream_rows<R / 4, XA, 768>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
-                                                    d.res, d.alpha);
+                        if constexpr (WIDE) {
+                            stream_rows_wide<R / 4, 4, XA, 768>(wv, PlainX{x}, y, cols, row_first,
+                                                                row_end, lane, d.res, d.alpha);
+                        } else {
+                            stream_rows<R / 4, XA, 768>(wv, PlainX{x}, y, cols, row_first, row_end,
+                                                        lane, d.res, d.alpha);
+                        }
                     } else {
                         stream_rows<R / 2, XA, 768>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
                                                     d.res, d.alpha);

@@ -631,7 +631,7 @@ inline unsigned strided_blocks_of(uint32_t n, uint32_t per) {
 
 template <int L, int R, int TB, bool XA>
 hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &args, int tails,
-                       bool fused) {
+                       bool fused, bool wide) {
     const uint32_t groups = (args.total_tiles + 3u) / 4u;
     if constexpr (L == q8::PACKED && TB == 1) {
         const bool norm = fused; // the planner only fuses into aligned launches of the decode kernel
@@ -660,7 +660,18 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &arg
                 }
                 return hipErrorInvalidValue;
             }
-            if (tails == 1) {
+            if (wide) { // short tiles under a long K: the instantiation with steps of several chunks
+                if (tails == 1) {
+                    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1, q8::GEMV_FEW_DESCS, false, true>),
+                              dim3(groups), dim3(256), 0, ctx->stream, stop, few);
+                } else if (tails == 2) {
+                    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 2, q8::GEMV_FEW_DESCS, false, true>),
+                              dim3(groups), dim3(256), 0, ctx->stream, stop, few);
+                } else {
+                    Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 0, q8::GEMV_FEW_DESCS, false, true>),
+                              dim3(groups), dim3(256), 0, ctx->stream, stop, few);
+                }
+            } else if (tails == 1) {
                 Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1, q8::GEMV_FEW_DESCS>), dim3(groups),
                           dim3(256), 0, ctx->stream, stop, few);
             } else if (tails == 2) {
@@ -961,6 +972,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     // which column tails with a streaming path of their own the products have:
     // 0 none, 1 128 columns (and maybe 768), 2 768 columns only
     int tails = 0;
+    bool wide = false; // some sealed product in short tiles has two chunks and more per row
     size_t at = 0; // the product's place in the launch's list (the fusions are recorded per product)
     for (const Op *op : ops) {
         const uint32_t tail = op->cols & 1023u;
@@ -1004,6 +1016,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
             if ((op->rows + R / 2 - 1) / (R / 2) < 512u) {
                 d.rows_per_tile = (uint32_t)R / 4u;
             }
+            wide = wide || (key.packed && op->cols >= 2048u);
         }
         d.pad = 0;
         const bool pair_first = launch.glu[at] != nullptr;
@@ -1066,7 +1079,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     if (key.packed == (P) && key.variant == ((T) == 1 ? V_DECODE : V_GENERAL) &&             \
         key.flag == (A)) {                                                                   \
         return launch_gemv<(P) ? q8::PACKED : q8::RAW, (T) == 1 ? kGemvR1 : kGemvR4, T, A>(  \
-            ctx, stop, args, tails, fused);                                                         \
+            ctx, stop, args, tails, fused, wide);                                                   \
     }
     TM_GEMV_CASE(true, 1, true)
     TM_GEMV_CASE(true, 1, false)
