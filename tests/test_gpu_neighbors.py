@@ -102,6 +102,10 @@ def test_argmax_matches_the_cpu_greedy_rule_exactly(ctx):
         v[ln - 1] = 2.0
         v[ln // 2] = 2.0
         cases.append(v)
+    for ln in (5, 6, 7, 70_003):  # the only maximum among the last n % 4 elements
+        v = np.ones(ln, np.float32)
+        v[ln - 1] = 3.0
+        cases.append(v)
     partial = ctx.buffer(H.ARGMAX_PARTIAL_BYTES)
     out = ctx.buffer(8)
     for c, x in enumerate(cases):

@@ -342,7 +342,23 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float *x, flo
     __shared__ uint32_t ti[4];
     float v = -__builtin_inff();
     uint32_t i = ARGMAX_NONE;
-    for (uint32_t k = blockIdx.x * 256u + threadIdx.x; k < n; k += ARGMAX_GROUPS * 256u) {
+    // (the rule is a total order on (value, index): any partition of the elements
+    // gives the same winner; four per lane and step, so that a vocabulary takes
+    // three or four dependent loads per lane, not sixteen)
+    const uint32_t n4 = n & ~3u;
+    for (uint32_t k = (blockIdx.x * 256u + threadIdx.x) * 4u; k < n4; k += ARGMAX_GROUPS * 1024u) {
+        const f32x4 q = *(const f32x4 *)(x + k);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float xv = q[e];
+            if (xv == xv && argmax_better(xv, k + (uint32_t)e, v, i)) {
+                v = xv;
+                i = k + (uint32_t)e;
+            }
+        }
+    }
+    if (blockIdx.x == 0u && threadIdx.x < n - n4) {
+        const uint32_t k = n4 + threadIdx.x;
         const float xv = x[k];
         if (xv == xv && argmax_better(xv, k, v, i)) {
             v = xv;
