@@ -584,14 +584,19 @@ CHAIN_MODELS = {
 }
 
 
-def bench_chain(host, ctx, steps, warmup, recorded=True, model="qwen"):
+def bench_chain(host, ctx, steps, warmup, recorded=True, model="qwen", tokens=1):
     """The decode step with its data dependencies: per layer rmsnorm -> q,k,v -> o ->
     residual -> rmsnorm -> gate,up -> silu_mul -> down -> residual, then final norm,
     lm_head and greedy argmax, Qwen3-0.6B shapes (or Gemma-3-1B's), one dispatch group per token
     (attention, RoPE and the KV cache are not part of this path: o reads q in place of
     the attention output, which has the same length and the same dependence). Products that do not depend on each other still share a launch (q,k,v and
     gate,up), everything else is ordered, so the step is bound by launch latency, not by
-    HBM: this is the figure a graph replay or wider fusion would have to beat."""
+    HBM: this is the figure a graph replay or wider fusion would have to beat.
+    `tokens` > 1: the same step over that many tokens with the exact small-batch GEMM
+    (`q8_0_gemm`), the shape of a speculative step that verifies a draft with the
+    decode arithmetic (crates/tuckcore/src/engine/metal.rs:2170-2192: two tokens);
+    the operators run over `tokens` rows, the argmax over the first row."""
+    T = int(tokens)
     model_name, hidden, qdim, kvdim, ffn, vocab, layers, act = CHAIN_MODELS[model]
     act_kind = TMH_SILU_MUL if act == "silu" else TMH_GELU_MUL
     keep, prods = [], []
@@ -608,39 +613,42 @@ def bench_chain(host, ctx, steps, warmup, recorded=True, model="qwen"):
         keep.append(m)
         return m
 
-    h, n, t = fbuf(hidden, 1), fbuf(hidden), fbuf(hidden)
-    q, k, v = fbuf(qdim), fbuf(kvdim), fbuf(kvdim)
-    gate, up = fbuf(ffn), fbuf(ffn)
-    logits, partial, token = fbuf(vocab), ctx.buffer(H.ARGMAX_PARTIAL_BYTES), ctx.buffer(8)
+    h, n, t = fbuf(T * hidden, 1), fbuf(T * hidden), fbuf(T * hidden)
+    q, k, v = fbuf(T * qdim), fbuf(T * kvdim), fbuf(T * kvdim)
+    gate, up = fbuf(T * ffn), fbuf(T * ffn)
+    logits, partial, token = fbuf(T * vocab), ctx.buffer(H.ARGMAX_PARTIAL_BYTES), ctx.buffer(8)
     keep += [partial, token]
     wbytes = 0
 
     def product(m, x, y, rows, cols):
         nonlocal wbytes
         wbytes += S.gemv_bytes(rows, cols)
-        prods.append(tmh_product(m.buf.raw, x.raw, y.raw, rows, cols, 1, TMH_GEMV))
+        prods.append(tmh_product(m.buf.raw, x.raw, y.raw, rows, cols, T,
+                                 TMH_GEMV if T == 1 else TMH_GEMM))
 
     for layer in range(layers):
         g1, g2 = fbuf(hidden, 100 + layer), fbuf(hidden, 200 + layer)
-        prods.append(tmh_product(g1.raw, h.raw, n.raw, 1, hidden, 1, TMH_RMSNORM))
+        prods.append(tmh_product(g1.raw, h.raw, n.raw, T, hidden, 1, TMH_RMSNORM))
         product(mat(qdim, hidden, 5000 + 7 * layer), n, q, qdim, hidden)
         product(mat(kvdim, hidden, 5001 + 7 * layer), n, k, kvdim, hidden)
         product(mat(kvdim, hidden, 5002 + 7 * layer), n, v, kvdim, hidden)
         product(mat(hidden, qdim, 5003 + 7 * layer), q, t, hidden, qdim)
-        prods.append(tmh_product(h.raw, t.raw, h.raw, 1, hidden, 1, TMH_AXPY))
-        prods.append(tmh_product(g2.raw, h.raw, n.raw, 1, hidden, 1, TMH_RMSNORM))
+        prods.append(tmh_product(h.raw, t.raw, h.raw, 1, T * hidden, 1, TMH_AXPY))
+        prods.append(tmh_product(g2.raw, h.raw, n.raw, T, hidden, 1, TMH_RMSNORM))
         product(mat(ffn, hidden, 5004 + 7 * layer), n, gate, ffn, hidden)
         product(mat(ffn, hidden, 5005 + 7 * layer), n, up, ffn, hidden)
-        prods.append(tmh_product(gate.raw, up.raw, gate.raw, 1, ffn, 1, act_kind))
+        prods.append(tmh_product(gate.raw, up.raw, gate.raw, 1, T * ffn, 1, act_kind))
         product(mat(hidden, ffn, 5006 + 7 * layer), gate, t, hidden, ffn)
-        prods.append(tmh_product(h.raw, t.raw, h.raw, 1, hidden, 1, TMH_AXPY))
+        prods.append(tmh_product(h.raw, t.raw, h.raw, 1, T * hidden, 1, TMH_AXPY))
     gf = fbuf(hidden, 999)
-    prods.append(tmh_product(gf.raw, h.raw, n.raw, 1, hidden, 1, TMH_RMSNORM))
+    prods.append(tmh_product(gf.raw, h.raw, n.raw, T, hidden, 1, TMH_RMSNORM))
     product(mat(vocab, hidden, 6000), n, logits, vocab, hidden)
     prods.append(tmh_product(partial.raw, logits.raw, token.raw, 1, vocab, 1, TMH_ARGMAX))
     ctx.fence()
     tg = run_steps(host, ctx, prods, warmup, steps, grouped=True)
-    out = {"workload": f"{model_name} decode step with data dependencies (no attention)",
+    out = {"workload": f"{model_name} decode step with data dependencies (no attention)" +
+                       (f", {T} tokens through the exact small-batch GEMM" if T > 1 else ""),
+           "tokens": T,
            "operators_per_step": len(prods), "algorithmic_bytes": wbytes,
            "grouped": {"us": tg.wall_ms / steps * 1e3, "gpu_us": tg.gpu_ms / steps * 1e3,
                        "launches_per_step": tg.launches / steps,
@@ -758,6 +766,9 @@ def main():
                     help="one commit per GEMV instead of one group per step")
     ap.add_argument("--model", choices=sorted(CHAIN_MODELS), default="qwen",
                     help="chain workload: whose shapes the dependent decode step has")
+    ap.add_argument("--tokens", type=int, default=1, choices=range(1, 33), metavar="1..32",
+                    help="chain workload: tokens per step (more than one: the exact small-batch "
+                         "GEMM, as a speculative step verifies its draft)")
     ap.add_argument("--unsealed", action="store_true",
                     help="decode workload: leave the weights in the layout they are uploaded in "
                          "(what a binding that never calls tm_hip_q8_0_pack runs on)")
@@ -781,7 +792,7 @@ def main():
     if args.workload != "decode":
         fn = {"gemma": bench_gemma, "sweep": bench_sweep, "chain": bench_chain,
               "f16": bench_f16, "layer": bench_layer}[args.workload]
-        extra = ({"recorded": not args.no_recorded, "model": args.model}
+        extra = ({"recorded": not args.no_recorded, "model": args.model, "tokens": args.tokens}
                  if args.workload == "chain" else {})
         print(json.dumps(fn(host, ctx, args.steps, args.warmup, **extra)), flush=True)
         ctx.close()
