@@ -347,6 +347,93 @@ def test_gated_activation_behind_gate_and_up_is_fused(ctx, act, in_place, with_n
     del wd
 
 
+@pytest.mark.parametrize("tokens", [2, 3, 4])
+@pytest.mark.parametrize("hidden,qdim,kvdim,ffn,act", [(1024, 2048, 1024, 3072, "silu"),   # Qwen3-0.6B
+                                                       (1152, 1024, 256, 6912, "gelu")])   # Gemma-3-1B
+def test_a_few_tokens_take_the_same_fusions_as_one(ctx, tokens, hidden, qdim, kvdim, ffn, act):
+    # A speculative step verifies [token, draft] with a small batch through the exact
+    # product (crates/tuckcore/src/engine/metal.rs:2170-2192). A whole layer at 2 to 4
+    # tokens: norm -> q, k, v -> o with its update -> norm -> gate, up -> activation ->
+    # down with its update. Grouped, every token is a descriptor of the one-token kernel
+    # and the operators ride along as they do for one token (4 launches for 12); every
+    # buffer must hold the bits of the separate run.
+    T = tokens
+    mats = {}
+    for i, (name, rows, cols) in enumerate([("q", qdim, hidden), ("k", kvdim, hidden),
+                                            ("v", kvdim, hidden), ("o", hidden, qdim),
+                                            ("gate", ffn, hidden), ("up", ffn, hidden),
+                                            ("down", hidden, ffn)]):
+        w = S.make_weights(rows, cols, 500 + i)
+        mats[name] = (w, rows, cols, weights_buffer(ctx, w, rows, cols, True))
+    h0 = S.make_activations(T * hidden, 510)
+    g1 = (0.5 + np.abs(S.make_activations(hidden, 511))).astype(np.float32)
+    g2 = (0.5 + np.abs(S.make_activations(hidden, 512))).astype(np.float32)
+    attn = S.make_activations(T * qdim, 513)
+    g1b, g2b, attnb = upload_new(ctx, g1), upload_new(ctx, g2), upload_new(ctx, attn)
+    runs = []
+    for grouped in (False, True):
+        hb = upload_new(ctx, h0)
+        nb, n2b, tb = (ctx.buffer(T * hidden * 4) for _ in range(3))
+        out = {k: ctx.buffer(T * mats[k][1] * 4) for k in ("q", "k", "v", "gate", "up")}
+        launches = ctx.kernel_launches()
+        if grouped:
+            ctx.begin_group()
+        ctx.rmsnorm(hb, g1b, nb, T, hidden, 1e-6)
+        for k in ("q", "k", "v"):
+            ctx.q8_0_gemm(mats[k][3], nb, out[k], mats[k][1], hidden, T)
+        ctx.q8_0_gemm(mats["o"][3], attnb, tb, hidden, qdim, T)
+        ctx.f32_axpy(tb, hb, 1.0, T * hidden)
+        ctx.rmsnorm(hb, g2b, n2b, T, hidden, 1e-6)
+        for k in ("gate", "up"):
+            ctx.q8_0_gemm(mats[k][3], n2b, out[k], mats[k][1], hidden, T)
+        (ctx.silu_mul if act == "silu" else ctx.gelu_tanh_mul)(out["gate"], out["up"], out["gate"],
+                                                               T * ffn)
+        ctx.q8_0_gemm(mats["down"][3], out["gate"], tb, hidden, ffn, T)
+        ctx.f32_axpy(tb, hb, 1.0, T * hidden)
+        if grouped:
+            ctx.end_group()
+        ctx.fence()
+        used = ctx.kernel_launches() - launches
+        assert used == (4 if grouped else 12), used
+        got = {k: out[k].download_f32(0, T * mats[k][1]).copy() for k in out}
+        got.update(n=nb.download_f32(0, T * hidden).copy(), n2=n2b.download_f32(0, T * hidden).copy(),
+                   h=hb.download_f32(0, T * hidden).copy(), t=tb.download_f32(0, T * hidden).copy())
+        runs.append(got)
+    for k in runs[0]:
+        assert np.array_equal(bits(runs[0][k]), bits(runs[1][k])), k
+    # and the separate run is the oracle's, token by token
+    for t in range(T):
+        n = O.rmsnorm(h0[t * hidden:(t + 1) * hidden], g1, 1e-6)
+        assert close(runs[1]["n"][t * hidden:(t + 1) * hidden], n)
+        q = O.gemv_q8_0_f32(mats["q"][0], qdim, hidden, runs[1]["n"][t * hidden:(t + 1) * hidden])
+        assert np.max(np.abs(runs[1]["q"][t * qdim:(t + 1) * qdim] - q)) <= 1e-5 * np.max(np.abs(q))
+
+
+def test_fusions_of_a_few_tokens_need_matching_token_counts(ctx):
+    # a norm over 2 rows in front of a product of 3 tokens over the same buffer: the
+    # product reads a third row that the norm does not write, nothing may be fused
+    hidden, rows = 1024, 256
+    w = S.make_weights(rows, hidden, 520)
+    wb = weights_buffer(ctx, w, rows, hidden, True)
+    h = S.make_activations(3 * hidden, 521)
+    g = (0.5 + np.abs(S.make_activations(hidden, 522))).astype(np.float32)
+    hb, gb = upload_new(ctx, h), upload_new(ctx, g)
+    nb, yb = upload_new(ctx, h), ctx.buffer(3 * rows * 4)
+    launches = ctx.kernel_launches()
+    ctx.begin_group()
+    ctx.rmsnorm(hb, gb, nb, 2, hidden, 1e-6)
+    ctx.q8_0_gemm(wb, nb, yb, rows, hidden, 3)
+    ctx.end_group()
+    ctx.fence()
+    assert ctx.kernel_launches() - launches == 2
+    x = nb.download_f32(0, 3 * hidden)
+    assert np.array_equal(bits(x[2 * hidden:]), bits(h[2 * hidden:]))
+    for t in range(3):
+        want = O.gemv_q8_0_f32(w, rows, hidden, x[t * hidden:(t + 1) * hidden])
+        got = yb.download_f32(0, 3 * rows)[t * rows:(t + 1) * rows]
+        assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
+
+
 def test_gated_activation_is_not_fused_when_out_is_the_up_buffer(ctx):
     hidden, ffn = 1024, 256
     wg, wu = S.make_weights(ffn, hidden, 411), S.make_weights(ffn, hidden, 412)

@@ -35,7 +35,7 @@ struct GemvDesc {
     // multiply then add, exactly what a separate axpy over y would compute.
     float *res;
     float alpha;
-    uint32_t pad2;
+    uint32_t pad2;         // the row of the launch's fused RMSNorm that this descriptor reads
 };
 
 // The list travels in the kernel-argument segment (read through the scalar
@@ -56,7 +56,9 @@ template <int ND> struct GemvArgsT {
     // At most one fused RMSNorm per launch (norm_w == nullptr: none):
     // n = h / sqrt(mean(h^2) + eps) * w over norm_cols elements, a multiple of
     // 1024; products flagged GEMV_X_NORMED read n without it going through
-    // memory, one of them also stores it to norm_out.
+    // memory, one of them also stores it to norm_out. A few tokens (rows of
+    // the norm) go as one descriptor per product and token, GemvDesc::pad2
+    // saying which row; one descriptor per row stores it.
     float norm_eps;
     uint32_t pad;
     const float *norm_h;
@@ -912,18 +914,22 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
         if (d.pad & (GEMV_X_NORMED | GEMV_PAIR)) {
             // Every wave recomputes the row's scale (a few hundred operations)
             // instead of waiting for a separate kernel to publish it.
+            // (d.pad2: which row of the norm this descriptor's token is, when a
+            // few tokens go through the launch as one descriptor each)
+            const float *norm_h = args.norm_h + (size_t)d.pad2 * cols;
+            float *norm_out = args.norm_out + (size_t)d.pad2 * cols;
             float inv = 0.0f;
             if (d.pad & GEMV_X_NORMED) {
-                const float sumsq = row_sumsq(args.norm_h, cols, lane);
+                const float sumsq = row_sumsq(norm_h, cols, lane);
                 inv = 1.0f / sqrtf(sumsq / (float)cols + args.norm_eps);
             }
-            const NormedX xn{args.norm_h, args.norm_w, inv};
+            const NormedX xn{norm_h, args.norm_w, inv};
             const uint32_t tail = cols & 1023u; // 0, or (TAILS == 1) 128: the host fuses nothing else
             if ((d.pad & GEMV_WRITES_NORM) && tile == d.tile_begin) {
                 for (uint32_t c = 0; c < full; ++c) {
                     float o[16];
                     xn.template load16<true>((c << 10) + lane * 16u, o);
-                    float4 *dst = (float4 *)(args.norm_out + (c << 10) + lane * 16u);
+                    float4 *dst = (float4 *)(norm_out + (c << 10) + lane * 16u);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         dst[i] = make_float4(o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]);
@@ -933,7 +939,7 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
                     if (tail == 128u) {
                         float o[2];
                         xn.template loadn<2, true>(tail0 + lane * 2u, o);
-                        *(float2 *)(args.norm_out + tail0 + lane * 2u) = make_float2(o[0], o[1]);
+                        *(float2 *)(norm_out + tail0 + lane * 2u) = make_float2(o[0], o[1]);
                     }
                 }
             }

@@ -474,6 +474,13 @@ struct GemvKey {
     }
     // one token, sealed weights, aligned activations: the kernel the planner's fusions target
     bool decode() const { return kind == OP_GEMV_LIST && variant == V_DECODE && packed && flag; }
+    // up to four tokens through the exact small-batch product, sealed weights,
+    // aligned activations: with a fusion such a launch goes to the one-token
+    // kernel, a descriptor per product and token
+    bool few_tokens() const {
+        return kind == OP_GEMV_LIST && variant == V_SPLIT && packed && flag && p0 == 1;
+    }
+    bool fusable() const { return decode() || few_tokens(); }
 };
 
 // Which prefill GEMMs over sealed weights run on the bf16 matrix cores: from 17
@@ -731,6 +738,11 @@ struct Launch {
     uint64_t bx3_split_tiles = 0, bx3_partial_floats = 0, bx3_xs_bytes = 0;
     int bx3_inputs = 0;
     uint32_t descs = 0; // descriptors the listed products take (token groups count one each)
+    uint32_t token_descs = 0; // the same at one descriptor per product and token
+    // A launch of GemvKey::few_tokens products with a fusion in it: it runs on
+    // the one-token kernel (which has the fused forms), one descriptor per
+    // product and token.
+    bool per_token = false;
     // V_BF16X3: bit i set = the launch's i-th distinct input (in list order)
     // arrives split already, written by the launch just before this one.
     uint32_t bx3_presplit = 0;
@@ -923,7 +935,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     args.norm_h = launch.norm != nullptr ? (const float *)launch.norm->a[0]->ptr : nullptr;
     args.norm_w = launch.norm != nullptr ? (const float *)launch.norm->a[1]->ptr : nullptr;
     args.norm_out = launch.norm != nullptr ? (float *)launch.norm->a[2]->ptr : nullptr;
-    bool norm_written = false;
+    uint32_t norm_written = 0; // bit t: a descriptor stores row t of the fused norm
     bool fused = launch.norm != nullptr; // the launch needs the kernel variant with fused forms
     const int R = key.variant == V_GENERAL ? kGemvR4 : kGemvR1;
     uint32_t tiles = 0;
@@ -949,8 +961,13 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     // 10.3 -> 6.6 and 10.2 -> 9.0). With more rows the weights read once per
     // token cost more than the waves bring (q,k,v at 4 tokens 4.8 -> 6.1 us; Gemma's,
     // 192 such workgroups, at 3 tokens 4.4 -> 7.4).
-    bool per_token = false;
-    if (small_split) {
+    // (A launch with one of the planner's fusions in it goes there whatever its
+    // size: those forms exist in that kernel only, and the dependent launch a
+    // fusion saves, about 4 us, is more than the difference.)
+    bool per_token = launch.per_token;
+    if (per_token) {
+        key.variant = V_DECODE;
+    } else if (small_split) {
         uint32_t max_batch = 0, descs = 0;
         uint64_t row_groups = 0;
         for (const Op *op : ops) {
@@ -973,25 +990,11 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     // 0 none, 1 128 columns (and maybe 768), 2 768 columns only
     int tails = 0;
     bool wide = false; // some sealed product in short tiles has two chunks and more per row
-    size_t at = 0; // the product's place in the launch's list (the fusions are recorded per product)
-    for (const Op *op : ops) {
+    // One descriptor: token group `grp` of the product at place `at` of the
+    // launch's list (the fusions are recorded per product).
+    auto emit = [&](size_t at, uint32_t grp, uint32_t groups, uint32_t group_tokens) {
+        const Op *op = ops[at];
         const uint32_t tail = op->cols & 1023u;
-        if (op->cols >= 1024u && tail == 128u) {
-            tails = 1;
-        } else if (op->cols >= 1024u && tail == 768u && tails == 0) {
-            tails = 2;
-        }
-        // The token-split kernel covers waves x tokens-per-wave tokens per
-        // descriptor: a larger batch goes as several descriptors over the same
-        // weights, each with its own rows of X and Y.
-        const uint32_t group_tokens = per_token                  ? 1u
-                                      : key.variant == V_SPLIT ? (uint32_t)key.p0 * key.p1
-                                                               : op->batch;
-        const uint32_t groups = per_token ? op->batch : split_token_groups(key, op->batch);
-        if (args.n + groups > (uint32_t)q8::GEMV_MAX_DESCS) {
-            return hipErrorInvalidValue;
-        }
-      for (uint32_t grp = 0; grp < groups; ++grp) {
         q8::GemvDesc &d = args.d[args.n++];
         d.w = (const uint8_t *)op->a[0]->ptr;
         d.x = (const float *)op->a[1]->ptr + op->x_off + (size_t)grp * group_tokens * op->cols;
@@ -1026,24 +1029,58 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
             d.pad |= q8::GEMV_PAIR;
             fused = true;
         }
+        // (with a fusion in the launch a descriptor is one token: grp is the
+        // token, the row of the norm, of the residual and of the activation)
+        d.pad2 = 0;
         if (launch.norm != nullptr && launch.normed[at]) {
-            d.x = args.norm_h; // not read through: the kernel normalises norm_h itself
-            d.pad |= q8::GEMV_X_NORMED | (norm_written ? 0u : q8::GEMV_WRITES_NORM);
-            norm_written = true;
+            d.x = args.norm_h; // not read through: the kernel normalises its row of norm_h itself
+            d.pad2 = grp;
+            d.pad |= q8::GEMV_X_NORMED |
+                     ((norm_written >> grp) & 1u ? 0u : q8::GEMV_WRITES_NORM);
+            norm_written |= 1u << grp;
         }
         const Op *update = residual[at];
-        d.res = update != nullptr ? (float *)update->a[1]->ptr : nullptr;
+        d.res = update != nullptr ? (float *)update->a[1]->ptr + (size_t)grp * op->rows : nullptr;
         d.alpha = update != nullptr ? update->scalar : 0.0f;
-        d.pad2 = 0;
         if (pair_second) { // owns no tiles; carries the activation's output and kind
             const Op *act = launch.glu[at - 1];
-            d.res = (float *)act->a[2]->ptr;
+            d.res = (float *)act->a[2]->ptr + (size_t)grp * op->rows;
             d.alpha = act->kind == OP_GELU_MUL ? 1.0f : 0.0f;
         } else {
             tiles += (op->rows + d.rows_per_tile - 1) / d.rows_per_tile;
         }
-      }
-        ++at;
+    };
+    for (size_t at = 0; at < ops.size(); ++at) {
+        const Op *op = ops[at];
+        const uint32_t tail = op->cols & 1023u;
+        if (op->cols >= 1024u && tail == 128u) {
+            tails = 1;
+        } else if (op->cols >= 1024u && tail == 768u && tails == 0) {
+            tails = 2;
+        }
+        // The token-split kernel covers waves x tokens-per-wave tokens per
+        // descriptor: a larger batch goes as several descriptors over the same
+        // weights, each with its own rows of X and Y.
+        const uint32_t group_tokens = per_token                  ? 1u
+                                      : key.variant == V_SPLIT ? (uint32_t)key.p0 * key.p1
+                                                               : op->batch;
+        const uint32_t groups = per_token ? op->batch : split_token_groups(key, op->batch);
+        if (args.n + groups > (uint32_t)q8::GEMV_MAX_DESCS) {
+            return hipErrorInvalidValue;
+        }
+        if (at > 0 && launch.glu[at - 1] != nullptr) {
+            continue; // the up projection of a fused pair: listed right behind its gate, below
+        }
+        const bool pair_first = launch.glu[at] != nullptr;
+        if (pair_first && args.n + 2u * groups > (uint32_t)q8::GEMV_MAX_DESCS) {
+            return hipErrorInvalidValue;
+        }
+        for (uint32_t grp = 0; grp < groups; ++grp) {
+            emit(at, grp, groups, group_tokens);
+            if (pair_first) {
+                emit(at + 1, grp, groups, group_tokens);
+            }
+        }
     }
     args.total_tiles = tiles;
 #define TM_SPLIT_CASE(P, W, T, A, TL)                                                        \
@@ -1394,7 +1431,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             // products may join its launch; the ones that read the norm's
             // whole output as their activations take it in without it going
             // through memory.
-            const bool decode_kind = key.decode();
+            const bool decode_kind = key.fusable();
             // (Not into a large product: the kernel variant with the fused forms
             // runs three waves per SIMD where the plain one runs four, which
             // costs a vocabulary projection three times the launch it saves:
@@ -1402,7 +1439,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             const bool large = (uint64_t)op.rows * op.cols > (16ull << 20);
             const bool normed = cur.norm != nullptr && decode_kind && !large &&
                                 op.a[1] == cur.norm->a[2] && op.x_off == 0 &&
-                                op.cols == cur.norm->cols;
+                                op.cols == cur.norm->cols && op.batch == cur.norm->rows;
             if (cur.norm != nullptr && (!decode_kind || large)) {
                 flush();
             }
@@ -1446,7 +1483,10 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                            cur.bx3_partial_floats + mine.partial_floats > kBx3MaxPartialFloats ||
                            (new_input && cur.bx3_inputs == q8::SPLIT_MAX_DESCS);
             }
-            const uint32_t need = split_token_groups(key, op.batch); // descriptors of this product
+            // descriptors of this product (behind a pending norm, or in a launch
+            // with a fusion already, a few tokens take one each)
+            const bool each_token = key.few_tokens() && (cur.per_token || cur.norm != nullptr);
+            const uint32_t need = each_token ? op.batch : split_token_groups(key, op.batch);
             if (open && (conflict || (!cur.list.empty() && !(key == cur.key)) ||
                          (int)(cur.descs + need) > cap)) {
                 flush();
@@ -1463,7 +1503,9 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             }
             const bool takes_norm = normed && cur.norm != nullptr; // still pending after a flush?
             cur.key = key;
-            cur.descs += need;
+            cur.per_token = cur.per_token || (key.few_tokens() && cur.norm != nullptr);
+            cur.descs += cur.per_token ? op.batch : split_token_groups(key, op.batch);
+            cur.token_descs += op.batch;
             cur.list.push_back(&op);
             cur.residual.push_back(nullptr);
             cur.glu.push_back(nullptr);
@@ -1474,11 +1516,12 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             if (op.a[3] != nullptr) {
                 op.a[3]->write_epoch = epoch;
             }
-        } else if (op.kind == OP_RMSNORM && op.rows == 1 && op.cols >= 1024u &&
+        } else if (op.kind == OP_RMSNORM && op.rows <= 4u && op.cols >= 1024u &&
                    ((op.cols & 1023u) == 0u || (op.cols & 1023u) == 128u) && op.a[0] != op.a[2]) {
-            // One row in front of its consumers (the norm before q/k/v, before
-            // gate/up, before the vocabulary projection): held back and fused
-            // into the launch of the products that read it, if any follow.
+            // One row (or the few of a speculative step) in front of its
+            // consumers (the norm before q/k/v, before gate/up, before the
+            // vocabulary projection): held back and fused into the launch of
+            // the products that read it, if any follow.
             flush();
             cur.norm = &op;
             op.a[0]->read_epoch = epoch;
@@ -1494,17 +1537,22 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             // consumes (same activations, same shape, decode kernel): both
             // rows of a pair are computed by one wave, which applies the
             // activation itself. `out` may be the gate buffer (in place).
+            // With up to four tokens all of this holds per token: the launch
+            // then takes a descriptor per product and token (Launch::per_token),
+            // if they fit the kernel's list.
+            const bool few_fit = cur.key.few_tokens() &&
+                                 cur.token_descs <= (uint32_t)q8::GEMV_MAX_DESCS;
             if ((op.kind == OP_SILU_MUL || op.kind == OP_GELU_MUL) && cur.list.size() >= 2 &&
-                cur.key.decode()) {
+                (cur.key.decode() || few_fit)) {
                 const size_t n = cur.list.size();
                 const Op *pg = cur.list[n - 2], *pu = cur.list[n - 1];
                 Alloc *out = op.a[2];
-                const bool shapes = pg->batch == 1 && pu->batch == 1 && pg->a[1] == pu->a[1] &&
+                const bool shapes = pg->batch == pu->batch && pg->a[1] == pu->a[1] &&
                                     pg->x_off == pu->x_off && pg->rows == pu->rows &&
                                     pg->cols == pu->cols && pg->cols >= 1024u &&
                                     ((pg->cols & 1023u) == 0u || (pg->cols & 1023u) == 128u) &&
                                     pg->y_off == 0 && pu->y_off == 0 &&
-                                    op.extra == pg->rows;
+                                    op.extra == (uint64_t)pg->rows * pg->batch;
                 const bool wiring = pg->a[2] == op.a[0] && pu->a[2] == op.a[1] &&
                                     pg->a[2] != pu->a[2] && out != pu->a[2];
                 const bool free_entries = cur.residual[n - 2] == nullptr &&
@@ -1517,6 +1565,10 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 if (shapes && wiring && free_entries && out_free) {
                     cur.glu[n - 2] = &op;
                     out->write_epoch = epoch;
+                    if (few_fit) {
+                        cur.per_token = true;
+                        cur.descs = cur.token_descs;
+                    }
                     continue;
                 }
             }
@@ -1525,12 +1577,17 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 Alloc *h = op.a[1];
                 const size_t n = cur.list.size();
                 const bool in_pair = cur.glu[n - 1] != nullptr || (n >= 2 && cur.glu[n - 2] != nullptr);
-                if (!in_pair && cur.residual.back() == nullptr && prod->batch == 1 &&
+                if (!in_pair && cur.residual.back() == nullptr && (prod->batch == 1 || few_fit) &&
                     prod->a[2] == op.a[0] &&
-                    prod->y_off == 0 && prod->rows == op.extra && h != op.a[0] &&
+                    prod->y_off == 0 && (uint64_t)prod->rows * prod->batch == op.extra &&
+                    h != op.a[0] &&
                     h->read_epoch != epoch && h->write_epoch != epoch) {
                     cur.residual.back() = &op;
                     h->write_epoch = epoch;
+                    if (few_fit) {
+                        cur.per_token = true;
+                        cur.descs = cur.token_descs;
+                    }
                     continue;
                 }
             }
