@@ -434,6 +434,28 @@ def test_fusions_of_a_few_tokens_need_matching_token_counts(ctx):
         assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
 
 
+def test_a_norm_over_a_few_rows_that_nobody_reads_still_runs(ctx):
+    hidden, rows, T = 2048, 64, 2
+    h = S.make_activations(T * hidden, 530)
+    g = (0.5 + np.abs(S.make_activations(hidden, 531))).astype(np.float32)
+    w = S.make_weights(rows, hidden, 532)
+    wb = weights_buffer(ctx, w, rows, hidden, True)
+    hb, gb = upload_new(ctx, h), upload_new(ctx, g)
+    nb, yb = ctx.buffer(T * hidden * 4), ctx.buffer(T * rows * 4)
+    ctx.begin_group()
+    ctx.rmsnorm(hb, gb, nb, T, hidden, 1e-5)
+    ctx.q8_0_gemm(wb, hb, yb, rows, hidden, T)  # reads h, not the norm's output
+    ctx.end_group()
+    ctx.fence()
+    for t in range(T):
+        ht = h[t * hidden:(t + 1) * hidden]
+        assert close(nb.download_f32(0, T * hidden)[t * hidden:(t + 1) * hidden],
+                     O.rmsnorm(ht, g, 1e-5))
+        want = O.gemv_q8_0_f32(w, rows, hidden, ht)
+        got = yb.download_f32(0, T * rows)[t * rows:(t + 1) * rows]
+        assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
+
+
 def test_gated_activation_is_not_fused_when_out_is_the_up_buffer(ctx):
     hidden, ffn = 1024, 256
     wg, wu = S.make_weights(ffn, hidden, 411), S.make_weights(ffn, hidden, 412)

@@ -1411,6 +1411,12 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 one.single = cur.norm;
                 plan.push_back(std::move(one));
                 cur.norm = nullptr;
+                // a few tokens stay one descriptor each only for a fusion that is left
+                bool other = false;
+                for (size_t i = 0; i < cur.list.size(); ++i) {
+                    other = other || cur.residual[i] != nullptr || cur.glu[i] != nullptr;
+                }
+                cur.per_token = cur.per_token && other;
             }
         }
         if (!cur.list.empty()) {
