@@ -116,3 +116,17 @@ def test_small_batch_gemm_keeps_two_waves_per_simd(resource_remarks):
         occupancy = int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", block).group(1))
         spill = int(re.search(r"VGPRs Spill: (\d+)", block).group(1))
         assert occupancy >= 2 and spill == 0, block
+
+
+def test_two_token_form_of_the_small_batch_gemm_fits_sixteen_workgroups_per_cu(resource_remarks):
+    """One wave with two tokens over sealed weights without column tails stages
+    half of a step's rows in LDS and loads the other half directly: 8 KB of LDS and
+    at most 128 registers, so that 16 one-wave workgroups (4 waves per SIMD) keep
+    128 KB per CU on their way instead of the 80 KB that 16 KB of LDS each allow."""
+    pattern = re.compile(r"Function Name: _ZN2q822gemm_split_list_kernelILi1ELi1ELi2ELb[01]ELb0EEE")
+    blocks = _blocks(resource_remarks, pattern)
+    assert len(blocks) == 2
+    for block in blocks:
+        assert int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", block).group(1)) >= 4, block
+        assert int(re.search(r"LDS Size \[bytes/block\]: (\d+)", block).group(1)) == 8192, block
+        assert int(re.search(r"VGPRs Spill: (\d+)", block).group(1)) == 0, block

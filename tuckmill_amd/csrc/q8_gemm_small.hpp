@@ -45,11 +45,25 @@ template <int L, int NW, int TW, bool XA, bool TAIL>
 __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvArgs args) {
     constexpr int R = SMALL_R;
     constexpr uint32_t ROWB = L == PACKED ? 1024u : RAW_CHUNK_BYTES; // a staged row
+    // One wave with two tokens (the big launches of a two-token step) is short of
+    // bytes in flight, not of registers: with all 8 rows of a step in LDS, LDS
+    // holds 10 workgroups per CU, 80 KB on their way at any time, where the
+    // one-token kernel has 128 KB. Half of the rows of a step then travel
+    // through registers instead (SR rows staged, R - SR loaded by the lanes
+    // directly), which halves the workgroup's LDS and lets 16 of them run: 128 KB
+    // on their way, 127 registers (2 B-class shapes, 535 MB at two tokens:
+    // 113 -> 105 us). With four tokens per wave the same (6 rows staged, 163
+    // registers, 96 KB) gains nothing measurable: that form waits for its
+    // multiply-adds, and keeps all rows in LDS. The column-tail variant
+    // would fall to two waves per SIMD.
+    constexpr bool HYBRID = NW == 1 && TW == 2 && L == PACKED && !TAIL;
+    constexpr int SR = HYBRID ? R / 2 : R; // rows of a step that go through LDS
+    constexpr int DR = HYBRID ? R - SR : 1; // rows of a step loaded directly (1: unused)
     // Two separate objects (not one array indexed by parity): the compiler then
     // sees that reads of one buffer cannot alias the fetch into the other and
     // does not wait for the prefetch before reading.
-    __shared__ __attribute__((aligned(16))) uint8_t stage_a[R * ROWB];
-    __shared__ __attribute__((aligned(16))) uint8_t stage_b[R * ROWB];
+    __shared__ __attribute__((aligned(16))) uint8_t stage_a[SR * ROWB];
+    __shared__ __attribute__((aligned(16))) uint8_t stage_b[SR * ROWB];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t tile = blockIdx.x; // one tile per workgroup; the grid is exactly total_tiles
@@ -103,8 +117,8 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
         (void *)tile_q, 0, tile_len > 0xffffffffull ? 0xffffffffu : (uint32_t)tile_len, 0x00020000);
     auto fetch = [&](uint32_t r0, uint32_t c, uint8_t *stage) {
 #pragma unroll
-        for (int i = 0; i < R / NW; ++i) {
-            const uint32_t r = wave * (R / NW) + i;
+        for (int i = 0; i < SR / NW; ++i) {
+            const uint32_t r = wave * (SR / NW) + i;
             const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
             const uint32_t base =
                 __builtin_amdgcn_readfirstlane((row - row_first) * row_stride + c * ROWB);
@@ -119,6 +133,14 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
                         lane * 16u + 1024u, base, 0, 0);
                 }
             }
+        }
+    };
+    // (the rows of a step that do not go through LDS: rows SR .. R-1)
+    auto load_direct = [&](uint32_t r0, uint32_t c, uint32_t (&qq)[DR][4]) {
+#pragma unroll
+        for (int r = SR; r < R; ++r) {
+            const uint32_t row = (r0 + r < row_end) ? r0 + r : row_end - 1u;
+            wv.template load_quants<16, true>(row, (c << 10) + lane * 16u, qq[r - SR]);
         }
     };
     auto load_scales = [&](uint32_t r0, uint32_t c, uint32_t (&ss)[R]) {
@@ -136,7 +158,11 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
     const uint32_t raw_sel = raw_high ? 0x07060504u : 0x05040302u;
 
     uint32_t sb[R], sn[R];
+    uint32_t qd[DR][4], qdn[DR][4]; // this step's and the next one's direct rows
     fetch(row_first, 0, stage_a);
+    if constexpr (HYBRID) {
+        load_direct(row_first, 0, qd);
+    }
     load_scales(row_first, 0, sb);
     uint32_t r0 = row_first, c = 0;
     float acc[R][TW];
@@ -171,6 +197,9 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
         // would drain the prefetch too.
         const bool last = step + 1u == nsteps;
         fetch(last ? r0 : rn, last ? c : cn, nxt);
+        if constexpr (HYBRID) {
+            load_direct(last ? r0 : rn, last ? c : cn, qdn);
+        }
         load_scales(last ? r0 : rn, last ? c : cn, sn);
         if (has_tokens) {
             if (c == 0u) {
@@ -217,12 +246,22 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 uint32_t q[4];
+                if constexpr (HYBRID) {
+                    if (r >= SR) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            q[i] = qd[r - SR][i];
+                        }
+                    }
+                }
                 if constexpr (L == PACKED) {
-                    const uint4 qv = *(const uint4 *)(cur + r * ROWB + lane * 16u);
-                    q[0] = qv.x;
-                    q[1] = qv.y;
-                    q[2] = qv.z;
-                    q[3] = qv.w;
+                    if (r < SR) {
+                        const uint4 qv = *(const uint4 *)(cur + r * ROWB + lane * 16u);
+                        q[0] = qv.x;
+                        q[1] = qv.y;
+                        q[2] = qv.z;
+                        q[3] = qv.w;
+                    }
                 } else {
                     const uint32_t *w = (const uint32_t *)(cur + r * ROWB + (raw_off & ~3u));
                     const uint32_t d0 = w[0], d1 = w[1], d2 = w[2], d3 = w[3], d4 = w[4];
@@ -268,6 +307,15 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 sb[r] = sn[r];
+            }
+        }
+        if constexpr (HYBRID) {
+#pragma unroll
+            for (int r = 0; r < R - SR; ++r) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    qd[r][i] = qdn[r][i];
+                }
             }
         }
         c = cn;
