@@ -204,6 +204,39 @@ def test_residual_update_behind_its_product_shares_the_launch(ctx, packed):
     assert np.array_equal(bits(results[1][1]), bits(O.axpy(results[1][0], 0.5, h0)))
 
 
+@pytest.mark.parametrize("packed", [True, False])
+@pytest.mark.parametrize("batch", [5, 8, 20, 32])
+def test_residual_update_behind_a_small_batch_product_shares_the_launch(ctx, packed, batch):
+    # the same behind the exact small-batch product at more tokens than the one-token
+    # kernel takes: the token-split kernel has the same epilogue (20 tokens: two
+    # descriptors of up to 16, each updating its own rows of h)
+    rows, cols = 1024, 2048
+    w = S.make_weights(rows, cols, 96)
+    x = S.make_activations(batch * cols, 97)
+    h0 = S.make_activations(batch * rows, 98)
+    wb = weights_buffer(ctx, w, rows, cols, packed)
+    xb = upload_new(ctx, x)
+    results = []
+    for grouped in (False, True):
+        hb, tb = upload_new(ctx, h0), ctx.buffer(batch * rows * 4)
+        launches = ctx.kernel_launches()
+        if grouped:
+            ctx.begin_group()
+        ctx.q8_0_gemm(wb, xb, tb, rows, cols, batch)
+        ctx.f32_axpy(tb, hb, -0.25, batch * rows)
+        if grouped:
+            ctx.end_group()
+        ctx.fence()
+        assert ctx.kernel_launches() - launches == (1 if grouped else 2)
+        results.append((tb.download_f32(0, batch * rows).copy(),
+                        hb.download_f32(0, batch * rows).copy()))
+    assert np.array_equal(bits(results[0][0]), bits(results[1][0]))
+    assert np.array_equal(bits(results[0][1]), bits(results[1][1]))
+    assert np.array_equal(bits(results[1][1]), bits(O.axpy(results[1][0], -0.25, h0)))
+    t0 = O.gemv_q8_0_f32(w, rows, cols, x[:cols])
+    assert np.max(np.abs(results[1][0][:rows] - t0)) <= 1e-5 * np.max(np.abs(t0))
+
+
 def test_residual_update_is_not_fused_when_it_would_reorder_accesses(ctx):
     # h is also the product's input: the update must wait for the whole product.
     rows = cols = 1024

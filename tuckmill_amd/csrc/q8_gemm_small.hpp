@@ -298,8 +298,11 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
                     for (int r = 0; r < R; ++r) {
                         col_acc[r] = acc[r][t];
                     }
-                    reduce_store<R>(col_acc, y + (size_t)(wave * TW + t) * rows, r0, row_end, lane,
-                                    tok_ok[t]);
+                    // (an optional residual update of the token's row rides along,
+                    // as in the one-token kernel)
+                    const size_t token_off = (size_t)(wave * TW + t) * rows;
+                    reduce_store<R>(col_acc, y + token_off, r0, row_end, lane, tok_ok[t],
+                                    d.res != nullptr ? d.res + token_off : nullptr, d.alpha);
                 }
             }
         }

@@ -31,8 +31,9 @@ struct GemvDesc {
     uint32_t tile_begin;   // index of this product's first tile in the launch
     uint32_t rows_per_tile;
     uint32_t pad;
-    // Optional fused residual update (one token only): res[r] += alpha * y[r],
-    // multiply then add, exactly what a separate axpy over y would compute.
+    // Optional fused residual update: res[r] += alpha * y[r] (row r of every
+    // token of the descriptor, res laid out like y), multiply then add, exactly
+    // what a separate axpy over y would compute.
     float *res;
     float alpha;
     uint32_t pad2;         // the row of the launch's fused RMSNorm that this descriptor reads

@@ -1040,7 +1040,9 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
             norm_written |= 1u << grp;
         }
         const Op *update = residual[at];
-        d.res = update != nullptr ? (float *)update->a[1]->ptr + (size_t)grp * op->rows : nullptr;
+        d.res = update != nullptr
+                    ? (float *)update->a[1]->ptr + (size_t)grp * group_tokens * op->rows
+                    : nullptr;
         d.alpha = update != nullptr ? update->scalar : 0.0f;
         if (pair_second) { // owns no tiles; carries the activation's output and kind
             const Op *act = launch.glu[at - 1];
@@ -1583,7 +1585,10 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 Alloc *h = op.a[1];
                 const size_t n = cur.list.size();
                 const bool in_pair = cur.glu[n - 1] != nullptr || (n >= 2 && cur.glu[n - 2] != nullptr);
-                if (!in_pair && cur.residual.back() == nullptr && (prod->batch == 1 || few_fit) &&
+                // (the token-split kernel has the same epilogue: any batch it takes)
+                const bool split = cur.key.variant == V_SPLIT;
+                if (!in_pair && cur.residual.back() == nullptr &&
+                    (prod->batch == 1 || few_fit || split) &&
                     prod->a[2] == op.a[0] &&
                     prod->y_off == 0 && (uint64_t)prod->rows * prod->batch == op.extra &&
                     h != op.a[0] &&
