@@ -205,12 +205,14 @@ def test_residual_update_behind_its_product_shares_the_launch(ctx, packed):
 
 
 @pytest.mark.parametrize("packed", [True, False])
-@pytest.mark.parametrize("batch", [5, 8, 20, 32])
-def test_residual_update_behind_a_small_batch_product_shares_the_launch(ctx, packed, batch):
+@pytest.mark.parametrize("batch,rows", [(5, 1024), (8, 1024), (20, 1024), (32, 1024), (2, 2048),
+                                        (4, 1536)])
+def test_residual_update_behind_a_small_batch_product_shares_the_launch(ctx, packed, batch, rows):
     # the same behind the exact small-batch product at more tokens than the one-token
     # kernel takes: the token-split kernel has the same epilogue (20 tokens: two
-    # descriptors of up to 16, each updating its own rows of h)
-    rows, cols = 1024, 2048
+    # descriptors of up to 16, each updating its own rows of h; 2 and 4 tokens over
+    # enough rows stay on that kernel as well)
+    cols = 2048
     w = S.make_weights(rows, cols, 96)
     x = S.make_activations(batch * cols, 97)
     h0 = S.make_activations(batch * rows, 98)
@@ -487,6 +489,36 @@ def test_a_norm_over_a_few_rows_that_nobody_reads_still_runs(ctx):
         want = O.gemv_q8_0_f32(w, rows, hidden, ht)
         got = yb.download_f32(0, T * rows)[t * rows:(t + 1) * rows]
         assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
+
+
+def test_large_products_of_a_few_tokens_are_not_read_once_per_token(ctx):
+    # gate and up of more than 16 M weights each at 2 tokens: fused with their
+    # activation they would go through the one-token kernel, every token reading the
+    # weights again; they stay one launch of the token-split kernel, the activation
+    # behind them on its own.
+    rows, hidden, T = 16400, 1024, 2
+    wg, wu = S.make_weights(rows, hidden, 540), S.make_weights(rows, hidden, 541)
+    wgb, wub = weights_buffer(ctx, wg, rows, hidden, True), weights_buffer(ctx, wu, rows, hidden, True)
+    x = S.make_activations(T * hidden, 542)
+    xb = upload_new(ctx, x)
+    runs = []
+    for grouped in (False, True):
+        gb, ub = ctx.buffer(T * rows * 4), ctx.buffer(T * rows * 4)
+        launches = ctx.kernel_launches()
+        if grouped:
+            ctx.begin_group()
+        ctx.q8_0_gemm(wgb, xb, gb, rows, hidden, T)
+        ctx.q8_0_gemm(wub, xb, ub, rows, hidden, T)
+        ctx.silu_mul(gb, ub, gb, T * rows)
+        if grouped:
+            ctx.end_group()
+        ctx.fence()
+        assert ctx.kernel_launches() - launches == (2 if grouped else 3)
+        runs.append((gb.download_f32(0, T * rows).copy(), ub.download_f32(0, T * rows).copy()))
+    for a, b in zip(runs[0], runs[1]):
+        assert np.array_equal(bits(a), bits(b))
+    u = O.gemv_q8_0_f32(wu, rows, hidden, x[hidden:])
+    assert np.max(np.abs(runs[1][1][rows:] - u)) <= 1e-5 * np.max(np.abs(u))
 
 
 def test_gated_activation_is_not_fused_when_out_is_the_up_buffer(ctx):

@@ -739,9 +739,9 @@ struct Launch {
     int bx3_inputs = 0;
     uint32_t descs = 0; // descriptors the listed products take (token groups count one each)
     uint32_t token_descs = 0; // the same at one descriptor per product and token
-    // A launch of GemvKey::few_tokens products with a fusion in it: it runs on
-    // the one-token kernel (which has the fused forms), one descriptor per
-    // product and token.
+    // A launch of GemvKey::few_tokens products with a fused norm or gated
+    // activation in it: it runs on the one-token kernel (which has those forms),
+    // one descriptor per product and token.
     bool per_token = false;
     // V_BF16X3: bit i set = the launch's i-th distinct input (in list order)
     // arrives split already, written by the launch just before this one.
@@ -961,9 +961,10 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     // 10.3 -> 6.6 and 10.2 -> 9.0). With more rows the weights read once per
     // token cost more than the waves bring (q,k,v at 4 tokens 4.8 -> 6.1 us; Gemma's,
     // 192 such workgroups, at 3 tokens 4.4 -> 7.4).
-    // (A launch with one of the planner's fusions in it goes there whatever its
-    // size: those forms exist in that kernel only, and the dependent launch a
-    // fusion saves, about 4 us, is more than the difference.)
+    // (A launch with a fused norm or gated activation in it goes there whatever
+    // its row count: those forms exist in that kernel only, and the dependent
+    // launch a fusion saves, about 4 us, is more than the difference; the planner
+    // keeps products of more than 16 M weights out of such launches.)
     bool per_token = launch.per_token;
     if (per_token) {
         key.variant = V_DECODE;
@@ -1413,10 +1414,10 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 one.single = cur.norm;
                 plan.push_back(std::move(one));
                 cur.norm = nullptr;
-                // a few tokens stay one descriptor each only for a fusion that is left
+                // a few tokens stay one descriptor each only for a fusion that needs it
                 bool other = false;
                 for (size_t i = 0; i < cur.list.size(); ++i) {
-                    other = other || cur.residual[i] != nullptr || cur.glu[i] != nullptr;
+                    other = other || cur.glu[i] != nullptr;
                 }
                 cur.per_token = cur.per_token && other;
             }
@@ -1448,8 +1449,8 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
             const bool normed = cur.norm != nullptr && decode_kind && !large &&
                                 op.a[1] == cur.norm->a[2] && op.x_off == 0 &&
                                 op.cols == cur.norm->cols && op.batch == cur.norm->rows;
-            if (cur.norm != nullptr && (!decode_kind || large)) {
-                flush();
+            if ((cur.norm != nullptr && (!decode_kind || large)) || (cur.per_token && large)) {
+                flush(); // (a large product does not go a token at a time either)
             }
             // a[0] = w (read), a[1] = x (read), a[2] = y (written), a[3] =
             // optional second output: the product joins the open launch
@@ -1563,7 +1564,10 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                                     op.extra == (uint64_t)pg->rows * pg->batch;
                 const bool wiring = pg->a[2] == op.a[0] && pu->a[2] == op.a[1] &&
                                     pg->a[2] != pu->a[2] && out != pu->a[2];
-                const bool free_entries = cur.residual[n - 2] == nullptr &&
+                // (a few tokens: not with large products, which would then be read
+                // once per token; the same bound as for the norm)
+                const bool fits = !few_fit || (uint64_t)pg->rows * pg->cols <= (16ull << 20);
+                const bool free_entries = fits && cur.residual[n - 2] == nullptr &&
                                           cur.residual[n - 1] == nullptr &&
                                           cur.glu[n - 2] == nullptr && cur.glu[n - 1] == nullptr &&
                                           (n < 3 || cur.glu[n - 3] == nullptr) &&
@@ -1585,20 +1589,16 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 Alloc *h = op.a[1];
                 const size_t n = cur.list.size();
                 const bool in_pair = cur.glu[n - 1] != nullptr || (n >= 2 && cur.glu[n - 2] != nullptr);
-                // (the token-split kernel has the same epilogue: any batch it takes)
+                // (the token-split kernel has the same epilogue: any batch it takes;
+                // which of the two kernels a few tokens run on is decided at the launch)
                 const bool split = cur.key.variant == V_SPLIT;
-                if (!in_pair && cur.residual.back() == nullptr &&
-                    (prod->batch == 1 || few_fit || split) &&
+                if (!in_pair && cur.residual.back() == nullptr && (prod->batch == 1 || split) &&
                     prod->a[2] == op.a[0] &&
                     prod->y_off == 0 && (uint64_t)prod->rows * prod->batch == op.extra &&
                     h != op.a[0] &&
                     h->read_epoch != epoch && h->write_epoch != epoch) {
                     cur.residual.back() = &op;
                     h->write_epoch = epoch;
-                    if (few_fit) {
-                        cur.per_token = true;
-                        cur.descs = cur.token_descs;
-                    }
                     continue;
                 }
             }
