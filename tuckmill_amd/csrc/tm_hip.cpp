@@ -943,12 +943,19 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     for (const Op *op : ops) {
         launch_bytes += (uint64_t)op->rows * (op->cols / 32u) * 34u;
     }
-    const bool small_launch = launch_bytes < (16u << 20);
     // The token-split kernel in a launch that is all latency (the projections
     // of one layer between two dependent operators, a few tokens of a
     // speculative step): one pass of rows per workgroup, and the same tokens
     // over twice the waves. A token's result does not depend on either.
-    const bool small_split = key.variant == V_SPLIT && launch_bytes < (32u << 20);
+    // (the same for a larger launch that has few workgroups anyway, few rows
+    // under a long K: 4096 x 14336 at 8 tokens 42.5 -> 32.3 us)
+    uint64_t split_wgs = 0;
+    for (const Op *op : ops) {
+        const uint32_t rpt = pick_rows_per_tile(op->rows, op->cols, 32768u, R);
+        split_wgs += (uint64_t)split_token_groups(key, op->batch) * ((op->rows + rpt - 1) / rpt);
+    }
+    const bool small_split = key.variant == V_SPLIT &&
+                             (launch_bytes < (32u << 20) || split_wgs < 1024u);
     if (small_split && key.p1 == 4 && key.p0 <= 2) {
         key.p0 = (uint8_t)(key.p0 * 2);
         key.p1 = 2;
@@ -987,6 +994,12 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     const uint32_t tile_bytes = key.variant == V_SPLIT ? (small_split ? 8192u : 32768u)
                                 : (!key.packed && key.variant == V_DECODE) ? 16384u
                                                                            : 8192u;
+    // tiles the launch has at one pass of R rows per tile (a product of a few
+    // tokens that goes a token a descriptor counts once per token)
+    uint64_t full_tiles = 0;
+    for (const Op *op : ops) {
+        full_tiles += (uint64_t)(per_token ? op->batch : 1u) * ((op->rows + R - 1) / R);
+    }
     // which column tails with a streaming path of their own the products have:
     // 0 none, 1 128 columns (and maybe 768), 2 768 columns only
     int tails = 0;
@@ -1010,14 +1023,20 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
         const bool streams = tail == 0u || (op->cols >= 1024u && (tail == 128u || tail == 768u));
         const bool one_token = key.kind == OP_GEMV_LIST && key.variant == V_DECODE;
-        if (small_launch && one_token && d.rows_per_tile == (uint32_t)R && streams &&
-            (op->rows + R - 1) / R < 256u) {
-            // Fewer than 256 tiles even at one pass per wave, in a launch that
-            // is all latency (a projection of a few MB between two dependent
-            // operators): half-height tiles put twice as many waves on it.
-            // Inside a large launch full-height tiles stream better.
+        if (one_token && d.rows_per_tile == (uint32_t)R && streams && full_tiles < 1024u) {
+            // Fewer than 1024 tiles in the whole launch even at one pass per
+            // wave (a projection or two between two dependent operators, up to
+            // the 4096 x 14336 of an 8 B model): a wave a tile, that leaves
+            // three quarters of the chip's wave slots empty, and a tile is one
+            // long row pass with 8 KB in flight. Half- and quarter-height
+            // tiles put two and four times as many waves on it (quarter-height
+            // ones under a very long K only if the launch would otherwise stay
+            // under 1024 tiles: 4096 x 14336 runs better on 1024 tiles of 4
+            // rows). Lone 4096 x 4096: 8.2 -> 5.6 us, 4096 x 14336: 23.0 ->
+            // 13.9, 2048 x 8192: 11.6 -> 6.3. Inside a large launch full-height
+            // tiles stream better.
             d.rows_per_tile = (uint32_t)R / 2u;
-            if ((op->rows + R / 2 - 1) / (R / 2) < 512u) {
+            if (2u * full_tiles < (op->cols >= 8192u ? 1024u : 2048u)) {
                 d.rows_per_tile = (uint32_t)R / 4u;
             }
             wide = wide || (key.packed && op->cols >= 2048u);
