@@ -76,7 +76,11 @@ def test_batch_one_gemm_is_bit_identical_to_gemv(ctx):
                                              (100, 3072, 2), (33, 1024, 4), (4099, 6144, 16),
                                              (41, 6912, 9), (64, 1056, 3), (50, 2016, 5),
                                              (8, 1024, 17), (9, 4096, 31),
-                                             (70, 1152, 20), (41, 6912, 32), (33, 2016, 25)])
+                                             (70, 1152, 20), (41, 6912, 32), (33, 2016, 25),
+                                             # few rows under a long K, up to 4 tokens: steps of 4 rows
+                                             (1300, 3072, 2), (1301, 4224, 4), (2050, 6912, 6),
+                                             (1290, 3072, 7), (1283, 4096, 3), (4096, 4096, 8),
+                                             (1300, 2048, 2), (1290, 6912, 4)])
 def test_every_token_of_the_small_gemm_equals_its_own_gemv(ctx, rows, cols, batch, x_off):
     # Stronger than the reference's batch = 1 identity: the exact (speculative
     # verify) path must reproduce decode for every token. Covers every

@@ -41,9 +41,14 @@ constexpr int SMALL_R = 8; // rows per step
 // the bytes into place, and the block's scale comes out of the same bytes
 // (q8_gemv.hpp's stream_rows_raw has the details). The arithmetic is the sealed
 // form's.
-template <int L, int NW, int TW, bool XA, bool TAIL>
+//
+// R: rows per step, 8, or 4 for launches of few rows under a long K (a product
+// of 4096 x 14336 has 512 workgroups of 8 rows on 256 CUs, each with one step
+// of 8 KB on its way: with 4 rows a step it has 1024).
+template <int L, int NW, int TW, bool XA, bool TAIL, int R = SMALL_R>
 __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvArgs args) {
-    constexpr int R = SMALL_R;
+    static_assert(R == 8 || R == 4, "rows per step");
+    static_assert(R % NW == 0, "every wave fetches whole rows of a step");
     constexpr uint32_t ROWB = L == PACKED ? 1024u : RAW_CHUNK_BYTES; // a staged row
     // One wave with two tokens (the big launches of a two-token step) is short of
     // bytes in flight, not of registers: with all 8 rows of a step in LDS, LDS
@@ -56,7 +61,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_split_list_kernel(const GemvA
     // registers, 96 KB) gains nothing measurable: that form waits for its
     // multiply-adds, and keeps all rows in LDS. The column-tail variant
     // would fall to two waves per SIMD.
-    constexpr bool HYBRID = NW == 1 && TW == 2 && L == PACKED && !TAIL;
+    constexpr bool HYBRID = NW == 1 && TW == 2 && L == PACKED && !TAIL && R == 8;
     constexpr int SR = HYBRID ? R / 2 : R; // rows of a step that go through LDS
     constexpr int DR = HYBRID ? R - SR : 1; // rows of a step loaded directly (1: unused)
     // Two separate objects (not one array indexed by parity): the compiler then

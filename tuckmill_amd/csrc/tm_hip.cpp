@@ -988,6 +988,27 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
             key.variant = V_DECODE;
         }
     }
+    // The token-split kernel's step: 8 rows, or 4 where a launch of up to 4
+    // tokens over sealed weights has at most 512 workgroups of 8 rows and
+    // every row is long (3072 columns and more: the plain reduction of the
+    // 4-row form is paid once per row pass; 2048 x 2048 at 3 tokens 4.8 -> 5.6
+    // us with it). Few rows under a long K then get twice the workgroups, each
+    // with a step on its way: lone 4096 x 14336 at 2 / 4 tokens 20.2 / 29.1
+    // -> 16.4 / 19.7 us, 2048 x 8192 at 2 tokens 11.5 -> 8.6. (With more
+    // workgroups or tokens the 8-row step is ahead: 6144 x 4096 at 4 tokens 10.5
+    // against 12.4 us, 4096 x 4096 at 8 tokens 10.7 against 13.7.)
+    int split_rows = 8;
+    if (key.variant == V_SPLIT && small_split && key.packed && key.p1 == 2 && key.p0 <= 2) {
+        uint64_t wgs = 0;
+        uint32_t min_cols = 0xffffffffu;
+        for (const Op *op : ops) {
+            wgs += (uint64_t)split_token_groups(key, op->batch) * ((op->rows + 7u) / 8u);
+            min_cols = op->cols < min_cols ? op->cols : min_cols;
+        }
+        if (wgs <= 512u && min_cols >= 3072u) {
+            split_rows = 4;
+        }
+    }
     // a workgroup's tile in the token-split kernel, a wave's tile otherwise (one
     // token over raw weights: two passes per wave, so that the second pass's
     // loads fly while the first goes through LDS)
@@ -1020,7 +1041,8 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
                                       ? op->batch - grp * group_tokens
                                       : group_tokens);
         d.tile_begin = tiles;
-        d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes, R);
+        d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes,
+                                             key.variant == V_SPLIT ? split_rows : R);
         const bool streams = tail == 0u || (op->cols >= 1024u && (tail == 128u || tail == 768u));
         const bool one_token = key.kind == OP_GEMV_LIST && key.variant == V_DECODE;
         if (one_token && d.rows_per_tile == (uint32_t)R && streams && full_tiles < 1024u) {
@@ -1107,7 +1129,7 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     args.total_tiles = tiles;
 #define TM_SPLIT_CASE(P, W, T, A, TL)                                                        \
     if (key.variant == V_SPLIT && key.packed == (P) && key.p0 == (W) && key.p1 == (T) &&     \
-        key.p2 == ((TL) ? 1 : 0) && key.flag == (A)) {                                       \
+        key.p2 == ((TL) ? 1 : 0) && key.flag == (A) && split_rows == 8) {                    \
         Q8_LAUNCH((q8::gemm_split_list_kernel<(P) ? q8::PACKED : q8::RAW, W, T, A, TL>),     \
                   dim3(tiles), dim3((W) * 64), 0, ctx->stream, stop, args);                  \
         return hipGetLastError();                                                            \
@@ -1134,6 +1156,22 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
     TM_SPLIT_CASE(false, 4, 8, false, false)
 #undef TM_SPLIT_ALL
 #undef TM_SPLIT_CASE
+#define TM_SPLIT_ROWS4(W, A, TL)                                                             \
+    if (key.variant == V_SPLIT && key.packed && key.p0 == (W) && key.p1 == 2 &&              \
+        key.p2 == ((TL) ? 1 : 0) && key.flag == (A) && split_rows == 4) {                    \
+        Q8_LAUNCH((q8::gemm_split_list_kernel<q8::PACKED, W, 2, A, TL, 4>), dim3(tiles),     \
+                  dim3((W) * 64), 0, ctx->stream, stop, args);                               \
+        return hipGetLastError();                                                            \
+    }
+#define TM_SPLIT_ROWS4_ALL(W)                                                                \
+    TM_SPLIT_ROWS4(W, true, false)                                                           \
+    TM_SPLIT_ROWS4(W, false, false)                                                          \
+    TM_SPLIT_ROWS4(W, true, true)                                                            \
+    TM_SPLIT_ROWS4(W, false, true)
+    TM_SPLIT_ROWS4_ALL(1)
+    TM_SPLIT_ROWS4_ALL(2)
+#undef TM_SPLIT_ROWS4_ALL
+#undef TM_SPLIT_ROWS4
 #define TM_GEMV_CASE(P, T, A)                                                                \
     if (key.packed == (P) && key.variant == ((T) == 1 ? V_DECODE : V_GENERAL) &&             \
         key.flag == (A)) {                                                                   \
