@@ -221,20 +221,48 @@ struct NormedX {
 // Sum of squares of a row in the order every kernel that must agree uses: lane
 // l adds its elements 1024*c + 16*l + i sequentially (c, then i, ascending;
 // multiply, then add), the 64 partials go through q8::wave_sum.
+// The loads of four chunks are requested before the first of them is added up
+// (the additions keep their order): a row of 4096 waits for memory once, not
+// four times, which every wave of a launch with a fused norm does before it
+// streams anything. XA: h is 16-byte aligned.
+template <bool XA = false>
 __device__ __forceinline__ float row_sumsq(const float *h, uint32_t cols, uint32_t lane) {
     float acc = 0.0f;
-    for (uint32_t e0 = lane * 16u; e0 < cols; e0 += 1024u) {
-        if (e0 + 16u <= cols) {
-            float hv[16];
-            load_x<16, false>(h + e0, hv);
+    const uint32_t full = cols >> 10; // whole chunks: the same for every lane
+    uint32_t c = 0;
+    for (; c + 4u <= full; c += 4u) {
+        float hv[4][16];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            load_x<16, XA>(h + ((c + (uint32_t)j) << 10) + lane * 16u, hv[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                acc += hv[i] * hv[i];
+                acc += hv[j][i] * hv[j][i];
             }
-        } else {
-            for (uint32_t e = e0; e < cols; ++e) {
-                acc += h[e] * h[e];
-            }
+        }
+    }
+    for (; c < full; ++c) {
+        float hv[16];
+        load_x<16, XA>(h + (c << 10) + lane * 16u, hv);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            acc += hv[i] * hv[i];
+        }
+    }
+    const uint32_t e0 = (full << 10) + lane * 16u; // the lane's run in the last, partial chunk
+    if (e0 + 16u <= cols) {
+        float hv[16];
+        load_x<16, XA>(h + e0, hv);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            acc += hv[i] * hv[i];
+        }
+    } else {
+        for (uint32_t e = e0; e < cols; ++e) {
+            acc += h[e] * h[e];
         }
     }
     return wave_sum(acc);
@@ -923,7 +951,7 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
             float *norm_out = args.norm_out + (size_t)d.pad2 * cols;
             float inv = 0.0f;
             if (d.pad & GEMV_X_NORMED) {
-                const float sumsq = row_sumsq(norm_h, cols, lane);
+                const float sumsq = row_sumsq<true>(norm_h, cols, lane);
                 inv = 1.0f / sqrtf(sumsq / (float)cols + args.norm_eps);
             }
             const NormedX xn{norm_h, args.norm_w, inv};

@@ -234,11 +234,10 @@ __global__ __launch_bounds__(64 * RMSNORM_ROWS) void rmsnorm_kernel(float *x, co
             }
         }
     }
-    const float sumsq = row_sumsq(xr, cols, lane);
+    const float sumsq = vec ? row_sumsq<true>(xr, cols, lane) : row_sumsq<false>(xr, cols, lane);
     const float inv = 1.0f / sqrtf(sumsq / (float)cols + eps);
-    auto four = [&](uint32_t e) { // elements e .. e+3 of the row: normalise, store, split
-        const float4 xv = *(const float4 *)(xr + e);
-        const float4 wv = *(const float4 *)(weight + e);
+    // elements e .. e+3 of the row: normalise, store, split
+    auto four_of = [&](uint32_t e, const float4 xv, const float4 wv) {
         const float4 v = make_float4(xv.x * inv * wv.x, xv.y * inv * wv.y, xv.z * inv * wv.z,
                                      xv.w * inv * wv.w);
         *(float4 *)(yr + e) = v;
@@ -255,6 +254,9 @@ __global__ __launch_bounds__(64 * RMSNORM_ROWS) void rmsnorm_kernel(float *x, co
             *(uint2 *)(dst + piece) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
             *(uint2 *)(dst + 2u * piece) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
         }
+    };
+    auto four = [&](uint32_t e) {
+        four_of(e, *(const float4 *)(xr + e), *(const float4 *)(weight + e));
     };
     if (add != nullptr) {
         for (uint32_t e0 = lane * 16u; e0 < cols; e0 += 1024u) {
@@ -276,9 +278,26 @@ __global__ __launch_bounds__(64 * RMSNORM_ROWS) void rmsnorm_kernel(float *x, co
         return;
     }
     if (vec) {
-        // four consecutive elements per lane, a wave's 1 KiB in one piece
-        for (uint32_t e = lane * 4u; e < cols; e += 256u) {
-            four(e);
+        // four consecutive elements per lane, a wave's 1 KiB in one piece; the
+        // loads of four such pieces are requested together (a lane reads and
+        // writes its own elements only, in place too)
+        for (uint32_t e = lane * 4u; e < cols; e += 1024u) {
+            float4 xv[4], wv[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t ee = e + 256u * (uint32_t)j;
+                if (ee < cols) {
+                    xv[j] = *(const float4 *)(xr + ee);
+                    wv[j] = *(const float4 *)(weight + ee);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t ee = e + 256u * (uint32_t)j;
+                if (ee < cols) {
+                    four_of(ee, xv[j], wv[j]);
+                }
+            }
         }
         return;
     }
