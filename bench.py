@@ -581,6 +581,7 @@ def bench_f16(host, ctx, steps, warmup):
 CHAIN_MODELS = {
     "qwen": ("Qwen3-0.6B", 1024, 2048, 1024, 3072, 151_936, S.QWEN3_0_6B_LAYERS, "silu"),
     "gemma": ("Gemma-3-1B", 1152, 1024, 256, 6912, 262_144, 26, "gelu_tanh"),
+    "1.7b": ("Qwen3-1.7B", 2048, 2048, 1024, 6144, 151_936, 28, "silu"),
     # an 8 B-class model's widths (4096 hidden, 14336 FFN, grouped-query k/v of 1024), 8 of its
     # 32 layers so that the synthetic weights stay at 2.3 GB: launches of 18-125 MB each
     "8b": ("8B-class widths, 8 layers", 4096, 4096, 1024, 14336, 128_256, 8, "silu"),

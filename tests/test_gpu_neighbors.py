@@ -330,15 +330,17 @@ def test_a_norm_nobody_reads_still_runs(ctx):
     assert np.max(np.abs(yb.download_f32(0, 64) - want)) <= 1e-5 * np.max(np.abs(want))
 
 
-@pytest.mark.parametrize("hidden", [1024, 1152, 2048 + 128])
+@pytest.mark.parametrize("hidden,ffn", [(1024, 3072 + 8), (1152, 3072 + 8), (2048 + 128, 3072 + 6),
+                                        (1024, 8192 + 12)])
 @pytest.mark.parametrize("act,in_place,with_norm", [("silu", True, True), ("silu", False, False),
                                                     ("gelu", True, False), ("gelu", False, True)])
-def test_gated_activation_behind_gate_and_up_is_fused(ctx, act, in_place, with_norm, hidden):
+def test_gated_activation_behind_gate_and_up_is_fused(ctx, act, in_place, with_norm, hidden, ffn):
     # [norm ->] gate, up -> act(gate) * up -> down with its residual update: grouped,
     # one wave computes a row of gate and of up and applies the activation itself.
     # Every buffer must hold the bits of the separate operators. (Widths with a column
-    # tail of 128 behind the 1024-column chunks too: Gemma-3-1B's 1152.)
-    ffn = 3072 + 8  # a row count that leaves a partial last tile
+    # tail of 128 behind the 1024-column chunks too: Gemma-3-1B's 1152. Row counts that
+    # leave a partial last tile; few rows go in tiles of 2 rows of each matrix, 8204 rows
+    # in tiles of 4.)
     wg, wu = S.make_weights(ffn, hidden, 401), S.make_weights(ffn, hidden, 402)
     wd = S.make_weights(hidden, 1024 * 3, 403)
     wgb, wub = weights_buffer(ctx, wg, ffn, hidden, True), weights_buffer(ctx, wu, ffn, hidden, True)

@@ -847,6 +847,51 @@ __device__ __forceinline__ float glu_act(float g, float u, uint32_t kind) {
     return 0.5f * g * (1.0f + tanhf(inner)) * u;
 }
 
+// The same with passes of 2 gate rows and 2 up rows (a pair of few rows cut
+// into short tiles, so that more waves share it): acc = [g0, g1, u0, u1]; the
+// butterfly halves the values per lane at the shuffles over 32 and 16 lanes,
+// every addition with the two operands q8::wave_sum gives it.
+template <bool XA, int TAILMASK, class XS>
+__device__ __forceinline__ void stream_rows_glu_short(const WView<PACKED> &wg,
+                                                      const WView<PACKED> &wu, const XS xs,
+                                                      float *gate_out, float *up_out, float *out,
+                                                      uint32_t kind, uint32_t cols,
+                                                      uint32_t row_first, uint32_t row_end,
+                                                      uint32_t lane) {
+    constexpr int R = 4;
+    stream_rows_to<R, XA, TAILMASK>(
+        PairRows{wg, wu}, xs, cols, row_first, row_end, lane,
+        [&](const float (&acc)[R], uint32_t r0) {
+            float a2[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const float keep = (lane & 32u) ? acc[i + 2] : acc[i];
+                const float send = (lane & 32u) ? acc[i] : acc[i + 2];
+                a2[i] = keep + __shfl_xor(send, 32, WAVE);
+            }
+            const float keep = (lane & 16u) ? a2[1] : a2[0];
+            const float send = (lane & 16u) ? a2[0] : a2[1];
+            float a1 = keep + __shfl_xor(send, 16, WAVE);
+            a1 += __shfl_xor(a1, 8, WAVE);
+            a1 += __shfl_xor(a1, 4, WAVE);
+            a1 += __shfl_xor(a1, 2, WAVE);
+            a1 += __shfl_xor(a1, 1, WAVE);
+            const float other = __shfl_xor(a1, 32, WAVE);
+            const uint32_t row = r0 + ((lane >> 4) & 1u);
+            if ((lane & 15u) == 0u && row < row_end) {
+                if (lane & 32u) {
+                    up_out[row] = a1;
+                } else {
+                    const float act = glu_act(a1, other, kind);
+                    if (out != gate_out) {
+                        gate_out[row] = a1;
+                    }
+                    out[row] = act;
+                }
+            }
+        });
+}
+
 template <bool XA, int TAILMASK, class XS>
 __device__ __forceinline__ void stream_rows_glu(const WView<PACKED> &wg, const WView<PACKED> &wu,
                                                 const XS xs, float *gate_out, float *up_out,
@@ -982,9 +1027,19 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
         const GemvDesc &d2 = args.d[lo + 1];                                                     \
         const WView<PACKED> wu(d2.w, rows, cols);                                                \
         const uint32_t kind = (uint32_t)d2.alpha;                                                \
+        /* (tiles of 2 rows of each: the short form, for whole chunks only) */                   \
+        const bool short_pair = (TAILMASK) == 0 && d.rows_per_tile % 4u != 0u;                   \
         if (d.pad & GEMV_X_NORMED) {                                                             \
-            stream_rows_glu<true, TAILMASK>(wv, wu, xn, y, d2.y, d2.res, kind, cols, row_first,  \
-                                            row_end, lane);                                      \
+            if (short_pair) {                                                                    \
+                stream_rows_glu_short<true, TAILMASK>(wv, wu, xn, y, d2.y, d2.res, kind, cols,   \
+                                                      row_first, row_end, lane);                 \
+            } else {                                                                             \
+                stream_rows_glu<true, TAILMASK>(wv, wu, xn, y, d2.y, d2.res, kind, cols,         \
+                                                row_first, row_end, lane);                       \
+            }                                                                                    \
+        } else if (short_pair) {                                                                 \
+            stream_rows_glu_short<true, TAILMASK>(wv, wu, PlainX{x}, y, d2.y, d2.res, kind,      \
+                                                  cols, row_first, row_end, lane);               \
         } else {                                                                                 \
             stream_rows_glu<true, TAILMASK>(wv, wu, PlainX{x}, y, d2.y, d2.res, kind, cols,      \
                                             row_first, row_end, lane);                           \

@@ -1068,6 +1068,17 @@ hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &laun
         const bool pair_second = at > 0 && launch.glu[at - 1] != nullptr;
         if (pair_first) { // a tile covers the same rows of both matrices: half the rows each
             d.rows_per_tile = pick_rows_per_tile(op->rows, op->cols, tile_bytes / 2u, 4);
+            if (d.rows_per_tile == 4u && tail == 0u &&
+                (full_tiles < 1024u || (full_tiles < 2048u && op->cols >= 2048u))) {
+                // Few tiles in the launch: tiles of 2 rows of each matrix, as for
+                // single products (3072 x 1024 twice, 768 tiles: 6.0 -> 5.6 us;
+                // 6144 x 2048 twice, 1536 tiles: 11.6 -> 11.0). Short rows in
+                // more tiles lose instead: every wave pays the norm's sum and
+                // its share of the activations again (6912 x 1152 twice, 1728
+                // tiles: 8.9 -> 11.2 us). Whole chunks only: the instantiation with
+                // the 128-column tail is short of registers as it is.
+                d.rows_per_tile = 2u;
+            }
             d.pad |= q8::GEMV_PAIR;
             fused = true;
         }
