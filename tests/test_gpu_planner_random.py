@@ -22,8 +22,10 @@ from q8util import bits, require_gpu, upload_new, weights_buffer
 
 pytestmark = pytest.mark.gpu
 
-# Qwen3-0.6B's widths, and Gemma-3-1B's (column tails of 128 and 768 behind the 1024-column steps)
-DIMS = [(1024, 3072), (1152, 6912)]
+# Qwen3-0.6B's widths, Gemma-3-1B's (column tails of 128 and 768 behind the 1024-column steps)
+# and Qwen3-1.7B's (rows of 2048 and 6144 columns: short tiles in steps of several chunks,
+# the token-split kernel's 4-row steps, short gated pairs)
+DIMS = [(1024, 3072), (1152, 6912), (2048, 6144)]
 
 
 @pytest.fixture(scope="module")
