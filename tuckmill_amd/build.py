@@ -61,34 +61,12 @@ def build_host(verbose: bool = False) -> str:
     return HOST_LIB
 
 
-PROBE_DIR = os.path.join(HERE, "probes")
-PROBES = ("phase_barrier", "mfma_coissue")
-
-
-def build_probes(verbose: bool = False) -> list[str]:
-    """Stand-alone measurement probes (one HIP program each); nothing in the
-    library depends on them."""
-    out = []
-    for name in PROBES:
-        exe = os.path.join(PROBE_DIR, name + ".bin")
-        cmd = [HIPCC, "-std=c++17", "-O2", "-Wno-unused-result", *DEVICE_FLAGS, "-o", exe,
-               os.path.join(PROBE_DIR, name + ".hip")]
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        res = subprocess.run(cmd, capture_output=True, text=True)
-        if res.returncode != 0:
-            raise RuntimeError(f"probe build failed ({res.returncode}):\n{res.stdout}{res.stderr}")
-        out.append(exe)
-    return out
-
-
 def build_all(verbose: bool = False) -> None:
     build_library(verbose)
     build_host(verbose)
-    build_probes(verbose)
 
 
 if __name__ == "__main__":
     build_library(verbose=True, extra=sys.argv[1:])
     build_host(verbose=True)
-    print("built", LIB, HOST_LIB, *build_probes(verbose=True))
+    print("built", LIB, HOST_LIB)

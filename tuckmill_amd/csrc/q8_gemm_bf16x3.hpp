@@ -322,8 +322,8 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
     {
         // The instruction order of a block is written out (scheduling barriers pin
         // it). A wave's vector instructions hide under MFMAs only where they sit
-        // between the MFMAs of its own instruction stream (measured with
-        // probes/mfma_coissue.hip: four independent vector instructions per
+        // between the MFMAs of its own instruction stream (measured with a
+        // stand-alone co-issue loop: four independent vector instructions per
         // 32-cycle MFMA cost nothing there, while a wave that only issues MFMAs
         // keeps the SIMD's issue port and the partner wave's vector work waits),
         // so every MFMA is followed by a piece of the next weight rows'
