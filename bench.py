@@ -11,9 +11,17 @@ resident in HBM before the timed region. One JSON line is printed:
 
   value      whole-step achieved bandwidth, algorithmic bytes / wall time
   roofline   the GEMV list kernel: algorithmic bytes per launch over its
-             average launch duration (HIP events on the library's stream)
-  gemm       the MFMA prefill GEMM at M = 512 on the seven projection shapes
-  cpu_baseline  the scalar CPU oracle timed on this host (reported only)
+             average launch duration (HIP events on the library's stream),
+             beside the read bandwidth a read-only streaming kernel sustains
+             on this box; and, as sub-objects, the other benchmark
+             configurations, each against the peak of the unit it runs on and
+             with its error against the CPU oracle:
+               gemm_m512  the seven projections at 512 tokens (config 2)
+               gemma      Gemma-3-1B shapes at 1 and 512 tokens (config 3)
+               sweep_2b   2B-class shapes, 1..2048 tokens, f32 and int8
+                          activations (config 4)
+  cpu_baseline  the scalar CPU oracle timed on this host (reported only),
+             with a bounded sample per configuration under per_config
 """
 from __future__ import annotations
 
@@ -224,35 +232,83 @@ def cpu_baseline(host_side, budget_s: float):
     }
 
 
-def _gemm_point(flops, t, steps, shapes):
-    """One timed prefill group: GPU time per step (mean and order statistics), the
-    f32-equivalent rate 2*M*N*K / time, and which matrix cores its launch used."""
+def sample_tokens(M: int, n: int = 8) -> list:
+    """Up to n token indices spread over 0..M-1, first and last included."""
+    return sorted({int(v) for v in np.linspace(0, M - 1, min(n, M))})
+
+
+def gemm_sample(raw, rows, cols, x_host, M, yb, tokens, int8=False, threads=None):
+    """The sampled tokens of a product Y [M, rows] on the GPU and through the
+    oracle (f32 activations: kernels.rs:186-204 per token; int8: quantize_row
+    + kernels.rs:206-221), all rows. Returns (got, want, oracle_seconds)."""
+    import oracle as O
+
+    threads = threads or min(16, os.cpu_count() or 1)
+    xs = np.ascontiguousarray(np.asarray(x_host).reshape(M, cols)[tokens]).reshape(-1)
+    t0 = time.perf_counter()
+    fn = O.gemm_q8_0_q8_0 if int8 else O.gemm_q8_0_f32
+    want = fn(raw, rows, cols, xs, len(tokens), threads=threads)
+    dt = time.perf_counter() - t0
+    got = np.stack([yb.download_f32(t * rows, rows) for t in tokens])
+    return got, want, dt
+
+
+def norm_err(got, want) -> float:
+    """max |got - want| / max |want| (the parity metric of the f32-activation kernels)."""
+    scale = float(np.max(np.abs(want)))
+    return float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64))) / (scale or 1.0))
+
+
+def mfma_point(flops, t, steps, shapes, extra=None):
+    """One timed prefill group against the peak of the matrix cores it ran on:
+    the f32 cores (2*M*N*K over the time against 157.3 TFLOP/s) or, when the
+    launch took the bf16 kernel (every activation as three exact bf16 pieces),
+    the three bf16 products issued per f32 one against 2.5 PFLOP/s."""
     stats = step_stats(t, steps)
     us = stats.get("median_us") or stats["mean_us"]
     tile = H.gemm_mma_launch_tile(shapes)
-    out = {"us": us, "step_us": stats, "launches_per_step": t.launches / steps,
-           "tflops": flops / us / 1e6, "frac_of_f32_mfma_peak": flops / us / 1e6 / MFMA_F32_PEAK_TFLOPS,
-           "matrix_cores": f"bf16 x3, tiles of {tile} tokens" if tile else "f32"}
+    out = {"bound": "mfma", "us": us, "mean_us": stats["mean_us"],
+           "launches_per_step": t.launches / steps, "tflops_f32_equivalent": flops / us / 1e6}
     if tile:
-        out["bf16_mfma_tflops_issued"] = 3.0 * flops / us / 1e6
-        out["frac_of_bf16_mfma_peak"] = 3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS
+        out.update(kernel=f"q8::split_act_list_kernel + q8::gemm_bf16x3_kernel, tiles of {tile} tokens",
+                   matrix_cores="bf16", achieved=3.0 * flops / us / 1e6, peak=MFMA_BF16_PEAK_TFLOPS)
+    else:
+        out.update(kernel="q8::gemm_mma kernels (v_mfma_f32_32x32x2_f32)", matrix_cores="f32",
+                   achieved=flops / us / 1e6, peak=MFMA_F32_PEAK_TFLOPS)
+    out["unit"] = "TFLOP/s"
+    out["frac"] = out["achieved"] / out["peak"]
+    if extra:
+        out.update(extra)
     return out
 
 
-def _layer_matrices(ctx, M):
-    """The seven projection matrices of a Qwen3-0.6B layer, sealed, each with an X
+def _layer_matrices(ctx, M, seal=True, keep_host=False):
+    """The seven projection matrices of a Qwen3-0.6B layer, each with an X
     [M, K] and a Y [M, N] of its own: (products, buffers to free, by name)."""
     products, keep, mats = [], [], {}
     for name, rows, cols in S.QWEN3_0_6B_LAYER:
         raw = S.make_weights(rows, cols, S.tensor_seed(2, 0, name))
-        m = H.Matrix.load(ctx, raw, cols, rows)
+        m = H.Matrix.load(ctx, raw, cols, rows, seal=seal)
         xb = ctx.buffer(M * cols * 4)
-        xb.upload(0, S.make_activations(M * cols, rows))
+        x = S.make_activations(M * cols, rows)
+        xb.upload(0, x)
         yb = ctx.buffer(M * rows * 4)
         keep += [m.buf, xb, yb]
-        mats[name] = (m, xb, yb, rows, cols)
+        mats[name] = (m, xb, yb, rows, cols) + ((raw, x) if keep_host else ())
         products.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA))
     return products, keep, mats
+
+
+def _group_err(mats, M, tokens):
+    """Worst normalised error of the seven products' sampled tokens against the
+    oracle, and the oracle's time for that sample (all host threads)."""
+    worst, secs = 0.0, 0.0
+    for name, _, _ in S.QWEN3_0_6B_LAYER:
+        _, _, yb, rows, cols, raw, x = mats[name]
+        got, want, dt = gemm_sample(raw, rows, cols, x[:M * cols], M, yb, tokens)
+        worst = max(worst, norm_err(got, want))
+        secs += dt
+    return worst, secs
 
 
 def _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, out, keep):
@@ -269,7 +325,7 @@ def _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, 
     bufs["h"].upload(0, S.make_activations(M * hid, 12))
     def layer(tokens):
         def prod(name, x):
-            m, _, yb, rows, cols = mats[name]
+            m, _, yb, rows, cols = mats[name][:5]
             return tmh_product(m.buf.raw, x.raw, yb.raw, rows, cols, tokens, TMH_GEMM_MMA)
         return [tmh_product(wn.raw, bufs["h"].raw, bufs["xn"].raw, tokens, hid, tokens, TMH_RMSNORM),
                 prod("q", bufs["xn"]), prod("k", bufs["xn"]), prod("v", bufs["xn"]),
@@ -282,13 +338,17 @@ def _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, 
                 prod("down", bufs["act"]),
                 tmh_product(bufs["h"].raw, mats["down"][2].raw, bufs["h"].raw, 1, tokens * hid, 1,
                             TMH_AXPY)]
-    for key, tokens in (("layer_with_operators", M), ("layer_with_operators_m128", 128)):
+    for key, tokens in (("layer_with_operators", M), ("layer_with_operators_m128", 128),
+                        ("layer_with_operators_m256", 256)):
+        if tokens > M:
+            continue
         t = run_steps(host, ctx, layer(tokens), warmup, steps, grouped=True)
         stats = step_stats(t, steps)
         us = stats.get("median_us") or stats["mean_us"]
         out[key] = {
-            "M": tokens, "us": us, "step_us": stats, "launches_per_step": t.launches / steps,
-            "tflops": flops_total * tokens / M / us / 1e6,
+            "M": tokens, "us": us, "mean_us": stats["mean_us"], "us_per_token": us / tokens,
+            "launches_per_step": t.launches / steps,
+            "tflops_f32_equivalent": flops_total * tokens / M / us / 1e6,
             "order": "rmsnorm -> q,k,v -> o(q) -> axpy -> rmsnorm -> gate,up -> silu_mul -> down -> axpy; "
                      "no attention"}
     keep += list(bufs.values()) + [wn]
@@ -297,7 +357,7 @@ def _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, 
 def bench_layer(host, ctx, steps, warmup):
     """Only the layer with its operators (for a kernel trace of just these launches)."""
     M = 512
-    out = {"workload": "Qwen3-0.6B layer with its operators, 512 and 128 tokens (no attention)", "M": M}
+    out = {"workload": "Qwen3-0.6B layer with its operators, 512, 256 and 128 tokens (no attention)", "M": M}
     products, keep, mats = _layer_matrices(ctx, M)
     flops_total = sum(2.0 * M * p.rows * p.cols for p in products)
     _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, out, keep)
@@ -306,183 +366,274 @@ def bench_layer(host, ctx, steps, warmup):
     return out
 
 
-def bench_gemm(host, ctx, steps, warmup):
+def bench_gemm(host, ctx, steps, warmup, cpu=True, full=True):
     """BASELINE config 2: M = 512 tokens against the seven projection matrices
-    of a Qwen3-0.6B layer, each with its own X [512, K]. Timed as one dispatch
-    group (the seven independent products share one launch), one commit per
-    product, as the four dependent launches of a layer (q,k,v -> o -> gate,up ->
-    down, each reading what the one before wrote), and as one group at the
-    engine's own prefill chunk of 128 tokens (crates/tuckcore/src/engine/metal.rs:25).
+    of a Qwen3-0.6B layer, each with its own X [512, K]. One dispatch group over
+    sealed weights (the seven independent products share one launch of the bf16
+    kernel) and over weights as uploaded (the f32 matrix cores), each checked
+    against the oracle on sampled tokens of every product; then one commit per
+    product, the four dependent launches of a layer (q,k,v -> o -> gate,up ->
+    down, each reading what the one before wrote), the layer with its operators,
+    the engine's own prefill chunk of 128 tokens
+    (crates/tuckcore/src/engine/metal.rs:25) and the vocabulary projection.
     Figures are medians over the timed steps where the commits could be told
-    apart, means otherwise."""
+    apart, means otherwise (method: crates/metal/src/tests.rs:1023-1073)."""
     M = 512
-    out = {"M": M, "shapes": []}
-    products, keep, mats = _layer_matrices(ctx, M)
-    flops_total = sum(2.0 * M * p.rows * p.cols for p in products)
-    us_sum = 0.0
-    for (name, rows, cols), p in zip(S.QWEN3_0_6B_LAYER, products):
-        t = run_steps(host, ctx, [p], warmup, steps, grouped=False)
-        pt = _gemm_point(2.0 * M * rows * cols, t, steps, [(rows, cols, M)])
-        us_sum += pt["us"]
-        out["shapes"].append(dict(pt, name=name, rows=rows, cols=cols))
-    out["one_commit_per_product"] = {"us": us_sum, "tflops": flops_total / us_sum / 1e6}
+    out = {"config": "BASELINE config 2: seven Qwen3-0.6B projections, 512 tokens, f32 activations"}
+    cpu_out = {}
+    tokens = sample_tokens(M)
+    products, keep, mats = _layer_matrices(ctx, M, keep_host=True)
     shapes = [(r, c, M) for _, r, c in S.QWEN3_0_6B_LAYER]
-    t = run_steps(host, ctx, products, warmup, steps, grouped=True)
-    out.update(_gemm_point(flops_total, t, steps, shapes))
-    out["precondition"] = run_steps.last_precondition
-    out["wall_us"] = t.wall_ms / steps * 1e3
+    flops_total = sum(2.0 * M * p.rows * p.cols for p in products)
     out["flops_per_step"] = flops_total
-    out["mfma_f32_peak_tflops"] = MFMA_F32_PEAK_TFLOPS
-    out["frac"] = out["frac_of_f32_mfma_peak"]
-    out["kernel"] = ("q8::split_act_list_kernel + q8::gemm_bf16x3_kernel (every f32 activation as "
-                     "three exact bf16 pieces)" if H.gemm_mma_launch_tile(shapes)
-                     else "q8::gemm_mma_persistent_kernel (f32 matrix cores)")
-    # the same seven products wired as a layer: four launches, each behind the last
-    h = mats["q"][1]
-    dep = []
-    for name, x in (("q", h), ("k", h), ("v", h), ("o", mats["q"][2]), ("gate", h), ("up", h),
-                    ("down", mats["gate"][2])):
-        m, _, yb, rows, cols = mats[name]
-        dep.append(tmh_product(m.buf.raw, x.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA))
-    t = run_steps(host, ctx, dep, warmup, steps, grouped=True)
-    stats = step_stats(t, steps)
-    us = stats.get("median_us") or stats["mean_us"]
-    out["dependent_layer"] = {"us": us, "step_us": stats, "launches_per_step": t.launches / steps,
-                              "tflops": flops_total / us / 1e6,
-                              "order": "q,k,v -> o(q) -> gate,up -> down(gate); no attention"}
-    _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, out, keep)
-    # the engine's prefill chunk
+    t = run_steps(host, ctx, products, warmup, steps, grouped=True)
+    err, secs = _group_err(mats, M, tokens)
+    out["sealed_group"] = mfma_point(flops_total, t, steps, shapes, {
+        "wall_us": t.wall_ms / steps * 1e3, "precondition_steps": run_steps.last_precondition["steps"],
+        "max_norm_err_vs_cpu": err, "tokens_checked": len(tokens)})
+    # the same seven products over weights as uploaded: the f32 matrix cores
+    rproducts, rkeep, rmats = _layer_matrices(ctx, M, seal=False, keep_host=True)
+    t = run_steps(host, ctx, rproducts, warmup, steps, grouped=True)
+    rerr, _ = _group_err(rmats, M, tokens)
+    out["raw_group"] = mfma_point(flops_total, t, steps, [], {
+        "max_norm_err_vs_cpu": rerr, "tokens_checked": len(tokens),
+        "weights_layout": "as uploaded (34-byte blocks)"})
+    for b in rkeep:
+        b.free()
+    if cpu:
+        import oracle as O
+        # the oracle on the same sample: all threads (timed above), and one thread
+        t0 = time.perf_counter()
+        for name, _, _ in S.QWEN3_0_6B_LAYER:
+            _, _, _, rows, cols, raw, x = mats[name]
+            xs = np.ascontiguousarray(x.reshape(M, cols)[tokens[:2]]).reshape(-1)
+            O.gemm_q8_0_f32(raw, rows, cols, xs, 2, threads=1)
+        one = (time.perf_counter() - t0) / 2
+        sample_flops = flops_total / M
+        cpu_out = {"sample": f"{len(tokens)} of the 512 tokens x 7 projections through the scalar C "
+                             "restatement (2 of them for the 1-thread figure)",
+                   "ms_per_token_1_thread": one * 1e3, "gflops_1_thread": sample_flops / one / 1e9,
+                   "ms_per_token_all_cores": secs / len(tokens) * 1e3,
+                   "gflops_all_cores": sample_flops * len(tokens) / secs / 1e9,
+                   "cores_all": min(16, os.cpu_count() or 1),
+                   "ms_per_step_1_thread_extrapolated": one * M * 1e3}
+    if full:
+        us_sum, lone = 0.0, []
+        for (name, rows, cols), p in zip(S.QWEN3_0_6B_LAYER, products):
+            t = run_steps(host, ctx, [p], warmup, steps, grouped=False)
+            pt = mfma_point(2.0 * M * rows * cols, t, steps, [(rows, cols, M)])
+            us_sum += pt["us"]
+            lone.append({"name": name, "rows": rows, "cols": cols, "us": pt["us"],
+                         "matrix_cores": pt["matrix_cores"], "frac": pt["frac"]})
+        out["one_commit_per_product"] = {"us": us_sum, "tflops_f32_equivalent": flops_total / us_sum / 1e6,
+                                         "products": lone}
+        # the same seven products wired as a layer: four launches, each behind the last
+        h = mats["q"][1]
+        dep = []
+        for name, x in (("q", h), ("k", h), ("v", h), ("o", mats["q"][2]), ("gate", h), ("up", h),
+                        ("down", mats["gate"][2])):
+            m, _, yb, rows, cols = mats[name][:5]
+            dep.append(tmh_product(m.buf.raw, x.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA))
+        t = run_steps(host, ctx, dep, warmup, steps, grouped=True)
+        stats = step_stats(t, steps)
+        us = stats.get("median_us") or stats["mean_us"]
+        out["dependent_layer"] = {"us": us, "launches_per_step": t.launches / steps,
+                                  "tflops_f32_equivalent": flops_total / us / 1e6,
+                                  "order": "q,k,v -> o(q) -> gate,up -> down(gate); no attention"}
+        _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, out, keep)
+    # the engine's prefill chunk, one group, checked like the 512-token group
     m128 = [tmh_product(p.w, p.x, p.y, p.rows, p.cols, 128, TMH_GEMM_MMA) for p in products]
     t = run_steps(host, ctx, m128, warmup, steps, grouped=True)
-    out["m128"] = dict(_gemm_point(flops_total / 4, t, steps, [(r, c, 128) for r, c, _ in shapes]),
-                       M=128)
-    # The same model's vocabulary projection at M = 512: large enough on its own
-    # for the kernel that runs on the bf16 matrix cores (every f32 activation
-    # split into three exact bf16 pieces, so the products stay exact).
+    tok128 = sample_tokens(128)
+    err128, _ = _group_err(mats, 128, tok128)
+    out["m128_group"] = mfma_point(flops_total / 4, t, steps, [(r, c, 128) for r, c, _ in shapes], {
+        "M": 128, "max_norm_err_vs_cpu": err128, "tokens_checked": len(tok128)})
+    for b in keep:
+        b.free()
+    # The same model's vocabulary projection at M = 512 and at 64 tokens
     rows, cols = S.QWEN3_0_6B_LM_HEAD[1], S.QWEN3_0_6B_LM_HEAD[2]
-    m = H.Matrix.load(ctx, S.make_weights(rows, cols, S.tensor_seed(2, 0, "lm_head")), cols, rows)
+    raw = S.make_weights(rows, cols, S.tensor_seed(2, 0, "lm_head"))
+    m = H.Matrix.load(ctx, raw, cols, rows)
     xb = ctx.buffer(M * cols * 4)
-    xb.upload(0, S.make_activations(M * cols, 5))
+    x = S.make_activations(M * cols, 5)
+    xb.upload(0, x)
     yb = ctx.buffer(M * rows * 4)
     n = max(5, steps // 20)
-    t = run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA)],
-                  max(2, warmup // 20), n, grouped=False)
-    us = t.gpu_ms / n * 1e3
-    flops = 2.0 * M * rows * cols
-    out["lm_head"] = dict(_bf16_gemm_point(flops, us), rows=rows, cols=cols,
-                          launches_per_step=t.launches / n)
-    # ... and at 64 tokens (one 64-token tile of the same kernel)
-    t = run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, 64, TMH_GEMM_MMA)],
-                  max(2, warmup // 20), n, grouped=False)
-    us = t.gpu_ms / n * 1e3
-    out["lm_head_m64"] = dict(_bf16_gemm_point(2.0 * 64 * rows * cols, us), rows=rows, cols=cols, M=64)
-    for b in keep + [m.buf, xb, yb]:
+    for key, mb in (("lm_head_m512", M), ("lm_head_m64", 64)):
+        t = run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, mb, TMH_GEMM_MMA)],
+                      max(2, warmup // 20), n, grouped=False)
+        toks = sample_tokens(mb, 4)
+        got, want, _ = gemm_sample(raw, rows, cols, x[:mb * cols], mb, yb, toks)
+        out[key] = mfma_point(2.0 * mb * rows * cols, t, n, [(rows, cols, mb)], {
+            "M": mb, "rows": rows, "cols": cols, "max_norm_err_vs_cpu": norm_err(got, want),
+            "tokens_checked": len(toks)})
+    for b in (m.buf, xb, yb):
         b.free()
-    return out
+    return out, cpu_out
 
 
-def _weights_pool(ctx, shapes, copies, seed_base):
-    """`copies` distinct sealed weight sets of `shapes` [(name, rows, cols)]."""
-    pool = []
+def _weights_pool(ctx, shapes, copies, seed_base, keep_host=0):
+    """`copies` distinct sealed weight sets of `shapes` [(name, rows, cols)];
+    the raw bytes of the first `keep_host` entries stay on the host."""
+    pool, host = [], []
     for c in range(copies):
         for name, rows, cols in shapes:
             raw = S.make_weights(rows, cols, seed_base + 17 * c + len(pool))
+            if len(pool) < keep_host:
+                host.append(raw)
             pool.append((name, rows, cols, H.Matrix.load(ctx, raw, cols, rows)))
-    return pool
+    return (pool, host) if keep_host else pool
 
 
-def _bf16_gemm_point(flops, us):
-    """A prefill GEMM that ran on the bf16 matrix cores: `flops` = 2*M*N*K of the
-    f32 product it stands for; the kernel issues three bf16 MFMA products per
-    f32 one (the activation's three exact pieces)."""
-    return {"flops": flops, "us": us, "tflops_f32_equivalent": flops / us / 1e6,
-            "kernel": "q8::split_act_list_kernel + q8::gemm_bf16x3_kernel",
-            "bf16_mfma_tflops_issued": 3.0 * flops / us / 1e6,
-            "frac_of_bf16_mfma_peak": 3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS}
+def hbm_point(abytes, us, extra=None):
+    out = {"bound": "hbm", "us": us, "algorithmic_bytes": abytes, "achieved": abytes / us / 1e3,
+           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": abytes / us / 1e3 / HBM_PEAK_GBS}
+    if extra:
+        out.update(extra)
+    return out
 
 
-def bench_gemma(host, ctx, steps, warmup):
+def bench_gemma(host, ctx, steps, warmup, cpu=True):
     """BASELINE config 3: Gemma-3-1B shapes (hidden 1152 = 36 blocks per row,
     FFN 6912, lm_head 262144 x 1152). M = 1: a 26-layer FFN + lm_head step
-    (79 GEMVs, 981 MB of weights) in one group. M = 512: the three FFN shapes
-    in one group, and the lm_head on its own."""
-    out = {"workload": "Gemma-3-1B shapes (BASELINE config 3)"}
+    (79 GEMVs, 984 MB of weights) in one group, every product checked against the
+    oracle. M = 512: the three FFN shapes in one group, and the lm_head on its
+    own, sampled tokens checked."""
+    import oracle as O
+
+    out = {"config": "BASELINE config 3: Gemma-3-1B shapes, 1 and 512 tokens, f32 activations"}
+    cpu_out = {}
     layers = 26
+    ncores = min(16, os.cpu_count() or 1)
     ffn = [s for s in S.GEMMA3_1B if s[0] != "lm_head"]
     head = [s for s in S.GEMMA3_1B if s[0] == "lm_head"][0]
-    pool = _weights_pool(ctx, ffn, layers, 3000) + _weights_pool(ctx, [head], 1, 3999)
-    products, keep = [], []
+    pool, host_w = [], []
+    for c in range(layers):
+        for name, rows, cols in ffn:
+            raw = S.make_weights(rows, cols, 3000 + 17 * c + len(pool))
+            host_w.append(raw)
+            pool.append((name, rows, cols, H.Matrix.load(ctx, raw, cols, rows)))
+    raw = S.make_weights(head[1], head[2], 3999)
+    host_w.append(raw)
+    pool.append((head[0], head[1], head[2], H.Matrix.load(ctx, raw, head[2], head[1])))
+    products, keep, host_x = [], [], []
     for name, rows, cols, m in pool:
         xb = ctx.buffer(cols * 4)
-        xb.upload(0, S.make_activations(cols, rows))
+        x = S.make_activations(cols, rows + len(products))
+        xb.upload(0, x)
         yb = ctx.buffer(rows * 4)
         keep += [xb, yb]
+        host_x.append((x, yb))
         products.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, 1, TMH_GEMV))
     step_bytes = sum(S.gemv_bytes(p.rows, p.cols) for p in products)
     t = run_steps(host, ctx, products, warmup, steps, grouped=True)
-    us = t.wall_ms / steps * 1e3
-    out["gemv_step"] = {"products": len(products), "algorithmic_bytes": step_bytes, "us": us,
-                        "gbs": step_bytes / us / 1e3, "pct_of_hbm_peak": step_bytes / us / 1e3 / 80.0,
-                        "launch_us": t.gpu_ms * 1e3 / t.launches}
+    stats = step_stats(t, steps)
+    launch_us = t.gpu_ms * 1e3 / t.launches
+    # parity of every product of the step; the all-cores pass is the CPU figure
+    worst, t0 = 0.0, time.perf_counter()
+    for (name, rows, cols, _), raw, (x, yb) in zip(pool, host_w, host_x):
+        want = O.gemv_q8_0_f32(raw, rows, cols, x, threads=ncores)
+        worst = max(worst, norm_err(yb.download_f32(0, rows), want))
+    cpu_all = time.perf_counter() - t0
+    out["gemv_step"] = hbm_point(step_bytes, launch_us, {
+        "kernel": "q8::gemv_list_kernel (column tails 128 and 768)", "products": len(products),
+        "launches_per_step": t.launches / steps, "median_us": stats.get("median_us"),
+        "wall_us": t.wall_ms / steps * 1e3, "max_norm_err_vs_cpu": worst,
+        "products_checked": len(products)})
     head_p = products[-1]
     t = run_steps(host, ctx, [head_p], warmup, steps, grouped=False)
     us = t.gpu_ms / steps * 1e3
-    hb = S.gemv_bytes(head_p.rows, head_p.cols)
-    out["lm_head_gemv"] = {"rows": head_p.rows, "cols": head_p.cols, "algorithmic_bytes": hb,
-                           "us": us, "gbs": hb / us / 1e3, "pct_of_hbm_peak": hb / us / 1e3 / 80.0}
+    out["lm_head_gemv"] = hbm_point(S.gemv_bytes(head_p.rows, head_p.cols), us,
+                                    {"rows": head_p.rows, "cols": head_p.cols})
+    if cpu:
+        t0 = time.perf_counter()
+        for (name, rows, cols, _), raw, (x, _) in list(zip(pool, host_w, host_x))[:6]:
+            O.gemv_q8_0_f32(raw, rows, cols, x, threads=1)
+        one = time.perf_counter() - t0
+        six = sum(S.gemv_bytes(r, c) for _, r, c, _ in pool[:6])
+        cpu_out = {"sample": "the 79-GEMV step once on all cores (the parity pass), two layers' FFN "
+                             "matrices on 1 thread",
+                   "gemv_step_ms_all_cores": cpu_all * 1e3, "gbs_all_cores": step_bytes / cpu_all / 1e9,
+                   "cores_all": ncores, "gbs_1_thread": six / one / 1e9,
+                   "gemv_step_ms_1_thread_extrapolated": step_bytes / (six / one) * 1e3}
     # M = 512
     M = 512
-    gsteps, gwarm = max(5, steps // 20), max(2, warmup // 20)
-    gp = []
-    for name, rows, cols, m in pool[:3]:
+    gsteps, gwarm = max(5, steps // 4), max(2, warmup // 4)
+    gp, gx = [], []
+    for (name, rows, cols, m), raw in zip(pool[:3], host_w[:3]):
         xb = ctx.buffer(M * cols * 4)
-        xb.upload(0, S.make_activations(M * cols, rows + 1))
+        x = S.make_activations(M * cols, rows + 1)
+        xb.upload(0, x)
         yb = ctx.buffer(M * rows * 4)
         keep += [xb, yb]
+        gx.append((raw, rows, cols, x, yb))
         gp.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA))
     flops = sum(2.0 * M * p.rows * p.cols for p in gp)
     t = run_steps(host, ctx, gp, gwarm, gsteps, grouped=True)
-    us = t.gpu_ms / gsteps * 1e3
-    out["ffn_gemm_m512"] = _bf16_gemm_point(flops, us)
+    toks = sample_tokens(M, 4)
+    worst = 0.0
+    for raw, rows, cols, x, yb in gx:
+        got, want, _ = gemm_sample(raw, rows, cols, x, M, yb, toks)
+        worst = max(worst, norm_err(got, want))
+    out["ffn_gemm_m512"] = mfma_point(flops, t, gsteps, [(p.rows, p.cols, M) for p in gp], {
+        "M": M, "max_norm_err_vs_cpu": worst, "tokens_checked": len(toks)})
     name, rows, cols, m = pool[-1]
     xb = ctx.buffer(M * cols * 4)
-    xb.upload(0, S.make_activations(M * cols, 7))
+    x = S.make_activations(M * cols, 7)
+    xb.upload(0, x)
     yb = ctx.buffer(M * rows * 4)
     keep += [xb, yb]
     flops = 2.0 * M * rows * cols
+    n = max(5, steps // 20)
     t = run_steps(host, ctx, [tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, M, TMH_GEMM_MMA)],
-                  2, 5, grouped=False)
-    us = t.gpu_ms / 5 * 1e3
-    out["lm_head_gemm_m512"] = _bf16_gemm_point(flops, us)
+                  2, n, grouped=False)
+    got, want, secs = gemm_sample(host_w[-1], rows, cols, x, M, yb, toks)
+    out["lm_head_gemm_m512"] = mfma_point(flops, t, n, [(rows, cols, M)], {
+        "M": M, "rows": rows, "cols": cols, "max_norm_err_vs_cpu": norm_err(got, want),
+        "tokens_checked": len(toks)})
+    if cpu:
+        cpu_out["lm_head_m512_ms_per_token_all_cores"] = secs / len(toks) * 1e3
     for b in keep:
         b.free()
     for _, _, _, m in pool:
         m.buf.free()
-    return out
+    return out, cpu_out
 
 
-def bench_sweep(host, ctx, steps, warmup):
+SWEEP_HEADLINE_M = (1, 8, 64, 512, 2048)  # the batches BASELINE config 4 names
+
+
+def bench_sweep(host, ctx, steps, warmup, cpu=True, batches=None):
     """BASELINE config 4: 2B-class shapes (hidden 2048, FFN 6144), M in
     {1, 8, 64, 512, 2048} plus the small batches in between, f32 activations
     and the int8-activation profile.
     Each point runs over 20 distinct weight copies per shape (535 MB in all),
-    so small M is measured against HBM, not against the caches."""
+    so small M is measured against HBM, not against the caches. Every point
+    carries both rooflines (algorithmic bytes against 8 TB/s, operations against
+    the peak of the matrix cores the launch used) and its error against the
+    oracle on sampled tokens of one copy of each shape (int8: bit equality)."""
+    import oracle as O
+
     copies = 20
-    pool = _weights_pool(ctx, list(S.SWEEP_2B), copies, 4000)
+    pool, host_w = _weights_pool(ctx, list(S.SWEEP_2B), copies, 4000, keep_host=len(S.SWEEP_2B))
     wbytes = sum(S.q8_0_bytes(r, c) for _, r, c, _ in pool)
-    out = {"workload": "2B-class sweep (BASELINE config 4)", "weight_copies": copies,
+    out = {"config": "BASELINE config 4: 2B-class shapes (6144 x 2048, 2048 x 6144), "
+                     f"{copies} copies of each = {len(pool)} products per step",
            "weights_bytes": wbytes, "points": []}
     maxM = 2048
     maxc = max(c for _, _, c, _ in pool)
     maxr = max(r for _, r, _, _ in pool)
     xb = ctx.buffer(maxM * maxc * 4)
-    xb.upload(0, S.make_activations(maxM * maxc, 99))
+    x_host = S.make_activations(maxM * maxc, 99)
+    xb.upload(0, x_host)
     widths = sorted({c for _, _, c, _ in pool})
     xqs = {c: ctx.buffer(H.xq_bytes(c, maxM)) for c in widths}
     ys = [ctx.buffer(maxM * maxr * 4) for _ in pool]
-    slice_x, slice_y = [], []
-    for M in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 2048):
-        n = max(3, steps // (10 if M < 64 else 200 if M < 512 else 1000))
+    slice_x, slice_y, slice_host = [], [], []
+    ncores = min(16, os.cpu_count() or 1)
+    for M in (batches or (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 2048)):
+        n = max(10 if M < 64 else 5 if M < 512 else 3,
+                steps // (10 if M < 64 else 200 if M < 512 else 1000))
         w = max(2, n // 5)
         flops = sum(2.0 * M * r * c for _, r, c, _ in pool)
         abytes = sum(S.q8_0_bytes(r, c) + 4 * M * c + 4 * M * r for _, r, c, _ in pool)
@@ -492,10 +643,10 @@ def bench_sweep(host, ctx, steps, warmup):
         if 1 < M <= 32:
             paths.append(("f32 gemm (gemv arithmetic)", TMH_GEMM, M))
         if 2 <= M <= 512:
-            paths.append(("f32 mfma", TMH_GEMM_MMA, M))
+            paths.append(("f32 mfma entry point", TMH_GEMM_MMA, M))
         if M > 512:
-            paths.append(("f32 mfma (slices of 512)", TMH_GEMM_MMA, 512))
-        paths.append(("i8 streaming dot4" if M <= 4 else "i8 mfma", TMH_GEMM_I8, M))
+            paths.append(("f32 mfma entry point (slices of 512)", TMH_GEMM_MMA, 512))
+        paths.append(("int8 activations", TMH_GEMM_I8, M))
         for label, kind, mb in paths:
             prods = []
             slices = (M + mb - 1) // mb
@@ -503,7 +654,7 @@ def bench_sweep(host, ctx, steps, warmup):
             if kind == TMH_GEMM_I8:
                 # activations are quantized once per distinct width (timed apart)
                 qprods = [tmh_product(None, xb.raw, xqs[c].raw, 1, c, M, TMH_QUANT) for c in widths]
-                tq = run_steps(host, ctx, qprods, 1, 3, grouped=True)
+                tq = run_steps(host, ctx, qprods, 1, 3, grouped=True, settle=False)
                 quant_us = tq.gpu_ms / 3 * 1e3
                 for (name, r, c, m), yb in zip(pool, ys):
                     prods.append(tmh_product(m.buf.raw, xqs[c].raw, yb.raw, r, c, M, kind))
@@ -513,8 +664,10 @@ def bench_sweep(host, ctx, steps, warmup):
                 # runner's products carry no offsets)
                 while len(slice_x) < slices - 1:
                     sx = ctx.buffer(mb * maxc * 4)
-                    sx.upload(0, S.make_activations(mb * maxc, 100 + len(slice_x)))
+                    sh = S.make_activations(mb * maxc, 100 + len(slice_x))
+                    sx.upload(0, sh)
                     slice_x.append(sx)
+                    slice_host.append(sh)
                     slice_y.append([ctx.buffer(mb * maxr * 4) for _ in pool])
                 for i, ((name, r, c, m), yb) in enumerate(zip(pool, ys)):
                     prods.append(tmh_product(m.buf.raw, xb.raw, yb.raw, r, c, mb, kind))
@@ -523,25 +676,114 @@ def bench_sweep(host, ctx, steps, warmup):
                                                  r, c, mb, kind))
             t = run_steps(host, ctx, prods, w, n, grouped=True)
             us = t.gpu_ms / n * 1e3
-            out["points"].append({
-                "M": M, "path": label, "us": us, "launches": t.launches / n,
-                "gbs": abytes / us / 1e3, "pct_of_hbm_peak": abytes / us / 1e3 / 80.0,
-                "tflops": flops / us / 1e6,
-                "frac_of_mfma_peak": flops / us / 1e6 / (MFMA_I8_PEAK_TOPS if kind == TMH_GEMM_I8
-                                                        else MFMA_F32_PEAK_TFLOPS),
-                "quantize_act_us": quant_us})
-            if kind == TMH_GEMM_MMA and mb >= H.GEMM_MMA_BF16_MIN_BATCH and \
+            # parity: sampled tokens of the first copy of each shape (for 2048 tokens in
+            # slices: of the first and of the last slice)
+            toks = sample_tokens(mb, 4)
+            err, equal = 0.0, True
+            for i, raw in enumerate(host_w):
+                _, r, c, _ = pool[i]
+                checks = [(x_host, ys[i])]
+                if slices > 1:
+                    checks.append((slice_host[slices - 2], slice_y[slices - 2][i]))
+                for xh, yb in checks:
+                    got, want, _ = gemm_sample(raw, r, c, xh[:mb * c], mb, yb, toks,
+                                               int8=kind == TMH_GEMM_I8, threads=ncores)
+                    err = max(err, norm_err(got, want))
+                    equal = equal and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+            pt = {"M": M, "path": label, "us": us, "launches": t.launches / n,
+                  "gbs": abytes / us / 1e3, "frac_hbm": abytes / us / 1e3 / HBM_PEAK_GBS,
+                  "tflops": flops / us / 1e6, "max_norm_err_vs_cpu": err}
+            if kind == TMH_GEMM_I8:
+                pt.update(mfma_peak="int8 5.0 POP/s", frac_mfma=flops / us / 1e6 / MFMA_I8_PEAK_TOPS,
+                          quantize_act_us=quant_us, bit_equal_to_cpu=bool(equal),
+                          kernel="q8::gemv_i8_list_kernel (v_dot4)" if M <= 4
+                          else "q8::gemm_i8_lds_kernel (v_mfma_i32_16x16x32_i8)")
+            elif kind == TMH_GEMM_MMA and mb >= H.GEMM_MMA_BF16_MIN_BATCH and \
                     H.gemm_mma_launch_tile([(r, c, mb) for _, r, c, _ in pool]):
-                # the products that share the launch are large enough together for the
-                # kernel on the bf16 matrix cores, which issues three bf16 products per f32 one
-                pt = out["points"][-1]
-                pt["path"] = label.replace("f32 mfma", "bf16 mfma x3")
-                pt["frac_of_mfma_peak"] = 3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS
+                # three bf16 products are issued per f32 one
+                pt.update(path=label + ": bf16 matrix cores, exact products",
+                          mfma_peak="bf16 2.5 PFLOP/s",
+                          frac_mfma=3.0 * flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS)
+            elif kind == TMH_GEMM_MMA and mb > 16:
+                pt.update(path=label + ": f32 matrix cores", mfma_peak="f32 157.3 TFLOP/s",
+                          frac_mfma=flops / us / 1e6 / MFMA_F32_PEAK_TFLOPS)
+            else:  # the vector kernels: f32 multiply-adds, no matrix cores
+                pt.update(mfma_peak=None, frac_mfma=None)
+            out["points"].append(pt)
+    out["points"].sort(key=lambda pt: (pt["M"], pt["path"].startswith("int8")))
+    # where the matrix cores take over from the vector (GEMV-arithmetic) kernels
+    best = {}
+    for pt in out["points"]:
+        if pt["path"].startswith("int8"):
+            continue
+        cur = best.get(pt["M"])
+        if cur is None or pt["us"] < cur["us"]:
+            best[pt["M"]] = pt
+    mfma_from = [M for M, pt in sorted(best.items()) if pt["frac_mfma"] is not None]
+    hbm_to = [M for M, pt in sorted(best.items()) if pt["frac_hbm"] >= 0.5]
+    out["crossover"] = {
+        "fastest_f32_path_by_M": {str(M): pt["path"] for M, pt in sorted(best.items())},
+        "matrix_cores_fastest_from_M": mfma_from[0] if mfma_from else None,
+        "at_least_half_of_hbm_peak_up_to_M": hbm_to[-1] if hbm_to else None,
+        "ridge_estimate": "2*M flops per weight byte x 34/32: the f32 vector rate (157 TFLOP/s) meets "
+                          "8 TB/s near M = 10, the measured crossover is where the vector kernels' "
+                          "issue rate, not HBM, starts to bound them"}
+    cpu_out = {}
+    if cpu:
+        # one copy of each shape, one token: both oracles, one thread and all cores
+        x1 = x_host[:maxc]
+        res = {}
+        for label, fn in (("f32", O.gemv_q8_0_f32), ("int8", O.gemv_q8_0_q8_0)):
+            for th in (1, ncores):
+                t0 = time.perf_counter()
+                for i, raw in enumerate(host_w):
+                    _, r, c, _ = pool[i]
+                    fn(raw, r, c, x1[:c], threads=th)
+                res[(label, th)] = time.perf_counter() - t0
+        one_bytes = sum(S.gemv_bytes(pool[i][1], pool[i][2]) for i in range(len(host_w)))
+        one_flops = sum(2.0 * pool[i][1] * pool[i][2] for i in range(len(host_w)))
+        cpu_out = {"sample": "one copy of each of the two shapes, one token (the CPU path is a loop "
+                             "of such GEMVs over tokens: forward.rs:703-735)",
+                   "f32_ms_per_token_1_thread": res[("f32", 1)] * 1e3,
+                   "f32_gbs_1_thread": one_bytes / res[("f32", 1)] / 1e9,
+                   "f32_ms_per_token_all_cores": res[("f32", ncores)] * 1e3,
+                   "int8_ms_per_token_1_thread": res[("int8", 1)] * 1e3,
+                   "int8_gops_1_thread": one_flops / res[("int8", 1)] / 1e9,
+                   "int8_ms_per_token_all_cores": res[("int8", ncores)] * 1e3,
+                   "cores_all": ncores,
+                   "step_of_40_products_ms_1_thread_extrapolated_per_token":
+                       res[("f32", 1)] * copies * 1e3}
     for b in [xb] + list(xqs.values()) + ys + slice_x + [y for per in slice_y for y in per]:
         b.free()
     for _, _, _, m in pool:
         m.buf.free()
-    return out
+    return out, cpu_out
+
+
+def read_ceiling(ctx, gib=1, reps=10):
+    """The read bandwidth this box sustains for a kernel that does nothing but
+    read: tm_hip_xor_checksum_u32 over `gib` GiB (non-temporal 16-byte loads, 8 KiB
+    per wave at a time, 8 KiB written per launch), median of `reps` commits."""
+    n = gib << 28  # 32-bit words
+    if n >= 1 << 32:
+        raise SystemExit("read_ceiling: at most 15 GiB")
+    src, part = ctx.buffer(n * 4), ctx.buffer(H.CHECKSUM_PARTIAL_BYTES)
+    ctx.fence()
+    for _ in range(4):
+        ctx.xor_checksum_u32(src, 0, n, part)
+    ctx.fence()
+    ctx.set_commit_log(True)
+    for _ in range(reps):
+        ctx.xor_checksum_u32(src, 0, n, part)
+    ctx.fence()
+    us = np.sort(np.asarray(ctx.read_commit_log(), dtype=np.float64)[-reps:]) / 1e3
+    ctx.set_commit_log(False)
+    src.free()
+    part.free()
+    med = float(np.median(us))
+    return {"kernel": "q8::xor_checksum_kernel", "bytes_read": n * 4, "median_us": med,
+            "min_us": float(us[0]), "gbs": n * 4 / med / 1e3, "gbs_best": n * 4 / float(us[0]) / 1e3,
+            "frac_of_published_peak": n * 4 / med / 1e3 / HBM_PEAK_GBS}
 
 
 def bench_f16(host, ctx, steps, warmup):
@@ -687,7 +929,8 @@ def run_traffic(host, ctx):
     the kernel trace that goes with them: every kernel family a few times, each
     preceded by enough untimed work of its own to be at its steady clocks.
       1. a plain f32 copy of known size (the calibration kernel: 256 MiB read,
-         256 MiB written per dispatch)
+         256 MiB written per dispatch), then the read-only streaming kernel over
+         1 GiB (xor_checksum_kernel: the read bandwidth this box sustains)
       2. the decode step (gemv_list_kernel, one dispatch per step)
       3. the seven Qwen3-0.6B projections at M = 512 as one group over sealed
          weights (split_act_list_kernel + gemm_bf16x3_kernel, 128-token tiles)
@@ -705,6 +948,8 @@ def run_traffic(host, ctx):
     src.free()
     dst.free()
     report = {"copy_f32_kernel": {"read_bytes": n * 4, "written_bytes": n * 4, "dispatches": 3}}
+    # 1b. the read-only streaming kernel over 1 GiB (the measured read ceiling)
+    report["xor_checksum_kernel"] = read_ceiling(ctx, gib=1, reps=10)
     products, keep, _ = build_decode_step(ctx, keep_host=False)
     step_bytes = sum(S.gemv_bytes(pr.rows, pr.cols) for pr in products)
     run_steps(host, ctx, products, 0, 5, grouped=True)
@@ -762,7 +1007,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="budget of the CPU-baseline leg (0 skips it)")
-    ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--no-gemm", action="store_true",
+                    help="decode workload: leave out roofline.gemm_m512 (BASELINE config 2)")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="decode workload: leave out roofline.gemma and roofline.sweep_2b "
+                         "(BASELINE configs 3 and 4)")
     ap.add_argument("--no-recorded", action="store_true",
                     help="chain workload: leave out the recorded-step leg (rocprofv3's kernel trace "
                          "crashed on stream capture here)")
@@ -776,10 +1025,12 @@ def main():
     ap.add_argument("--unsealed", action="store_true",
                     help="decode workload: leave the weights in the layout they are uploaded in "
                          "(what a binding that never calls tm_hip_q8_0_pack runs on)")
-    ap.add_argument("--workload", choices=["decode", "gemma", "sweep", "chain", "f16", "layer", "traffic"],
+    ap.add_argument("--workload", choices=["decode", "gemm", "gemma", "sweep", "chain", "f16", "layer",
+                                           "traffic"],
                     default="decode",
-                    help="decode (default, the headline line); gemma / sweep print the "
-                         "BASELINE config 3 / 4 measurements as one JSON object")
+                    help="decode (default, the headline line, which carries every BASELINE "
+                         "configuration); gemm / gemma / sweep print configs 2 / 3 / 4 on their own, "
+                         "the sweep with every batch")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one MI355X: this path runs on a single GPU "
@@ -795,13 +1046,17 @@ def main():
         return
     if args.workload != "decode":
         fn = {"gemma": bench_gemma, "sweep": bench_sweep, "chain": bench_chain,
-              "f16": bench_f16, "layer": bench_layer}[args.workload]
+              "f16": bench_f16, "layer": bench_layer, "gemm": bench_gemm}[args.workload]
         extra = ({"recorded": not args.no_recorded, "model": args.model, "tokens": args.tokens}
                  if args.workload == "chain" else {})
-        print(json.dumps(fn(host, ctx, args.steps, args.warmup, **extra)), flush=True)
+        res = fn(host, ctx, args.steps, args.warmup, **extra)
+        if isinstance(res, tuple):  # (roofline entry, CPU sample)
+            res = {"roofline": res[0], "cpu_baseline": res[1]}
+        print(json.dumps(res), flush=True)
         ctx.close()
         return
 
+    ceiling = read_ceiling(ctx)
     products, keep, host_side = build_decode_step(ctx, keep_host=args.cpu_seconds > 0,
                                                   seal=not args.unsealed)
     step_bytes = sum(S.gemv_bytes(pr.rows, pr.cols) for pr in products)
@@ -833,6 +1088,9 @@ def main():
             "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
             "precondition": dict(pre, rule="untimed windows of steps until three in a row agree "
                                  "within 1 % on GPU time per step; then --warmup, then --steps"),
+            "other_configs": "roofline.gemm_m512 (config 2), roofline.gemma (config 3), "
+                             "roofline.sweep_2b (config 4); their CPU samples under "
+                             "cpu_baseline.per_config",
         },
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -850,14 +1108,26 @@ def main():
                                if median_launch_us > 0 else None),
             "step_us": stats,
             "algorithmic_bytes_per_launch": launch_bytes,
+            "measured_read_ceiling": ceiling,
+            "frac_of_measured_ceiling": achieved / ceiling["gbs"],
         },
     }
+    per_config = {}
     if args.cpu_seconds > 0:
         line["cpu_baseline"] = cpu_baseline(host_side, args.cpu_seconds)
+        line["cpu_baseline"]["per_config"] = per_config
     for obj in keep:
         (obj.buf if isinstance(obj, H.Matrix) else obj).free()
+    host_side = None
+    cpu = args.cpu_seconds > 0
     if not args.no_gemm:
-        line["gemm"] = bench_gemm(host, ctx, max(10, args.steps // 4), max(3, args.warmup // 4))
+        line["roofline"]["gemm_m512"], per_config["config2_gemm_m512"] = bench_gemm(
+            host, ctx, max(10, args.steps // 4), max(3, args.warmup // 4), cpu=cpu)
+    if not args.no_configs:
+        line["roofline"]["gemma"], per_config["config3_gemma"] = bench_gemma(
+            host, ctx, max(10, args.steps // 4), max(3, args.warmup // 4), cpu=cpu)
+        line["roofline"]["sweep_2b"], per_config["config4_sweep_2b"] = bench_sweep(
+            host, ctx, max(20, args.steps // 4), 0, cpu=cpu, batches=SWEEP_HEADLINE_M + (16, 32, 128))
     ctx.close()
     print(json.dumps(line), flush=True)
 

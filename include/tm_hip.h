@@ -326,6 +326,18 @@ int tm_hip_q8_0_gemm_i8(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm
 
 /* ---- measurement surface (native/metal/tm_metal.h:293-325) ---- */
 
+/* XOR of the n 32-bit words at word offset src_off (a multiple of 4) of `src`,
+ * left as TM_HIP_CHECKSUM_PARTIAL_BYTES / 4 partial words in `partial` whose
+ * XOR is the result (any buffer contents, sealed weights included: the bytes
+ * are read as they lie on the device). Usable inside a group. The kernel only
+ * reads (non-temporal 16-byte loads, a wave's tile 8 KiB like the decode
+ * GEMV's) and writes 8 KiB whatever n is: over a gibibyte it measures the
+ * sustained HBM read bandwidth the streaming kernels are set against, and it
+ * checks an upload without a download. No counterpart in the reference. */
+#define TM_HIP_CHECKSUM_PARTIAL_BYTES 8192u
+int tm_hip_xor_checksum_u32(tm_hip_ctx *ctx, tm_hip_buffer *src, uint32_t src_off, uint32_t n,
+                            tm_hip_buffer *partial, char *err, size_t err_cap);
+
 uint64_t tm_hip_committed_dispatches(const tm_hip_ctx *ctx);
 uint64_t tm_hip_completed_dispatches(const tm_hip_ctx *ctx);
 /* GPU milliseconds of the most recently completed commit (HIP events on the

@@ -201,6 +201,51 @@ def test_copy_f32_moves_exact_slices_and_refuses_out_of_range(ctx):
     assert np.array_equal(got[7:], raw[5:]) and not got[:7].any()
 
 
+def test_xor_checksum_reads_every_word_once(ctx):
+    """The read-only streaming kernel (the HBM read-bandwidth calibration): its
+    partial words XOR to numpy's XOR of the same words, on lengths around its
+    8 KiB tiles and 16-byte pieces, at an offset, inside a group, and over a
+    sealed weight buffer (whose device bytes are the host statement of the
+    sealed layout)."""
+    rng = np.random.default_rng(31)
+    n_max = (17 << 20) + 777  # past one sweep of the grid: 8192 waves x 2048 words
+    raw = rng.integers(0, 1 << 32, n_max, dtype=np.uint64).astype(np.uint32)
+    buf = ctx.buffer(n_max * 4)
+    buf.upload(0, raw.view(np.uint8))
+    part = ctx.buffer(H.CHECKSUM_PARTIAL_BYTES)
+    for off, n in [(0, 1), (0, 3), (0, 4), (4, 2047), (0, 2048), (8, 2049), (0, 2048 * 4 * 2048),
+                   (12, 2048 * 4 * 2048 + 2048 * 3 + 5), (0, n_max), (n_max - 777 - 1, 777)]:
+        off -= off % 4
+        ctx.xor_checksum_u32(buf, off, n, part)
+        ctx.fence()
+        want = int(np.bitwise_xor.reduce(raw[off:off + n]))
+        assert H.HipContext.checksum_of(part) == want, (off, n)
+    # inside a group, behind the copy that writes what it reads
+    dst = ctx.buffer(4096 * 4)
+    ctx.begin_group()
+    ctx.copy_f32(buf, 64, dst, 0, 4096)
+    ctx.xor_checksum_u32(dst, 0, 4096, part)
+    ctx.end_group()
+    ctx.fence()
+    assert H.HipContext.checksum_of(part) == int(np.bitwise_xor.reduce(raw[64:64 + 4096]))
+    # a sealed matrix: the checksum of the device layout, no download needed
+    rows, cols = 96, 1152
+    w = S.make_weights(rows, cols, 5)
+    m = H.Matrix.load(ctx, w, cols, rows)
+    ctx.xor_checksum_u32(m.buf, 0, w.nbytes // 4, part)
+    ctx.fence()
+    sealed = S.pack_q8_0(w, rows, cols)
+    assert H.HipContext.checksum_of(part) == int(np.bitwise_xor.reduce(sealed.view(np.uint32)))
+    for args, code in [((buf, 2, 8, part), H.TM_HIP_ERR_UNSUPPORTED),
+                       ((buf, 0, 0, part), H.TM_HIP_ERR_BOUNDS),
+                       ((buf, 0, n_max + 1, part), H.TM_HIP_ERR_BOUNDS),
+                       ((buf, 0, 8, dst if False else ctx.buffer(64)), H.TM_HIP_ERR_BOUNDS),
+                       ((part, 0, 8, part), H.TM_HIP_ERR_UNSUPPORTED)]:
+        with pytest.raises(H.TuckmillError) as e:
+            ctx.xor_checksum_u32(*args)
+        assert e.value.abi_code == code
+
+
 def test_copy_f32_inside_a_group_follows_the_product_that_wrote_its_source(ctx):
     wb, xb, yb = ones_problem(ctx, xval=3.0)
     keep = ctx.buffer(8 * 4)

@@ -106,6 +106,52 @@ def test_config1_projection_shapes_alone_at_one_token(ctx, rows, cols):
     xb.free()
 
 
+# ---------------------------------------------------------------- config 2 --
+
+@pytest.mark.parametrize("batch,seal", [(512, True), (128, True), (512, False)])
+def test_config2_group_as_benchmarked(ctx, batch, seal):
+    """The workload bench.py times for config 2: the seven Qwen3-0.6B projections,
+    each with its own X, as ONE dispatch group: over sealed weights at 512 tokens
+    (one launch of the bf16 kernel on 128-token tiles behind one split pass), at
+    the engine's prefill chunk of 128 tokens (64-token tiles), and over weights
+    as uploaded (the f32 matrix cores). Every product within 1e-5 of the oracle on
+    sampled tokens, all rows. Which kernel a product takes depends on what
+    shares its launch, so each product alone proves nothing about this group."""
+    items = []
+    for name, rows, cols in S.QWEN3_0_6B_LAYER:
+        raw = S.make_weights(rows, cols, S.tensor_seed(2, 0, name))
+        x = S.make_activations(batch * cols, rows)
+        m = H.Matrix.load(ctx, raw, cols, rows, seal=seal)
+        items.append((name, rows, cols, raw, x, m, upload_new(ctx, x), ctx.buffer(batch * rows * 4)))
+    shapes = [(rows, cols, batch) for _, rows, cols in S.QWEN3_0_6B_LAYER]
+    tile = H.gemm_mma_launch_tile(shapes) if seal else 0
+    assert tile == ((128 if batch == 512 else 64) if seal else 0)
+    launches = ctx.kernel_launches()
+    ctx.begin_group()
+    for name, rows, cols, raw, x, m, xb, yb in items:
+        m.gemm(ctx, xb, yb, batch, exact=False)
+    ctx.end_group()
+    ctx.fence()
+    if seal:  # the split pass and one product launch
+        assert ctx.kernel_launches() == launches + 2
+    picked = token_sample(batch)
+    worst = 0.0
+    for name, rows, cols, raw, x, m, xb, yb in items:
+        xs = np.ascontiguousarray(x.reshape(batch, cols)[picked]).reshape(-1)
+        want = O.gemm_q8_0_f32(raw, rows, cols, xs, len(picked), threads=8)
+        scale = float(np.max(np.abs(want)))
+        for i, t in enumerate(picked):
+            got = yb.download_f32(t * rows, rows)
+            err = float(np.max(np.abs(got - want[i]))) / scale
+            assert err <= 1e-5, (name, t, err)
+            worst = max(worst, err)
+    print(f"config 2 group, {batch} tokens, {'sealed' if seal else 'raw'}: worst {worst:.2e}")
+    for it in items:
+        it[5].buf.free()
+        it[6].free()
+        it[7].free()
+
+
 # ---------------------------------------------------------------- config 3 --
 
 @pytest.fixture(scope="module")

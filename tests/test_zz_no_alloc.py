@@ -2,7 +2,8 @@
 nothing: its results against tm_hip_q8_0_gemm_mma's (same kernels, so bit for
 bit) and against the CPU oracle, on calls in a row that share the library's
 static device workspace, the second smaller than the first; its refusals; its
-leases; and that the device's free memory does not move.
+leases; that the device's free memory does not move; and calls from two contexts,
+which the library orders on the one workspace.
 """
 import ctypes
 
@@ -153,3 +154,35 @@ def test_refusals(ctx):
     assert e.value.abi_code == H.TM_HIP_ERR_UNSUPPORTED and "group" in e.value.message
     ctx.abort_group()
     ctx.fence()
+
+
+def test_two_contexts_share_the_static_workspace_in_order(ctx):
+    """Every context of a GPU uses that GPU's one static workspace, each on its own
+    stream: calls from two contexts with no fence between them are ordered by the
+    library (the later call's stream waits for the earlier context's), so each
+    product has the bits of the allocating entry point."""
+    other = H.HipContext.open()
+    try:
+        pa = [problem(ctx, 6144, 2048, 512, 300 + i) for i in range(2)]
+        pb = [problem(other, 4096, 3072, 384, 310 + i) for i in range(2)]
+        ctx.fence()
+        other.fence()
+        for round_ in range(3):  # A B A B ..., nothing in between
+            for c, p in ((ctx, pa[round_ % 2]), (other, pb[round_ % 2]),
+                         (ctx, pa[(round_ + 1) % 2]), (other, pb[(round_ + 1) % 2])):
+                c.q8_0_gemm_mma_noalloc(p["wb"], p["xb"], p["y_new"], p["rows"], p["cols"],
+                                        p["batch"], 0, 3)
+        ctx.fence()
+        other.fence()
+        for c, probs in ((ctx, pa), (other, pb)):
+            for p in probs:
+                c.q8_0_gemm_mma(p["wb"], p["xb"], p["y_old"], p["rows"], p["cols"], p["batch"], 0, 3)
+            c.fence()
+            for p in probs:
+                n = 3 + p["batch"] * p["rows"]
+                assert np.array_equal(bits(p["y_new"].download_f32(0, n)),
+                                      bits(p["y_old"].download_f32(0, n)))
+                for name in ("wb", "xb", "y_new", "y_old"):
+                    p[name].free()
+    finally:
+        other.close()

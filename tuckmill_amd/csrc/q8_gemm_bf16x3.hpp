@@ -562,6 +562,9 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
         if (arrived != chunks - 1u) {
             return;
         }
+        // (the loads below are issued after the count has come back; this keeps
+        // the compiler from moving them above the branch)
+        asm volatile("" ::: "memory");
         if (threadIdx.x == 0u) {
             __hip_atomic_store(&args.arrivals[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }

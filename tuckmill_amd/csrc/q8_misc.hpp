@@ -75,6 +75,60 @@ __global__ __launch_bounds__(256) void copy_f32_kernel(const float *src, float *
     }
 }
 
+// XOR of n 32-bit words, read once with non-temporal 16-byte loads: a wave
+// takes a tile of 8 KiB at a time, the shape in which the decode GEMV streams
+// its weights (eight 1 KiB rows in flight per wave). It writes one word per
+// workgroup, so what it measures is the read path alone: the sustained HBM
+// read bandwidth that the streaming kernels can be set against. `src` is
+// 16-byte aligned.
+constexpr uint32_t CHECKSUM_GROUPS = 2048;
+
+__global__ __launch_bounds__(256) void xor_checksum_kernel(const uint32_t *__restrict__ src,
+                                                           uint32_t *__restrict__ partial,
+                                                           uint32_t n) {
+    const uint32_t lane = threadIdx.x & 63u, wave_in = threadIdx.x >> 6;
+    const uint32_t pieces = n >> 2; // whole 16-byte pieces
+    const uint32_t full_tiles = pieces >> 9; // 512 pieces = 8 KiB
+    const uint32_t waves = gridDim.x * 4u;
+    const u32x4 *base = (const u32x4 *)src;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    uint32_t tile = blockIdx.x * 4u + wave_in;
+    for (; tile < full_tiles; tile += waves) {
+        const u32x4 *p = base + (size_t)tile * 512u + lane;
+        u32x4 v[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            v[r] = __builtin_nontemporal_load(p + r * 64);
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            acc ^= v[r];
+        }
+    }
+    if (tile == full_tiles) { // the ragged last tile: piece by piece
+#pragma unroll 1
+        for (uint32_t i = (full_tiles << 9) + lane; i < pieces; i += 64u) {
+            acc ^= base[i];
+        }
+        if (lane < (n & 3u)) { // and the last one to three words
+            acc.x ^= src[(size_t)pieces * 4u + lane];
+        }
+    }
+    uint32_t x = acc.x ^ acc.y ^ acc.z ^ acc.w;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        x ^= (uint32_t)__shfl_xor((int)x, off, 64);
+    }
+    __shared__ uint32_t per_wave[4];
+    if (lane == 0u) {
+        per_wave[wave_in] = x;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0u) {
+        partial[blockIdx.x] = per_wave[0] ^ per_wave[1] ^ per_wave[2] ^ per_wave[3];
+    }
+}
+
 // Clears n dwords (counters that must read zero when the next kernel starts).
 __global__ __launch_bounds__(256) void zero_u32_kernel(uint32_t *dst, uint32_t n) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;

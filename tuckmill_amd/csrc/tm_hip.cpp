@@ -19,6 +19,7 @@
 #include <deque>
 #include <mutex>
 #include <string>
+#include <type_traits>
 #include <unistd.h>
 #include <vector>
 
@@ -51,6 +52,7 @@ constexpr size_t kScratchPartialBytes = kScratchBytes - kScratchPartialOff;
 static_assert(kScratchArrivalsOff + q8::BX3_MAX_SPLIT_TILES * 4u <= kScratchXsOff, "counters");
 static_assert(q8::MMA_SHARED_PARTIAL_FLOATS * 4u <= kScratchPartialBytes, "f32 partial tiles");
 static_assert(q8::MMA_SHARED_MAX_TILES <= q8::BX3_MAX_SPLIT_TILES, "f32 arrival counters");
+static_assert(q8::CHECKSUM_GROUPS * 4u == TM_HIP_CHECKSUM_PARTIAL_BYTES, "checksum partial words");
 static __device__ __align__(256) uint8_t scratch[kScratchBytes];
 
 namespace {
@@ -61,6 +63,15 @@ namespace {
 constexpr int kMaxDevices = 64;
 uint8_t *g_scratch_ptr[kMaxDevices];
 std::mutex g_scratch_mu;
+// Every context of a GPU shares that GPU's array, and each launches on its own
+// stream. Calls of tm_hip_q8_0_gemm_mma_noalloc are ordered across contexts:
+// the context whose call used the array last is remembered per device, and a
+// call from another context first makes its stream wait for that one's (an
+// event recorded on the last user's stream, one per device, created with the
+// device's first context; nothing is allocated per call). All under
+// g_scratch_mu, which a call holds from its wait to its last launch.
+hipEvent_t g_scratch_event[kMaxDevices];
+::tm_hip_ctx *g_scratch_last[kMaxDevices];
 
 hipError_t scratch_on_current_device(int device, uint8_t **out) {
     if (device < 0 || device >= kMaxDevices) {
@@ -77,6 +88,13 @@ hipError_t scratch_on_current_device(int device, uint8_t **out) {
             return hipErrorInvalidSymbol;
         }
         g_scratch_ptr[device] = (uint8_t *)ptr;
+    }
+    if (g_scratch_event[device] == nullptr) {
+        const hipError_t e = hipEventCreateWithFlags(&g_scratch_event[device], hipEventDisableTiming);
+        if (e != hipSuccess) {
+            g_scratch_event[device] = nullptr;
+            return e;
+        }
     }
     *out = g_scratch_ptr[device];
     return hipSuccess;
@@ -122,7 +140,8 @@ void alloc_release(Alloc *a) {
 enum OpKind {
     OP_GEMV_LIST, OP_MMA, OP_ROW, OP_ROW_INDIRECT, OP_COPY, OP_PACK, OP_QUANT, OP_I8,
     OP_SCALE, OP_AXPY, OP_SILU_MUL, OP_GELU_MUL, OP_RMSNORM, OP_ARGMAX,
-    OP_F16_GEMM, OP_F16_ROW, OP_F16_ROW_INDIRECT, OP_CAST_F16_F32, OP_CAST_F32_F16
+    OP_F16_GEMM, OP_F16_ROW, OP_F16_ROW_INDIRECT, OP_CAST_F16_F32, OP_CAST_F32_F16,
+    OP_CHECKSUM
 };
 
 struct Op {
@@ -724,13 +743,99 @@ hipError_t launch_gemv(tm_hip_ctx *ctx, hipEvent_t stop, const q8::GemvArgs &arg
 constexpr int kGemvR1 = 8; // rows per pass at one token per pass
 constexpr int kGemvR4 = 2; // rows per pass at four tokens per pass
 
+// A vector of trivially copyable elements whose first N live inside the object:
+// a launch of a few products (every launch of the entry point that allocates
+// nothing has one) never touches the heap; longer lists spill to it.
+template <typename T, size_t N> class InlineVec {
+    static_assert(std::is_trivially_copyable<T>::value, "elements are copied with memcpy");
+
+  public:
+    InlineVec() = default;
+    InlineVec(const InlineVec &o) { assign(o); }
+    InlineVec(InlineVec &&o) noexcept { steal(o); }
+    InlineVec &operator=(const InlineVec &o) {
+        if (this != &o) {
+            clear();
+            assign(o);
+        }
+        return *this;
+    }
+    InlineVec &operator=(InlineVec &&o) noexcept {
+        if (this != &o) {
+            release();
+            steal(o);
+        }
+        return *this;
+    }
+    ~InlineVec() { release(); }
+    size_t size() const { return n_; }
+    bool empty() const { return n_ == 0; }
+    void clear() { n_ = 0; }
+    T &operator[](size_t i) { return data()[i]; }
+    const T &operator[](size_t i) const { return data()[i]; }
+    T &back() { return data()[n_ - 1]; }
+    const T &back() const { return data()[n_ - 1]; }
+    T *begin() { return data(); }
+    T *end() { return data() + n_; }
+    const T *begin() const { return data(); }
+    const T *end() const { return data() + n_; }
+    void push_back(const T &v) {
+        if (n_ == cap_) {
+            grow();
+        }
+        data()[n_++] = v;
+    }
+
+  private:
+    T *data() { return heap_ != nullptr ? heap_ : inline_; }
+    const T *data() const { return heap_ != nullptr ? heap_ : inline_; }
+    void grow() {
+        const size_t cap = cap_ * 2;
+        T *fresh = new T[cap];
+        memcpy(fresh, data(), n_ * sizeof(T));
+        delete[] heap_;
+        heap_ = fresh;
+        cap_ = cap;
+    }
+    void assign(const InlineVec &o) {
+        for (const T &v : o) {
+            push_back(v);
+        }
+    }
+    void steal(InlineVec &o) {
+        n_ = o.n_;
+        if (o.heap_ != nullptr) {
+            heap_ = o.heap_;
+            cap_ = o.cap_;
+            o.heap_ = nullptr;
+            o.cap_ = N;
+        } else {
+            heap_ = nullptr;
+            cap_ = N;
+            memcpy(inline_, o.inline_, o.n_ * sizeof(T));
+        }
+        o.n_ = 0;
+    }
+    void release() {
+        delete[] heap_;
+        heap_ = nullptr;
+        cap_ = N;
+        n_ = 0;
+    }
+    T inline_[N];
+    T *heap_ = nullptr;
+    size_t n_ = 0, cap_ = N;
+};
+
+using OpList = InlineVec<const Op *, 4>;
+
 // One kernel launch of a commit: a list of products, or a single operation.
 struct Launch {
-    std::vector<const Op *> list; // empty: `single`
-    std::vector<const Op *> residual; // per list entry: an axpy fused into it, or null
-    std::vector<const Op *> glu;      // per list entry: this product and the next are the gate
-                                      // and up projections of this fused gated activation
-    std::vector<bool> normed;         // per list entry: reads the fused RMSNorm's output
+    OpList list;     // empty: `single`
+    OpList residual; // per list entry: an axpy fused into it, or null
+    OpList glu;      // per list entry: this product and the next are the gate
+                     // and up projections of this fused gated activation
+    InlineVec<uint8_t, 4> normed; // per list entry: reads the fused RMSNorm's output
     const Op *norm = nullptr;         // an RMSNorm fused in front of the flagged entries
     GemvKey key{};
     const Op *single = nullptr;
@@ -761,7 +866,7 @@ bool same_input(const Op &a, const Op &b) {
 }
 size_t bx3_xs_bytes_of(const Op &op) { return ((size_t)op.batch * op.cols * 6u + 255u) & ~(size_t)255u; }
 
-hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
+hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const OpList &ops,
                            GemvKey key, const Workspace &ws) {
     q8::MmaProduct prods[q8::MMA_MAX_DESCS];
     int n = 0;
@@ -782,7 +887,7 @@ hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<c
 // ensure_bx3_workspace() when the launches were planned.
 hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch,
                            const Workspace &ws) {
-    const std::vector<const Op *> &ops = launch.list;
+    const OpList &ops = launch.list;
     if (launch.bx3_xs_bytes > ws.xs_bytes || launch.bx3_partial_floats * 4u > ws.partial_bytes) {
         return hipErrorInvalidValue;
     }
@@ -873,7 +978,7 @@ hipError_t ensure_bx3_workspace(tm_hip_ctx *ctx, const std::vector<Launch> &plan
     return e;
 }
 
-hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const std::vector<const Op *> &ops,
+hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const OpList &ops,
                           GemvKey key) {
     q8::I8Product prods[q8::I8_MAX_DESCS];
     int n = 0;
@@ -904,8 +1009,8 @@ uint32_t split_token_groups(const GemvKey &key, uint32_t batch) {
 
 hipError_t launch_gemv_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch,
                             const Workspace &ws) {
-    const std::vector<const Op *> &ops = launch.list;
-    const std::vector<const Op *> &residual = launch.residual;
+    const OpList &ops = launch.list;
+    const OpList &residual = launch.residual;
     GemvKey key = launch.key;
     if (key.variant == V_BF16X3) {
         return launch_bx3_list(ctx, stop, launch, ws);
@@ -1243,6 +1348,10 @@ hipError_t launch_single(tm_hip_ctx *ctx, hipEvent_t stop, const Op &op,
                   stop, src, dst, op.extra);
         break;
     }
+    case OP_CHECKSUM:
+        Q8_LAUNCH(q8::xor_checksum_kernel, dim3(q8::CHECKSUM_GROUPS), dim3(256), 0, st, stop,
+                  (const uint32_t *)op.a[0]->ptr + op.x_off, (uint32_t *)op.a[1]->ptr, op.extra);
+        break;
     case OP_SCALE:
         Q8_LAUNCH(q8::scale_kernel, dim3(strided_blocks_of(op.extra, 256u)), dim3(256), 0, st,
                   stop, (const float *)op.a[0]->ptr, (float *)op.a[1]->ptr, op.scalar, op.extra);
@@ -2073,6 +2182,13 @@ void tm_hip_destroy(tm_hip_ctx *ctx) {
         ctx->event_pool.clear();
     }
     noalloc_release(ctx);
+    {
+        // (its stream is idle: no other context has anything left to wait for)
+        std::lock_guard<std::mutex> g(g_scratch_mu);
+        if (ctx->device >= 0 && ctx->device < kMaxDevices && g_scratch_last[ctx->device] == ctx) {
+            g_scratch_last[ctx->device] = nullptr;
+        }
+    }
     for (void *p : {(void *)ctx->ws.mma_queue, (void *)ctx->ws.mma_partials,
                     (void *)ctx->ws.arrivals, (void *)ctx->ws.xs, (void *)ctx->ws.partials}) {
         if (p != nullptr) {
@@ -2319,6 +2435,44 @@ int tm_hip_copy_f32(tm_hip_ctx *ctx, tm_hip_buffer *src, uint32_t src_off, tm_hi
     return submit(ctx, op, "copy_f32", err, err_cap);
 }
 
+int tm_hip_xor_checksum_u32(tm_hip_ctx *ctx, tm_hip_buffer *src, uint32_t src_off, uint32_t n,
+                            tm_hip_buffer *partial, char *err, size_t err_cap) {
+    if (check_ctx(ctx, err, err_cap, "xor_checksum_u32") != TM_HIP_OK) {
+        return TM_HIP_ERR_UNSUPPORTED;
+    }
+    if (n == 0) {
+        return fail(err, err_cap, TM_HIP_ERR_BOUNDS, "xor_checksum_u32: zero length");
+    }
+    if ((src_off & 3u) != 0u) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "xor_checksum_u32: src_off %u is not a multiple of 4 words (16 bytes)", src_off);
+    }
+    int rc;
+    if ((rc = check_buffer(ctx, src, ((size_t)src_off + n) * 4u, err, err_cap,
+                           "xor_checksum_u32.src")) != TM_HIP_OK ||
+        (rc = check_buffer(ctx, partial, TM_HIP_CHECKSUM_PARTIAL_BYTES, err, err_cap,
+                           "xor_checksum_u32.partial")) != TM_HIP_OK) {
+        return rc;
+    }
+    if (partial->alloc->packed) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "xor_checksum_u32: partial is a sealed weight buffer");
+    }
+    if (partial->alloc == src->alloc) {
+        return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
+                    "xor_checksum_u32: partial must not be the buffer that is read");
+    }
+    Op op;
+    op.kind = OP_CHECKSUM;
+    op.a[0] = src->alloc;
+    op.a[1] = partial->alloc;
+    op.n_alloc = 2;
+    op.writes_mask = 2;
+    op.x_off = src_off;
+    op.extra = n;
+    return submit(ctx, op, "xor_checksum_u32", err, err_cap);
+}
+
 // ---- the small f32 operators either side of a product ----------------------
 
 namespace {
@@ -2547,6 +2701,9 @@ int tm_hip_end_group_recorded(tm_hip_ctx *ctx, tm_hip_step **out, char *err, siz
         delete step;
         return hip_fail(err, err_cap, "end_group_recorded: workspace", e);
     }
+    // (No other context may put its ordering event on this stream while it
+    // records: see tm_hip_q8_0_gemm_mma_noalloc.)
+    std::lock_guard<std::mutex> scratch_guard(g_scratch_mu);
     // Relaxed mode: the launchers may query occupancy while the stream records.
     e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed);
     if (e != hipSuccess) {
@@ -2765,6 +2922,19 @@ int tm_hip_q8_0_gemm_mma_noalloc(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffe
                     "fence first",
                     what, ctx->noalloc_keep.size());
     }
+    // The array is this GPU's, not this context's: behind another context's calls
+    // this one's launches wait for that context's stream first.
+    std::lock_guard<std::mutex> scratch_guard(g_scratch_mu);
+    if (g_scratch_last[ctx->device] != nullptr && g_scratch_last[ctx->device] != ctx) {
+        hipError_t e = hipEventRecord(g_scratch_event[ctx->device], g_scratch_last[ctx->device]->stream);
+        if (e == hipSuccess) {
+            e = hipStreamWaitEvent(ctx->stream, g_scratch_event[ctx->device], 0);
+        }
+        if (e != hipSuccess) {
+            return hip_fail(err, err_cap, "q8_0_gemm_mma_noalloc: ordering behind another context", e);
+        }
+    }
+    g_scratch_last[ctx->device] = ctx;
     ctx->loose_work = true; // launched outside any commit: a fence asks the runtime
     // Held until the next commit adopts them or a fence has passed them (the list
     // has its capacity from tm_hip_create on).

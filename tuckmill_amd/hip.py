@@ -117,6 +117,7 @@ NOALLOC_XS_BYTES = 20 << 20
 GEMM_I8_MAX_BATCH = 2048
 ARGMAX_NONE = 0xFFFFFFFF  # crates/metal/src/lib.rs (ARGMAX_NONE), native/metal/kernels.metal:143
 ARGMAX_PARTIAL_BYTES = 512
+CHECKSUM_PARTIAL_BYTES = 8192  # include/tm_hip.h TM_HIP_CHECKSUM_PARTIAL_BYTES
 STAGING_CHUNK_BYTES = 4 << 20  # crates/tuckcore/src/qwen35_gpu.rs:1176
 
 TM_HIP_ERR_NO_DEVICE = -1
@@ -287,6 +288,9 @@ _SIGS = {
     "tm_hip_copy_f32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
                                        ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32,
                                        ctypes.c_char_p, ctypes.c_size_t]),
+    "tm_hip_xor_checksum_u32": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
+                                               ctypes.c_uint32, ctypes.c_void_p, ctypes.c_char_p,
+                                               ctypes.c_size_t]),
     "tm_hip_begin_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_end_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
     "tm_hip_abort_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]),
@@ -552,6 +556,18 @@ class HipContext:
     def copy_f32(self, src, src_off, dst, dst_off, n):
         self._check_owned(src, dst)
         self._operate("copy_f32", self._lib.tm_hip_copy_f32, src.raw, src_off, dst.raw, dst_off, n)
+
+    def xor_checksum_u32(self, src, src_off, n, partial):
+        """Records the XOR of n 32-bit words of `src` as CHECKSUM_PARTIAL_BYTES / 4 partial
+        words in `partial` (XOR them after a fence: `checksum_of`)."""
+        self._check_owned(src, partial)
+        self._operate("xor_checksum_u32", self._lib.tm_hip_xor_checksum_u32, src.raw, src_off, n,
+                      partial.raw)
+
+    @staticmethod
+    def checksum_of(partial) -> int:
+        words = np.frombuffer(partial.download(0, CHECKSUM_PARTIAL_BYTES), dtype=np.uint32)
+        return int(np.bitwise_xor.reduce(words))
 
     # -- additions ---------------------------------------------------------
     def q8_0_pack(self, w, rows: int, cols: int):
