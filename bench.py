@@ -70,6 +70,7 @@ class tmh_timing(ctypes.Structure):
 
 TMH_GEMV, TMH_GEMM, TMH_GEMM_MMA, TMH_GEMM_I8, TMH_QUANT = range(5)
 TMH_RMSNORM, TMH_SILU_MUL, TMH_AXPY, TMH_ARGMAX, TMH_F16_GEMM, TMH_GELU_MUL = range(5, 11)
+TMH_GEMM_I8_FMA = 11
 
 
 def load_host():
@@ -647,11 +648,13 @@ def bench_sweep(host, ctx, steps, warmup, cpu=True, batches=None):
         if M > 512:
             paths.append(("f32 mfma entry point (slices of 512)", TMH_GEMM_MMA, 512))
         paths.append(("int8 activations", TMH_GEMM_I8, M))
+        if M >= 5:
+            paths.append(("int8 activations, fused tail", TMH_GEMM_I8_FMA, M))
         for label, kind, mb in paths:
             prods = []
             slices = (M + mb - 1) // mb
             quant_us = None
-            if kind == TMH_GEMM_I8:
+            if kind in (TMH_GEMM_I8, TMH_GEMM_I8_FMA):
                 # activations are quantized once per distinct width (timed apart)
                 qprods = [tmh_product(None, xb.raw, xqs[c].raw, 1, c, M, TMH_QUANT) for c in widths]
                 tq = run_steps(host, ctx, qprods, 1, 3, grouped=True, settle=False)
@@ -687,13 +690,14 @@ def bench_sweep(host, ctx, steps, warmup, cpu=True, batches=None):
                     checks.append((slice_host[slices - 2], slice_y[slices - 2][i]))
                 for xh, yb in checks:
                     got, want, _ = gemm_sample(raw, r, c, xh[:mb * c], mb, yb, toks,
-                                               int8=kind == TMH_GEMM_I8, threads=ncores)
+                                               int8=kind in (TMH_GEMM_I8, TMH_GEMM_I8_FMA),
+                                               threads=ncores)
                     err = max(err, norm_err(got, want))
                     equal = equal and np.array_equal(got.view(np.uint32), want.view(np.uint32))
             pt = {"M": M, "path": label, "us": us, "launches": t.launches / n,
                   "gbs": abytes / us / 1e3, "frac_hbm": abytes / us / 1e3 / HBM_PEAK_GBS,
                   "tflops": flops / us / 1e6, "max_norm_err_vs_cpu": err}
-            if kind == TMH_GEMM_I8:
+            if kind in (TMH_GEMM_I8, TMH_GEMM_I8_FMA):
                 pt.update(mfma_peak="int8 5.0 POP/s", frac_mfma=flops / us / 1e6 / MFMA_I8_PEAK_TOPS,
                           quantize_act_us=quant_us, bit_equal_to_cpu=bool(equal),
                           kernel="q8::gemv_i8_list_kernel (v_dot4)" if M <= 4

@@ -250,9 +250,13 @@ int tm_hip_q8_0_gemm_mma(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *x, tm
  *     until the next commit of the context completes or a fence has passed;
  *     after TM_HIP_NOALLOC_MAX_PENDING calls without either, the call is refused.
  *   - All calls on one GPU share the one array, which keeps the last call's
- *     contents (what must start at zero is cleared by the call itself): calls
- *     that overlap on one GPU, from two contexts or two processes' worth of
- *     streams in one process, race. One context orders its own calls. */
+ *     contents (what must start at zero is cleared by the call itself). One
+ *     context orders its own calls; calls from different contexts of one process
+ *     are ordered by the library (a call that follows another context's makes
+ *     its stream wait for that context's stream first, under a process-wide
+ *     lock held for the duration of the call), so they may come from different
+ *     threads without a fence between them. The call allocates nothing on the
+ *     host either. Two PROCESSES each hold their own copy of the array. */
 #define TM_HIP_NOALLOC_WORKSPACE_BYTES (64u << 20)
 #define TM_HIP_NOALLOC_XS_BYTES (20u << 20)
 #define TM_HIP_NOALLOC_MAX_PENDING 1024u
@@ -323,6 +327,20 @@ int tm_hip_q8_0_quantize_act(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *x
 int tm_hip_q8_0_gemm_i8(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm_hip_buffer *y,
                         tm_hip_buffer *sumi, uint32_t rows, uint32_t cols, uint32_t batch,
                         uint32_t y_off, char *err, size_t err_cap);
+
+/* tm_hip_q8_0_gemm_i8 with a declared, faster tail: the same exact i32 block
+ * dots and the same scale product d_w * d_x, but each block's term enters the
+ * sum with one fused multiply-add, acc = fma(d_w * d_x, (float)sumi, acc),
+ * where crates/tuckcore/src/kernels.rs:206-221 rounds the product and then the
+ * sum. One rounding fewer per block: the f32 result is within the 1e-5
+ * (normalised) tolerance of the CPU's, not bit-identical to it. Never chosen by
+ * the library on its own: a caller that wants the CPU's bits calls
+ * tm_hip_q8_0_gemm_i8. Batches that the bit-exact kernels serve at the speed of
+ * the weight stream (up to 4 tokens, or weights as uploaded) take those kernels
+ * and their bits. No counterpart in the reference. */
+int tm_hip_q8_0_gemm_i8_fma(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm_hip_buffer *y,
+                            uint32_t rows, uint32_t cols, uint32_t batch, uint32_t y_off, char *err,
+                            size_t err_cap);
 
 /* ---- measurement surface (native/metal/tm_metal.h:293-325) ---- */
 

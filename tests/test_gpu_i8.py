@@ -170,3 +170,60 @@ def test_lds_staged_i8_gemm_is_bit_exact(ctx, rows, cols, batch):
     assert not out[:5].any()
     want = O.gemm_q8_0_q8_0(w, rows, cols, x, batch, threads=8)
     assert np.array_equal(bits(out[5:]), bits(want.reshape(-1)))
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(300, 1152, 5), (129, 2080, 17), (100, 352, 48),
+                                             (513, 160, 41), (200, 1024, 96), (64, 1152, 256),
+                                             (257, 6144, 129), (513, 3072, 300), (1000, 64, 512),
+                                             (6144, 2048, 512), (300, 1152, 3), (96, 1024, 1)])
+def test_fused_tail_variant_is_within_tolerance_and_never_silent(ctx, rows, cols, batch):
+    """tm_hip_q8_0_gemm_i8_fma: the same exact block dots, every term fused into
+    the f32 sum. Within 1e-5 (normalised) of the CPU's dot_q8_0_q8_0 and of the
+    bit-exact entry point; where the fused multiply-add rounds differently the
+    bits differ, which is why it is an entry point of its own. Up to four tokens
+    the bit-exact streaming kernel serves it."""
+    w = S.make_weights(rows, cols, 7 * rows + cols)
+    x = S.make_activations(cols * batch, batch + 3)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    xq, qs, ds = quantize_on_gpu(ctx, x, cols, batch)
+    y_fma, y_exact = ctx.buffer((5 + batch * rows) * 4), ctx.buffer(batch * rows * 4)
+    ctx.begin_group()  # both in one group: they never share a launch
+    ctx.q8_0_gemm_i8_fma(wb, xq, y_fma, rows, cols, batch, 5)
+    ctx.q8_0_gemm_i8(wb, xq, y_exact, rows, cols, batch, 0)
+    ctx.end_group()
+    ctx.fence()
+    out = y_fma.download_f32(0, 5 + batch * rows)
+    assert not out[:5].any()
+    want = O.gemm_q8_0_q8_0(w, rows, cols, x, batch, threads=8).reshape(-1)
+    exact = y_exact.download_f32(0, batch * rows)
+    assert np.array_equal(bits(exact), bits(want))
+    scale = float(np.max(np.abs(want)))
+    assert float(np.max(np.abs(out[5:] - want))) / scale <= 1e-5
+    if batch <= 4:
+        assert np.array_equal(bits(out[5:]), bits(want))
+    for b in (wb, xq, y_fma, y_exact):
+        b.free()
+
+
+def test_matrix_takes_the_fused_tail_only_when_asked(ctx):
+    rows, cols, batch = 512, 2048, 64
+    w = S.make_weights(rows, cols, 11)
+    x = S.make_activations(cols * batch, 12)
+    xb = upload_new(ctx, x)
+    want = O.gemm_q8_0_q8_0(w, rows, cols, x, batch, threads=8)
+    outs = {}
+    for fused in (False, True):
+        m = H.Matrix.load(ctx, w, cols, rows, profile=H.NumericalProfile.LLAMA_CPU,
+                          fused_i8_tail=fused)
+        yb = ctx.buffer(batch * rows * 4)
+        m.gemm(ctx, xb, yb, batch, exact=False)
+        ctx.fence()
+        outs[fused] = yb.download_f32(0, batch * rows).reshape(batch, rows)
+        m.buf.free()
+        yb.free()
+    assert np.array_equal(bits(outs[False]), bits(want)), "the default keeps the CPU's bits"
+    assert float(np.max(np.abs(outs[True] - want))) / float(np.max(np.abs(want))) <= 1e-5
+    with pytest.raises(H.TuckmillError) as e:
+        H.Matrix.load(ctx, w, cols, rows, fused_i8_tail=True)  # oracle-f32 has no int8 tail
+    assert e.value.code == "InvalidRequest"
+    xb.free()

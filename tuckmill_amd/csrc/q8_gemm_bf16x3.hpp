@@ -609,6 +609,7 @@ struct Bx3Product {
     const uint16_t *xs;
     float *y;
     uint32_t rows, cols, batch;
+    uint32_t chunks; // K chunks of this product, as bx3_plan_launch cut the launch
 };
 
 // How a product is cut into work units (output tile x K chunk): a function of
@@ -661,6 +662,190 @@ inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint3
     return p;
 }
 
+// ---- K chunks: decided per launch ------------------------------------------
+//
+// What bx3_plan_with says about a product's chunks is what the product would get
+// alone; bx3_launch_tile keeps using those unit counts as its measure of "enough
+// work". How the products of a launch are actually cut is decided for the launch
+// as a whole, because a work unit has a fixed cost that 16-block chunks pay too
+// often: measured (1024 units of one product at 512 tokens, K = 512 ... 4096)
+// a unit takes about 6 us plus 1.43 us per Q8_0 block, and a unit of a chunked
+// tile about 10 us more (its 128 KiB partial tile goes to memory and comes back;
+// a whole round of them is 33 MB at once). The seven projections of a Qwen3-0.6B
+// layer at 512 tokens, each cut as if alone, were 480 units of 16 blocks, two
+// rounds of the chip and 61 MB of partial tiles: 82 us. Cut for the launch they
+// are 240 units of 32 blocks, one round, the five K = 1024 products whole: 66 us.
+//
+// The rule: every product gets chunks_i = ceil(blocks_i / L) (at most
+// bx3_chunk_cap) for one target length L per launch; L runs over the lengths at
+// which some product's chunk count changes, each candidate is priced by handing
+// its units, longest first (the kernel's order), to the chip's workgroup slots
+// as they come free, and the cheapest wins (ties: fewer units).
+struct Bx3Shape3 {
+    uint32_t rows, cols, batch;
+};
+
+// At most eight chunks, none below 512 columns, and no more than it takes to
+// give a product about two rounds of units on its own: a product with many
+// output tiles is never cut.
+inline uint32_t bx3_chunk_cap(uint32_t rows, uint32_t cols, uint32_t batch, uint32_t tile_tokens) {
+    const uint32_t blocks = cols / 32u;
+    const uint64_t tiles = (uint64_t)((batch + tile_tokens - 1u) / tile_tokens) *
+                           ((rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS);
+    uint32_t cap = blocks / BX3_CHUNK_BLOCKS;
+    cap = cap < BX3_MAX_CHUNKS ? cap : BX3_MAX_CHUNKS;
+    const uint64_t by_tiles = (2u * 256u + tiles - 1u) / tiles;
+    cap = by_tiles < cap ? (uint32_t)by_tiles : cap;
+    return cap < 1u ? 1u : cap;
+}
+
+// The plan of a product cut into `chunks` chunks (as many as bx3_plan_launch gave it).
+inline Bx3Plan bx3_plan_chunked(uint32_t rows, uint32_t cols, uint32_t batch, uint32_t tile_tokens,
+                                uint32_t chunks) {
+    Bx3Plan p;
+    p.tile_tokens = tile_tokens;
+    const uint32_t blocks = cols / 32u;
+    p.tiles = (uint64_t)((batch + tile_tokens - 1u) / tile_tokens) *
+              ((rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS);
+    chunks = chunks < 1u ? 1u : chunks;
+    p.chunk_blocks = (blocks + chunks - 1u) / chunks;
+    p.chunks = (blocks + p.chunk_blocks - 1u) / p.chunk_blocks;
+    p.units = p.tiles * p.chunks;
+    p.split_tiles = p.chunks > 1u ? p.tiles : 0u;
+    p.partial_floats = p.split_tiles * p.chunks * tile_tokens * BX3_TILE_ROWS;
+    return p;
+}
+
+// Estimated duration (ns) of a launch whose products are cut as `chunks` says:
+// units in descending length to `slots` workgroup slots, each to the slot that
+// comes free first. Units of one product are alike, so the slots are tracked as
+// groups that come free together.
+inline uint64_t bx3_price(const Bx3Shape3 *shapes, const uint32_t *chunks, int n,
+                          uint32_t tile_tokens) {
+    const uint32_t slots = tile_tokens == 128u ? 256u : 512u;
+    const uint64_t unit_ns = tile_tokens == 128u ? 6000u : 4500u;
+    const uint64_t block_ns = tile_tokens == 128u ? 1430u : 1100u;
+    const uint64_t chunked_ns = tile_tokens == 128u ? 10000u : 5000u;
+    struct Kind {
+        uint64_t ns, units;
+    };
+    Kind kinds[BX3_MAX_DESCS];
+    for (int i = 0; i < n; ++i) { // insertion sort, longest first
+        const Bx3Plan p = bx3_plan_chunked(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens,
+                                           chunks[i]);
+        const Kind k{unit_ns + block_ns * p.chunk_blocks + (p.chunks > 1u ? chunked_ns + 1000u * p.chunks : 0u),
+                     p.units};
+        int at = i;
+        while (at > 0 && kinds[at - 1].ns < k.ns) {
+            kinds[at] = kinds[at - 1];
+            --at;
+        }
+        kinds[at] = k;
+    }
+    struct Group {
+        uint64_t free_at, count;
+    };
+    constexpr int MAX_GROUPS = 4 * BX3_MAX_DESCS + 4;
+    Group groups[MAX_GROUPS]; // ascending free_at
+    int ng = 1;
+    groups[0] = Group{0u, slots};
+    uint64_t end = 0;
+    for (int i = 0; i < n; ++i) {
+        uint64_t left = kinds[i].units;
+        while (left > 0) {
+            // whole rounds of every slot at once when the class is large
+            if (ng == 1 && left >= groups[0].count) {
+                const uint64_t rounds = left / groups[0].count;
+                groups[0].free_at += rounds * kinds[i].ns;
+                left -= rounds * groups[0].count;
+                end = groups[0].free_at > end ? groups[0].free_at : end;
+                continue;
+            }
+            const uint64_t take = left < groups[0].count ? left : groups[0].count;
+            const uint64_t done = groups[0].free_at + kinds[i].ns;
+            end = done > end ? done : end;
+            groups[0].count -= take;
+            left -= take;
+            if (groups[0].count == 0) { // drop it
+                for (int g = 1; g < ng; ++g) {
+                    groups[g - 1] = groups[g];
+                }
+                --ng;
+            }
+            // insert (done, take), merging with a group of the same time
+            int at = 0;
+            while (at < ng && groups[at].free_at < done) {
+                ++at;
+            }
+            if (at < ng && groups[at].free_at == done) {
+                groups[at].count += take;
+            } else if (ng < MAX_GROUPS) {
+                for (int g = ng; g > at; --g) {
+                    groups[g] = groups[g - 1];
+                }
+                groups[at] = Group{done, take};
+                ++ng;
+            } else { // (cannot happen with these bounds; stay correct anyway)
+                groups[ng - 1].count += take;
+            }
+        }
+    }
+    return end;
+}
+
+// chunks[i] for every product of a launch (see above). Deterministic: a function
+// of the shapes in list order and the tile.
+inline void bx3_plan_launch(const Bx3Shape3 *shapes, int n, uint32_t tile_tokens, uint32_t *chunks) {
+    uint32_t cap[BX3_MAX_DESCS];
+    uint64_t tiles = 0;
+    bool any = false;
+    for (int i = 0; i < n; ++i) {
+        cap[i] = bx3_chunk_cap(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens);
+        any = any || cap[i] > 1u;
+        chunks[i] = 1u;
+        tiles += bx3_plan_chunked(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens, 1u).tiles;
+    }
+    if (!any || tiles >= 1024u) {
+        return; // nothing to cut, or rounds enough as it is
+    }
+    // candidate lengths: where some product's chunk count changes
+    uint32_t lengths[BX3_MAX_DESCS * BX3_MAX_CHUNKS];
+    int nl = 0;
+    for (int i = 0; i < n; ++i) {
+        const uint32_t blocks = shapes[i].cols / 32u;
+        for (uint32_t c = 1; c <= cap[i]; ++c) {
+            const uint32_t len = (blocks + c - 1u) / c;
+            bool seen = false;
+            for (int j = 0; j < nl; ++j) {
+                seen = seen || lengths[j] == len;
+            }
+            if (!seen) {
+                lengths[nl++] = len;
+            }
+        }
+    }
+    uint64_t best_ns = ~0ull, best_units = ~0ull;
+    uint32_t trial[BX3_MAX_DESCS];
+    for (int j = 0; j < nl; ++j) {
+        uint64_t units = 0;
+        for (int i = 0; i < n; ++i) {
+            const uint32_t blocks = shapes[i].cols / 32u;
+            uint32_t c = (blocks + lengths[j] - 1u) / lengths[j];
+            c = c > cap[i] ? cap[i] : c;
+            trial[i] = c;
+            units += bx3_plan_chunked(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens, c).units;
+        }
+        const uint64_t ns = bx3_price(shapes, trial, n, tile_tokens);
+        if (ns < best_ns || (ns == best_ns && units < best_units)) {
+            best_ns = ns;
+            best_units = units;
+            for (int i = 0; i < n; ++i) {
+                chunks[i] = trial[i];
+            }
+        }
+    }
+}
+
 // Which tile the products of one launch take together, or 0 when the kernel does
 // not pay for them: the rule of a single product, with the launch's sums in the
 // place of the product's own figures (`shapes` = rows, cols, batch of every
@@ -692,10 +877,6 @@ inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint3
 // large tile 8192 x 1024 49 against 93, 6144 x 2048 69 against 133. Together: the
 // seven Qwen3-0.6B projections at 512 tokens 78 us on the large tile against 144
 // on the f32 kernel.
-struct Bx3Shape3 {
-    uint32_t rows, cols, batch;
-};
-
 inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
     if (n <= 0) {
         return 0;
@@ -780,15 +961,27 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
     args.n = (uint32_t)n;
     args.partials = partials;
     args.arrivals = arrivals;
-    // Longest K first (the order of the list changes no product's result).
+    // Longest work unit first (the order of the list changes no product's
+    // result). A unit is an output tile x K chunk and lasts one stage per Q8_0
+    // block of its chunk; the chip takes units in list order as workgroups
+    // retire, so the long ones must not come last. Products whose K is cut into
+    // chunks have the SHORT units: listed by K, the seven projections of a
+    // Qwen3-0.6B layer at 512 tokens (160 units of 32 stages, 160 of 16) ran
+    // the short ones first and finished after 48 stages; long ones first, 32.
     Bx3Product prods[BX3_MAX_DESCS];
+    uint32_t unit_blocks[BX3_MAX_DESCS];
     for (int i = 0; i < n; ++i) {
+        const uint32_t mine = bx3_plan_chunked(prods_in[i].rows, prods_in[i].cols, prods_in[i].batch,
+                                               (uint32_t)Sh::tokens, prods_in[i].chunks).chunk_blocks;
         int at = i;
-        while (at > 0 && prods[at - 1].cols < prods_in[i].cols) {
+        while (at > 0 && (unit_blocks[at - 1] < mine ||
+                          (unit_blocks[at - 1] == mine && prods[at - 1].cols < prods_in[i].cols))) {
             prods[at] = prods[at - 1];
+            unit_blocks[at] = unit_blocks[at - 1];
             --at;
         }
         prods[at] = prods_in[i];
+        unit_blocks[at] = mine;
     }
     uint64_t units = 0, split_tiles = 0, partial_tiles = 0;
     for (int i = 0; i < n; ++i) {
@@ -800,9 +993,9 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
         d.cols = prods[i].cols;
         d.batch = prods[i].batch;
         d.tile_begin = (uint32_t)units;
-        // K chunks as the product's shape and the launch's tile say
-        const Bx3Plan plan = bx3_plan_with(prods[i].rows, prods[i].cols, prods[i].batch,
-                                           (uint32_t)Sh::tokens);
+        // K chunks as the launch was cut
+        const Bx3Plan plan = bx3_plan_chunked(prods[i].rows, prods[i].cols, prods[i].batch,
+                                              (uint32_t)Sh::tokens, prods[i].chunks);
         d.tiles_t = (prods[i].batch + Sh::tokens - 1) / Sh::tokens;
         d.chunk_blocks = plan.chunk_blocks;
         d.chunks = plan.chunks;
@@ -828,8 +1021,8 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
 }
 
 // Sealed weights, every region below 4 GiB (32-bit buffer offsets): the caller
-// checks these before choosing this kernel; every product is planned with
-// bx3_plan_with(..., tile_tokens). `partials` holds the sum of the products' partial_floats,
+// checks these before choosing this kernel; every product carries the chunk
+// count bx3_plan_launch gave it. `partials` holds the sum of the products' partial_floats,
 // `arrivals` BX3_MAX_SPLIT_TILES counters that are zero between launches (both
 // may be null when no product's K is cut into chunks).
 inline hipError_t launch_gemm_bf16x3_list(hipStream_t stream, hipEvent_t stop, uint32_t tile_tokens,

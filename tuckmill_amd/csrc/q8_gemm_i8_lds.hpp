@@ -51,7 +51,14 @@ __device__ __forceinline__ uint32_t i8_swz(uint32_t r, uint32_t p) {
     return p ^ ((r / Sh::rows_per_bankrow) % (Sh::pieces < 16 ? Sh::pieces : 16));
 }
 
-template <int WM, int WN, int KS, int TM = 4, int TN = 4>
+// FMA = false: the tail of crates/tuckcore/src/kernels.rs:206-221 operation for
+// operation, (d_w * d_x) * sumi rounded, then the addition: the f32 result has the
+// CPU's bits. FMA = true (the declared fast variant, tm_hip_q8_0_gemm_i8_fma): the
+// same exact i32 block dots and the same scale product, but the term goes into
+// the sum with one fused multiply-add (one rounding fewer per block, three vector
+// operations per output and block instead of four): within 1e-5 of the CPU's
+// result, not its bits.
+template <int WM, int WN, int KS, int TM = 4, int TN = 4, bool FMA = false>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_i8_lds_kernel(const I8Args args) {
     using Sh = I8LdsShape<WM, WN, KS, TM, TN>;
     constexpr int NW = WM * WN; // 16x16 tiles per wave: 16*TM tokens x 16*TN rows
@@ -204,8 +211,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_i8_lds_kernel(const I8Args 
                     for (int v = 0; v < 4; ++v) {
                         // (d_w * d_x) * sumi, then the add: unfused, block order
                         const float scale = __fmul_rn(dw[j], dxv[v]);
-                        const float term = __fmul_rn(scale, (float)s[v]);
-                        acc[i][j][v] = __fadd_rn(acc[i][j][v], term);
+                        if constexpr (FMA) {
+                            acc[i][j][v] = __builtin_fmaf(scale, (float)s[v], acc[i][j][v]);
+                        } else {
+                            const float term = __fmul_rn(scale, (float)s[v]);
+                            acc[i][j][v] = __fadd_rn(acc[i][j][v], term);
+                        }
                     }
                 }
             }
@@ -249,7 +260,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_i8_lds_kernel(const I8Args 
     }
 }
 
-template <int WM, int WN, int KS, int TM = 4, int TN = 4>
+template <int WM, int WN, int KS, int TM = 4, int TN = 4, bool FMA = false>
 inline hipError_t launch_i8_lds_cfg(hipStream_t stream, hipEvent_t stop, const I8Product *prods,
                                     int n) {
     using Sh = I8LdsShape<WM, WN, KS, TM, TN>;
@@ -273,8 +284,8 @@ inline hipError_t launch_i8_lds_cfg(hipStream_t stream, hipEvent_t stop, const I
     args.total_tiles = (uint32_t)tiles;
     args.chunk_wgs = args.d[0].tiles_t;
     args.pad = 0;
-    Q8_LAUNCH((gemm_i8_lds_kernel<WM, WN, KS, TM, TN>), dim3((unsigned)tiles), dim3(WM * WN * 64), 0,
-              stream, stop, args);
+    Q8_LAUNCH((gemm_i8_lds_kernel<WM, WN, KS, TM, TN, FMA>), dim3((unsigned)tiles),
+              dim3(WM * WN * 64), 0, stream, stop, args);
     return hipGetLastError();
 }
 
@@ -303,9 +314,19 @@ inline int i8_lds_shape(uint32_t batch) {
 }
 
 inline hipError_t launch_gemm_i8_lds_list(hipStream_t stream, hipEvent_t stop, int shape,
-                                          const I8Product *prods, int n) {
+                                          const I8Product *prods, int n, bool fma = false) {
     if (n <= 0 || n > I8_MAX_DESCS) {
         return hipErrorInvalidValue;
+    }
+    if (fma) {
+        switch (shape) {
+        case 0: return launch_i8_lds_cfg<1, 4, 8, 1, 1, true>(stream, stop, prods, n);
+        case 1: return launch_i8_lds_cfg<1, 4, 4, 2, 1, true>(stream, stop, prods, n);
+        case 2: return launch_i8_lds_cfg<1, 4, 4, 3, 1, true>(stream, stop, prods, n);
+        case 3: return launch_i8_lds_cfg<1, 4, 4, 4, 1, true>(stream, stop, prods, n);
+        case 4: return launch_i8_lds_cfg<2, 2, 2, 4, 4, true>(stream, stop, prods, n);
+        default: return hipErrorInvalidValue;
+        }
     }
     switch (shape) {
     case 0: return launch_i8_lds_cfg<1, 4, 8, 1, 1>(stream, stop, prods, n);

@@ -477,7 +477,8 @@ enum Variant : uint8_t {
                   // p0 = tokens per tile / 64
     V_I8_TILE,    // register-fed int8 MFMA GEMM: p0 = tile configuration
     V_I8_STREAM,  // int8 streaming kernel: p0 = tokens per pass
-    V_I8_LDS,     // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (q8::i8_lds_shape)
+    V_I8_LDS,     // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (q8::i8_lds_shape),
+                  // p1 = 1: the term goes into the sum fused (tm_hip_q8_0_gemm_i8_fma)
     V_F16         // F16-weight list kernel: p0 = tokens per sweep, flag = every row 16-byte aligned
 };
 
@@ -530,8 +531,15 @@ bool bx3_admissible(const Op &op) {
            (uint64_t)op.batch * op.cols < (1ull << 30);
 }
 
+// The most a product can need of the workspace, however its launch is cut
+// (q8::bx3_plan_launch decides the chunks once the launch's list is known).
+q8::Bx3Plan bx3_plan_bound(const Op &op, uint32_t tile_tokens) {
+    return q8::bx3_plan_chunked(op.rows, op.cols, op.batch, tile_tokens,
+                                q8::bx3_chunk_cap(op.rows, op.cols, op.batch, tile_tokens));
+}
+
 bool bx3_fits(const Op &op, uint32_t tile_tokens) {
-    const q8::Bx3Plan plan = q8::bx3_plan_with(op.rows, op.cols, op.batch, tile_tokens);
+    const q8::Bx3Plan plan = bx3_plan_bound(op, tile_tokens);
     return plan.split_tiles <= q8::BX3_MAX_SPLIT_TILES && plan.partial_floats <= kBx3MaxPartialFloats;
 }
 
@@ -577,6 +585,7 @@ GemvKey gemv_key(const Op &op) {
             small_regions) {
             k.variant = V_I8_LDS;
             k.p0 = (uint8_t)q8::i8_lds_shape(op.batch);
+            k.p1 = (uint8_t)(op.extra & 1u); // the fused tail (the other int8 kernels have none)
         } else if (op.packed && op.batch <= q8::GEMV_I8_MAX_BATCH) {
             k.variant = V_I8_STREAM;
             k.p0 = (uint8_t)q8::gemv_i8_tokens(op.batch);
@@ -839,8 +848,11 @@ struct Launch {
     const Op *norm = nullptr;         // an RMSNorm fused in front of the flagged entries
     GemvKey key{};
     const Op *single = nullptr;
-    // V_BF16X3: what the listed products need of the context's workspace
+    // V_BF16X3: what the listed products need of the context's workspace (while
+    // the launch is open, the most they can need; exact once cut_bx3_launch has
+    // decided the K chunks of every product, `bx3_chunks`, per list entry)
     uint64_t bx3_split_tiles = 0, bx3_partial_floats = 0, bx3_xs_bytes = 0;
+    InlineVec<uint8_t, 4> bx3_chunks;
     int bx3_inputs = 0;
     uint32_t descs = 0; // descriptors the listed products take (token groups count one each)
     uint32_t token_descs = 0; // the same at one descriptor per product and token
@@ -888,7 +900,8 @@ hipError_t launch_mma_list(tm_hip_ctx *ctx, hipEvent_t stop, const OpList &ops,
 hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launch,
                            const Workspace &ws) {
     const OpList &ops = launch.list;
-    if (launch.bx3_xs_bytes > ws.xs_bytes || launch.bx3_partial_floats * 4u > ws.partial_bytes) {
+    if (launch.bx3_chunks.size() != ops.size() || launch.bx3_xs_bytes > ws.xs_bytes ||
+        launch.bx3_partial_floats * 4u > ws.partial_bytes) {
         return hipErrorInvalidValue;
     }
     q8::SplitInput inputs[q8::SPLIT_MAX_DESCS];
@@ -911,9 +924,10 @@ hipError_t launch_bx3_list(tm_hip_ctx *ctx, hipEvent_t stop, const Launch &launc
             xs_used += bx3_xs_bytes_of(*op);
             ++n_in;
         }
-        prods[n++] = q8::Bx3Product{(const uint8_t *)op->a[0]->ptr, inputs[at].xs,
-                                    (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
-                                    op->batch};
+        prods[n] = q8::Bx3Product{(const uint8_t *)op->a[0]->ptr, inputs[at].xs,
+                                  (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
+                                  op->batch, launch.bx3_chunks[(size_t)n]};
+        ++n;
     }
     // Inputs that the launch before this one has split already stay out of the
     // split pass (none left: no split pass).
@@ -989,7 +1003,7 @@ hipError_t launch_i8_list(tm_hip_ctx *ctx, hipEvent_t stop, const OpList &ops,
                                    op->rows, op->cols, op->batch};
     }
     if (key.variant == V_I8_LDS) {
-        return q8::launch_gemm_i8_lds_list(ctx->stream, stop, key.p0, prods, n);
+        return q8::launch_gemm_i8_lds_list(ctx->stream, stop, key.p0, prods, n, key.p1 != 0);
     }
     if (key.variant == V_I8_STREAM) {
         return q8::launch_gemv_i8_list(ctx->stream, stop, key.flag, key.p0, prods, n);
@@ -1513,6 +1527,32 @@ std::vector<GemvKey> assign_mma_keys(tm_hip_ctx *ctx, const std::vector<Op> &ops
     return keys;
 }
 
+// The K chunks of a bf16-matrix-core launch, decided for the launch as a whole
+// once its list is known, and what it then needs of the workspace.
+void cut_bx3_launch(Launch &l) {
+    if (l.single != nullptr || l.key.variant != V_BF16X3) {
+        return;
+    }
+    q8::Bx3Shape3 shapes[q8::BX3_MAX_DESCS];
+    uint32_t chunks[q8::BX3_MAX_DESCS];
+    const int n = (int)l.list.size();
+    for (int i = 0; i < n; ++i) {
+        shapes[i] = q8::Bx3Shape3{l.list[i]->rows, l.list[i]->cols, l.list[i]->batch};
+    }
+    const uint32_t tile = l.key.p0 * 64u;
+    q8::bx3_plan_launch(shapes, n, tile, chunks);
+    l.bx3_chunks.clear();
+    l.bx3_split_tiles = 0;
+    l.bx3_partial_floats = 0;
+    for (int i = 0; i < n; ++i) {
+        const q8::Bx3Plan p = q8::bx3_plan_chunked(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile,
+                                                  chunks[i]);
+        l.bx3_chunks.push_back((uint8_t)p.chunks);
+        l.bx3_split_tiles += p.split_tiles;
+        l.bx3_partial_floats += p.partial_floats;
+    }
+}
+
 // A bf16-matrix-core launch reads its activations in split form, which a pass
 // of its own makes first: a dependent launch of about 5 us. Where the launch
 // right before it is the RMSNorm or gated activation that writes those
@@ -1663,7 +1703,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                     new_input = new_input && !same_input(*other, op);
                 }
                 // the launch's share of the workspace stays within its limits
-                const q8::Bx3Plan mine = q8::bx3_plan_with(op.rows, op.cols, op.batch, key.p0 * 64u);
+                const q8::Bx3Plan mine = bx3_plan_bound(op, key.p0 * 64u);
                 conflict = conflict ||
                            cur.bx3_split_tiles + mine.split_tiles > q8::BX3_MAX_SPLIT_TILES ||
                            cur.bx3_partial_floats + mine.partial_floats > kBx3MaxPartialFloats ||
@@ -1679,7 +1719,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
                 new_input = true;
             }
             if (key.variant == V_BF16X3) {
-                const q8::Bx3Plan mine = q8::bx3_plan_with(op.rows, op.cols, op.batch, key.p0 * 64u);
+                const q8::Bx3Plan mine = bx3_plan_bound(op, key.p0 * 64u);
                 cur.bx3_split_tiles += mine.split_tiles;
                 cur.bx3_partial_floats += mine.partial_floats;
                 if (new_input) {
@@ -1800,6 +1840,9 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
         }
     }
     flush();
+    for (Launch &l : plan) {
+        cut_bx3_launch(l);
+    }
     fuse_split_passes(plan);
     return plan;
 }
@@ -2899,9 +2942,7 @@ int tm_hip_q8_0_gemm_mma_noalloc(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffe
     launch.normed.push_back(false);
     bool counters = launch.key.kind == OP_MMA; // the work-queue form of the f32 kernel may run
     if (launch.key.variant == V_BF16X3) {
-        const q8::Bx3Plan plan = q8::bx3_plan_with(rows, cols, batch, launch.key.p0 * 64u);
-        launch.bx3_split_tiles = plan.split_tiles;
-        launch.bx3_partial_floats = plan.partial_floats;
+        cut_bx3_launch(launch);
         launch.bx3_xs_bytes = bx3_xs_bytes_of(op);
         launch.bx3_inputs = 1;
         if (launch.bx3_xs_bytes > ctx->fixed.xs_bytes ||
@@ -2914,7 +2955,7 @@ int tm_hip_q8_0_gemm_mma_noalloc(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffe
                         (unsigned long long)(launch.bx3_partial_floats * 4u), ctx->fixed.xs_bytes,
                         ctx->fixed.partial_bytes);
         }
-        counters = plan.split_tiles > 0;
+        counters = launch.bx3_split_tiles > 0;
     }
     if (ctx->noalloc_keep.size() + 3u > kNoallocKeepCap) {
         return fail(err, err_cap, TM_HIP_ERR_UNSUPPORTED,
@@ -3244,9 +3285,10 @@ int tm_hip_q8_0_quantize_act(tm_hip_ctx *ctx, tm_hip_buffer *x, tm_hip_buffer *x
     return submit(ctx, op, "q8_0_quantize_act", err, err_cap);
 }
 
-int tm_hip_q8_0_gemm_i8(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm_hip_buffer *y,
-                        tm_hip_buffer *sumi, uint32_t rows, uint32_t cols, uint32_t batch,
-                        uint32_t y_off, char *err, size_t err_cap) {
+// `fused_tail`: the declared fast variant (tm_hip_q8_0_gemm_i8_fma).
+static int gemm_i8_submit(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm_hip_buffer *y,
+                          tm_hip_buffer *sumi, uint32_t rows, uint32_t cols, uint32_t batch,
+                          uint32_t y_off, bool fused_tail, char *err, size_t err_cap) {
     if (check_ctx(ctx, err, err_cap, "q8_0_gemm_i8") != TM_HIP_OK) {
         return TM_HIP_ERR_UNSUPPORTED;
     }
@@ -3292,7 +3334,20 @@ int tm_hip_q8_0_gemm_i8(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm
     op.batch = batch;
     op.y_off = y_off;
     op.packed = w->alloc->packed;
-    return submit(ctx, op, "q8_0_gemm_i8", err, err_cap);
+    op.extra = fused_tail ? 1u : 0u;
+    return submit(ctx, op, fused_tail ? "q8_0_gemm_i8_fma" : "q8_0_gemm_i8", err, err_cap);
+}
+
+int tm_hip_q8_0_gemm_i8(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm_hip_buffer *y,
+                        tm_hip_buffer *sumi, uint32_t rows, uint32_t cols, uint32_t batch,
+                        uint32_t y_off, char *err, size_t err_cap) {
+    return gemm_i8_submit(ctx, w, xq, y, sumi, rows, cols, batch, y_off, false, err, err_cap);
+}
+
+int tm_hip_q8_0_gemm_i8_fma(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffer *xq, tm_hip_buffer *y,
+                            uint32_t rows, uint32_t cols, uint32_t batch, uint32_t y_off, char *err,
+                            size_t err_cap) {
+    return gemm_i8_submit(ctx, w, xq, y, nullptr, rows, cols, batch, y_off, true, err, err_cap);
 }
 
 // -------------------------------------------------------- measurement ----

@@ -512,6 +512,15 @@ class HipContext {
         });
     }
 
+    // The declared fast variant: exact block dots, each term fused into the sum.
+    void q8_0_gemm_i8_fma(const HipBuffer &w, const HipBuffer &xq, const HipBuffer &y, uint32_t rows,
+                          uint32_t cols, uint32_t batch, uint32_t y_off) const {
+        operate("q8_0_gemm_i8_fma", [&](char *e) {
+            return tm_hip_q8_0_gemm_i8_fma(raw(), w.raw(), xq.raw(), y.raw(), rows, cols, batch, y_off,
+                                           e, ERR_CAP);
+        });
+    }
+
     uint64_t committed_dispatches() const { return tm_hip_committed_dispatches(raw()); }
     uint64_t completed_dispatches() const { return tm_hip_completed_dispatches(raw()); }
     double last_gpu_ms() const { return tm_hip_last_gpu_ms(raw()); }
@@ -649,6 +658,10 @@ class Matrix {
     uint32_t type_id = 8;
     uint64_t in_dim = 0, out_dim = 0;
     NumericalProfile profile = NumericalProfile::OracleF32;
+    // llama-cpu only, off unless the caller sets it: the int8 products take
+    // tm_hip_q8_0_gemm_i8_fma (exact block dots, fused f32 tail: within 1e-5 of the
+    // CPU's result instead of bit-identical to it, faster from 5 tokens).
+    bool fused_i8_tail = false;
 
   private:
     // forward.rs:783-821 on the device: quantize the activations once per
@@ -666,7 +679,11 @@ class Matrix {
                 xq = gpu.buffer(need, true);
             }
             gpu.q8_0_quantize_act(x, xq, cols, n, t0 * cols);
-            gpu.q8_0_gemm_i8(buf, xq, y, rows, cols, n, t0 * rows);
+            if (fused_i8_tail) {
+                gpu.q8_0_gemm_i8_fma(buf, xq, y, rows, cols, n, t0 * rows);
+            } else {
+                gpu.q8_0_gemm_i8(buf, xq, y, rows, cols, n, t0 * rows);
+            }
             t0 += n;
         }
     }

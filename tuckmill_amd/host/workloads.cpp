@@ -26,7 +26,8 @@ enum {
     TMH_AXPY = 7,     // y += x (alpha = 1), w unused (pass y)
     TMH_ARGMAX = 8,   // x -> y[0], w = 512 bytes of scratch
     TMH_F16_GEMM = 9, // w holds rows*cols f16 values
-    TMH_GELU_MUL = 10 // as TMH_SILU_MUL with ggml's tanh GELU
+    TMH_GELU_MUL = 10, // as TMH_SILU_MUL with ggml's tanh GELU
+    TMH_GEMM_I8_FMA = 11 // as TMH_GEMM_I8 through the declared fast variant
 };
 
 struct tmh_product {
@@ -60,6 +61,7 @@ static void issue(const HipContext &gpu, const tmh_product *p, const std::vector
         case TMH_GEMM: gpu.q8_0_gemm(w, x, y, q.rows, q.cols, q.batch, 0, 0); break;
         case TMH_GEMM_MMA: gpu.q8_0_gemm_mma(w, x, y, q.rows, q.cols, q.batch, 0, 0); break;
         case TMH_GEMM_I8: gpu.q8_0_gemm_i8(w, x, y, q.rows, q.cols, q.batch, 0); break;
+        case TMH_GEMM_I8_FMA: gpu.q8_0_gemm_i8_fma(w, x, y, q.rows, q.cols, q.batch, 0); break;
         case TMH_QUANT: gpu.q8_0_quantize_act(x, y, q.cols, q.batch, 0); break;
         case TMH_RMSNORM: gpu.rmsnorm(x, w, y, q.rows, q.cols, 1e-6f); break;
         case TMH_SILU_MUL: gpu.silu_mul(w, x, y, q.cols); break;
