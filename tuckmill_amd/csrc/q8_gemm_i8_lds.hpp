@@ -59,7 +59,7 @@ __device__ __forceinline__ uint32_t i8_swz(uint32_t r, uint32_t p) {
 // operations per output and block instead of four): within 1e-5 of the CPU's
 // result, not its bits.
 template <int WM, int WN, int KS, int TM = 4, int TN = 4, bool FMA = false>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_i8_lds_kernel(const I8Args args) {
+__global__ __launch_bounds__(WM * WN * 64, 2) void gemm_i8_lds_kernel(const I8Args args) {
     using Sh = I8LdsShape<WM, WN, KS, TM, TN>;
     constexpr int NW = WM * WN; // 16x16 tiles per wave: 16*TM tokens x 16*TN rows
     // two stage buffers as separate objects (reads of one provably do not alias
