@@ -22,22 +22,41 @@ DEVICE_FLAGS = [
 ]
 
 
+# The library is two translation units: the host logic (tm_hip.cpp: no device
+# code, seconds to compile) and the kernels with their launchers (tm_launch.cpp).
+SOURCES = ("tm_hip.cpp", "tm_launch.cpp")
+
+
 def build_library(verbose: bool = False, extra: list[str] | None = None) -> str:
-    cmd = [HIPCC, "-x", "hip", "-std=c++17", "-O3", "-fPIC", "-shared",
-           "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
-           *DEVICE_FLAGS,
-           "-I", os.path.join(ROOT, "include"), "-I", CSRC,
-           *(extra or []),
-           "-o", LIB, os.path.join(CSRC, "tm_hip.cpp")]
+    from concurrent.futures import ThreadPoolExecutor
+
+    common = [HIPCC, "-x", "hip", "-std=c++17", "-O3", "-fPIC",
+              "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
+              *DEVICE_FLAGS,
+              "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+              *(extra or [])]
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        out = "\n".join(l for l in (res.stdout + res.stderr).splitlines()
+                        if "packed-fp32-ops" not in l and l.strip())
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
+        return out
+
+    objs = [os.path.join(objdir, src.replace(".cpp", ".o")) for src in SOURCES]
+    with ThreadPoolExecutor(max_workers=len(SOURCES)) as pool:
+        outs = list(pool.map(run, [[*common, "-c", "-o", obj, os.path.join(CSRC, src)]
+                                   for src, obj in zip(SOURCES, objs)]))
+    outs.append(run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB, *objs]))
     if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    out = "\n".join(l for l in (res.stdout + res.stderr).splitlines()
-                    if "packed-fp32-ops" not in l and l.strip())
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
-    if verbose and out:
-        print(out)
+        for out in outs:
+            if out:
+                print(out)
     return LIB
 
 

@@ -21,8 +21,6 @@ namespace q8 {
 
 typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
-constexpr uint32_t F16_GEMM_MAX_BATCH = 32; // native/metal/tm_metal.m:1279-1283 (max_batch 32)
-
 __device__ __forceinline__ float f16_lo(uint32_t v) { return f16_bits_to_f32(v & 0xffffu); }
 __device__ __forceinline__ float f16_hi(uint32_t v) { return f16_bits_to_f32(v >> 16); }
 
@@ -201,8 +199,6 @@ __global__ __launch_bounds__(256) void f16_row_indirect_kernel(const uint16_t *_
     const uint32_t row = ids[slot];
     out[i] = row < rows ? f16_bits_to_f32(w[(size_t)row * cols + i]) : 0.0f;
 }
-
-inline int f16_tokens(uint32_t batch) { return batch == 1u ? 1 : (batch == 2u ? 2 : (batch <= 4u ? 4 : 8)); }
 
 // About 16 KiB of weights per wave, at least one pass of 8 rows; a matrix that
 // would give fewer than 1024 tiles gets one-pass tiles so that it still spreads.

@@ -11,6 +11,8 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
+#include "q8_plan.hpp"
+
 // Launch with an optional stop event attached to the dispatch itself: the
 // event completes with the kernel and costs no extra packet on the stream
 // (a separate hipEventRecord after each launch measured +3 us per launch).

@@ -49,8 +49,6 @@ struct SplitDesc {
     uint32_t pad;
 };
 
-constexpr int SPLIT_MAX_DESCS = 16;
-
 struct SplitArgs {
     uint32_t n;
     uint32_t pad;
@@ -97,10 +95,6 @@ struct Bx3Desc {
     uint32_t part_begin; // first arrival counter of this product (one per output tile)
     uint32_t part_tile;  // first partial tile of this product in `partials`
 };
-
-constexpr int BX3_MAX_DESCS = 64;
-constexpr uint32_t BX3_CHUNK_BLOCKS = 16;   // K is cut into chunks of 512 columns or more
-constexpr uint32_t BX3_MAX_SPLIT_TILES = 16384; // arrival counters per context
 
 struct Bx3Args {
     uint32_t n;
@@ -611,346 +605,6 @@ struct Bx3Product {
     uint32_t rows, cols, batch;
     uint32_t chunks; // K chunks of this product, as bx3_plan_launch cut the launch
 };
-
-// How a product is cut into work units (output tile x K chunk): a function of
-// the product's shape and of the tile its launch uses.
-//
-// Tile: 256 rows x 128 tokens (2 x 4 waves, two per SIMD), or x 64 tokens (1 x 4
-// waves, one per SIMD) for some products that would make fewer than 192 units
-// of the large tile (bx3_plan below). Measured alone, the small tile is 1.1-1.6 times as fast on such
-// products (4096 x 1024 at 512 tokens: 35 against 40 us, 6144 x 2048 at 128
-// tokens: 33 us against 48 on the f32 kernel) and 10-25 % slower on large ones
-// (a quarter more operand bytes per product).
-//
-// K chunks: a product with few output tiles cuts K into at most BX3_MAX_CHUNKS
-// chunks of 512 columns or more, as many as it takes to give the chip about
-// BX3_UNITS_WANTED work units; one with many tiles does not cut K at all
-// (14336 x 4096 at 512 tokens: 295 TFLOP/s whole, less in chunks). Measured
-// alone with the large tile: chunks of 512 instead of 1024 columns make
-// 6144 x 2048 at 256 tokens 47 us instead of 59 (f32 kernel: 69) and 8192 x 1024
-// at 512 tokens 49 instead of 56 (f32: 93); chunks of 256 columns and less made
-// the 0.6B projections slower, alone and together.
-constexpr uint32_t BX3_TILE_ROWS = 256;
-constexpr uint32_t BX3_UNITS_WANTED = 192;
-constexpr uint32_t BX3_MAX_CHUNKS = 8;
-
-struct Bx3Plan {
-    uint32_t tile_tokens;  // 128 or 64
-    uint32_t chunk_blocks; // Q8_0 blocks per K chunk
-    uint32_t chunks;
-    uint64_t tiles;        // output tiles
-    uint64_t units;        // tiles x chunks
-    uint64_t split_tiles;  // tiles that need an arrival counter (chunks > 1)
-    uint64_t partial_floats; // floats of partial tiles (chunks > 1)
-};
-
-inline Bx3Plan bx3_plan_with(uint32_t rows, uint32_t cols, uint32_t batch, uint32_t tile_tokens) {
-    Bx3Plan p;
-    p.tile_tokens = tile_tokens;
-    const uint32_t blocks = cols / 32u;
-    p.tiles = (uint64_t)((batch + tile_tokens - 1u) / tile_tokens) *
-              ((rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS);
-    uint32_t most = (blocks + BX3_CHUNK_BLOCKS - 1u) / BX3_CHUNK_BLOCKS;
-    most = most < BX3_MAX_CHUNKS ? most : BX3_MAX_CHUNKS;
-    const uint64_t want = (BX3_UNITS_WANTED + p.tiles - 1u) / p.tiles;
-    const uint32_t chunks = want < most ? (uint32_t)want : most;
-    p.chunk_blocks = (blocks + chunks - 1u) / chunks;
-    p.chunks = (blocks + p.chunk_blocks - 1u) / p.chunk_blocks;
-    p.units = p.tiles * p.chunks;
-    p.split_tiles = p.chunks > 1u ? p.tiles : 0u;
-    p.partial_floats = p.split_tiles * p.chunks * tile_tokens * BX3_TILE_ROWS;
-    return p;
-}
-
-// ---- K chunks: decided per launch ------------------------------------------
-//
-// What bx3_plan_with says about a product's chunks is what the product would get
-// alone; bx3_launch_tile keeps using those unit counts as its measure of "enough
-// work". How the products of a launch are actually cut is decided for the launch
-// as a whole, because a work unit has a fixed cost that 16-block chunks pay too
-// often: measured (1024 units of one product at 512 tokens, K = 512 ... 4096)
-// a unit takes about 6 us plus 1.43 us per Q8_0 block, and a unit of a chunked
-// tile about 10 us more (its 128 KiB partial tile goes to memory and comes back;
-// a whole round of them is 33 MB at once). The seven projections of a Qwen3-0.6B
-// layer at 512 tokens, each cut as if alone, were 480 units of 16 blocks, two
-// rounds of the chip and 61 MB of partial tiles: 82 us. Cut for the launch they
-// are 240 units of 32 blocks, one round, the five K = 1024 products whole: 66 us.
-//
-// The rule: every product gets chunks_i = ceil(blocks_i / L) (at most
-// bx3_chunk_cap) for one target length L per launch; L runs over the lengths at
-// which some product's chunk count changes, each candidate is priced by handing
-// its units, longest first (the kernel's order), to the chip's workgroup slots
-// as they come free, and the cheapest wins (ties: fewer units).
-struct Bx3Shape3 {
-    uint32_t rows, cols, batch;
-};
-
-// At most eight chunks, none below 512 columns, and no more than it takes to
-// give a product about two rounds of units on its own: a product with many
-// output tiles is never cut.
-inline uint32_t bx3_chunk_cap(uint32_t rows, uint32_t cols, uint32_t batch, uint32_t tile_tokens) {
-    const uint32_t blocks = cols / 32u;
-    const uint64_t tiles = (uint64_t)((batch + tile_tokens - 1u) / tile_tokens) *
-                           ((rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS);
-    uint32_t cap = blocks / BX3_CHUNK_BLOCKS;
-    cap = cap < BX3_MAX_CHUNKS ? cap : BX3_MAX_CHUNKS;
-    const uint64_t by_tiles = (2u * 256u + tiles - 1u) / tiles;
-    cap = by_tiles < cap ? (uint32_t)by_tiles : cap;
-    return cap < 1u ? 1u : cap;
-}
-
-// The plan of a product cut into `chunks` chunks (as many as bx3_plan_launch gave it).
-inline Bx3Plan bx3_plan_chunked(uint32_t rows, uint32_t cols, uint32_t batch, uint32_t tile_tokens,
-                                uint32_t chunks) {
-    Bx3Plan p;
-    p.tile_tokens = tile_tokens;
-    const uint32_t blocks = cols / 32u;
-    p.tiles = (uint64_t)((batch + tile_tokens - 1u) / tile_tokens) *
-              ((rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS);
-    chunks = chunks < 1u ? 1u : chunks;
-    p.chunk_blocks = (blocks + chunks - 1u) / chunks;
-    p.chunks = (blocks + p.chunk_blocks - 1u) / p.chunk_blocks;
-    p.units = p.tiles * p.chunks;
-    p.split_tiles = p.chunks > 1u ? p.tiles : 0u;
-    p.partial_floats = p.split_tiles * p.chunks * tile_tokens * BX3_TILE_ROWS;
-    return p;
-}
-
-// Estimated duration (ns) of a launch whose products are cut as `chunks` says:
-// units in descending length to `slots` workgroup slots, each to the slot that
-// comes free first. Units of one product are alike, so the slots are tracked as
-// groups that come free together.
-inline uint64_t bx3_price(const Bx3Shape3 *shapes, const uint32_t *chunks, int n,
-                          uint32_t tile_tokens) {
-    const uint32_t slots = tile_tokens == 128u ? 256u : 512u;
-    const uint64_t unit_ns = tile_tokens == 128u ? 6000u : 4500u;
-    const uint64_t block_ns = tile_tokens == 128u ? 1430u : 1100u;
-    const uint64_t chunked_ns = tile_tokens == 128u ? 10000u : 5000u;
-    struct Kind {
-        uint64_t ns, units;
-    };
-    Kind kinds[BX3_MAX_DESCS];
-    for (int i = 0; i < n; ++i) { // insertion sort, longest first
-        const Bx3Plan p = bx3_plan_chunked(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens,
-                                           chunks[i]);
-        const Kind k{unit_ns + block_ns * p.chunk_blocks + (p.chunks > 1u ? chunked_ns + 1000u * p.chunks : 0u),
-                     p.units};
-        int at = i;
-        while (at > 0 && kinds[at - 1].ns < k.ns) {
-            kinds[at] = kinds[at - 1];
-            --at;
-        }
-        kinds[at] = k;
-    }
-    struct Group {
-        uint64_t free_at, count;
-    };
-    constexpr int MAX_GROUPS = 4 * BX3_MAX_DESCS + 4;
-    Group groups[MAX_GROUPS]; // ascending free_at
-    int ng = 1;
-    groups[0] = Group{0u, slots};
-    uint64_t end = 0;
-    for (int i = 0; i < n; ++i) {
-        uint64_t left = kinds[i].units;
-        while (left > 0) {
-            // whole rounds of every slot at once when the class is large
-            if (ng == 1 && left >= groups[0].count) {
-                const uint64_t rounds = left / groups[0].count;
-                groups[0].free_at += rounds * kinds[i].ns;
-                left -= rounds * groups[0].count;
-                end = groups[0].free_at > end ? groups[0].free_at : end;
-                continue;
-            }
-            const uint64_t take = left < groups[0].count ? left : groups[0].count;
-            const uint64_t done = groups[0].free_at + kinds[i].ns;
-            end = done > end ? done : end;
-            groups[0].count -= take;
-            left -= take;
-            if (groups[0].count == 0) { // drop it
-                for (int g = 1; g < ng; ++g) {
-                    groups[g - 1] = groups[g];
-                }
-                --ng;
-            }
-            // insert (done, take), merging with a group of the same time
-            int at = 0;
-            while (at < ng && groups[at].free_at < done) {
-                ++at;
-            }
-            if (at < ng && groups[at].free_at == done) {
-                groups[at].count += take;
-            } else if (ng < MAX_GROUPS) {
-                for (int g = ng; g > at; --g) {
-                    groups[g] = groups[g - 1];
-                }
-                groups[at] = Group{done, take};
-                ++ng;
-            } else { // (cannot happen with these bounds; stay correct anyway)
-                groups[ng - 1].count += take;
-            }
-        }
-    }
-    return end;
-}
-
-// chunks[i] for every product of a launch (see above). Deterministic: a function
-// of the shapes in list order and the tile.
-inline void bx3_plan_launch(const Bx3Shape3 *shapes, int n, uint32_t tile_tokens, uint32_t *chunks) {
-    uint32_t cap[BX3_MAX_DESCS];
-    uint64_t tiles = 0;
-    bool any = false;
-    for (int i = 0; i < n; ++i) {
-        cap[i] = bx3_chunk_cap(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens);
-        any = any || cap[i] > 1u;
-        chunks[i] = 1u;
-        tiles += bx3_plan_chunked(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens, 1u).tiles;
-    }
-    if (!any || tiles >= 1024u) {
-        return; // nothing to cut, or rounds enough as it is
-    }
-    // candidate lengths: where some product's chunk count changes
-    uint32_t lengths[BX3_MAX_DESCS * BX3_MAX_CHUNKS];
-    int nl = 0;
-    for (int i = 0; i < n; ++i) {
-        const uint32_t blocks = shapes[i].cols / 32u;
-        for (uint32_t c = 1; c <= cap[i]; ++c) {
-            const uint32_t len = (blocks + c - 1u) / c;
-            bool seen = false;
-            for (int j = 0; j < nl; ++j) {
-                seen = seen || lengths[j] == len;
-            }
-            if (!seen) {
-                lengths[nl++] = len;
-            }
-        }
-    }
-    uint64_t best_ns = ~0ull, best_units = ~0ull;
-    uint32_t trial[BX3_MAX_DESCS];
-    for (int j = 0; j < nl; ++j) {
-        uint64_t units = 0;
-        for (int i = 0; i < n; ++i) {
-            const uint32_t blocks = shapes[i].cols / 32u;
-            uint32_t c = (blocks + lengths[j] - 1u) / lengths[j];
-            c = c > cap[i] ? cap[i] : c;
-            trial[i] = c;
-            units += bx3_plan_chunked(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens, c).units;
-        }
-        const uint64_t ns = bx3_price(shapes, trial, n, tile_tokens);
-        if (ns < best_ns || (ns == best_ns && units < best_units)) {
-            best_ns = ns;
-            best_units = units;
-            for (int i = 0; i < n; ++i) {
-                chunks[i] = trial[i];
-            }
-        }
-    }
-}
-
-// Which tile the products of one launch take together, or 0 when the kernel does
-// not pay for them: the rule of a single product, with the launch's sums in the
-// place of the product's own figures (`shapes` = rows, cols, batch of every
-// product; all with batch <= 32, all with 33..64, or all above).
-//
-// Up to 64 tokens there is one small tile of tokens. The kernel's time hardly
-// depends on the batch here (27 us for 8192 x 1024, 97 us for 151936 x 1024), the
-// f32 kernel's does: from 33 tokens (its 64-token tile) 16 M weights are the
-// break-even (16384 x 1024 at 64 tokens: 30 against 29 us; 4096 x 4096: 34 against
-// 47; 151936 x 1024: 97 against 219). At 32 tokens and below only the largest
-// matrices would gain, and little: from 17 tokens (below, the exact small-batch
-// kernel serves the entry point) the bar is 32 M weights.
-//
-// Above 64 tokens, in order of preference: the large tile with 192 units or more;
-// the small tile with 192 units or more, in however many K chunks (alone, split
-// pass included: 1024 x 4096 at 512 tokens in six chunks 37 us, against 47 on the
-// large tile and 46 on the f32 kernel; 896 x 4864 39 against 51; 2048 x 4096 at 256
-// tokens 35 against 45; 1024 x 3072 at 512 tokens 33 against 31 on the f32 kernel,
-// 28 when the gated activation in front of it has written its split form; the
-// seven Qwen3-0.6B projections at 128 tokens 34 us against 54 on the f32
-// kernels); the large tile with 128 units or more (a product alone is then
-// about even with the f32 kernel, products that share a launch far ahead);
-// the small tile again for products of 3072 columns and more with at least 32
-// units (alone, at 128 tokens: 1024 x 3072 29 us against 34 on the f32 kernel,
-// 1024 x 4096 32 against 44, 1152 x 6912 38 against 71, 1536 x 8960 45 against 90;
-// at 256 tokens 1024 x 4096 34 against 39; 2048 columns lose, 27 against 24). Measured alone at 512 tokens
-// against the f32 kernel: small tile 3072 x 1024 34 against 35 us, 2048 x 2048 39
-// against 49, 4096 x 1024 36 against 48, 2048 x 1024 (128 units) 31 against 28;
-// large tile 8192 x 1024 49 against 93, 6144 x 2048 69 against 133. Together: the
-// seven Qwen3-0.6B projections at 512 tokens 78 us on the large tile against 144
-// on the f32 kernel.
-inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
-    if (n <= 0) {
-        return 0;
-    }
-    uint64_t large = 0, small = 0, weights = 0;
-    uint32_t least_cols = shapes[0].cols;
-    for (int i = 0; i < n; ++i) {
-        least_cols = shapes[i].cols < least_cols ? shapes[i].cols : least_cols;
-        small += bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 64u).units;
-        large += bx3_plan_with(shapes[i].rows, shapes[i].cols, shapes[i].batch, 128u).units;
-        weights += (uint64_t)shapes[i].rows * shapes[i].cols;
-    }
-    if (shapes[0].batch <= 32u) {
-        // half of the one token tile is padding: only twice the weights pay (the
-        // f32 kernel's own tile is 32 tokens here; 20 x (6144 x 2048 + 2048 x 6144) at
-        // 32 tokens: 385 us on the f32 kernels, about 300 us here)
-        return weights >= (1ull << 25) && small >= 128u ? 64u : 0u;
-    }
-    if (shapes[0].batch <= 64u) {
-        return weights >= (1ull << 24) && small >= 128u ? 64u : 0u;
-    }
-    if (large >= BX3_UNITS_WANTED) {
-        return 128u;
-    }
-    if (small >= BX3_UNITS_WANTED) {
-        return 64u;
-    }
-    if (large >= 128u) {
-        return 128u;
-    }
-    // Few output tiles under a deep K: this kernel cuts K into chunks and takes
-    // 22.5 + 2.3 us per 1024 columns, its split pass included. A wave of the f32
-    // kernel takes 0.72 us per block of a 32-token tile (twice that for 64
-    // tokens) after 4.5 us, over K divided by its 4 waves and by the workgroups
-    // that share a tile (q8::mma_shared_parts), once per round of 256
-    // workgroups: 1024 x 3072 at 128 tokens 14.8 us against 29.1 here, 1024 x 4096
-    // at 192 tokens 26.4 against 33.1, but 1152 x 6912 at 128 tokens 42.0 against
-    // 37.9 and 2048 x 8192 at 96 tokens 49.0 against 41.3. The cheaper estimate wins.
-    if (least_cols < 3072u || small < 32u) {
-        return 0u;
-    }
-    MmaProduct prods[MMA_MAX_DESCS];
-    const int m = n < MMA_MAX_DESCS ? n : MMA_MAX_DESCS;
-    uint32_t min_blocks = 0xffffffffu, max_blocks = 0;
-    for (int i = 0; i < m; ++i) {
-        prods[i] = MmaProduct{nullptr, nullptr, nullptr, shapes[i].rows, shapes[i].cols, shapes[i].batch};
-        const uint32_t blocks = shapes[i].cols / 32u;
-        min_blocks = blocks < min_blocks ? blocks : min_blocks;
-        max_blocks = blocks > max_blocks ? blocks : max_blocks;
-    }
-    const MmaConfig c = pick_mma_config(prods, m);
-    uint64_t tiles = 0;
-    for (int i = 0; i < m; ++i) {
-        tiles += mma_tiles(prods[i], c);
-    }
-    const uint32_t z = c.s == 4 ? mma_shared_parts(tiles, min_blocks) : 1u;
-    const uint64_t rounds = (tiles * z + 255u) / 256u;
-    const uint64_t per_wave = (max_blocks + 4u * z - 1u) / (4u * z);
-    const uint64_t f32_us_x100 = 450u + 72u * (uint64_t)c.tmw * per_wave * rounds;
-    const uint64_t here_us_x100 = 2250u + 230u * (uint64_t)(max_blocks * 32u) / 1024u;
-    return here_us_x100 < f32_us_x100 ? 64u : 0u;
-}
-
-// A product on its own: its plan, and whether the kernel pays for it (`worth`).
-inline Bx3Plan bx3_plan(uint32_t rows, uint32_t cols, uint32_t batch, bool *worth) {
-    const Bx3Shape3 one{rows, cols, batch};
-    const uint32_t tile = bx3_launch_tile(&one, 1);
-    *worth = tile != 0u;
-    return bx3_plan_with(rows, cols, batch, tile != 0u ? tile : (batch <= 64u ? 64u : 128u));
-}
-inline Bx3Plan bx3_plan(uint32_t rows, uint32_t cols, uint32_t batch) {
-    bool worth;
-    return bx3_plan(rows, cols, batch, &worth);
-}
 
 template <int WM, int WN, int TM, int NS>
 inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3Product *prods_in,

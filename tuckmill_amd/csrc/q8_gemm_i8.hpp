@@ -16,15 +16,6 @@ namespace q8 {
 
 typedef int intx4 __attribute__((ext_vector_type(4)));
 
-// Layout of a quantized-activation buffer for `batch` rows of `cols`:
-//   [batch][cols] int8 quants, then [cols/32][bpad] f32 scales with
-//   bpad = batch rounded up to 4 (block-major, so that the four tokens a lane
-//   rescales per MFMA are one aligned 16-byte load).
-__host__ __device__ inline uint32_t xq_bpad(uint32_t batch) { return (batch + 3u) & ~3u; }
-__host__ __device__ inline size_t xq_bytes(uint32_t cols, uint32_t batch) {
-    return (size_t)batch * cols + (size_t)(cols / 32u) * xq_bpad(batch) * 4u;
-}
-
 // Activation quantizer, crates/tuckcore/src/tensor.rs:184-206: per block of
 // 32, d = amax/127, id = 1/d (0 when d == 0), q = clamp(rte(x*id), +-127),
 // stored scale = f32 value of the f16 rounding of d. One half-wave per block.
@@ -88,8 +79,6 @@ struct I8Desc {
     uint32_t tiles_t;    // token tiles per row tile
     uint32_t pad;
 };
-
-constexpr int I8_MAX_DESCS = 64;
 
 struct I8Args {
     uint32_t n;
@@ -254,13 +243,6 @@ struct I8Product {
     int32_t *sumi;
     uint32_t rows, cols, batch;
 };
-
-// 0: 16 tokens x 64 rows (batch <= 16), 1: 32 x 32 (batch <= 32), 2: 64 x 32,
-// 3: 64 x 64 (large batches: operands are re-read from L2 per wave, so the
-// larger tile halves that traffic per MFMA).
-inline int pick_i8_config(uint32_t batch) {
-    return batch <= 16u ? 0 : (batch <= 32u ? 1 : (batch < 128u ? 2 : 3));
-}
 
 template <int L, int TM, int TN, bool SUMI>
 inline hipError_t launch_i8_cfg(hipStream_t stream, hipEvent_t stop, const I8Product *prods, int n) {

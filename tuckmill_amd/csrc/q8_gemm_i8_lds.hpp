@@ -291,28 +291,6 @@ inline hipError_t launch_i8_lds_cfg(hipStream_t stream, hipEvent_t stop, const I
 
 // Sealed weights, no verification output, every region below 4 GiB (32-bit
 // buffer offsets): the caller checks these before choosing this kernel.
-constexpr uint32_t GEMM_I8_LDS_MIN_BATCH = 5; // below: the streaming kernel (q8_gemv_i8.hpp)
-
-// Workgroup shape for a batch. The bits do not depend on the shape.
-//   0..3  batches up to 256: four waves side by side, each 16 rows for 1..4 token
-//         tiles of 16; larger batches take several such tiles of equal height
-//         (96 tokens: two of 48). While a weight byte is used a few times only,
-//         what counts is the weight stream: whole 128-byte lines per fetched row
-//         piece (stages of 4 blocks; 8 for one token tile, where LDS leaves
-//         room), and many small workgroups per CU so that many stages are in
-//         flight. Measured on 535 MB of 2B-class matrices: M = 128 364 us against
-//         521 us for shape 4, M = 256 671 against 705, M = 512 1273 against 1165.
-//   4     above 256: 2x2 waves over 128 tokens x 128 rows, stages of 2 blocks
-//         (bound by the epilogue's f32 operations, not by the fetch).
-inline int i8_lds_shape(uint32_t batch) {
-    if (batch > 256u) {
-        return 4;
-    }
-    const uint32_t tiles = (batch + 63u) / 64u;
-    const uint32_t per_tile = (batch + tiles - 1u) / tiles;
-    return (int)((per_tile + 15u) / 16u) - 1;
-}
-
 inline hipError_t launch_gemm_i8_lds_list(hipStream_t stream, hipEvent_t stop, int shape,
                                           const I8Product *prods, int n, bool fma = false) {
     if (n <= 0 || n > I8_MAX_DESCS) {

@@ -54,8 +54,6 @@ struct MmaDesc {
     uint32_t pad;
 };
 
-constexpr int MMA_MAX_DESCS = 64;
-
 struct MmaArgs {
     uint32_t n;
     uint32_t total_tiles;
@@ -65,23 +63,6 @@ struct MmaArgs {
     uint32_t *arrivals; // z > 1: one counter per output tile, zero between launches
     MmaDesc d[MMA_MAX_DESCS];
 };
-
-// How many workgroups share each output tile of a launch, each with its own
-// part of K: a launch with few output tiles and a long K otherwise leaves most
-// of the chip idle (1024 x 2048 at 32 tokens is 32 tiles of 64 blocks each).
-// Doubled while the launch's tiles, times it, stay within 256 workgroups and
-// every wave keeps at least 4 blocks of the shortest K. It depends on what
-// shares the launch, and with it the order of a product's f32 sums (the same
-// launch gives the same bits every time).
-constexpr uint32_t MMA_SHARED_MAX_TILES = 128;  // tiles x parts <= 256, parts >= 2
-constexpr size_t MMA_SHARED_PARTIAL_FLOATS = 256u * 2u * 16u * 64u; // 256 partial tiles of 64 x 32
-inline uint32_t mma_shared_parts(uint64_t tiles, uint32_t min_blocks) {
-    uint32_t z = 1;
-    while (z < 8u && tiles * (z * 2u) <= 256u && min_blocks / (4u * z * 2u) >= 4u) {
-        z *= 2u;
-    }
-    return z;
-}
 
 // Operands of one Q8_0 block for a wave's TMW x TNW tiles, as loaded.
 template <int TMW, int TNW> struct MmaRaw {
@@ -717,55 +698,6 @@ __global__ __launch_bounds__(256, 2) void gemm_mma_queue_kernel(const MmaArgs ar
             atomicExch(&queue[1], 0u);
         }
     }
-}
-
-struct MmaConfig {
-    int tmw, tnw, s;
-};
-
-struct MmaProduct {
-    const uint8_t *w;
-    const float *x;
-    float *y;
-    uint32_t rows, cols, batch;
-};
-
-inline uint64_t mma_tiles(const MmaProduct &p, const MmaConfig &c) {
-    return (uint64_t)((p.batch + 32u * c.tmw - 1) / (32u * c.tmw)) *
-           ((p.rows + 32u * c.tnw - 1) / (32u * c.tnw));
-}
-
-// Tile and K split. Measured on MI355X at M = 512 over the Qwen3-0.6B
-// projection shapes, alone and as one list launch: a 64-token x 32-row wave
-// tile with K split over the 4 waves of a workgroup is best or tied
-// everywhere (f32 MFMA is slow enough that filling all 1024 SIMDs with short
-// MFMA streams matters more than operand reuse). Narrow batches use a
-// 32-token tile; K is split no finer than one Q8_0 block per wave.
-inline MmaConfig pick_mma_config(const MmaProduct *prods, int n) {
-    uint32_t max_batch = 0, min_blocks = 0xffffffffu;
-    for (int i = 0; i < n; ++i) {
-        max_batch = prods[i].batch > max_batch ? prods[i].batch : max_batch;
-        const uint32_t blocks = prods[i].cols / 32u;
-        min_blocks = blocks < min_blocks ? blocks : min_blocks;
-    }
-    // Tokens per wave tile: 64, or 32 for narrow batches and for launches whose
-    // last round of workgroups would be less than half full with 64 (the chip
-    // runs 256 of these workgroups at a time; a 32-token tile makes twice the
-    // workgroups, each half as long). Up to 128 output tiles of 64 tokens x 32
-    // rows: 1024 x 2048 at 128 tokens 24 -> 15 us, 1024 x 1024 14 -> 9, 256 x 4096
-    // 43 -> 26, 512 x 2048 at 512 tokens 23 -> 15; 257 to 384 tiles: the 0.6B gate
-    // and up projections together at 128 tokens 27 -> 24; at 192 and at 256 tiles
-    // the 64-token tile is ahead (1536 x 1024 at 256 tokens 14 against 16 us).
-    uint64_t tiles64 = 0;
-    for (int i = 0; i < n; ++i) {
-        tiles64 += (uint64_t)((prods[i].batch + 63u) / 64u) * ((prods[i].rows + 31u) / 32u);
-    }
-    const bool short_last_round = tiles64 <= 128u || (tiles64 > 256u && tiles64 <= 384u);
-    MmaConfig c;
-    c.tmw = max_batch > 32u && !short_last_round ? 2 : 1;
-    c.tnw = 1;
-    c.s = min_blocks >= 4u ? 4 : (min_blocks >= 2u ? 2 : 1);
-    return c;
 }
 
 // Resident workgroups of a 256-thread kernel on the current device (a multiple of 8).

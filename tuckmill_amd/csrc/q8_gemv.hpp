@@ -39,11 +39,6 @@ struct GemvDesc {
     uint32_t pad2;         // the row of the launch's fused RMSNorm that this descriptor reads
 };
 
-// The list travels in the kernel-argument segment (read through the scalar
-// cache): 224 * 64 + 40 = 14376 bytes, enough for a whole decode step of a
-// 28-layer model (197 products) in one launch.
-constexpr int GEMV_MAX_DESCS = 224;
-
 // Descriptor flag bits (GemvDesc::pad): the product's activations are the
 // launch's fused RMSNorm output, and this product's first tile writes it out.
 constexpr uint32_t GEMV_X_NORMED = 1u, GEMV_WRITES_NORM = 2u;
@@ -68,13 +63,6 @@ template <int ND> struct GemvArgsT {
     GemvDesc d[ND];
 };
 using GemvArgs = GemvArgsT<GEMV_MAX_DESCS>;
-
-// Most launches of a real step carry one to three products (q/k/v, gate/up, a
-// lone projection between two dependent operators), at up to four tokens with
-// a descriptor each: they use a short argument block (808 bytes) instead of the
-// 14 KB one, which is copied and fetched per launch (q,k,v at 2 tokens: 6
-// descriptors, a step of 115 such launches 727 -> 718 us).
-constexpr int GEMV_FEW_DESCS = 12;
 
 template <int NB, bool XA>
 __device__ __forceinline__ void load_x(const float *p, float *out) {

@@ -225,12 +225,6 @@ inline hipError_t launch_gemv_i8_cfg(hipStream_t stream, hipEvent_t stop, const 
     return hipGetLastError();
 }
 
-constexpr uint32_t GEMV_I8_MAX_BATCH = 16; // above this the MFMA kernels only
-
-inline int gemv_i8_tokens(uint32_t batch) {
-    return batch == 1u ? 1 : (batch == 2u ? 2 : (batch <= 4u ? 4 : 8));
-}
-
 // Sealed weights only; tb is gemv_i8_tokens(batch) of every product in the list.
 inline hipError_t launch_gemv_i8_list(hipStream_t stream, hipEvent_t stop, bool sumi, int tb,
                                       const I8Product *prods, int n) {

@@ -81,7 +81,6 @@ __global__ __launch_bounds__(256) void copy_f32_kernel(const float *src, float *
 // workgroup, so what it measures is the read path alone: the sustained HBM
 // read bandwidth that the streaming kernels can be set against. `src` is
 // 16-byte aligned.
-constexpr uint32_t CHECKSUM_GROUPS = 2048;
 
 __global__ __launch_bounds__(256) void xor_checksum_kernel(const uint32_t *__restrict__ src,
                                                            uint32_t *__restrict__ partial,

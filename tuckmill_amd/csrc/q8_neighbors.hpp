@@ -139,7 +139,6 @@ __global__ __launch_bounds__(256) void gelu_tanh_mul_kernel(const float *gate, c
 // order, not the CPU's sequential one, hence tolerance-qualified like the
 // reference's own GPU kernel; the GEMV kernel's fused form computes the same
 // bits. In place (x == y) is safe: a lane rereads only what it writes itself.
-constexpr uint32_t RMSNORM_ROWS = 1;
 
 // `add` non-null: the residual update x += alpha * add of the same rows comes
 // first (axpy_kernel's operations: multiply, then add; x is written back), for
@@ -315,8 +314,6 @@ __global__ __launch_bounds__(64 * RMSNORM_ROWS) void rmsnorm_kernel(float *x, co
 // "a is better than b" is a strict total order on (value, index) pairs, so any
 // reduction tree returns the sequential scan's answer.
 constexpr uint32_t ARGMAX_NONE = 0xffffffffu;
-constexpr uint32_t ARGMAX_GROUPS = 64;   // partial results: 64 f32 values, then 64 u32 indices
-constexpr uint32_t ARGMAX_PARTIAL_BYTES = ARGMAX_GROUPS * 8u;
 
 __device__ __forceinline__ bool argmax_better(float av, uint32_t ai, float bv, uint32_t bi) {
     if (ai == ARGMAX_NONE) {
