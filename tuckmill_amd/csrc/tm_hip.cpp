@@ -2362,6 +2362,7 @@ int tm_hip_q8_0_pack(tm_hip_ctx *ctx, tm_hip_buffer *w, uint32_t rows, uint32_t 
     op.writes_mask = 2;
     op.rows = rows;
     op.cols = cols;
+    op.what = "q8_0_pack";
     std::vector<Op> one(1, op);
     rc = commit_ops(ctx, one, "q8_0_pack", "q8_0_pack", err, err_cap);
     // The handle now names the sealed copy; the raw bytes stay leased by the
