@@ -28,7 +28,7 @@ def resource_remarks(tmp_path_factory):
     out = tmp_path_factory.mktemp("resources") / "device.o"
     cmd = [hipcc, "-x", "hip", "-std=c++17", "-O3", *B.DEVICE_FLAGS, "--cuda-device-only",
            "-I", os.path.join(B.ROOT, "include"), "-I", B.CSRC,
-           "-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(B.CSRC, "tm_hip.cpp"),
+           "-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(B.CSRC, "tm_launch.cpp"),
            "-o", str(out)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     assert res.returncode == 0, res.stderr[-2000:]
