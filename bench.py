@@ -47,10 +47,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 # HBM bytes per launch of the decode step's GEMV list kernel, from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in profiles/gemv_list_kernel__decode_step__pmc_traffic.txt
 # (fetch counter x 2.000 + write counter x 1.000, factors from a plain copy kernel).
-DECODE_STEP_TRAFFIC_BYTES = 644.77e6
+DECODE_STEP_TRAFFIC_BYTES = 644.75e6
 DECODE_STEP_TRAFFIC_SOURCE = ("constant from profiles/gemv_list_kernel__decode_step__pmc_traffic.txt "
                               "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --workload "
-                              "traffic` on q8::gemv_list_kernel<1, 8, 1, true, 0, 224, false>); not "
+                              "traffic` on q8::gemv_list_kernel<1, 8, 1, true, 0, 224, false, false>); not "
                               "measured in this run")
 
 
@@ -941,7 +941,8 @@ def run_traffic(host, ctx):
       4. the same over raw weights (gemm_mma kernels, f32 matrix cores)
       5. the Gemma-3-1B vocabulary projection at M = 512 (gemm_bf16x3_kernel)
       6. 2B-class shapes, int8-activation profile at M = 512
-         (quantize_act_kernel + gemm_i8_lds_kernel), 8 copies of each matrix
+         (quantize_act_kernel + gemm_i8_lds_kernel), 8 copies of each matrix, through
+         the bit-exact entry point and then through the one with the fused tail
     Prints the algorithmic bytes / operations of each so that the counter values
     per dispatch can be set beside them."""
     n = 64 << 20  # f32 elements
@@ -994,13 +995,15 @@ def run_traffic(host, ctx):
     xb.upload(0, S.make_activations(M * max(widths), 99))
     xqs = {c: ctx.buffer(H.xq_bytes(c, M)) for c in widths}
     ys = [ctx.buffer(M * r * 4) for _, r, _, _ in pool]
-    prods = [tmh_product(None, xb.raw, xqs[c].raw, 1, c, M, TMH_QUANT) for c in widths]
-    prods += [tmh_product(m.buf.raw, xqs[c].raw, yb.raw, r, c, M, TMH_GEMM_I8)
-              for (_, r, c, m), yb in zip(pool, ys)]
-    run_steps(host, ctx, prods, 0, 5, grouped=True)
-    report["gemm_i8_lds_kernel, 2B shapes"] = {
-        "int8_ops_per_group": sum(2.0 * M * r * c for _, r, c, _ in pool), "timed_groups": 5,
-        "products_per_group": len(pool)}
+    for label, kind in (("gemm_i8_lds_kernel, 2B shapes", TMH_GEMM_I8),
+                        ("gemm_i8_lds_kernel with the fused tail, 2B shapes", TMH_GEMM_I8_FMA)):
+        prods = [tmh_product(None, xb.raw, xqs[c].raw, 1, c, M, TMH_QUANT) for c in widths]
+        prods += [tmh_product(m.buf.raw, xqs[c].raw, yb.raw, r, c, M, kind)
+                  for (_, r, c, m), yb in zip(pool, ys)]
+        run_steps(host, ctx, prods, 0, 5, grouped=True)
+        report[label] = {
+            "int8_ops_per_group": sum(2.0 * M * r * c for _, r, c, _ in pool), "timed_groups": 5,
+            "products_per_group": len(pool)}
     print(json.dumps(report), flush=True)
 
 
