@@ -11,6 +11,8 @@
 #include <string>
 #include <vector>
 
+#include <mutex>
+
 #include "recorder.hpp"
 
 using namespace tmh;
@@ -19,6 +21,15 @@ namespace rec {
 std::vector<std::string> log;
 std::string (*name_of)(const void *) = nullptr;
 } // namespace rec
+
+namespace {
+// Contexts may launch from several threads at once (each on its own stream).
+std::mutex rec_mu;
+void record(std::string line) {
+    std::lock_guard<std::mutex> g(rec_mu);
+    rec::log.push_back(std::move(line));
+}
+} // namespace
 
 namespace {
 
@@ -94,9 +105,11 @@ hipError_t tmdev::kernels_present() { return hipSuccess; }
 
 hipError_t tmdev::scratch_on_current_device(int device, uint8_t **out) {
     static uint8_t *scratch = nullptr; // (lives as long as the process, like the real one)
+    static std::mutex mu;
     if (device != 0) {
         return hipErrorInvalidDevice;
     }
+    std::lock_guard<std::mutex> g(mu);
     if (scratch == nullptr) {
         scratch = (uint8_t *)malloc(kScratchBytes);
     }
@@ -111,7 +124,7 @@ hipError_t tmdev::zero_words(hipStream_t stream, uint32_t *dst, uint32_t n) {
     if (!fake::enqueue(stream, "zero_words")) {
         return hipErrorInvalidValue;
     }
-    rec::log.push_back("{\"k\":\"zero_words\",\"n\":" + std::to_string(n) + "}");
+    record("{\"k\":\"zero_words\",\"n\":" + std::to_string(n) + "}");
     return hipSuccess;
 }
 
@@ -244,7 +257,7 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
         }
         fake::attach_event(stop, stream);
     }
-    rec::log.push_back(out);
+    record(out);
     return hipSuccess;
 }
 
@@ -324,6 +337,6 @@ hipError_t tmdev::launch_single(hipStream_t stream, hipEvent_t stop, const Op &o
         }
         fake::attach_event(stop, stream);
     }
-    rec::log.push_back(out);
+    record(out);
     return hipSuccess;
 }

@@ -53,9 +53,9 @@ def driver(tmp_path_factory):
 def run_program(driver, lines):
     """Runs the commands; returns the parsed output lines. The sanitizers abort the
     process on a finding, the driver exits non-zero on an unexpected return code."""
-    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0:halt_on_error=1",
+    env = dict(os.environ,
+               ASAN_OPTIONS="detect_leaks=1:abort_on_error=0:halt_on_error=1:verify_asan_link_order=0",
                UBSAN_OPTIONS="print_stacktrace=1:halt_on_error=1")
-    env.pop("LD_PRELOAD", None)
     res = subprocess.run([driver], input="\n".join(lines) + "\n", capture_output=True, text=True,
                          timeout=300, env=env)
     assert res.returncode == 0, f"exit {res.returncode}\n{res.stderr[-4000:]}\n{res.stdout[-2000:]}"
@@ -460,3 +460,29 @@ def test_the_no_allocation_calls_are_refused_past_their_lease_list(driver):
     after = [o for o in sec["again"] if o["k"] == "stats"]
     # the commit behind the call adopts its leases (and adds its own on x and y)
     assert after[0]["in_flight"] == per_call + batch * (cols + rows) * 4 and after[1]["in_flight"] == 0
+
+
+# ------------------------------------------------------------------ threads --
+
+def test_two_contexts_and_their_readers_on_four_threads_under_the_thread_sanitizer(tmp_path):
+    """What the library promises about threads (tests/host_cpu/threads.cpp): two
+    owner threads drive a context each (groups, calls that allocate nothing on the
+    one static workspace, frees with work in flight, fences) while a reader thread
+    per context calls tm_hip_download_after and the dispatch counters, which take
+    no lock in the reference's typed layer (crates/metal/src/lib.rs:2618-2633)."""
+    gxx = shutil.which(os.environ.get("CXX", "g++"))
+    out = str(tmp_path / "threads")
+    cmd = [gxx, "-std=c++17", "-O1", "-g", "-fsanitize=thread", "-fno-omit-frame-pointer", "-Wall",
+           "-Wextra", "-Wno-format-truncation", "-I", HERE, "-I", os.path.join(ROOT, "include"),
+           "-I", os.path.join(ROOT, "tuckmill_amd", "csrc"), "-o", out,
+           os.path.join(ROOT, "tuckmill_amd", "csrc", "tm_hip.cpp"),
+           os.path.join(HERE, "fake_runtime.cpp"), os.path.join(HERE, "stub_launch.cpp"),
+           os.path.join(HERE, "threads.cpp"), "-lpthread"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stdout + res.stderr
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1:exitcode=66")
+    run = subprocess.run([out, "300"], capture_output=True, text=True, timeout=300, env=env)
+    assert run.returncode == 0, f"exit {run.returncode}\n{run.stderr[-6000:]}"
+    assert "ThreadSanitizer" not in run.stderr, run.stderr[-6000:]
+    end = json.loads(run.stdout.strip().splitlines()[-1])
+    assert end["k"] == "exit" and end["failures"] == 0 and end["enqueued"] > 1000
