@@ -1128,13 +1128,15 @@ def main():
     host_side = None
     cpu = args.cpu_seconds > 0
     if not args.no_gemm:
+        # (the other configurations' legs last milliseconds: they take enough steps for
+        # stable means whatever --steps says)
         line["roofline"]["gemm_m512"], per_config["config2_gemm_m512"] = bench_gemm(
-            host, ctx, max(10, args.steps // 4), max(3, args.warmup // 4), cpu=cpu)
+            host, ctx, max(100, args.steps // 4), max(10, args.warmup // 4), cpu=cpu)
     if not args.no_configs:
         line["roofline"]["gemma"], per_config["config3_gemma"] = bench_gemma(
-            host, ctx, max(10, args.steps // 4), max(3, args.warmup // 4), cpu=cpu)
+            host, ctx, max(100, args.steps // 4), max(10, args.warmup // 4), cpu=cpu)
         line["roofline"]["sweep_2b"], per_config["config4_sweep_2b"] = bench_sweep(
-            host, ctx, max(20, args.steps // 4), 0, cpu=cpu, batches=SWEEP_HEADLINE_M + (16, 32, 128))
+            host, ctx, max(40, args.steps // 4), 0, cpu=cpu, batches=SWEEP_HEADLINE_M + (16, 32, 128))
     ctx.close()
     print(json.dumps(line), flush=True)
 
