@@ -191,6 +191,27 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
                 xs_bytes += bx3_xs_bytes_of(op);
             }
         }
+        if (l.bx3_tail.row_tiles != 0u) { // one product's last rows as a segment with chunks of its own
+            const q8::Bx3Tail &t = l.bx3_tail;
+            if (t.product >= n || l.bx3_chunks[t.product] != 1u || n + 1 > (size_t)q8::BX3_MAX_DESCS) {
+                die("bf16 launch: tail segment on a product that cannot have one");
+            }
+            const Op &op = *l.list[t.product];
+            const uint32_t row_tiles = (op.rows + q8::BX3_TILE_ROWS - 1u) / q8::BX3_TILE_ROWS;
+            if (t.row_tiles >= row_tiles) {
+                die("bf16 launch: tail segment leaves its product no head");
+            }
+            const uint32_t head = q8::bx3_head_rows(op.rows, t.row_tiles);
+            const q8::Bx3Plan p = q8::bx3_plan_chunked(op.rows - head, op.cols, op.batch, key.p0 * 64u, t.chunks);
+            if (p.chunks != t.chunks || t.chunks < 2u || t.chunks > q8::BX3_TAIL_MAX_CHUNKS || key.p0 != 2 ||
+                p.chunk_blocks < q8::BX3_TAIL_CHUNK_BLOCKS) {
+                die("bf16 launch: tail segment with chunks it cannot have");
+            }
+            split_tiles += p.split_tiles;
+            partial_floats += p.partial_floats;
+            out += ",\"tail\":{\"product\":" + std::to_string(t.product) + ",\"row_tiles\":" +
+                   std::to_string(t.row_tiles) + ",\"chunks\":" + std::to_string(t.chunks) + "}";
+        }
         if (split_tiles != l.bx3_split_tiles || partial_floats != l.bx3_partial_floats ||
             xs_bytes != l.bx3_xs_bytes || inputs != l.bx3_inputs) {
             die("bf16 launch: workspace figures do not match its products");

@@ -350,6 +350,58 @@ def test_update_norm_and_products_in_one_group(ctx, batch):
         b.free()
 
 
+# Launches whose work units leave the last round of the chip's workgroup slots
+# partly empty: the units of that round are cut off one product's last rows as a
+# tail segment whose K goes in chunks (q8::bx3_plan_launch). 300 units on the 256
+# slots of the 128-token tile; ragged rows in the tail's last tile; the Qwen3-0.6B
+# vocabulary at 128 tokens (594 units).
+TAIL_SHAPES = [(76800, 1024, 128), (76801, 2048, 100), (151936, 1024, 128)]
+
+
+@pytest.mark.parametrize("rows,cols,batch", TAIL_SHAPES)
+def test_a_ragged_last_round_goes_as_a_tail_segment(ctx, rows, cols, batch):
+    w = S.make_weights(rows, cols, 3 * rows + cols)
+    x = S.make_activations(batch * cols, batch + rows)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    got = product(ctx, wb, x, rows, cols, batch, 0, 8)
+    assert not got[:8].any(), "nothing before y_off"
+    want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=16)
+    got = got[8:].reshape(batch, rows)
+    assert norm_err(got, want) <= 1e-5
+    # the boundary between the two segments and the last rows, row by row
+    scale = np.abs(want).max()
+    for r in (0, rows // 2, rows - 1, rows - 256, rows - 257):
+        assert np.abs(got[:, r] - want[:, r]).max() <= 1e-5 * scale, r
+    worst_row = np.abs(got - want).max(axis=0)
+    assert worst_row.max() <= 1e-5 * scale, int(worst_row.argmax())
+    again = product(ctx, wb, x, rows, cols, batch, 0, 8)[8:].reshape(batch, rows)
+    assert np.array_equal(bits(got), bits(again)), "the same launch gives the same bits"
+    wb.free()
+
+
+def test_a_tail_segment_inside_a_group(ctx):
+    """Two products share the launch; the larger one gives up its last rows."""
+    cols, batch = 1024, 128
+    shapes = [(70000, cols), (8192, cols)]
+    ws = [S.make_weights(r, c, 11 + r) for r, c in shapes]
+    wbs = [weights_buffer(ctx, w, r, c, True) for w, (r, c) in zip(ws, shapes)]
+    x = S.make_activations(batch * cols, 99)
+    xb = upload_new(ctx, x)
+    ybs = [ctx.buffer(batch * r * 4) for r, _ in shapes]
+    launches = ctx.kernel_launches()
+    ctx.begin_group()
+    for wb, yb, (r, c) in zip(wbs, ybs, shapes):
+        ctx.q8_0_gemm_mma(wb, xb, yb, r, c, batch, 0, 0)
+    ctx.end_group()
+    ctx.fence()
+    assert ctx.kernel_launches() == launches + 2
+    for w, yb, (r, c) in zip(ws, ybs, shapes):
+        want = O.gemm_q8_0_f32(w, r, c, x, batch, threads=16)
+        assert norm_err(yb.download_f32(0, batch * r).reshape(batch, r), want) <= 1e-5
+    for b in wbs + ybs + [xb]:
+        b.free()
+
+
 @pytest.mark.parametrize("rows,cols,batch", [(8192, 1024, 512), (8191, 1024, 512), (7936, 1024, 512),
                                              (32768, 1024, 65), (32768, 1024, 64), (32513, 1024, 65),
                                              (4096, 4096, 128), (4096, 4096, 129), (6144, 2048, 512),

@@ -87,7 +87,8 @@ struct Bx3Desc {
     const uint8_t *w;    // sealed weights
     const uint16_t *xs;  // the split activations of this product, [cols/32][3][batch][32] bf16
     float *y;            // y_off already applied
-    uint32_t rows, cols, batch;
+    uint32_t rows, cols, batch; // the whole matrix (rows: also the row stride of y)
+    uint32_t row_begin, row_end; // the rows this descriptor computes (a product, or a segment of one)
     uint32_t tile_begin; // first work unit of this product in the launch
     uint32_t tiles_t;    // token tiles per row tile
     uint32_t chunks;     // K chunks per output tile (work units per tile)
@@ -179,7 +180,10 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
     const uint32_t rows = d.rows, cols = d.cols, batch = d.batch;
     const uint32_t unit = tile - d.tile_begin;
     const uint32_t chunks = d.chunks, chunk = unit % chunks, local = unit / chunks;
-    const uint32_t t0 = (local % d.tiles_t) * Sh::tokens, n0 = (local / d.tiles_t) * Sh::rows;
+    const uint32_t t0 = (local % d.tiles_t) * Sh::tokens;
+    const uint32_t n0 = d.row_begin + (local / d.tiles_t) * Sh::rows;
+    // (rows of the tile at or beyond d.row_end, a segment's last tile, are computed
+    // from the matrix's own rows there and not stored)
     const uint32_t blocks = cols >> 5;
     const uint32_t kb_first = chunk * d.chunk_blocks;
     const uint32_t kb_last = kb_first + d.chunk_blocks < blocks ? kb_first + d.chunk_blocks : blocks;
@@ -525,16 +529,29 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
         constexpr uint32_t TILE_FLOATS = (uint32_t)NW * TM * TN * 16u * 64u;
         const uint32_t slot = d.part_begin + local;
         const size_t first_tile = (size_t)d.part_tile + (size_t)local * chunks;
-        float *mine = args.partials + (first_tile + chunk) * TILE_FLOATS +
-                      (size_t)wave * (TM * TN * 16u * 64u) + lane;
+        // Partial tiles travel in 16-byte pieces, a lane's four values of one MFMA
+        // result row group each (any layout does as long as writer and reader agree:
+        // the reader has the writer's place in its own workgroup). sc1 = device
+        // scope on this part: the access goes past this XCD's L2.
+        constexpr int AUX_SC1 = 16;
+        const __amdgpu_buffer_rsrc_t rs_part = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(args.partials + first_tile * TILE_FLOATS), 0, (int)(chunks * TILE_FLOATS * 4u), 0x00020000);
+        const uint32_t lane_bytes = (wave * (TM * TN * 4u) * 64u + lane) * 16u;
+        const uint32_t mine_bytes = chunk * TILE_FLOATS * 4u + lane_bytes;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    __hip_atomic_store(mine + ((i * TN + j) * 16 + v) * 64, acc[i][j][v], __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
+                for (int q = 0; q < 4; ++q) {
+                    // (through named floats: a bit cast applied to a vector element
+                    // directly reads element 0 with this compiler)
+                    const float f0 = acc[i][j][4 * q], f1 = acc[i][j][4 * q + 1];
+                    const float f2 = acc[i][j][4 * q + 2], f3 = acc[i][j][4 * q + 3];
+                    const u32x4 piece = {__builtin_bit_cast(uint32_t, f0), __builtin_bit_cast(uint32_t, f1),
+                                         __builtin_bit_cast(uint32_t, f2), __builtin_bit_cast(uint32_t, f3)};
+                    __builtin_amdgcn_raw_buffer_store_b128(
+                        piece, rs_part, (int)(mine_bytes + (uint32_t)(((i * TN + j) * 4 + q) * 1024)), 0, AUX_SC1);
                 }
             }
         }
@@ -562,19 +579,22 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
         if (threadIdx.x == 0u) {
             __hip_atomic_store(&args.arrivals[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        const float *first = args.partials + first_tile * TILE_FLOATS +
-                             (size_t)wave * (TM * TN * 16u * 64u) + lane;
         for (uint32_t c = 0; c < chunks; ++c) {
-            const float *part = first + (size_t)c * TILE_FLOATS;
+            const uint32_t part_bytes = c * TILE_FLOATS * 4u + lane_bytes;
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const float pv = __hip_atomic_load(part + ((i * TN + j) * 16 + v) * 64,
-                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        acc[i][j][v] = c == 0u ? pv : acc[i][j][v] + pv;
+                    for (int q = 0; q < 4; ++q) {
+                        const u32x4 piece = __builtin_amdgcn_raw_buffer_load_b128(
+                            rs_part, (int)(part_bytes + (uint32_t)(((i * TN + j) * 4 + q) * 1024)), 0, AUX_SC1);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t pu = piece[e];
+                            const float pv = __builtin_bit_cast(float, pu);
+                            acc[i][j][4 * q + e] = c == 0u ? pv : acc[i][j][4 * q + e] + pv;
+                        }
                     }
                 }
             }
@@ -590,7 +610,7 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const uint32_t t = t0 + wm * (32u * TM) + 32u * i + 8u * (v / 4) + 4u * half + (v % 4);
-                if (t < batch && n < rows) {
+                if (t < batch && n < d.row_end) {
                     d.y[(size_t)t * rows + n] = acc[i][j][v];
                 }
             }
@@ -604,6 +624,9 @@ struct Bx3Product {
     float *y;
     uint32_t rows, cols, batch;
     uint32_t chunks; // K chunks of this product, as bx3_plan_launch cut the launch
+    // the rows to compute: the whole product (0, rows), or one of the two
+    // segments of a product with a tail (bx3_plan_launch)
+    uint32_t row_begin, row_end;
 };
 
 template <int WM, int WN, int TM, int NS>
@@ -625,8 +648,13 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
     Bx3Product prods[BX3_MAX_DESCS];
     uint32_t unit_blocks[BX3_MAX_DESCS];
     for (int i = 0; i < n; ++i) {
-        const uint32_t mine = bx3_plan_chunked(prods_in[i].rows, prods_in[i].cols, prods_in[i].batch,
-                                               (uint32_t)Sh::tokens, prods_in[i].chunks).chunk_blocks;
+        if (prods_in[i].row_begin >= prods_in[i].row_end || prods_in[i].row_end > prods_in[i].rows ||
+            prods_in[i].row_begin % (uint32_t)Sh::rows != 0u) {
+            return hipErrorInvalidValue;
+        }
+        const uint32_t mine = bx3_plan_chunked(prods_in[i].row_end - prods_in[i].row_begin, prods_in[i].cols,
+                                               prods_in[i].batch, (uint32_t)Sh::tokens,
+                                               prods_in[i].chunks).chunk_blocks;
         int at = i;
         while (at > 0 && (unit_blocks[at - 1] < mine ||
                           (unit_blocks[at - 1] == mine && prods[at - 1].cols < prods_in[i].cols))) {
@@ -644,18 +672,21 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
         d.xs = prods[i].xs;
         d.y = prods[i].y;
         d.rows = prods[i].rows;
+        d.row_begin = prods[i].row_begin;
+        d.row_end = prods[i].row_end;
         d.cols = prods[i].cols;
         d.batch = prods[i].batch;
         d.tile_begin = (uint32_t)units;
         // K chunks as the launch was cut
-        const Bx3Plan plan = bx3_plan_chunked(prods[i].rows, prods[i].cols, prods[i].batch,
+        const uint32_t seg_rows = prods[i].row_end - prods[i].row_begin;
+        const Bx3Plan plan = bx3_plan_chunked(seg_rows, prods[i].cols, prods[i].batch,
                                               (uint32_t)Sh::tokens, prods[i].chunks);
         d.tiles_t = (prods[i].batch + Sh::tokens - 1) / Sh::tokens;
         d.chunk_blocks = plan.chunk_blocks;
         d.chunks = plan.chunks;
         d.part_begin = (uint32_t)split_tiles;
         d.part_tile = (uint32_t)partial_tiles;
-        const uint64_t tiles = (uint64_t)d.tiles_t * ((prods[i].rows + Sh::rows - 1) / Sh::rows);
+        const uint64_t tiles = (uint64_t)d.tiles_t * ((seg_rows + Sh::rows - 1) / Sh::rows);
         units += tiles * d.chunks;
         if (d.chunks > 1u) {
             split_tiles += tiles;

@@ -219,12 +219,29 @@ inline Bx3Plan bx3_plan_chunked(uint32_t rows, uint32_t cols, uint32_t batch, ui
     return p;
 }
 
-// Estimated duration (ns) of a launch whose products are cut as `chunks` says:
-// units in descending length to `slots` workgroup slots, each to the slot that
-// comes free first. Units of one product are alike, so the slots are tracked as
-// groups that come free together.
+// A product's last rows may be cut off as a segment of their own with K in
+// (more) chunks: the tail of a launch whose units do not fill its last round
+// (bx3_plan_launch). row_tiles == 0: none.
+struct Bx3Tail {
+    uint32_t product = 0;   // index in the launch's list
+    uint32_t row_tiles = 0; // row tiles (of BX3_TILE_ROWS rows) in the tail segment
+    uint32_t chunks = 0;    // its K chunks
+};
+constexpr uint32_t BX3_TAIL_CHUNK_BLOCKS = 8; // a tail's chunks: 256 columns or more,
+constexpr uint32_t BX3_TAIL_MAX_CHUNKS = 3;   // at most three
+
+// Rows of a product's head segment (what the tail leaves), and of the tail.
+inline uint32_t bx3_head_rows(uint32_t rows, uint32_t tail_row_tiles) {
+    const uint32_t row_tiles = (rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS;
+    return tail_row_tiles == 0u ? rows : (row_tiles - tail_row_tiles) * BX3_TILE_ROWS;
+}
+
+// Estimated duration (ns) of a launch whose products are cut as `chunks` says
+// (and `tail`, if any): units in descending length to `slots` workgroup slots,
+// each to the slot that comes free first. Units of one segment are alike, so
+// the slots are tracked as groups that come free together.
 inline uint64_t bx3_price(const Bx3Shape3 *shapes, const uint32_t *chunks, int n,
-                          uint32_t tile_tokens) {
+                          uint32_t tile_tokens, const Bx3Tail *tail = nullptr) {
     const uint32_t slots = tile_tokens == 128u ? 256u : 512u;
     const uint64_t unit_ns = tile_tokens == 128u ? 6000u : 4500u;
     const uint64_t block_ns = tile_tokens == 128u ? 1430u : 1100u;
@@ -232,28 +249,37 @@ inline uint64_t bx3_price(const Bx3Shape3 *shapes, const uint32_t *chunks, int n
     struct Kind {
         uint64_t ns, units;
     };
-    Kind kinds[BX3_MAX_DESCS];
-    for (int i = 0; i < n; ++i) { // insertion sort, longest first
-        const Bx3Plan p = bx3_plan_chunked(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens,
-                                           chunks[i]);
+    Kind kinds[BX3_MAX_DESCS + 1];
+    int nk = 0;
+    auto add = [&](uint32_t rows, uint32_t cols, uint32_t batch, uint32_t c) { // insertion sort, longest first
+        const Bx3Plan p = bx3_plan_chunked(rows, cols, batch, tile_tokens, c);
         const Kind k{unit_ns + block_ns * p.chunk_blocks + (p.chunks > 1u ? chunked_ns + 1000u * p.chunks : 0u),
                      p.units};
-        int at = i;
+        int at = nk++;
         while (at > 0 && kinds[at - 1].ns < k.ns) {
             kinds[at] = kinds[at - 1];
             --at;
         }
         kinds[at] = k;
+    };
+    for (int i = 0; i < n; ++i) {
+        if (tail != nullptr && tail->row_tiles != 0u && tail->product == (uint32_t)i) {
+            const uint32_t head = bx3_head_rows(shapes[i].rows, tail->row_tiles);
+            add(head, shapes[i].cols, shapes[i].batch, chunks[i]);
+            add(shapes[i].rows - head, shapes[i].cols, shapes[i].batch, tail->chunks);
+        } else {
+            add(shapes[i].rows, shapes[i].cols, shapes[i].batch, chunks[i]);
+        }
     }
     struct Group {
         uint64_t free_at, count;
     };
-    constexpr int MAX_GROUPS = 4 * BX3_MAX_DESCS + 4;
+    constexpr int MAX_GROUPS = 4 * BX3_MAX_DESCS + 8;
     Group groups[MAX_GROUPS]; // ascending free_at
     int ng = 1;
     groups[0] = Group{0u, slots};
     uint64_t end = 0;
-    for (int i = 0; i < n; ++i) {
+    for (int i = 0; i < nk; ++i) {
         uint64_t left = kinds[i].units;
         while (left > 0) {
             // whole rounds of every slot at once when the class is large
@@ -298,7 +324,7 @@ inline uint64_t bx3_price(const Bx3Shape3 *shapes, const uint32_t *chunks, int n
 
 // chunks[i] for every product of a launch (see above). Deterministic: a function
 // of the shapes in list order and the tile.
-inline void bx3_plan_launch(const Bx3Shape3 *shapes, int n, uint32_t tile_tokens, uint32_t *chunks) {
+inline void bx3_plan_chunks(const Bx3Shape3 *shapes, int n, uint32_t tile_tokens, uint32_t *chunks) {
     uint32_t cap[BX3_MAX_DESCS];
     uint64_t tiles = 0;
     bool any = false;
@@ -346,6 +372,77 @@ inline void bx3_plan_launch(const Bx3Shape3 *shapes, int n, uint32_t tile_tokens
                 chunks[i] = trial[i];
             }
         }
+    }
+}
+
+// The whole cut of a launch: chunks[i] for every product, and (when `tail` is
+// given) at most one tail segment. A launch of more units than the chip has
+// workgroup slots ends with a round that is partly empty: 594 whole-K units on
+// 512 slots are two rounds, the second 16 % full. The units of that last round
+// are then taken off the end of one whole-K product, as a segment of rows of its
+// own whose K is cut into chunks: several short units in the place of each long
+// one. Candidates: every whole-K product, 2 or 3 chunks of 256 columns or more;
+// priced like everything else; taken when the estimate drops by 5 % or more.
+// Measured (split pass included): 76800 x 1024 at 128 tokens, 300 units on 256
+// slots, 99.4 us whole, 89.3 / 86.9 / 90.5 with the last 44 row tiles in 2 / 3 / 4
+// chunks; 151936 x 1024 at 128 tokens (594 units) 152.8 whole, 147.0 / 150.2 /
+// 176.4. More chunks lose what they gain to their partial tiles, which cost more
+// the more of them are on their way at once; on the 64-token tile (512 slots, half
+// the arithmetic per partial byte) they cost too much for the estimate to be
+// trusted (151936 x 1024 at 64 tokens: 88.1 whole, 83.8 / 85.1 / 94.8): no tails
+// there. The tail's rows add in another order than the head's (another chunk
+// count), like any product whose K is cut.
+inline void bx3_plan_launch(const Bx3Shape3 *shapes, int n, uint32_t tile_tokens, uint32_t *chunks,
+                            Bx3Tail *tail = nullptr) {
+    bx3_plan_chunks(shapes, n, tile_tokens, chunks);
+    if (tail == nullptr) {
+        return;
+    }
+    *tail = Bx3Tail{};
+    const uint32_t slots = tile_tokens == 128u ? 256u : 512u;
+    uint64_t units = 0;
+    for (int i = 0; i < n; ++i) {
+        units += bx3_plan_chunked(shapes[i].rows, shapes[i].cols, shapes[i].batch, tile_tokens, chunks[i]).units;
+    }
+    const uint64_t ragged = units % slots;
+    if (tile_tokens != 128u || units <= slots || ragged == 0u || n >= BX3_MAX_DESCS) {
+        return;
+    }
+    const uint64_t base_ns = bx3_price(shapes, chunks, n, tile_tokens);
+    uint64_t best_ns = base_ns;
+    Bx3Tail best;
+    for (int i = 0; i < n; ++i) {
+        if (chunks[i] != 1u) {
+            continue;
+        }
+        const uint32_t blocks = shapes[i].cols / 32u;
+        uint32_t most = blocks / BX3_TAIL_CHUNK_BLOCKS;
+        most = most < BX3_TAIL_MAX_CHUNKS ? most : BX3_TAIL_MAX_CHUNKS;
+        const uint32_t tiles_t = (shapes[i].batch + tile_tokens - 1u) / tile_tokens;
+        const uint32_t row_tiles = (shapes[i].rows + BX3_TILE_ROWS - 1u) / BX3_TILE_ROWS;
+        const uint64_t t = (ragged + tiles_t - 1u) / tiles_t;
+        if (most < 2u || t >= row_tiles) {
+            continue; // (the head keeps at least one row tile)
+        }
+        // (one chunk more only for 5 % more: the estimate knows nothing of what
+        // many partial tiles at once cost each other)
+        Bx3Tail mine;
+        uint64_t mine_ns = ~0ull;
+        for (uint32_t c = 2; c <= most; ++c) {
+            const Bx3Tail trial{(uint32_t)i, (uint32_t)t, c};
+            const uint64_t ns = bx3_price(shapes, chunks, n, tile_tokens, &trial);
+            if (mine_ns == ~0ull || ns * 100u < mine_ns * 95u) {
+                mine_ns = ns;
+                mine = trial;
+            }
+        }
+        if (mine_ns < best_ns) {
+            best_ns = mine_ns;
+            best = mine;
+        }
+    }
+    if (best.row_tiles != 0u && best_ns * 100u <= base_ns * 95u) {
+        *tail = best;
     }
 }
 

@@ -639,7 +639,7 @@ std::vector<GemvKey> assign_mma_keys(tm_hip_ctx *ctx, const std::vector<Op> &ops
 
 // The K chunks of a bf16-matrix-core launch, decided for the launch as a whole
 // once its list is known, and what it then needs of the workspace.
-void cut_bx3_launch(Launch &l) {
+void cut_bx3_launch(Launch &l, uint64_t max_partial_floats = kBx3MaxPartialFloats) {
     if (l.single != nullptr || l.key.variant != V_BF16X3) {
         return;
     }
@@ -650,8 +650,10 @@ void cut_bx3_launch(Launch &l) {
         shapes[i] = q8::Bx3Shape3{l.list[i]->rows, l.list[i]->cols, l.list[i]->batch};
     }
     const uint32_t tile = l.key.p0 * 64u;
-    q8::bx3_plan_launch(shapes, n, tile, chunks);
+    q8::Bx3Tail tail;
+    q8::bx3_plan_launch(shapes, n, tile, chunks, &tail);
     l.bx3_chunks.clear();
+    l.bx3_tail = q8::Bx3Tail{};
     l.bx3_split_tiles = 0;
     l.bx3_partial_floats = 0;
     for (int i = 0; i < n; ++i) {
@@ -660,6 +662,20 @@ void cut_bx3_launch(Launch &l) {
         l.bx3_chunks.push_back((uint8_t)p.chunks);
         l.bx3_split_tiles += p.split_tiles;
         l.bx3_partial_floats += p.partial_floats;
+    }
+    if (tail.row_tiles != 0u) {
+        // (the tail's product has its K whole, so nothing of it is counted above;
+        // a tail that would not fit the workspace is left out)
+        const q8::Bx3Shape3 &sh = shapes[tail.product];
+        const uint32_t head = q8::bx3_head_rows(sh.rows, tail.row_tiles);
+        const q8::Bx3Plan p = q8::bx3_plan_chunked(sh.rows - head, sh.cols, sh.batch, tile, tail.chunks);
+        if (l.bx3_split_tiles + p.split_tiles <= q8::BX3_MAX_SPLIT_TILES &&
+            l.bx3_partial_floats + p.partial_floats <= max_partial_floats) {
+            l.bx3_tail = tail;
+            l.bx3_tail.chunks = p.chunks;
+            l.bx3_split_tiles += p.split_tiles;
+            l.bx3_partial_floats += p.partial_floats;
+        }
     }
 }
 
@@ -2063,7 +2079,7 @@ int tm_hip_q8_0_gemm_mma_noalloc(tm_hip_ctx *ctx, tm_hip_buffer *w, tm_hip_buffe
     launch.normed.push_back(false);
     bool counters = launch.key.kind == OP_MMA; // the work-queue form of the f32 kernel may run
     if (launch.key.variant == V_BF16X3) {
-        cut_bx3_launch(launch);
+        cut_bx3_launch(launch, ctx->fixed.partial_bytes / 4u); // (a tail only if the static array holds it)
         launch.bx3_xs_bytes = bx3_xs_bytes_of(op);
         launch.bx3_inputs = 1;
         if (launch.bx3_xs_bytes > ctx->fixed.xs_bytes ||

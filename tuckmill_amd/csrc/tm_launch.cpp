@@ -203,6 +203,7 @@ hipError_t launch_bx3_list(hipStream_t stream, hipEvent_t stop, const Launch &la
     const Op *input_of[q8::SPLIT_MAX_DESCS];
     q8::Bx3Product prods[q8::BX3_MAX_DESCS];
     int n_in = 0, n = 0;
+    uint32_t op_at = 0;
     size_t xs_used = 0;
     for (const Op *op : ops) {
         int at = 0;
@@ -219,10 +220,23 @@ hipError_t launch_bx3_list(hipStream_t stream, hipEvent_t stop, const Launch &la
             xs_used += bx3_xs_bytes_of(*op);
             ++n_in;
         }
-        prods[n] = q8::Bx3Product{(const uint8_t *)op->a[0]->ptr, inputs[at].xs,
-                                  (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
-                                  op->batch, launch.bx3_chunks[(size_t)n]};
-        ++n;
+        const uint32_t chunks = launch.bx3_chunks[(size_t)(op_at)];
+        const bool tailed = launch.bx3_tail.row_tiles != 0u && launch.bx3_tail.product == op_at;
+        const uint32_t head = tailed ? q8::bx3_head_rows(op->rows, launch.bx3_tail.row_tiles) : op->rows;
+        if (n + (tailed ? 2 : 1) > q8::BX3_MAX_DESCS || head == 0u) {
+            return hipErrorInvalidValue;
+        }
+        prods[n++] = q8::Bx3Product{(const uint8_t *)op->a[0]->ptr, inputs[at].xs,
+                                    (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
+                                    op->batch, chunks, 0u, head};
+        if (tailed) { // the product's last rows, K in chunks of their own
+            prods[n] = prods[n - 1];
+            prods[n].chunks = launch.bx3_tail.chunks;
+            prods[n].row_begin = head;
+            prods[n].row_end = op->rows;
+            ++n;
+        }
+        ++op_at;
     }
     // Inputs that the launch before this one has split already stay out of the
     // split pass (none left: no split pass).

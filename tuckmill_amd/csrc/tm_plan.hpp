@@ -221,6 +221,9 @@ struct Launch {
     // decided the K chunks of every product, `bx3_chunks`, per list entry)
     uint64_t bx3_split_tiles = 0, bx3_partial_floats = 0, bx3_xs_bytes = 0;
     InlineVec<uint8_t, 4> bx3_chunks;
+    // the rows that one of the products gives up to a tail segment with chunks of
+    // its own (q8::bx3_plan_launch); row_tiles == 0: none
+    q8::Bx3Tail bx3_tail{};
     int bx3_inputs = 0;
     uint32_t descs = 0; // descriptors the listed products take (token groups count one each)
     uint32_t token_descs = 0; // the same at one descriptor per product and token
