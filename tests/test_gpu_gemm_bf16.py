@@ -353,9 +353,9 @@ def test_update_norm_and_products_in_one_group(ctx, batch):
 # Launches whose work units leave the last round of the chip's workgroup slots
 # partly empty: the units of that round are cut off one product's last rows as a
 # tail segment whose K goes in chunks (q8::bx3_plan_launch). 300 units on the 256
-# slots of the 128-token tile; ragged rows in the tail's last tile; the Qwen3-0.6B
-# vocabulary at 128 tokens (594 units).
-TAIL_SHAPES = [(76800, 1024, 128), (76801, 2048, 100), (151936, 1024, 128)]
+# slots of the 128-token tile; one ragged row in the tail's last tile and a ragged
+# token tile; two token tiles per row tile, ragged both ways, K of 48 blocks.
+TAIL_SHAPES = [(76800, 1024, 128), (76801, 1024, 100), (38500, 1536, 250)]
 
 
 @pytest.mark.parametrize("rows,cols,batch", TAIL_SHAPES)

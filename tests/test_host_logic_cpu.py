@@ -463,28 +463,30 @@ def test_the_no_allocation_calls_are_refused_past_their_lease_list(driver):
 
 
 def test_a_ragged_last_round_is_cut_off_as_a_tail_segment(driver):
-    """594 whole-K units on the 256 workgroup slots of the 128-token tile (a 151936 x
-    1024 vocabulary at 128 tokens) are two rounds and a third that is a third full:
-    the units of the last round become a tail segment of rows whose K is cut in
-    chunks (q8::bx3_plan_launch). The same product at 512 tokens (2376 units, nine
-    full rounds and a bit) keeps its K whole everywhere, and so does the 64-token
-    tile, where tails do not pay. The recording launcher checks the segment
-    against the limits."""
+    """300 whole-K units on the 256 workgroup slots of the 128-token tile (76800 x
+    1024 at 128 tokens) are a full round and one that is a sixth full: the units of
+    the last round become a tail segment of rows whose K is cut in chunks
+    (q8::bx3_plan_launch). A launch with many rounds (the 151936 x 1024 vocabulary
+    at 512 tokens: 2376 units; at 128 tokens: 594, where the estimate gains too
+    little) keeps its K whole everywhere, and so does the 64-token tile, where
+    tails do not pay. The recording launcher checks the segment against the limits."""
     rows, cols = 151936, 1024
     lines = ["ctx main", f"buf w {rows * (cols // 32) * 34}", f"seal w {rows} {cols}",
+             f"buf w2 {76800 * (cols // 32) * 34}", f"seal w2 76800 {cols}",
              f"buf x {512 * cols * 4}", f"buf y {512 * rows * 4}", "fence",
+             "mark t128", f"mma w2 x y 76800 {cols} 128 0 0", "fence",
+             "mark noalloc", f"mma_noalloc w2 x y 76800 {cols} 128 0 0", "fence",
              "mark m64", f"mma w x y {rows} {cols} 64 0 0", "fence",
              "mark m128", f"mma w x y {rows} {cols} 128 0 0", "fence",
-             "mark m512", f"mma w x y {rows} {cols} 512 0 0", "fence",
-             "mark noalloc", f"mma_noalloc w x y {rows} {cols} 128 0 0", "fence", "stats"]
+             "mark m512", f"mma w x y {rows} {cols} 512 0 0", "fence", "stats"]
     sec = sections(run_program(driver, lines))
-    for name in ("m128", "noalloc"):
+    for name in ("t128", "noalloc"):
         (l,) = launches_of(sec[name])
         assert l["variant"] == "bf16x3" and l["p"][0] == 2, l
         tail = l["tail"]
-        assert tail["product"] == 0 and tail["row_tiles"] == 82 and 2 <= tail["chunks"] <= 3, l
+        assert tail["product"] == 0 and tail["row_tiles"] == 44 and 2 <= tail["chunks"] <= 3, l
         assert l["ops"][0]["chunks"] == 1
-    for name in ("m64", "m512"):
+    for name in ("m64", "m128", "m512"):
         (l,) = launches_of(sec[name])
         assert "tail" not in l and l["ops"][0]["chunks"] == 1
 

@@ -85,7 +85,7 @@ def test_raw_decode_kernel_with_column_tails_fits_three_workgroups_per_cu(resour
 
 
 # gemm_bf16x3_kernel<WM, 4, 2, NS>: the 128-token and the 64-token tile
-BF16_KERNEL = re.compile(r"Function Name: _ZN2q818gemm_bf16x3_kernelILi[12]ELi4ELi2ELi[34]EEE")
+BF16_KERNEL = re.compile(r"Function Name: _ZN2q818gemm_bf16x3_kernelILi[12]ELi4ELi2ELi[34]ELb[01]EEE")
 
 
 def test_bf16_gemm_keeps_its_results_in_vector_registers(resource_remarks):

@@ -133,7 +133,11 @@ __device__ __forceinline__ bf16x8_t sbytes_to_bf16x8(uint32_t lo, uint32_t hi) {
     return __builtin_bit_cast(bf16x8_t, v);
 }
 
-template <int WM, int WN, int TM, int NS>
+// SEG: some descriptor of the launch covers a range of its product's rows only
+// (a product with a tail segment, bx3_plan_launch). A separate instantiation:
+// the two extra descriptor words in the plain kernel's addressing cost its
+// hand-ordered loop 3-4 % (measured: 0.6B vocabulary at 512 tokens 505 -> 525 us).
+template <int WM, int WN, int TM, int NS, bool SEG = false>
 // (Two waves per SIMD, declared: with a register budget of 256 the compiler keeps
 // the MFMA results in ordinary vector registers, which the rescale reads
 // directly. With a single wave's budget it parked the small tile's results in
@@ -181,9 +185,9 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
     const uint32_t unit = tile - d.tile_begin;
     const uint32_t chunks = d.chunks, chunk = unit % chunks, local = unit / chunks;
     const uint32_t t0 = (local % d.tiles_t) * Sh::tokens;
-    const uint32_t n0 = d.row_begin + (local / d.tiles_t) * Sh::rows;
-    // (rows of the tile at or beyond d.row_end, a segment's last tile, are computed
-    // from the matrix's own rows there and not stored)
+    // (SEG: rows of the tile at or beyond d.row_end, a segment's last tile, are
+    // computed from the matrix's own rows there and not stored)
+    const uint32_t n0 = (SEG ? d.row_begin : 0u) + (local / d.tiles_t) * Sh::rows;
     const uint32_t blocks = cols >> 5;
     const uint32_t kb_first = chunk * d.chunk_blocks;
     const uint32_t kb_last = kb_first + d.chunk_blocks < blocks ? kb_first + d.chunk_blocks : blocks;
@@ -529,29 +533,16 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
         constexpr uint32_t TILE_FLOATS = (uint32_t)NW * TM * TN * 16u * 64u;
         const uint32_t slot = d.part_begin + local;
         const size_t first_tile = (size_t)d.part_tile + (size_t)local * chunks;
-        // Partial tiles travel in 16-byte pieces, a lane's four values of one MFMA
-        // result row group each (any layout does as long as writer and reader agree:
-        // the reader has the writer's place in its own workgroup). sc1 = device
-        // scope on this part: the access goes past this XCD's L2.
-        constexpr int AUX_SC1 = 16;
-        const __amdgpu_buffer_rsrc_t rs_part = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(args.partials + first_tile * TILE_FLOATS), 0, (int)(chunks * TILE_FLOATS * 4u), 0x00020000);
-        const uint32_t lane_bytes = (wave * (TM * TN * 4u) * 64u + lane) * 16u;
-        const uint32_t mine_bytes = chunk * TILE_FLOATS * 4u + lane_bytes;
+        float *mine = args.partials + (first_tile + chunk) * TILE_FLOATS +
+                      (size_t)wave * (TM * TN * 16u * 64u) + lane;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    // (through named floats: a bit cast applied to a vector element
-                    // directly reads element 0 with this compiler)
-                    const float f0 = acc[i][j][4 * q], f1 = acc[i][j][4 * q + 1];
-                    const float f2 = acc[i][j][4 * q + 2], f3 = acc[i][j][4 * q + 3];
-                    const u32x4 piece = {__builtin_bit_cast(uint32_t, f0), __builtin_bit_cast(uint32_t, f1),
-                                         __builtin_bit_cast(uint32_t, f2), __builtin_bit_cast(uint32_t, f3)};
-                    __builtin_amdgcn_raw_buffer_store_b128(
-                        piece, rs_part, (int)(mine_bytes + (uint32_t)(((i * TN + j) * 4 + q) * 1024)), 0, AUX_SC1);
+                for (int v = 0; v < 16; ++v) {
+                    __hip_atomic_store(mine + ((i * TN + j) * 16 + v) * 64, acc[i][j][v], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
         }
@@ -579,22 +570,19 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
         if (threadIdx.x == 0u) {
             __hip_atomic_store(&args.arrivals[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        const float *first = args.partials + first_tile * TILE_FLOATS +
+                             (size_t)wave * (TM * TN * 16u * 64u) + lane;
         for (uint32_t c = 0; c < chunks; ++c) {
-            const uint32_t part_bytes = c * TILE_FLOATS * 4u + lane_bytes;
+            const float *part = first + (size_t)c * TILE_FLOATS;
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const u32x4 piece = __builtin_amdgcn_raw_buffer_load_b128(
-                            rs_part, (int)(part_bytes + (uint32_t)(((i * TN + j) * 4 + q) * 1024)), 0, AUX_SC1);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const uint32_t pu = piece[e];
-                            const float pv = __builtin_bit_cast(float, pu);
-                            acc[i][j][4 * q + e] = c == 0u ? pv : acc[i][j][4 * q + e] + pv;
-                        }
+                    for (int v = 0; v < 16; ++v) {
+                        const float pv = __hip_atomic_load(part + ((i * TN + j) * 16 + v) * 64,
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        acc[i][j][v] = c == 0u ? pv : acc[i][j][v] + pv;
                     }
                 }
             }
@@ -610,7 +598,7 @@ __global__ __launch_bounds__(WM * WN * 64, 2) void gemm_bf16x3_kernel(const Bx3A
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const uint32_t t = t0 + wm * (32u * TM) + 32u * i + 8u * (v / 4) + 4u * half + (v % 4);
-                if (t < batch && n < d.row_end) {
+                if (t < batch && n < (SEG ? d.row_end : rows)) {
                     d.y[(size_t)t * rows + n] = acc[i][j][v];
                 }
             }
@@ -700,8 +688,17 @@ inline hipError_t launch_bx3_cfg(hipStream_t stream, hipEvent_t stop, const Bx3P
     args.total_tiles = (uint32_t)units;
     args.chunk_wgs = args.d[0].tiles_t * args.d[0].chunks;
     args.pad = 0;
-    Q8_LAUNCH((gemm_bf16x3_kernel<WM, WN, TM, NS>), dim3((unsigned)units), dim3(WM * WN * 64), 0, stream,
-              stop, args);
+    bool segments = false;
+    for (int i = 0; i < n; ++i) {
+        segments = segments || prods[i].row_begin != 0u || prods[i].row_end != prods[i].rows;
+    }
+    if (segments) {
+        Q8_LAUNCH((gemm_bf16x3_kernel<WM, WN, TM, NS, true>), dim3((unsigned)units), dim3(WM * WN * 64), 0,
+                  stream, stop, args);
+    } else {
+        Q8_LAUNCH((gemm_bf16x3_kernel<WM, WN, TM, NS, false>), dim3((unsigned)units), dim3(WM * WN * 64), 0,
+                  stream, stop, args);
+    }
     return hipGetLastError();
 }
 

@@ -382,11 +382,13 @@ inline void bx3_plan_chunks(const Bx3Shape3 *shapes, int n, uint32_t tile_tokens
 // are then taken off the end of one whole-K product, as a segment of rows of its
 // own whose K is cut into chunks: several short units in the place of each long
 // one. Candidates: every whole-K product, 2 or 3 chunks of 256 columns or more;
-// priced like everything else; taken when the estimate drops by 5 % or more.
-// Measured (split pass included): 76800 x 1024 at 128 tokens, 300 units on 256
-// slots, 99.4 us whole, 89.3 / 86.9 / 90.5 with the last 44 row tiles in 2 / 3 / 4
-// chunks; 151936 x 1024 at 128 tokens (594 units) 152.8 whole, 147.0 / 150.2 /
-// 176.4. More chunks lose what they gain to their partial tiles, which cost more
+// priced like everything else; taken when the estimate drops by 8 % or more (a
+// launch with a segment in it runs on an instantiation of the kernel that is
+// 3-4 % slower, gemm_bf16x3_kernel<..., SEG = true>).
+// Measured on that instantiation (split pass included): 76800 x 1024 at 128
+// tokens, 300 units on 256 slots, 99.4 us whole, 89.3 / 86.9 / 90.5 with the last
+// 44 row tiles in 2 / 3 / 4 chunks; 151936 x 1024 at 128 tokens (594 units) 152.8
+// whole, 147.0 / 150.2 / 176.4 (too little to pay for the instantiation: not taken). More chunks lose what they gain to their partial tiles, which cost more
 // the more of them are on their way at once; on the 64-token tile (512 slots, half
 // the arithmetic per partial byte) they cost too much for the estimate to be
 // trusted (151936 x 1024 at 64 tokens: 88.1 whole, 83.8 / 85.1 / 94.8): no tails
@@ -441,7 +443,7 @@ inline void bx3_plan_launch(const Bx3Shape3 *shapes, int n, uint32_t tile_tokens
             best = mine;
         }
     }
-    if (best.row_tiles != 0u && best_ns * 100u <= base_ns * 95u) {
+    if (best.row_tiles != 0u && best_ns * 100u <= base_ns * 92u) {
         *tail = best;
     }
 }
