@@ -439,11 +439,6 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
             }
             wide = wide || (key.packed && op->cols >= 2048u);
         }
-        if (one_token && key.packed && tail == 768u && op->cols >= 1024u &&
-            d.rows_per_tile == (uint32_t)R) {
-            // this tail's pass is half the rows: a tile a pass
-            d.rows_per_tile = (uint32_t)R / 2u;
-        }
         d.pad = 0;
         const bool pair_first = launch.glu[at] != nullptr;
         const bool pair_second = at > 0 && launch.glu[at - 1] != nullptr;
