@@ -64,13 +64,43 @@ def test_raw_and_packed_layouts_give_identical_bits(ctx):
                              # staged whole, odd and even numbers of rows in the last pass)
                              (1, 1152, 17), (7, 1152, 18), (301, 1152, 19), (1030, 1152, 20),
                              (13, 6912, 21), (260, 6912, 22),
-                             # other tails (general form)
-                             (40, 2176, 23), (24, 1792, 24)]:
+                             # full-height tiles of 1152 columns (a tile is a single step), ragged end
+                             (9001, 1152, 25),
+                             # whole chunks in front of a 128-column tail (pipelined), other tails
+                             (40, 2176, 23), (9000, 3200, 26), (24, 1792, 24)]:
         w = O.boundary_weights(rows, cols, seed)
         x = O.boundary_input(cols, seed + 100)
         a = gemv(ctx, weights_buffer(ctx, w, rows, cols, False), x, rows, cols)
         b = gemv(ctx, weights_buffer(ctx, w, rows, cols, True), x, rows, cols)
         assert np.array_equal(bits(a), bits(b))
+
+
+def test_rows_of_1152_columns_beside_longer_rows_with_the_same_tail(ctx):
+    """Alone, products of 1152 columns run tiles of a single step; in a launch with a
+    product whose rows have more whole chunks in front of the 128-column tail (3200
+    columns) they take the pipelined form like it. Same bits either way, and the
+    oracle's within 1e-5."""
+    shapes = [(9000, 1152), (2000, 3200), (300, 1152), (1152, 6912)]
+    ws = [S.make_weights(r, c, 40 + i) for i, (r, c) in enumerate(shapes)]
+    xs = [S.make_activations(c, 50 + i) for i, (r, c) in enumerate(shapes)]
+    wbs = [weights_buffer(ctx, w, r, c, True) for w, (r, c) in zip(ws, shapes)]
+    alone = [gemv(ctx, wb, x, r, c) for wb, x, (r, c) in zip(wbs, xs, shapes)]
+    for picked in ([0, 1, 2, 3], [0, 2], [0, 2, 3]):
+        xbs = [upload_new(ctx, xs[i]) for i in picked]
+        ybs = [ctx.buffer(shapes[i][0] * 4) for i in picked]
+        launches = ctx.kernel_launches()
+        ctx.begin_group()
+        for i, xb, yb in zip(picked, xbs, ybs):
+            ctx.q8_0_gemv(wbs[i], xb, yb, *shapes[i])
+        ctx.end_group()
+        ctx.fence()
+        assert ctx.kernel_launches() == launches + 1
+        for i, yb in zip(picked, ybs):
+            assert np.array_equal(bits(yb.download_f32(0, shapes[i][0])), bits(alone[i])), (picked, i)
+        for b in xbs + ybs:
+            b.free()
+    for w, x, got, (r, c) in zip(ws, xs, alone, shapes):
+        assert norm_err(got, O.gemv_q8_0_f32(w, r, c, x)) <= 1e-5
 
 
 @pytest.mark.parametrize("packed", [False, True])

@@ -450,6 +450,46 @@ __device__ __forceinline__ void stream_rows(const WView<PACKED> &wv, const XS xs
                                     });
 }
 
+// stream_rows for rows of exactly one whole chunk (1024 columns, or 1152 with
+// TAILMASK = 128) in tiles of at most R rows: the tile is a single step, so there
+// is nothing to run ahead of, no loop, and no second set of weight registers to
+// hold: every load of the tile is issued at once. Same arithmetic as stream_rows:
+// the tail piece first, then the chunk. Measured on the 262144 x 1152 vocabulary:
+// 47.2 -> 44.5 us (the kernel that carries this form instead of the pipelined one
+// for such rows needs 120 registers instead of 164: four waves per SIMD, which
+// is where the gain comes from). For rows of 1024 columns, whose kernel has four
+// waves anyway, the same form is slower than the pipelined one run for a single
+// step (Qwen3-0.6B decode step 95.4 -> 100.2 us): TAILMASK = 0 is not used.
+template <int R, bool XA, int TAILMASK, class XS = PlainX>
+__device__ __forceinline__ void stream_rows_once(const WView<PACKED> &wv, const XS xs, float *y,
+                                                 uint32_t row_first, uint32_t row_end,
+                                                 uint32_t lane, float *res, float alpha) {
+    static_assert(TAILMASK == 0 || TAILMASK == 128, "one whole chunk, with or without a 128-column tail");
+    constexpr bool T2 = TAILMASK == 128;
+    float x2[2], xv[16];
+    if constexpr (T2) xs.template loadn<2, XA>(1024u + lane * 2u, x2);
+    xs.template load16<XA>(lane * 16u, xv);
+    uint32_t q2[R][1], s2[R], q[R][4], sb[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t row = row_first + (uint32_t)r < row_end ? row_first + (uint32_t)r : row_end - 1u;
+        if constexpr (T2) {
+            wv.template load_quants<2, true>(row, 1024u + lane * 2u, q2[r]);
+            s2[r] = wv.scale_bits(row, (1024u + lane * 2u) >> 5);
+        }
+        wv.template load_quants<16, true>(row, lane * 16u, q[r]);
+        sb[r] = wv.scale_bits(row, lane >> 1);
+    }
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        float a = 0.0f;
+        if constexpr (T2) a = __builtin_fmaf(f16_bits_to_f32(s2[r]), piece_dot<2>(q2[r], x2), a);
+        acc[r] = __builtin_fmaf(f16_bits_to_f32(sb[r]), piece_dot<16>(q[r], xv), a);
+    }
+    reduce_store<R>(acc, y, row_first, row_end, lane, true, res, alpha);
+}
+
 // stream_rows for passes of few rows under a long K (a small product cut into
 // short tiles, so that more waves share it): a step covers C chunks of the R
 // rows instead of one, which keeps R x C kilobytes per wave in flight where the
@@ -929,9 +969,14 @@ __device__ __forceinline__ void stream_rows_glu(const WView<PACKED> &wg, const W
 // TAILS selects which column tails get the streaming decode path: 0 = none
 // (cols a multiple of 1024 only; fewest registers, the Qwen3 shapes), 1 = also
 // cols % 1024 == 128 and == 768 (the Gemma-3-1B shapes), 2 = also == 768 but
-// not 128 (a launch of Gemma's down projections only: the 128-column tail is
-// what costs the registers, without it four waves fit a SIMD). The host picks
-// the cheapest set that covers the products of a launch.
+// not 128 (a launch of Gemma's down projections only), 3 = as 1. In the plain
+// kernel (neither NORM nor WIDE) 1 stands for "every row with a 128-column tail
+// is 1152 columns long": its tiles are single steps (stream_rows_once), and
+// without the pipelined form for that tail, which is what costs the registers,
+// four waves fit a SIMD (120 registers against 164; Gemma-3-1B's 79-GEMV step
+// 152.2 -> 143.2 us, its vocabulary alone 47.2 -> 44.5); 3 is the pipelined
+// form for any number of whole chunks in front of the tail. The host picks the
+// cheapest set that covers the products of a launch.
 // NORM: the launch carries fused forms, an RMSNorm in front of its products
 // and/or gate-up pairs with their activation (a separate instantiation, so that
 // the plain decode kernel keeps its register budget).
@@ -1088,8 +1133,22 @@ __global__ __launch_bounds__(256) void gemv_list_kernel(const GemvArgsT<ND> args
                 return;
             }
             // (as above, a small product may be cut into shorter tiles)
-            if constexpr (TAILS == 1) {
-                if (tail == 128u) { // hidden 1152 (Gemma-3-1B)
+            if constexpr (TAILS == 1 && !NORM && !WIDE) {
+                // every product with this tail has one whole chunk per row (the host
+                // chose the instantiation by that): a tile is a single step
+                if (tail == 128u && full == 1u && d.rows_per_tile <= (uint32_t)R) {
+                    if (d.rows_per_tile % (R / 2) != 0u) {
+                        stream_rows_once<R / 4, XA, 128>(wv, PlainX{x}, y, row_first, row_end, lane, d.res, d.alpha);
+                    } else if (d.rows_per_tile % R != 0u) {
+                        stream_rows_once<R / 2, XA, 128>(wv, PlainX{x}, y, row_first, row_end, lane, d.res, d.alpha);
+                    } else {
+                        stream_rows_once<R, XA, 128>(wv, PlainX{x}, y, row_first, row_end, lane, d.res, d.alpha);
+                    }
+                    return;
+                }
+            }
+            if constexpr ((TAILS == 1 && (NORM || WIDE)) || TAILS == 3) {
+                if (tail == 128u) { // any number of whole chunks, pipelined
                     if (d.rows_per_tile % (R / 2) != 0u) {
                         stream_rows<R / 4, XA, 128>(wv, PlainX{x}, y, cols, row_first, row_end, lane,
                                                     d.res, d.alpha);

@@ -87,7 +87,7 @@ inline unsigned strided_blocks_of(uint32_t n, uint32_t per) {
 
 template <int L, int R, int TB, bool XA>
 hipError_t launch_gemv(hipStream_t stream, hipEvent_t stop, const q8::GemvArgs &args, int tails,
-                       bool fused, bool wide) {
+                       bool fused, bool wide, bool tail128_long = false) {
     const uint32_t groups = (args.total_tiles + 3u) / 4u;
     if constexpr (L == q8::PACKED && TB == 1) {
         const bool norm = fused; // the planner only fuses into aligned launches of the decode kernel
@@ -127,6 +127,9 @@ hipError_t launch_gemv(hipStream_t stream, hipEvent_t stop, const q8::GemvArgs &
                     Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 0, q8::GEMV_FEW_DESCS, false, true>),
                               dim3(groups), dim3(256), 0, stream, stop, few);
                 }
+            } else if (tails == 1 && tail128_long) { // some row has whole chunks in front of its 128-column tail
+                Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 3, q8::GEMV_FEW_DESCS>), dim3(groups),
+                          dim3(256), 0, stream, stop, few);
             } else if (tails == 1) {
                 Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1, q8::GEMV_FEW_DESCS>), dim3(groups),
                           dim3(256), 0, stream, stop, few);
@@ -154,6 +157,13 @@ hipError_t launch_gemv(hipStream_t stream, hipEvent_t stop, const q8::GemvArgs &
         }
     }
     if constexpr (TB == 1) { // (either layout: the column tails that stream)
+        if constexpr (L == q8::PACKED) {
+            if (tails == 1 && tail128_long) {
+                Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 3>), dim3(groups), dim3(256), 0,
+                          stream, stop, args);
+                return hipGetLastError();
+            }
+        }
         if (tails == 1) {
             Q8_LAUNCH((q8::gemv_list_kernel<L, R, TB, XA, 1>), dim3(groups), dim3(256), 0,
                       stream, stop, args);
@@ -400,6 +410,7 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
     // which column tails with a streaming path of their own the products have:
     // 0 none, 1 128 columns (and maybe 768), 2 768 columns only
     int tails = 0;
+    bool tail128_long = false; // some row with a 128-column tail has more than one whole chunk
     bool wide = false; // some sealed product in short tiles has two chunks and more per row
     // One descriptor: token group `grp` of the product at place `at` of the
     // launch's list (the fusions are recorded per product).
@@ -486,6 +497,7 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
         const uint32_t tail = op->cols & 1023u;
         if (op->cols >= 1024u && tail == 128u) {
             tails = 1;
+            tail128_long = tail128_long || op->cols != 1152u;
         } else if (op->cols >= 1024u && tail == 768u && tails == 0) {
             tails = 2;
         }
@@ -563,7 +575,7 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
     if (key.packed == (P) && key.variant == ((T) == 1 ? V_DECODE : V_GENERAL) &&             \
         key.flag == (A)) {                                                                   \
         return launch_gemv<(P) ? q8::PACKED : q8::RAW, (T) == 1 ? kGemvR1 : kGemvR4, T, A>(  \
-            stream, stop, args, tails, fused, wide);                                                   \
+            stream, stop, args, tails, fused, wide, tail128_long);                                    \
     }
     TM_GEMV_CASE(true, 1, true)
     TM_GEMV_CASE(true, 1, false)
