@@ -48,6 +48,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 # WRITE_SIZE counter runs summarised in profiles/gemv_list_kernel__decode_step__pmc_traffic.txt
 # (fetch counter x 2.000 + write counter x 1.000, factors from a plain copy kernel).
 DECODE_STEP_TRAFFIC_BYTES = 644.75e6
+GEMMA_STEP_TRAFFIC_BYTES = 991.37e6  # the same for the Gemma-3-1B 79-GEMV step (its own profile file)
 DECODE_STEP_TRAFFIC_SOURCE = ("constant from profiles/gemv_list_kernel__decode_step__pmc_traffic.txt "
                               "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --workload "
                               "traffic` on q8::gemv_list_kernel<1, 8, 1, true, 0, 224, false, false>); not "
@@ -540,7 +541,11 @@ def bench_gemma(host, ctx, steps, warmup, cpu=True):
         "kernel": "q8::gemv_list_kernel (column tails 128 and 768)", "products": len(products),
         "launches_per_step": t.launches / steps, "median_us": stats.get("median_us"),
         "wall_us": t.wall_ms / steps * 1e3, "max_norm_err_vs_cpu": worst,
-        "products_checked": len(products)})
+        "products_checked": len(products),
+        "traffic": GEMMA_STEP_TRAFFIC_BYTES if t.launches == steps else None,
+        "traffic_source": "constant from profiles/gemv_list_kernel__gemma3_1b_step__pmc_traffic.txt "
+                          "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --workload "
+                          "traffic`); not measured in this run"})
     head_p = products[-1]
     t = run_steps(host, ctx, [head_p], warmup, steps, grouped=False)
     us = t.gpu_ms / steps * 1e3
@@ -935,7 +940,8 @@ def run_traffic(host, ctx):
       1. a plain f32 copy of known size (the calibration kernel: 256 MiB read,
          256 MiB written per dispatch), then the read-only streaming kernel over
          1 GiB (xor_checksum_kernel: the read bandwidth this box sustains)
-      2. the decode step (gemv_list_kernel, one dispatch per step)
+      2. the decode step (gemv_list_kernel, one dispatch per step), then the
+         Gemma-3-1B FFN + vocabulary step (the instantiation with the column tails)
       3. the seven Qwen3-0.6B projections at M = 512 as one group over sealed
          weights (split_act_list_kernel + gemm_bf16x3_kernel, 128-token tiles)
       4. the same over raw weights (gemm_mma kernels, f32 matrix cores)
@@ -962,6 +968,27 @@ def run_traffic(host, ctx):
         "algorithmic_bytes_per_dispatch": step_bytes, "timed_dispatches": 5,
         "weights_bytes": sum(S.q8_0_bytes(p.rows, p.cols) for p in products)}
     for obj in keep:
+        (obj.buf if isinstance(obj, H.Matrix) else obj).free()
+    # 2b. the Gemma-3-1B step (79 GEMVs: rows of 1152 and of 6912 columns), one dispatch per step
+    gp, gkeep = [], []
+    for c in range(26):
+        for name, rows, cols in [s for s in S.GEMMA3_1B if s[0] != "lm_head"]:
+            gkeep.append(H.Matrix.load(ctx, S.make_weights(rows, cols, 3000 + 17 * c + len(gp)), cols, rows))
+            gp.append((gkeep[-1], rows, cols))
+    rows, cols = [s for s in S.GEMMA3_1B if s[0] == "lm_head"][0][1:]
+    gkeep.append(H.Matrix.load(ctx, S.make_weights(rows, cols, 3999), cols, rows))
+    gp.append((gkeep[-1], rows, cols))
+    gprods = []
+    for m, rows, cols in gp:
+        xb, yb = ctx.buffer(cols * 4), ctx.buffer(rows * 4)
+        xb.upload(0, S.make_activations(cols, rows))
+        gkeep += [xb, yb]
+        gprods.append(tmh_product(m.buf.raw, xb.raw, yb.raw, rows, cols, 1, TMH_GEMV))
+    run_steps(host, ctx, gprods, 0, 5, grouped=True)
+    report["gemv_list_kernel, Gemma-3-1B step"] = {
+        "algorithmic_bytes_per_dispatch": sum(S.gemv_bytes(p.rows, p.cols) for p in gprods),
+        "timed_dispatches": 5, "weights_bytes": sum(S.q8_0_bytes(p.rows, p.cols) for p in gprods)}
+    for obj in gkeep:
         (obj.buf if isinstance(obj, H.Matrix) else obj).free()
     M = 512
     for label, seal in (("gemm_bf16x3_kernel, seven projections, sealed", True),
