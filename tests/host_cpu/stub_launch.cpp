@@ -64,6 +64,7 @@ const char *variant_name(Variant v) {
     case V_SPLIT: return "split";
     case V_MMA: return "mma_f32";
     case V_BF16X3: return "bf16x3";
+    case V_MMA_SPLIT: return "mma_split";
     case V_I8_TILE: return "i8_tile";
     case V_I8_STREAM: return "i8_stream";
     case V_I8_LDS: return "i8_lds";
@@ -222,6 +223,20 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
             die("bf16 launch: partial tiles do not fit the workspace");
         }
         out += ",\"presplit\":" + std::to_string(l.bx3_presplit);
+    }
+    if (key.variant == V_MMA_SPLIT) { // every product reads the one split form the launch before has written
+        if (!key.packed || l.bx3_inputs != 1 || l.bx3_presplit != 1u) {
+            die("split-form f32-tile launch: not one input split by the launch before");
+        }
+        if (ws.xs == nullptr || l.bx3_xs_bytes > ws.xs_bytes || l.bx3_xs_bytes != bx3_xs_bytes_of(*l.list[0])) {
+            die("split-form f32-tile launch: split activations do not fit the workspace");
+        }
+        for (size_t i = 0; i < n; ++i) {
+            if (!same_input(*l.list[0], *l.list[i])) {
+                die("split-form f32-tile launch: products over different inputs");
+            }
+        }
+        out += ",\"presplit\":1";
     }
     if (l.norm != nullptr) {
         const Op &nrm = *l.norm;

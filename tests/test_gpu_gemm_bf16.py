@@ -294,6 +294,119 @@ def test_the_operator_in_front_writes_the_split_form_itself(ctx, kind, batch):
         m[4].free()
 
 
+# Launches with too few work units for the staged kernel (they keep the f32 kernel's
+# 32 x 32 tiles) right behind the operator that writes their one input: the operator
+# leaves the split form and the tiles run on the bf16 matrix cores. q,k,v at 128 tokens
+# (K over the four waves of a workgroup); one ragged product whose K is 33 blocks
+# (a last group of one block, scales off an 8-byte boundary) over two workgroups per
+# tile; K of 8 and of 2 blocks (two waves, one wave per tile); q,k,v at 256 tokens (two
+# row tiles per wave); the down projection behind the gated activation (K of 96 blocks,
+# two workgroups per tile).
+SMALL_BEHIND = [("rmsnorm", 128, 1024, [2048, 1024, 1024]), ("rmsnorm", 100, 1056, [1000]),
+                ("rmsnorm", 40, 256, [512, 33]), ("rmsnorm", 17, 64, [300]),
+                ("rmsnorm", 256, 1024, [2048, 1024, 1024]), ("silu_mul", 128, 3072, [1024]),
+                ("gelu_tanh_mul", 96, 3072, [1024])]
+
+
+@pytest.mark.parametrize("kind,batch,cols,rows_list", SMALL_BEHIND)
+def test_small_launches_behind_an_operator_read_its_split_form(ctx, kind, batch, cols, rows_list):
+    assert H.gemm_mma_launch_tile([(r, cols, batch) for r in rows_list]) == 0  # not the staged kernel
+    src = [upload_new(ctx, S.make_activations(batch * cols, 60 + i)) for i in range(2)]
+    wn = upload_new(ctx, (1.0 + 0.1 * S.make_activations(cols, 9)).astype(np.float32))
+    xb = ctx.buffer(batch * cols * 4)
+    mats = []
+    for i, rows in enumerate(rows_list):
+        w = S.make_weights(rows, cols, 900 + i)
+        mats.append((w, rows, weights_buffer(ctx, w, rows, cols, True), ctx.buffer(batch * rows * 4)))
+
+    def operator():
+        if kind == "rmsnorm":
+            ctx.rmsnorm(src[0], wn, xb, batch, cols, 1e-6)
+        elif kind == "silu_mul":
+            ctx.silu_mul(src[0], src[1], xb, batch * cols)
+        else:
+            ctx.gelu_tanh_mul(src[0], src[1], xb, batch * cols)
+
+    def products():
+        for w, rows, wb, yb in mats:
+            ctx.q8_0_gemm_mma(wb, xb, yb, rows, cols, batch, 0, 0)
+
+    def outputs():
+        ctx.fence()
+        return [m[3].download_f32(0, batch * m[1]).copy() for m in mats]
+
+    def clear():
+        xb.zero(0, batch * cols * 4)
+        for m in mats:
+            m[3].zero(0, batch * m[1] * 4)
+
+    operator()
+    ctx.fence()
+    x = xb.download_f32(0, batch * cols).copy()
+    wants = [O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8) for w, rows, _, _ in mats]
+    runs = []
+    for attempt in range(2):  # the second run finds the workspace as the first left it
+        clear()
+        before = ctx.kernel_launches()
+        ctx.begin_group()
+        operator()
+        products()
+        ctx.end_group()
+        runs.append(outputs())
+        assert ctx.kernel_launches() == before + 2  # the operator and the products: no split pass
+        assert np.array_equal(bits(xb.download_f32(0, batch * cols)), bits(x))
+    for i, want in enumerate(wants):
+        assert np.array_equal(bits(runs[0][i]), bits(runs[1][i])), f"product {i}"
+        assert norm_err(runs[0][i].reshape(batch, mats[i][1]), want) <= 1e-5, f"product {i}"
+
+    # recorded and replayed, with other work on the context in between
+    ctx.begin_group()
+    operator()
+    products()
+    step = ctx.end_group_recorded()
+    assert step.launches == 2
+    for replay in range(2):
+        clear()
+        step.run()
+        got = outputs()
+        for i in range(len(mats)):
+            assert np.array_equal(bits(got[i]), bits(runs[0][i])), f"replay {replay}, product {i}"
+    step.free()
+    for b in src + [wn, xb] + [m[2] for m in mats] + [m[3] for m in mats]:
+        b.free()
+
+
+def test_an_infinite_or_nan_activation_reaches_the_outputs_through_the_operators_split_form(ctx):
+    # silu_mul passes its second operand's non-finite values on; the products behind it
+    # then see them in the split form (whole in the first piece).
+    batch, cols, rows = 64, 1024, 512
+    g = S.make_activations(batch * cols, 71)
+    u = S.make_activations(batch * cols, 72)
+    u[5 * cols + 100] = np.inf
+    u[9 * cols + 7] = np.nan
+    gb, ub = upload_new(ctx, g), upload_new(ctx, u)
+    xb = ctx.buffer(batch * cols * 4)
+    w = S.make_weights(rows, cols, 950)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    yb = ctx.buffer(batch * rows * 4)
+    ctx.begin_group()
+    ctx.silu_mul(gb, ub, xb, batch * cols)
+    ctx.q8_0_gemm_mma(wb, xb, yb, rows, cols, batch, 0, 0)
+    ctx.end_group()
+    ctx.fence()
+    y = yb.download_f32(0, batch * rows).reshape(batch, rows)
+    x = xb.download_f32(0, batch * cols).reshape(batch, cols)
+    assert np.isinf(x[5, 100]) and np.isnan(x[9, 7])
+    assert not np.isfinite(y[5]).any() and np.isnan(y[9]).all()
+    ok = np.ones(batch, bool)
+    ok[[5, 9]] = False
+    assert np.isfinite(y[ok]).all()
+    want = O.gemm_q8_0_f32(w, rows, cols, np.ascontiguousarray(x[ok]).ravel(), int(ok.sum()), threads=8)
+    assert norm_err(y[ok], want) <= 1e-5
+    for b in [gb, ub, xb, wb, yb]:
+        b.free()
+
+
 @pytest.mark.parametrize("batch", [512, 128, 40])
 def test_update_norm_and_products_in_one_group(ctx, batch):
     # The seam between two blocks of a layer: h += t, xn = rmsnorm(h), then the

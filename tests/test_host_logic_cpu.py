@@ -491,6 +491,60 @@ def test_a_ragged_last_round_is_cut_off_as_a_tail_segment(driver):
         assert "tail" not in l and l["ops"][0]["chunks"] == 1
 
 
+def test_small_prefill_launches_behind_their_operator_take_its_split_form(driver):
+    """A layer at 128 tokens as an executor encodes it: every product launch has too
+    few work units for the staged bf16 kernel. The launches right behind the norm or
+    the gated activation that writes their one input (q,k,v; gate,up; down) run the
+    f32 kernel's tiles on the bf16 matrix cores, fed with the split form that the
+    operator leaves (fuse_split_passes); o, whose input no operator of the group
+    writes, stays on the f32 kernel, and so does everything over raw weights or when
+    the operator's result is read from an offset."""
+    M, hid, ffn = 128, 1024, 3072
+    lines = ["ctx main", f"buf nw {hid * 4}", f"buf h {M * hid * 4}", f"buf xn {(M * hid + 32) * 4}",
+             f"buf act {M * ffn * 4}"]
+    mats = (("q", 2048, hid), ("k", 1024, hid), ("v", 1024, hid), ("o", hid, 2048),
+            ("gate", ffn, hid), ("up", ffn, hid), ("down", hid, ffn))
+    for name, r, c in mats:
+        lines += [f"buf W{name} {r * (c // 32) * 34}", f"seal W{name} {r} {c}", f"buf Y{name} {M * r * 4}",
+                  f"buf R{name} {r * (c // 32) * 34}"]
+
+    def layer(prefix, x_off=0):
+        return ["begin", f"rmsnorm h nw xn {M} {hid}",
+                f"mma {prefix}q xn Yq 2048 {hid} {M} {x_off} 0", f"mma {prefix}k xn Yk 1024 {hid} {M} {x_off} 0",
+                f"mma {prefix}v xn Yv 1024 {hid} {M} {x_off} 0",
+                f"mma {prefix}o Yq Yo {hid} 2048 {M} 0 0", f"axpy Yo h 1.0 {M * hid}",  # (o reads q: no attention here)
+                f"rmsnorm h nw xn {M} {hid}",
+                f"mma {prefix}gate xn Ygate {ffn} {hid} {M} {x_off} 0",
+                f"mma {prefix}up xn Yup {ffn} {hid} {M} {x_off} 0",
+                f"silu Ygate Yup act {M * ffn}", f"mma {prefix}down act Ydown {hid} {ffn} {M} 0 0",
+                f"axpy Ydown h 1.0 {M * hid}", "end", "fence"]
+
+    lines += ["fence", "mark sealed"] + layer("W") + ["mark raw"] + layer("R") + ["mark offset"] + \
+             layer("W", x_off=32) + ["mark recorded", "begin"] + layer("W")[1:-2] + ["record s", "run s", "fence",
+                                                                                   "stepfree s", "stats"]
+    sec = sections(run_program(driver, lines))
+
+    def shape(ls):
+        return [(l["k"], l.get("variant") or l["what"], l.get("split", False)) for l in ls]
+
+    want = [("single", "rmsnorm", True), ("list", "mma_split", False), ("list", "mma_f32", False),
+            ("single", "rmsnorm", True), ("list", "mma_split", False), ("single", "silu_mul", True),
+            ("list", "mma_split", False), ("single", "f32_axpy", False)]
+    got = launches_of(sec["sealed"])
+    assert shape(got) == want, shape(got)
+    assert [len(l["ops"]) for l in got if l["k"] == "list"] == [3, 1, 2, 1]
+    assert all(l["presplit"] == 1 for l in got if l.get("variant") == "mma_split")
+    assert shape([l for l in launches_of(sec["recorded"]) if l.get("recording")]) == want
+    for name in ("raw", "offset"):
+        ls = launches_of(sec[name])
+        # (with the norm's result read from an offset, the down projection still takes the
+        # gated activation's whole result)
+        last = "mma_f32" if name == "raw" else "mma_split"
+        assert [l["variant"] for l in ls if l["k"] == "list"] == ["mma_f32"] * 3 + [last], shape(ls)
+        splits = [l.get("split", False) for l in ls if l["k"] == "single"]
+        assert splits == ([False] * 4 if name == "raw" else [False, False, True, False]), shape(ls)
+
+
 # ------------------------------------------------------------------ threads --
 
 def test_two_contexts_and_their_readers_on_four_threads_under_the_thread_sanitizer(tmp_path):

@@ -126,6 +126,25 @@ __device__ __forceinline__ float sbyte_to_float(uint32_t w, int i) {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+// 8 signed bytes (two dwords) -> 8 bf16: the conversion to f32 is exact and
+// its upper half is the bf16.
+__device__ __forceinline__ bf16x8_t sbytes_to_bf16x8(uint32_t lo, uint32_t hi) {
+    uint32_t p[4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t f0 = __builtin_bit_cast(uint32_t, sbyte_to_float(lo, 2 * i));
+        const uint32_t f1 = __builtin_bit_cast(uint32_t, sbyte_to_float(lo, 2 * i + 1));
+        p[i] = __builtin_amdgcn_perm(f1, f0, 0x07060302u);
+        const uint32_t g0 = __builtin_bit_cast(uint32_t, sbyte_to_float(hi, 2 * i));
+        const uint32_t g1 = __builtin_bit_cast(uint32_t, sbyte_to_float(hi, 2 * i + 1));
+        p[2 + i] = __builtin_amdgcn_perm(g1, g0, 0x07060302u);
+    }
+    const u32x4 v = {p[0], p[1], p[2], p[3]};
+    return __builtin_bit_cast(bf16x8_t, v);
+}
+
 
 template <bool NT, class T> __device__ __forceinline__ T load_maybe_nt(const T *p) {
     if constexpr (NT) {

@@ -35,7 +35,6 @@
 namespace q8 {
 
 typedef float floatx16_t __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 // xs holds, per Q8_0 block kb and piece p (0 = h, 1 = m, 2 = l), the 32 bf16
 // values of every token: [cols / 32][3][batch][32]. A workgroup's tokens of one
@@ -115,23 +114,6 @@ template <int WM, int WN, int TM> struct Bx3Shape {
     static constexpr int dw_bytes = rows * 4;            // per row the dword that holds its f16 scale
     static constexpr int stage_bytes = a_bytes + b_bytes + dw_bytes;
 };
-
-// 8 signed bytes (two dwords) -> 8 bf16: the conversion to f32 is exact and
-// its upper half is the bf16.
-__device__ __forceinline__ bf16x8_t sbytes_to_bf16x8(uint32_t lo, uint32_t hi) {
-    uint32_t p[4];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const uint32_t f0 = __builtin_bit_cast(uint32_t, sbyte_to_float(lo, 2 * i));
-        const uint32_t f1 = __builtin_bit_cast(uint32_t, sbyte_to_float(lo, 2 * i + 1));
-        p[i] = __builtin_amdgcn_perm(f1, f0, 0x07060302u);
-        const uint32_t g0 = __builtin_bit_cast(uint32_t, sbyte_to_float(hi, 2 * i));
-        const uint32_t g1 = __builtin_bit_cast(uint32_t, sbyte_to_float(hi, 2 * i + 1));
-        p[2 + i] = __builtin_amdgcn_perm(g1, g0, 0x07060302u);
-    }
-    const u32x4 v = {p[0], p[1], p[2], p[3]};
-    return __builtin_bit_cast(bf16x8_t, v);
-}
 
 // SEG: some descriptor of the launch covers a range of its product's rows only
 // (a product with a tail segment, bx3_plan_launch). A separate instantiation:

@@ -101,8 +101,16 @@ __device__ __forceinline__ void mma_load_block(const WView<L> &wv, const float *
 // at the tile's counter adds the z partial tiles in part order (whoever it is:
 // the result does not depend on the order of arrival), stores the sum and puts
 // the counter back to zero.
-template <int L, int TMW, int TNW, int S, bool XA, bool ZS = false>
-__global__ __launch_bounds__(256) void gemm_mma_kernel(const MmaArgs args) {
+//
+// XP: the activations come in split form (d.x points at [cols / 32][3][batch][32]
+// bf16, split_index; an operator in front of the launch has written it) and the
+// products run on the bf16 matrix cores, exactly (q8_gemm_bf16x3.hpp has the
+// argument): the lane's 16 quants of a block are exact in bf16, six
+// v_mfma_f32_32x32x16_bf16 (pieces l, m, h times the two halves of the lane's k
+// range) leave the block's sum of q*x in f32, and  acc += d * S  rescales it.
+// Six matrix instructions of 8 passes stand where sixteen of 16 passes stood.
+template <int L, int TMW, int TNW, int S, bool XA, bool ZS = false, bool XP = false>
+__global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs args) {
     static_assert(!ZS || S == 4, "shared tiles: one tile per workgroup");
     constexpr int P = 4 / S;
     constexpr int TILE_FLOATS = TMW * TNW * 16 * WAVE;
@@ -184,7 +192,137 @@ __global__ __launch_bounds__(256) void gemm_mma_kernel(const MmaArgs args) {
         }
     }
 
-    if (valid && kb_begin < kb_end) {
+    if constexpr (XP) {
+        // Activations in split form, sealed weights. What limits this path is what
+        // the waves pull through the L2, so nothing is fetched twice: the wave's
+        // K range is made of groups of four Q8_0 blocks, a group's weights are one
+        // whole 128-byte line per row (four 16-byte loads per lane, issued
+        // together) and its four scales one 8-byte load; the activations' pieces
+        // are whole lines as they are. The next group's weights and the
+        // activations of the next two blocks are on their way while a block is
+        // multiplied.
+        static_assert(L == PACKED, "split-form activations: sealed weights");
+        const uint32_t groups = (blocks + 3u) >> 2;
+        const uint32_t g_begin = (uint32_t)(((uint64_t)groups * kpart) / kparts);
+        const uint32_t g_end = (uint32_t)(((uint64_t)groups * (kpart + 1u)) / kparts);
+        const uint32_t xkb_begin = g_begin * 4u;
+        const uint32_t xkb_end = g_end * 4u < blocks ? g_end * 4u : blocks;
+        if (valid && g_begin < g_end) {
+            const uint16_t *xs = (const uint16_t *)x;
+            const bool scales8 = (blocks & 3u) == 0u; // a group's scales: one aligned 8-byte load
+            struct WGroup {
+                u32x4 q[TNW][4];
+                u32x2 sc[TNW];
+            };
+            struct XBlock {
+                u32x4 p[TMW][3][2];
+            };
+            auto load_w = [&](uint32_t grp, WGroup &into) {
+#pragma unroll
+                for (int j = 0; j < TNW; ++j) {
+                    const uint8_t *row = wv.q + (size_t)wrow[j] * cols + (half << 4);
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        uint32_t kb = grp * 4u + (uint32_t)b;
+                        kb = kb < blocks ? kb : blocks - 1u;
+                        into.q[j][b] = *(const u32x4 *)(row + (kb << 5));
+                    }
+                    const uint16_t *sp = wv.s + (size_t)wrow[j] * blocks + grp * 4u;
+                    if (scales8) {
+                        into.sc[j] = *(const u32x2 *)sp;
+                    } else {
+                        uint32_t h4[4];
+#pragma unroll
+                        for (int b = 0; b < 4; ++b) {
+                            h4[b] = grp * 4u + (uint32_t)b < blocks ? (uint32_t)sp[b] : 0u;
+                        }
+                        into.sc[j] = u32x2{h4[0] | (h4[1] << 16), h4[2] | (h4[3] << 16)};
+                    }
+                }
+            };
+            auto load_x = [&](uint32_t kb, XBlock &into) {
+#pragma unroll
+                for (int i = 0; i < TMW; ++i) {
+                    const uint16_t *base = xs + ((size_t)kb * 3u * batch + tok[i]) * 32u + (half << 4);
+#pragma unroll
+                    for (int pc = 0; pc < 3; ++pc) {
+#pragma unroll
+                        for (int k2 = 0; k2 < 2; ++k2) {
+                            into.p[i][pc][k2] = *(const u32x4 *)(base + (size_t)pc * batch * 32u + 8u * k2);
+                        }
+                    }
+                }
+            };
+            WGroup wg[2];
+            XBlock xb[2];
+            load_w(g_begin, wg[0]);
+            load_x(xkb_begin, xb[0]);
+            if (xkb_begin + 1u < xkb_end) {
+                load_x(xkb_begin + 1u, xb[1]);
+            }
+            for (uint32_t g0 = g_begin; g0 < g_end; g0 += 2u) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint32_t grp = g0 + (uint32_t)u;
+                    if (grp >= g_end) { // (uniform over the wave)
+                        break;
+                    }
+                    if (grp + 1u < g_end) {
+                        load_w(grp + 1u, wg[u ^ 1]);
+                    }
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        const uint32_t kb = grp * 4u + (uint32_t)b;
+                        if (kb >= xkb_end) {
+                            break;
+                        }
+                        bf16x8_t wb[TNW][2], xp[TMW][3][2];
+                        float dsc[TNW];
+#pragma unroll
+                        for (int j = 0; j < TNW; ++j) {
+                            const uint32_t pair = b < 2 ? wg[u].sc[j].x : wg[u].sc[j].y;
+                            dsc[j] = f16_bits_to_f32(b % 2 ? pair >> 16 : pair & 0xffffu);
+                            wb[j][0] = sbytes_to_bf16x8(wg[u].q[j][b].x, wg[u].q[j][b].y);
+                            wb[j][1] = sbytes_to_bf16x8(wg[u].q[j][b].z, wg[u].q[j][b].w);
+                        }
+#pragma unroll
+                        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+                            for (int pc = 0; pc < 3; ++pc) {
+#pragma unroll
+                                for (int k2 = 0; k2 < 2; ++k2) {
+                                    xp[i][pc][k2] = __builtin_bit_cast(bf16x8_t, xb[b % 2].p[i][pc][k2]);
+                                }
+                            }
+                        }
+                        if (kb + 2u < xkb_end) {
+                            load_x(kb + 2u, xb[b % 2]);
+                        }
+#pragma unroll
+                        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+                            for (int j = 0; j < TNW; ++j) {
+                                floatx16 sum = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
+                                                0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                                for (int piece = 2; piece >= 0; --piece) { // smallest pieces first
+#pragma unroll
+                                    for (int k2 = 0; k2 < 2; ++k2) {
+                                        sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xp[i][piece][k2], wb[j][k2],
+                                                                                      sum, 0, 0, 0);
+                                    }
+                                }
+#pragma unroll
+                                for (int v = 0; v < 16; ++v) {
+                                    acc[i][j][v] = __builtin_fmaf(dsc[j], sum[v], acc[i][j][v]);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    } else if (valid && kb_begin < kb_end) {
         MmaRaw<TMW, TNW> raw;
         mma_load_block<L, TMW, TNW, XA>(wv, x, cols, wrow, tok, kb_begin, half, raw);
         for (uint32_t kb = kb_begin; kb < kb_end; ++kb) {
@@ -831,6 +969,94 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
     Q8_LAUNCH((gemm_mma_kernel<L, TMW, TNW, S, XA>), dim3(groups), dim3(256), lds, stream, stop,
               args);
     return hipGetLastError();
+}
+
+// Products over sealed weights whose activations are in split form: prods[i].x
+// points at the split form ([cols / 32][3][batch][32] bf16) of the product's
+// activations, not at the activations.
+template <int TNW, int S>
+inline hipError_t launch_mma_split_cfg(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods_in,
+                                       int n, const MmaShared &shared) {
+    constexpr int P = 4 / S;
+    MmaArgs args;
+    args.n = (uint32_t)n;
+    args.z = 1;
+    args.partials = nullptr;
+    args.arrivals = nullptr;
+    const MmaConfig c{1, TNW, S};
+    // longest K first: the hardware hands the tiles out in list order
+    MmaProduct prods[MMA_MAX_DESCS];
+    for (int i = 0; i < n; ++i) {
+        int at = i;
+        while (at > 0 && prods[at - 1].cols < prods_in[i].cols) {
+            prods[at] = prods[at - 1];
+            --at;
+        }
+        prods[at] = prods_in[i];
+    }
+    uint64_t tiles = 0;
+    uint32_t min_blocks = 0xffffffffu;
+    for (int i = 0; i < n; ++i) {
+        MmaDesc &d = args.d[i];
+        d.w = prods[i].w;
+        d.x = prods[i].x;
+        d.y = prods[i].y;
+        d.rows = prods[i].rows;
+        d.cols = prods[i].cols;
+        d.batch = prods[i].batch;
+        d.tile_begin = (uint32_t)tiles;
+        d.tiles_t = (prods[i].batch + 31u) / 32u;
+        d.pad = 0;
+        tiles += mma_tiles(prods[i], c);
+        const uint32_t blocks = prods[i].cols / 32u;
+        min_blocks = blocks < min_blocks ? blocks : min_blocks;
+    }
+    if (tiles >= (1ull << 31)) {
+        return hipErrorInvalidValue;
+    }
+    args.total_tiles = (uint32_t)tiles;
+    args.chunk_wgs = args.d[0].tiles_t >= (uint32_t)P ? args.d[0].tiles_t / P : 1u;
+    const uint32_t groups = (uint32_t)((tiles + P - 1) / P);
+    if constexpr (S == 4 && TNW == 1) if (shared.partials != nullptr && shared.arrivals != nullptr) {
+        const uint32_t z = mma_shared_parts(tiles, min_blocks);
+        if (z > 1u) {
+            args.z = z;
+            args.partials = shared.partials;
+            args.arrivals = shared.arrivals;
+            const size_t lds = (size_t)(S - 1) * TNW * 16 * WAVE * sizeof(float);
+            Q8_LAUNCH((gemm_mma_kernel<PACKED, 1, TNW, S, true, true, true>), dim3(groups * z), dim3(256),
+                      lds, stream, stop, args);
+            return hipGetLastError();
+        }
+    }
+    const size_t lds = S > 1 ? (size_t)P * (S - 1) * TNW * 16 * WAVE * sizeof(float) : 0;
+    Q8_LAUNCH((gemm_mma_kernel<PACKED, 1, TNW, S, true, false, true>), dim3(groups), dim3(256), lds,
+              stream, stop, args);
+    return hipGetLastError();
+}
+
+inline hipError_t launch_gemm_mma_split_list(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods,
+                                             int n, const MmaShared &shared) {
+    if (n <= 0 || n > MMA_MAX_DESCS) {
+        return hipErrorInvalidValue;
+    }
+    for (int i = 0; i < n; ++i) {
+        // (the kernel indexes a product's split form in 32 bits of bf16 units)
+        if ((uint64_t)prods[i].batch * prods[i].cols * 3u >= (1ull << 32) || prods[i].cols % 32u != 0u) {
+            return hipErrorInvalidValue;
+        }
+    }
+    const MmaConfig c = pick_mma_split_config(prods, n);
+    if (c.tnw == 2) {
+        return launch_mma_split_cfg<2, 4>(stream, stop, prods, n, shared);
+    }
+    if (c.s == 4) {
+        return launch_mma_split_cfg<1, 4>(stream, stop, prods, n, shared);
+    }
+    if (c.s == 2) {
+        return launch_mma_split_cfg<1, 2>(stream, stop, prods, n, shared);
+    }
+    return launch_mma_split_cfg<1, 1>(stream, stop, prods, n, shared);
 }
 
 template <int L, bool XA>

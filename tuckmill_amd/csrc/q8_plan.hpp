@@ -106,6 +106,29 @@ inline MmaConfig pick_mma_config(const MmaProduct *prods, int n) {
 }
 
 
+// The same kernel fed with activations in split form (gemm_mma_kernel<..., XP>):
+// always the 32-token tile. Two row tiles per wave once the launch has more than
+// two rounds of workgroups (the activations' pieces are then fetched once for
+// both: at 256 tokens 4096 x 1024 takes 18 us against 22, 6144 x 1024 26 against
+// 30; with fewer workgroups the narrow tile is ahead, 1024 x 2048 at 256 tokens 12
+// us against 18). A wave's share of K is made of whole groups of four blocks, so
+// K is split over four waves from 16 blocks on.
+inline MmaConfig pick_mma_split_config(const MmaProduct *prods, int n) {
+    uint32_t min_blocks = 0xffffffffu;
+    uint64_t tiles = 0;
+    for (int i = 0; i < n; ++i) {
+        const uint32_t blocks = prods[i].cols / 32u;
+        min_blocks = blocks < min_blocks ? blocks : min_blocks;
+        tiles += (uint64_t)((prods[i].batch + 31u) / 32u) * ((prods[i].rows + 31u) / 32u);
+    }
+    MmaConfig c;
+    c.tmw = 1;
+    c.s = min_blocks >= 16u ? 4 : (min_blocks >= 8u ? 2 : 1);
+    c.tnw = c.s == 4 && tiles >= 1024u ? 2 : 1;
+    return c;
+}
+
+
 // ---- prefill GEMM on the bf16 matrix cores (q8_gemm_bf16x3.hpp) -------------
 
 constexpr int SPLIT_MAX_DESCS = 16;

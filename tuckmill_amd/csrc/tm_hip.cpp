@@ -527,7 +527,7 @@ uint32_t kernel_launches_of(const Launch &l) {
 hipError_t ensure_bx3_workspace(tm_hip_ctx *ctx, const std::vector<Launch> &plan) {
     size_t xs = 0, partial = 0;
     for (const Launch &l : plan) {
-        if (l.single == nullptr && l.key.variant == V_BF16X3) {
+        if (l.single == nullptr && (l.key.variant == V_BF16X3 || l.key.variant == V_MMA_SPLIT)) {
             xs = l.bx3_xs_bytes > xs ? (size_t)l.bx3_xs_bytes : xs;
             partial = l.bx3_partial_floats * 4u > partial ? (size_t)(l.bx3_partial_floats * 4u) : partial;
         }
@@ -699,11 +699,44 @@ void fuse_split_passes(std::vector<Launch> &plan) {
     for (size_t j = 1; j < plan.size(); ++j) {
         Launch &cons = plan[j];
         Launch &prod = plan[j - 1];
-        if (cons.single != nullptr || cons.key.variant != V_BF16X3 || prod.single == nullptr) {
+        if (cons.single != nullptr || prod.single == nullptr) {
             continue;
         }
         const Op &p = *prod.single;
         if (p.kind != OP_RMSNORM && p.kind != OP_SILU_MUL && p.kind != OP_GELU_MUL) {
+            continue;
+        }
+        auto written_whole_by = [&](const Op &op) { // `op` reads exactly what `p` writes
+            const bool whole = op.a[1] == p.a[2] && op.x_off == 0;
+            const bool shape = p.kind == OP_RMSNORM ? op.batch == p.rows && op.cols == p.cols
+                                                    : (uint64_t)op.batch * op.cols == p.extra;
+            return whole && shape;
+        };
+        if (cons.key.variant == V_MMA && cons.key.packed && prod.split_xs_off < 0) {
+            // Products left to the f32 matrix cores (too few work units for the
+            // staged kernel), all over the one input that `p` writes: with that
+            // input in split form the same tiles run on the bf16 matrix cores
+            // (gemm_mma_kernel<..., XP>), exact products in the place of f32 ones
+            // and 20-30 % less time at every size measured (at 128 tokens: 4096 x 1024
+            // 11.8 us against 16.4, 6144 x 1024 17.2 against 24.0, 1024 x 3072 12.1
+            // against 15.2). Without the operator in front a split pass of 5 us
+            // would have to make the split form: then the f32 kernel stays.
+            bool all = true;
+            for (const Op *op : cons.list) {
+                all = all && written_whole_by(*op) && same_input(*cons.list[0], *op) &&
+                      (uint64_t)op->batch * op->cols * 6u < (1ull << 32);
+            }
+            if (all) {
+                cons.key.variant = V_MMA_SPLIT;
+                cons.bx3_inputs = 1;
+                cons.bx3_presplit = 1u;
+                cons.bx3_xs_bytes = bx3_xs_bytes_of(*cons.list[0]);
+                prod.split_xs_off = 0;
+                prod.split_cols = cons.list[0]->cols;
+            }
+            continue;
+        }
+        if (cons.key.variant != V_BF16X3) {
             continue;
         }
         // the launch's distinct inputs in list order, as launch_bx3_list lays them out
@@ -722,11 +755,7 @@ void fuse_split_passes(std::vector<Launch> &plan) {
                 break;
             }
             input_of[n_in] = op;
-            const bool whole = op->a[1] == p.a[2] && op->x_off == 0;
-            const bool shape = p.kind == OP_RMSNORM
-                                   ? op->batch == p.rows && op->cols == p.cols
-                                   : (uint64_t)op->batch * op->cols == p.extra;
-            if (whole && shape && prod.split_xs_off < 0) {
+            if (written_whole_by(*op) && prod.split_xs_off < 0) {
                 prod.split_xs_off = (int64_t)off;
                 prod.split_cols = op->cols;
                 cons.bx3_presplit |= 1u << n_in;

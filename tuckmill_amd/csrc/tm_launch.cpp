@@ -199,6 +199,31 @@ hipError_t launch_mma_list(hipStream_t stream, hipEvent_t stop, const OpList &op
                                     ws.mma_queue, shared);
 }
 
+// The f32 kernel's tiles on the bf16 matrix cores: every product reads the one
+// split form that the launch before this one has left at the start of the
+// workspace.
+hipError_t launch_mma_split_list(hipStream_t stream, hipEvent_t stop, const Launch &launch,
+                                 const Workspace &ws) {
+    const OpList &ops = launch.list;
+    if (ops.empty() || launch.bx3_inputs != 1 || launch.bx3_presplit != 1u ||
+        launch.bx3_xs_bytes > ws.xs_bytes) {
+        return hipErrorInvalidValue;
+    }
+    q8::MmaProduct prods[q8::MMA_MAX_DESCS];
+    int n = 0;
+    for (const Op *op : ops) {
+        if (n == q8::MMA_MAX_DESCS || !same_input(*ops[0], *op) ||
+            bx3_xs_bytes_of(*op) > launch.bx3_xs_bytes) {
+            return hipErrorInvalidValue;
+        }
+        prods[n++] = q8::MmaProduct{(const uint8_t *)op->a[0]->ptr, (const float *)ws.xs,
+                                    (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
+                                    op->batch};
+    }
+    const q8::MmaShared shared{ws.mma_partials, ws.arrivals};
+    return q8::launch_gemm_mma_split_list(stream, stop, prods, n, shared);
+}
+
 // The split-float GEMM: one launch that splits every distinct input of the list
 // into its three bf16 planes, then the product list. The workspace was sized by
 // ensure_bx3_workspace() when the launches were planned.
@@ -295,6 +320,9 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
     GemvKey key = launch.key;
     if (key.variant == V_BF16X3) {
         return launch_bx3_list(stream, stop, launch, ws);
+    }
+    if (key.variant == V_MMA_SPLIT) {
+        return launch_mma_split_list(stream, stop, launch, ws);
     }
     if (key.kind == OP_MMA) {
         return launch_mma_list(stream, stop, ops, key, ws);

@@ -92,6 +92,8 @@ enum Variant : uint8_t {
     V_MMA,        // f32 MFMA GEMM: p0 = tmw, p1 = tnw, p2 = K split
     V_BF16X3,     // prefill GEMM on the bf16 matrix cores, activations split in three:
                   // p0 = tokens per tile / 64
+    V_MMA_SPLIT,  // the f32 kernel's tiles on the bf16 matrix cores, fed with the split form that
+                  // the operator right before the launch has written (fuse_split_passes)
     V_I8_TILE,    // register-fed int8 MFMA GEMM: p0 = tile configuration
     V_I8_STREAM,  // int8 streaming kernel: p0 = tokens per pass
     V_I8_LDS,     // LDS-staged int8 MFMA GEMM: p0 = workgroup shape (q8::i8_lds_shape),
@@ -232,7 +234,8 @@ struct Launch {
     // one descriptor per product and token.
     bool per_token = false;
     // V_BF16X3: bit i set = the launch's i-th distinct input (in list order)
-    // arrives split already, written by the launch just before this one.
+    // arrives split already, written by the launch just before this one
+    // (V_MMA_SPLIT: its one input always does).
     uint32_t bx3_presplit = 0;
     // An RMSNorm or gated activation on its own whose result is the next
     // launch's input: byte offset in the split workspace where it writes the
