@@ -228,9 +228,26 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
         if (!key.packed || l.bx3_inputs != 1 || l.bx3_presplit != 1u) {
             die("split-form f32-tile launch: not one input split by the launch before");
         }
-        if (ws.xs == nullptr || l.bx3_xs_bytes > ws.xs_bytes || l.bx3_xs_bytes != bx3_xs_bytes_of(*l.list[0])) {
+        const uint64_t in_end = l.xs_in_off + bx3_xs_bytes_of(*l.list[0]);
+        if (ws.xs == nullptr || l.bx3_xs_bytes > ws.xs_bytes || in_end > l.bx3_xs_bytes || l.xs_in_off % 256u != 0u) {
             die("split-form f32-tile launch: split activations do not fit the workspace");
         }
+        if (l.glu[0] != nullptr) { // gate, up and the gated activation; its split form goes behind the input's
+            const Op &act = *l.glu[0];
+            if (n != 2 || l.list[0]->rows != l.list[1]->rows || l.list[0]->cols != l.list[1]->cols ||
+                act.extra != (uint64_t)l.list[0]->rows * l.list[0]->batch) {
+                die("split-form f32-tile launch: gated pair of unlike projections");
+            }
+            if (l.split_xs_off >= 0 &&
+                ((uint64_t)l.split_xs_off < in_end ||
+                 (uint64_t)l.split_xs_off + (uint64_t)act.extra * 6u > l.bx3_xs_bytes || l.split_cols != l.list[0]->rows)) {
+                die("split-form f32-tile launch: the activation's split form overlaps the input's or the end");
+            }
+            out += std::string(",\"split_out\":") + (l.split_xs_off >= 0 ? "true" : "false");
+        } else if (l.split_xs_off >= 0 || in_end != l.bx3_xs_bytes) {
+            die("split-form f32-tile launch: workspace figures do not match its products");
+        }
+        out += ",\"xs_in_off\":" + std::to_string(l.xs_in_off);
         for (size_t i = 0; i < n; ++i) {
             if (!same_input(*l.list[0], *l.list[i])) {
                 die("split-form f32-tile launch: products over different inputs");

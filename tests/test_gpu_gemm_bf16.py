@@ -376,6 +376,97 @@ def test_small_launches_behind_an_operator_read_its_split_form(ctx, kind, batch,
         b.free()
 
 
+@pytest.mark.parametrize("kind,batch,hid,ffn,in_place",
+                         [("silu_mul", 128, 1024, 3072, False), ("gelu_tanh_mul", 100, 1056, 1120, False),
+                          ("silu_mul", 64, 1024, 3072, True), ("silu_mul", 40, 256, 512, False)])
+def test_the_gated_activation_rides_in_the_launch_of_gate_and_up(ctx, kind, batch, hid, ffn, in_place):
+    # The feed-forward half of a layer at a small prefill size: norm, gate and up, the
+    # gated activation, down. In one group that is three launches: gate and up with the
+    # activation in their launch, which also leaves the activation's split form for the
+    # down projection. Every buffer comes out bit for bit as from the same operations in
+    # two groups (norm, gate, up | activation, down), where the activation launches on
+    # its own. In place (the activation over the gate's buffer) the raw gate is not kept,
+    # as with the operator on its own.
+    h = upload_new(ctx, S.make_activations(batch * hid, 31))
+    wn = upload_new(ctx, (1.0 + 0.1 * S.make_activations(hid, 9)).astype(np.float32))
+    xn = ctx.buffer(batch * hid * 4)
+    wg, wu, wd = (S.make_weights(ffn, hid, 960), S.make_weights(ffn, hid, 961), S.make_weights(hid, ffn, 962))
+    bg, bu, bd = (weights_buffer(ctx, wg, ffn, hid, True), weights_buffer(ctx, wu, ffn, hid, True),
+                  weights_buffer(ctx, wd, hid, ffn, True))
+    yg, yu, yd = ctx.buffer(batch * ffn * 4), ctx.buffer(batch * ffn * 4), ctx.buffer(batch * hid * 4)
+    act = yg if in_place else ctx.buffer(batch * ffn * 4)
+    bufs = [(xn, batch * hid), (yg, batch * ffn), (yu, batch * ffn), (act, batch * ffn), (yd, batch * hid)]
+
+    def front():
+        ctx.rmsnorm(h, wn, xn, batch, hid, 1e-6)
+        ctx.q8_0_gemm_mma(bg, xn, yg, ffn, hid, batch, 0, 0)
+        ctx.q8_0_gemm_mma(bu, xn, yu, ffn, hid, batch, 0, 0)
+
+    def back():
+        (ctx.silu_mul if kind == "silu_mul" else ctx.gelu_tanh_mul)(yg, yu, act, batch * ffn)
+        ctx.q8_0_gemm_mma(bd, act, yd, hid, ffn, batch, 0, 0)
+
+    def state():
+        ctx.fence()
+        return [b.download_f32(0, n).copy() for b, n in bufs]
+
+    def clear():
+        for b, n in bufs:
+            b.zero(0, n * 4)
+
+    clear()
+    before = ctx.kernel_launches()
+    ctx.begin_group()
+    front()
+    ctx.end_group()
+    raw_gate = yg.download_f32(0, batch * ffn).copy()
+    ctx.begin_group()
+    back()
+    ctx.end_group()
+    apart = state()
+    assert ctx.kernel_launches() == before + 4
+
+    for attempt in range(2):
+        clear()
+        before = ctx.kernel_launches()
+        ctx.begin_group()
+        front()
+        back()
+        ctx.end_group()
+        fused = state()
+        assert ctx.kernel_launches() == before + 3
+        for i, (a, b) in enumerate(zip(apart, fused)):
+            assert np.array_equal(bits(a), bits(b)), f"attempt {attempt}, buffer {i}"
+
+    x = apart[0]
+    g_want = O.gemm_q8_0_f32(wg, ffn, hid, x, batch, threads=8)
+    assert norm_err(raw_gate.reshape(batch, ffn), g_want) <= 1e-5
+    u = apart[2].astype(np.float64)
+    g = raw_gate.astype(np.float64)
+    if kind == "silu_mul":
+        a_want = g / (1.0 + np.exp(-g)) * u
+    else:
+        a_want = 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * g * (1.0 + 0.044715 * g * g))) * u
+    assert np.abs(apart[3] - a_want).max() <= 1e-5 * max(1.0, np.abs(a_want).max())
+    d_want = O.gemm_q8_0_f32(wd, hid, ffn, apart[3], batch, threads=8)
+    assert norm_err(apart[4].reshape(batch, hid), d_want) <= 1e-5
+
+    ctx.begin_group()
+    front()
+    back()
+    step = ctx.end_group_recorded()
+    assert step.launches == 3
+    for replay in range(2):
+        clear()
+        step.run()
+        got = state()
+        for i, (a, b) in enumerate(zip(apart, got)):
+            assert np.array_equal(bits(a), bits(b)), f"replay {replay}, buffer {i}"
+    step.free()
+    for b in {h, wn, xn, bg, bu, bd, yg, yu, yd, act}:
+        b.free()
+
+
 def test_an_infinite_or_nan_activation_reaches_the_outputs_through_the_operators_split_form(ctx):
     # silu_mul passes its second operand's non-finite values on; the products behind it
     # then see them in the split form (whole in the first piece).

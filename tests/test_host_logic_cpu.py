@@ -527,13 +527,18 @@ def test_small_prefill_launches_behind_their_operator_take_its_split_form(driver
     def shape(ls):
         return [(l["k"], l.get("variant") or l["what"], l.get("split", False)) for l in ls]
 
+    # (the gated activation rides in the launch of gate and up, which leaves its split
+    # form for the down projection behind its own input's: 7 launches)
     want = [("single", "rmsnorm", True), ("list", "mma_split", False), ("list", "mma_f32", False),
-            ("single", "rmsnorm", True), ("list", "mma_split", False), ("single", "silu_mul", True),
-            ("list", "mma_split", False), ("single", "f32_axpy", False)]
+            ("single", "rmsnorm", True), ("list", "mma_split", False), ("list", "mma_split", False),
+            ("single", "f32_axpy", False)]
     got = launches_of(sec["sealed"])
     assert shape(got) == want, shape(got)
     assert [len(l["ops"]) for l in got if l["k"] == "list"] == [3, 1, 2, 1]
     assert all(l["presplit"] == 1 for l in got if l.get("variant") == "mma_split")
+    pair, down = got[4], got[5]
+    assert "glu" in pair["ops"][0] and pair["split_out"] and pair["xs_in_off"] == 0
+    assert down["xs_in_off"] == M * hid * 6 and "glu" not in down["ops"][0]
     assert shape([l for l in launches_of(sec["recorded"]) if l.get("recording")]) == want
     for name in ("raw", "offset"):
         ls = launches_of(sec[name])

@@ -55,6 +55,17 @@ __device__ __forceinline__ void split3_bf16(float x, uint32_t &h, uint32_t &m, u
     l = __builtin_bit_cast(uint32_t, r2) >> 16;
 }
 
+// act(g) * u of the gated activations fused into product kernels: silu (kind 0) or
+// ggml's tanh GELU (kind 1), the expressions of silu_mul_kernel / gelu_tanh_mul_kernel.
+__device__ __forceinline__ float glu_act(float g, float u, uint32_t kind) {
+    if (kind == 0u) {
+        const float s = g / (1.0f + expf(-g));
+        return s * u;
+    }
+    const float inner = 0.7978845608028654f * g * (1.0f + 0.044715f * g * g);
+    return 0.5f * g * (1.0f + tanhf(inner)) * u;
+}
+
 // Where the pieces of element (token t, column k) of a [batch][cols] matrix live
 // in its split form [cols / 32][3][batch][32] (bf16 units): the h piece at the
 // returned index, m and l each batch * 32 further on.

@@ -54,6 +54,17 @@ struct MmaDesc {
     uint32_t pad;
 };
 
+// A launch of gemm_mma_kernel<..., GLU>: its one descriptor is the gate projection,
+// this the up projection over the same activations and what becomes of the pair.
+struct MmaGlu {
+    const uint8_t *w2 = nullptr; // the up projection's weights (the descriptor's shape)
+    float *y2 = nullptr;         // its output
+    float *act = nullptr;        // act(gate) * up, [batch][rows]; may be the gate's output (in place)
+    uint16_t *act_split = nullptr; // the split form of `act` as [rows / 32][3][batch][32] bf16, or null
+    uint32_t kind = 0;           // 0 silu, 1 tanh GELU
+    uint32_t pad = 0;
+};
+
 struct MmaArgs {
     uint32_t n;
     uint32_t total_tiles;
@@ -61,6 +72,7 @@ struct MmaArgs {
     uint32_t z;         // workgroups that share one output tile, each with a part of K (1: none)
     float *partials;    // z > 1: total_tiles x z partial tiles
     uint32_t *arrivals; // z > 1: one counter per output tile, zero between launches
+    MmaGlu glu;
     MmaDesc d[MMA_MAX_DESCS];
 };
 
@@ -109,9 +121,18 @@ __device__ __forceinline__ void mma_load_block(const WView<L> &wv, const float *
 // v_mfma_f32_32x32x16_bf16 (pieces l, m, h times the two halves of the lane's k
 // range) leave the block's sum of q*x in f32, and  acc += d * S  rescales it.
 // Six matrix instructions of 8 passes stand where sixteen of 16 passes stood.
-template <int L, int TMW, int TNW, int S, bool XA, bool ZS = false, bool XP = false>
+//
+// GLU (with XP): the launch is the gate and the up projection of a gated unit
+// (same shape, same activations) and the activation behind them. A wave's two
+// accumulator tiles are the same 32 x 32 outputs of both; the wave that holds the
+// sums stores the projections, act(gate) * up and, for a product launched right
+// behind, its split form: one launch and one pass over the outputs in the place of
+// two. Every sum is formed as in the launch without the activation.
+template <int L, int TMW, int TNW, int S, bool XA, bool ZS = false, bool XP = false, bool GLU = false>
 __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs args) {
     static_assert(!ZS || S == 4, "shared tiles: one tile per workgroup");
+    static_assert(!GLU || (XP && TMW == 1 && TNW == 2 && !ZS), "gated pair: two accumulators over one 32 x 32 tile");
+    constexpr int TNG = GLU ? 1 : TNW; // row tiles of 32 that a wave's outputs span
     constexpr int P = 4 / S;
     constexpr int TILE_FLOATS = TMW * TNW * 16 * WAVE;
     extern __shared__ float red[]; // [P][S-1][TILE_FLOATS]
@@ -156,11 +177,12 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
     const uint32_t rows = d.rows, cols = d.cols, batch = d.batch;
     const uint32_t local = valid ? tile - d.tile_begin : 0u;
     const uint32_t tn = local / d.tiles_t, tt = local % d.tiles_t;
-    const uint32_t t0 = tt * (32u * TMW), n0 = tn * (32u * TNW);
+    const uint32_t t0 = tt * (32u * TMW), n0 = tn * (32u * TNG);
     const float *x = d.x;
     float *y = d.y;
 
     const WView<L> wv(d.w, rows, cols);
+    const WView<L> wv2(GLU ? args.glu.w2 : d.w, rows, cols); // GLU: the up projection
     const uint32_t blocks = cols >> 5;
     // this wave's part of K: one of S, or with shared tiles one of z x S
     const uint32_t kparts = ZS ? args.z * (uint32_t)S : (uint32_t)S;
@@ -171,7 +193,7 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
     uint32_t wrow[TNW], tok[TMW];
 #pragma unroll
     for (int j = 0; j < TNW; ++j) {
-        const uint32_t r = n0 + 32u * j + idx;
+        const uint32_t r = n0 + (GLU ? 0u : 32u * j) + idx;
         wrow[j] = r < rows ? r : rows - 1u;
     }
 #pragma unroll
@@ -220,14 +242,15 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
             auto load_w = [&](uint32_t grp, WGroup &into) {
 #pragma unroll
                 for (int j = 0; j < TNW; ++j) {
-                    const uint8_t *row = wv.q + (size_t)wrow[j] * cols + (half << 4);
+                    const WView<L> &view = GLU && j == 1 ? wv2 : wv;
+                    const uint8_t *row = view.q + (size_t)wrow[j] * cols + (half << 4);
 #pragma unroll
                     for (int b = 0; b < 4; ++b) {
                         uint32_t kb = grp * 4u + (uint32_t)b;
                         kb = kb < blocks ? kb : blocks - 1u;
                         into.q[j][b] = *(const u32x4 *)(row + (kb << 5));
                     }
-                    const uint16_t *sp = wv.s + (size_t)wrow[j] * blocks + grp * 4u;
+                    const uint16_t *sp = view.s + (size_t)wrow[j] * blocks + grp * 4u;
                     if (scales8) {
                         into.sc[j] = *(const u32x2 *)sp;
                     } else {
@@ -360,7 +383,87 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
         }
     }
 
-    if constexpr (S > 1) {
+    if constexpr (XP && !ZS && S > 1) {
+        // The matrix instructions of these launches are short, so what follows them
+        // counts: every wave leaves its partial tile in LDS, and wave s adds up (in
+        // wave order, as the one-wave form below does) and stores the 16 / S values
+        // per lane and tile that start at value (16 / S) * s.
+        constexpr int VQ = 16 / S;
+        float *slot = red + (size_t)p * S * TILE_FLOATS; // [S][TILE_FLOATS]
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+            for (int j = 0; j < TNW; ++j) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    slot[(size_t)s * TILE_FLOATS + ((i * TNW + j) * 16 + v) * WAVE + lane] = acc[i][j][v];
+                }
+            }
+        }
+        __syncthreads();
+        if (!valid) {
+            return;
+        }
+        float fin[TMW][TNW][VQ];
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+            for (int j = 0; j < TNW; ++j) {
+#pragma unroll
+                for (int vv = 0; vv < VQ; ++vv) {
+                    const uint32_t at = ((i * TNW + j) * 16 + (uint32_t)VQ * s + vv) * WAVE + lane;
+                    float sum = slot[at];
+#pragma unroll
+                    for (int o = 1; o < S; ++o) {
+                        sum += slot[(size_t)o * TILE_FLOATS + at];
+                    }
+                    fin[i][j][vv] = sum;
+                }
+            }
+        }
+        // value v of a 32x32 tile is (token 8*(v/4) + 4*half + v%4, row idx)
+        if constexpr (GLU) {
+            const uint32_t n = n0 + idx;
+            float *y2 = args.glu.y2, *act = args.glu.act;
+            uint16_t *act_split = args.glu.act_split;
+            const uint32_t kind = args.glu.kind;
+#pragma unroll
+            for (int vv = 0; vv < VQ; ++vv) {
+                const uint32_t v = (uint32_t)VQ * s + vv;
+                const uint32_t t = t0 + 8u * (v / 4u) + 4u * half + (v % 4u);
+                if (t < batch && n < rows) {
+                    const float gv = fin[0][0][vv], uv = fin[0][1][vv];
+                    const float a = glu_act(gv, uv, kind);
+                    const size_t at = (size_t)t * rows + n;
+                    if (act != y) {
+                        y[at] = gv;
+                    }
+                    y2[at] = uv;
+                    act[at] = a;
+                    if (act_split != nullptr) {
+                        split_store(act_split, batch, t, n, a);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+                for (int j = 0; j < TNW; ++j) {
+                    const uint32_t n = n0 + 32u * j + idx;
+#pragma unroll
+                    for (int vv = 0; vv < VQ; ++vv) {
+                        const uint32_t v = (uint32_t)VQ * s + vv;
+                        const uint32_t t = t0 + 32u * i + 8u * (v / 4u) + 4u * half + (v % 4u);
+                        if (t < batch && n < rows) {
+                            y[(size_t)t * rows + n] = fin[i][j][vv];
+                        }
+                    }
+                }
+            }
+        }
+        return;
+    } else if constexpr (S > 1) {
         if (s > 0u) {
             float *mine = red + ((size_t)p * (S - 1) + (s - 1u)) * TILE_FLOATS;
 #pragma unroll
@@ -457,6 +560,30 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
         }
     }
     // acc[v] of a 32x32 tile is (token 8*(v/4) + 4*half + v%4, row idx).
+    if constexpr (GLU) {
+        const uint32_t n = n0 + idx;
+        float *y2 = args.glu.y2, *act = args.glu.act;
+        uint16_t *act_split = args.glu.act_split;
+        const uint32_t kind = args.glu.kind;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const uint32_t t = t0 + 8u * (v / 4) + 4u * half + (v % 4);
+            if (t < batch && n < rows) {
+                const float gv = acc[0][0][v], uv = acc[0][1][v];
+                const float a = glu_act(gv, uv, kind);
+                const size_t at = (size_t)t * rows + n;
+                if (act != y) {
+                    y[at] = gv;
+                }
+                y2[at] = uv;
+                act[at] = a;
+                if (act_split != nullptr) {
+                    split_store(act_split, batch, t, n, a);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TMW; ++i) {
 #pragma unroll
@@ -976,7 +1103,7 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
 // activations, not at the activations.
 template <int TNW, int S>
 inline hipError_t launch_mma_split_cfg(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods_in,
-                                       int n, const MmaShared &shared) {
+                                       int n, const MmaShared &shared, const MmaGlu *glu = nullptr) {
     constexpr int P = 4 / S;
     MmaArgs args;
     args.n = (uint32_t)n;
@@ -1017,6 +1144,13 @@ inline hipError_t launch_mma_split_cfg(hipStream_t stream, hipEvent_t stop, cons
     args.total_tiles = (uint32_t)tiles;
     args.chunk_wgs = args.d[0].tiles_t >= (uint32_t)P ? args.d[0].tiles_t / P : 1u;
     const uint32_t groups = (uint32_t)((tiles + P - 1) / P);
+    if constexpr (TNW == 1) if (glu != nullptr) { // (n == 1: the gate projection's descriptor)
+        args.glu = *glu;
+        const size_t lds = S > 1 ? (size_t)P * S * 2 * 16 * WAVE * sizeof(float) : 0;
+        Q8_LAUNCH((gemm_mma_kernel<PACKED, 1, 2, S, true, false, true, true>), dim3(groups), dim3(256), lds,
+                  stream, stop, args);
+        return hipGetLastError();
+    }
     if constexpr (S == 4 && TNW == 1) if (shared.partials != nullptr && shared.arrivals != nullptr) {
         const uint32_t z = mma_shared_parts(tiles, min_blocks);
         if (z > 1u) {
@@ -1029,16 +1163,34 @@ inline hipError_t launch_mma_split_cfg(hipStream_t stream, hipEvent_t stop, cons
             return hipGetLastError();
         }
     }
-    const size_t lds = S > 1 ? (size_t)P * (S - 1) * TNW * 16 * WAVE * sizeof(float) : 0;
+    const size_t lds = S > 1 ? (size_t)P * S * TNW * 16 * WAVE * sizeof(float) : 0; // every wave's partial tile
     Q8_LAUNCH((gemm_mma_kernel<PACKED, 1, TNW, S, true, false, true>), dim3(groups), dim3(256), lds,
               stream, stop, args);
     return hipGetLastError();
 }
 
+// `glu`: the list is the gate projection alone; glu names the up projection, the
+// activation's kind and where its result goes (gemm_mma_kernel<..., GLU>).
 inline hipError_t launch_gemm_mma_split_list(hipStream_t stream, hipEvent_t stop, const MmaProduct *prods,
-                                             int n, const MmaShared &shared) {
+                                             int n, const MmaShared &shared, const MmaGlu *glu = nullptr) {
     if (n <= 0 || n > MMA_MAX_DESCS) {
         return hipErrorInvalidValue;
+    }
+    if (glu != nullptr) {
+        if (n != 1 || glu->w2 == nullptr || glu->y2 == nullptr || glu->act == nullptr || glu->kind > 1u ||
+            (uint64_t)prods[0].batch * prods[0].cols * 3u >= (1ull << 32) || prods[0].cols % 32u != 0u ||
+            (glu->act_split != nullptr &&
+             ((uint64_t)prods[0].batch * prods[0].rows * 3u >= (1ull << 32) || prods[0].rows % 32u != 0u))) {
+            return hipErrorInvalidValue;
+        }
+        const uint32_t blocks = prods[0].cols / 32u;
+        if (blocks >= 16u) {
+            return launch_mma_split_cfg<1, 4>(stream, stop, prods, 1, shared, glu);
+        }
+        if (blocks >= 8u) {
+            return launch_mma_split_cfg<1, 2>(stream, stop, prods, 1, shared, glu);
+        }
+        return launch_mma_split_cfg<1, 1>(stream, stop, prods, 1, shared, glu);
     }
     for (int i = 0; i < n; ++i) {
         // (the kernel indexes a product's split form in 32 bits of bf16 units)

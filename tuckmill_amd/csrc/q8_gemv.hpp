@@ -866,15 +866,6 @@ __device__ __forceinline__ void stream_rows_raw(const WView<RAW> &wv, const floa
 // r0..r0+3 and lanes 32, 40, 48, 56 the up rows; one exchange pairs them. The
 // raw projections are stored as well (the gate's only when `out` is another
 // buffer: in place, the activation replaces it as the separate operator would).
-__device__ __forceinline__ float glu_act(float g, float u, uint32_t kind) {
-    if (kind == 0u) {
-        const float s = g / (1.0f + expf(-g));
-        return s * u;
-    }
-    const float inner = 0.7978845608028654f * g * (1.0f + 0.044715f * g * g);
-    return 0.5f * g * (1.0f + tanhf(inner)) * u;
-}
-
 // The same with passes of 2 gate rows and 2 up rows (a pair of few rows cut
 // into short tiles, so that more waves share it): acc = [g0, g1, u0, u1]; the
 // butterfly halves the values per lane at the shuffles over 32 and 16 lanes,

@@ -695,6 +695,57 @@ void cut_bx3_launch(Launch &l, uint64_t max_partial_floats = kBx3MaxPartialFloat
 // place in the workspace where the product launch expects it, and the input
 // drops out of the split pass. Both launches are neighbours on one stream, so
 // nothing else touches the workspace in between.
+// plan[at] has just become a V_MMA_SPLIT launch. If it is the gate and the up
+// projection of a gated unit, plan[at + 1] the gated activation over exactly their
+// outputs and plan[at + 2] a launch of the same kind over exactly the activation's
+// result (the down projection), the activation moves into the pair's launch, which
+// then writes the projections, the activation and its split form (behind its own
+// input's in the workspace): a layer's feed-forward half is three launches instead
+// of four, every result with the same bits.
+void fuse_gated_pair(std::vector<Launch> &plan, size_t at) {
+    if (at + 2 >= plan.size()) {
+        return;
+    }
+    Launch &pair = plan[at];
+    Launch &actl = plan[at + 1];
+    Launch &down = plan[at + 2];
+    if (pair.list.size() != 2 || actl.single == nullptr || actl.update != nullptr || actl.split_xs_off >= 0 ||
+        down.single != nullptr || down.key.variant != V_MMA || !down.key.packed) {
+        return;
+    }
+    const Op &act = *actl.single;
+    if (act.kind != OP_SILU_MUL && act.kind != OP_GELU_MUL) {
+        return;
+    }
+    const Op *pg = pair.list[0], *pu = pair.list[1];
+    const Alloc *out = act.a[2];
+    const bool shapes = pg->rows == pu->rows && pg->cols == pu->cols && pg->y_off == 0 && pu->y_off == 0 &&
+                        act.extra == (uint64_t)pg->rows * pg->batch && pg->rows % 32u == 0u;
+    const bool wiring = pg->a[2] == act.a[0] && pu->a[2] == act.a[1] && pg->a[2] != pu->a[2] &&
+                        out != pu->a[2] && out != pg->a[0] && out != pu->a[0];
+    if (!shapes || !wiring) {
+        return;
+    }
+    for (const Op *op : down.list) {
+        const bool whole = op->a[1] == out && op->x_off == 0 &&
+                           (uint64_t)op->batch * op->cols == act.extra && op->cols == pg->rows;
+        if (!whole || !same_input(*down.list[0], *op) || (uint64_t)op->batch * op->cols * 6u >= (1ull << 32) ||
+            op->a[2] == out || op->a[2] == pg->a[2] || op->a[2] == pu->a[2]) {
+            return;
+        }
+    }
+    pair.glu[0] = &act;
+    pair.split_xs_off = (int64_t)pair.bx3_xs_bytes; // behind the pair's own input
+    pair.split_cols = down.list[0]->cols;
+    down.key.variant = V_MMA_SPLIT;
+    down.bx3_inputs = 1;
+    down.bx3_presplit = 1u;
+    down.xs_in_off = pair.bx3_xs_bytes;
+    down.bx3_xs_bytes = down.xs_in_off + bx3_xs_bytes_of(*down.list[0]);
+    pair.bx3_xs_bytes = down.bx3_xs_bytes;
+    plan.erase(plan.begin() + (ptrdiff_t)(at + 1));
+}
+
 void fuse_split_passes(std::vector<Launch> &plan) {
     for (size_t j = 1; j < plan.size(); ++j) {
         Launch &cons = plan[j];
@@ -730,9 +781,11 @@ void fuse_split_passes(std::vector<Launch> &plan) {
                 cons.key.variant = V_MMA_SPLIT;
                 cons.bx3_inputs = 1;
                 cons.bx3_presplit = 1u;
+                cons.xs_in_off = 0;
                 cons.bx3_xs_bytes = bx3_xs_bytes_of(*cons.list[0]);
                 prod.split_xs_off = 0;
                 prod.split_cols = cons.list[0]->cols;
+                fuse_gated_pair(plan, j);
             }
             continue;
         }

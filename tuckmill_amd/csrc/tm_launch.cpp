@@ -200,27 +200,46 @@ hipError_t launch_mma_list(hipStream_t stream, hipEvent_t stop, const OpList &op
 }
 
 // The f32 kernel's tiles on the bf16 matrix cores: every product reads the one
-// split form that the launch before this one has left at the start of the
-// workspace.
+// split form that the launch before this one has left in the workspace
+// (at Launch::xs_in_off).
 hipError_t launch_mma_split_list(hipStream_t stream, hipEvent_t stop, const Launch &launch,
                                  const Workspace &ws) {
     const OpList &ops = launch.list;
     if (ops.empty() || launch.bx3_inputs != 1 || launch.bx3_presplit != 1u ||
-        launch.bx3_xs_bytes > ws.xs_bytes) {
+        launch.bx3_xs_bytes > ws.xs_bytes || launch.xs_in_off + bx3_xs_bytes_of(*ops[0]) > launch.bx3_xs_bytes) {
         return hipErrorInvalidValue;
     }
     q8::MmaProduct prods[q8::MMA_MAX_DESCS];
     int n = 0;
     for (const Op *op : ops) {
-        if (n == q8::MMA_MAX_DESCS || !same_input(*ops[0], *op) ||
-            bx3_xs_bytes_of(*op) > launch.bx3_xs_bytes) {
+        if (n == q8::MMA_MAX_DESCS || !same_input(*ops[0], *op)) {
             return hipErrorInvalidValue;
         }
-        prods[n++] = q8::MmaProduct{(const uint8_t *)op->a[0]->ptr, (const float *)ws.xs,
+        prods[n++] = q8::MmaProduct{(const uint8_t *)op->a[0]->ptr,
+                                    (const float *)(ws.xs + launch.xs_in_off),
                                     (float *)op->a[2]->ptr + op->y_off, op->rows, op->cols,
                                     op->batch};
     }
     const q8::MmaShared shared{ws.mma_partials, ws.arrivals};
+    if (launch.glu.size() == ops.size() && launch.glu[0] != nullptr) {
+        // gate, up and the gated activation behind them as one launch
+        const Op &act = *launch.glu[0];
+        if (n != 2 || ops[0]->rows != ops[1]->rows || ops[0]->cols != ops[1]->cols ||
+            ops[0]->y_off != 0 || ops[1]->y_off != 0 || act.a[0] != ops[0]->a[2] || act.a[1] != ops[1]->a[2] ||
+            (act.kind != OP_SILU_MUL && act.kind != OP_GELU_MUL) ||
+            act.extra != (uint64_t)ops[0]->rows * ops[0]->batch ||
+            (launch.split_xs_off >= 0 &&
+             (uint64_t)launch.split_xs_off + (uint64_t)ops[0]->batch * ops[0]->rows * 6u > ws.xs_bytes)) {
+            return hipErrorInvalidValue;
+        }
+        q8::MmaGlu glu;
+        glu.w2 = prods[1].w;
+        glu.y2 = prods[1].y;
+        glu.act = (float *)act.a[2]->ptr;
+        glu.act_split = launch.split_xs_off >= 0 ? (uint16_t *)(ws.xs + launch.split_xs_off) : nullptr;
+        glu.kind = act.kind == OP_SILU_MUL ? 0u : 1u;
+        return q8::launch_gemm_mma_split_list(stream, stop, prods, 1, shared, &glu);
+    }
     return q8::launch_gemm_mma_split_list(stream, stop, prods, n, shared);
 }
 

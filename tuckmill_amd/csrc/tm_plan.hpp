@@ -237,9 +237,12 @@ struct Launch {
     // arrives split already, written by the launch just before this one
     // (V_MMA_SPLIT: its one input always does).
     uint32_t bx3_presplit = 0;
-    // An RMSNorm or gated activation on its own whose result is the next
-    // launch's input: byte offset in the split workspace where it writes the
-    // split form as well, or -1.
+    // V_MMA_SPLIT: byte offset in the split workspace of the launch's input.
+    uint64_t xs_in_off = 0;
+    // An RMSNorm or gated activation on its own (or a V_MMA_SPLIT launch with the
+    // gated activation fused in, glu[0]) whose result is the next launch's input:
+    // byte offset in the split workspace where it writes the split form as well,
+    // or -1.
     int64_t split_xs_off = -1;
     uint32_t split_cols = 0; // the row length that result is cut by
     // An RMSNorm on its own: the residual update of its input that it does first.
