@@ -104,9 +104,10 @@ __device__ __forceinline__ void mma_load_block(const WView<L> &wv, const float *
 // prefill chunk share their input and do not depend on each other).
 // Workgroup = 4 waves = P slots x S k-slices. Slot p of workgroup g owns
 // output tile g*P + p of the launch; its S waves each take a contiguous share
-// of the Q8_0 blocks and wave s = 0 adds the partial tiles of s = 1..S-1 in
-// that order. The k loop is software-pipelined: the operands of block kb+1
-// are requested before the 16*TMW*TNW MFMAs of block kb are issued.
+// of the Q8_0 blocks; the partial tiles are added in wave order, each wave
+// finishing and storing 16 / S of a lane's 16 values per tile. The k loop is
+// software-pipelined: the operands of block kb+1 are requested before the
+// 16*TMW*TNW MFMAs of block kb are issued.
 // ZS: args.z workgroups share an output tile (S == 4 only: one tile per
 // workgroup). Workgroup g takes part g % z of the K range of tile g / z; what its
 // four waves add up goes to args.partials, and the workgroup that arrives last
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
     constexpr int TNG = GLU ? 1 : TNW; // row tiles of 32 that a wave's outputs span
     constexpr int P = 4 / S;
     constexpr int TILE_FLOATS = TMW * TNW * 16 * WAVE;
-    extern __shared__ float red[]; // [P][S-1][TILE_FLOATS]
+    extern __shared__ float red[]; // S > 1: [P][S][TILE_FLOATS] (+ one word with shared tiles)
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -383,10 +384,10 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
         }
     }
 
-    if constexpr (XP && !ZS && S > 1) {
-        // The matrix instructions of these launches are short, so what follows them
-        // counts: every wave leaves its partial tile in LDS, and wave s adds up (in
-        // wave order, as the one-wave form below does) and stores the 16 / S values
+    if constexpr (S > 1) {
+        // What follows the matrix instructions counts in these launches (short K
+        // ranges, workgroups that share a tile): every wave leaves its partial tile
+        // in LDS, and wave s adds up (in wave order) and finishes the 16 / S values
         // per lane and tile that start at value (16 / S) * s.
         constexpr int VQ = 16 / S;
         float *slot = red + (size_t)p * S * TILE_FLOATS; // [S][TILE_FLOATS]
@@ -402,7 +403,7 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
         }
         __syncthreads();
         if (!valid) {
-            return;
+            return; // (with shared tiles a workgroup is one tile: all of its waves leave here)
         }
         float fin[TMW][TNW][VQ];
 #pragma unroll
@@ -418,6 +419,68 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
                         sum += slot[(size_t)o * TILE_FLOATS + at];
                     }
                     fin[i][j][vv] = sum;
+                }
+            }
+        }
+        if constexpr (ZS) {
+            // The tile's z workgroups exchange their sums through memory with
+            // device-scope accesses (sc1: past this XCD's L2, so no cache has to be
+            // written back or invalidated to publish them; what is needed is
+            // order). Producer: every wave waits until its stores are acknowledged
+            // (vmcnt(0)), the workgroup's barrier follows, and only then does one
+            // lane count the arrival. Consumer: the count comes back to every wave
+            // through LDS behind a second barrier, and the loads of the last
+            // workgroup to arrive are issued after it. The empty asm statements
+            // keep the compiler from moving the relaxed atomics across either
+            // point. Device-scope release and acquire fences in their place write
+            // back and invalidate the whole L2 under the other workgroups: measured
+            // 1.7 us per launch of 12-15 us, and far more on launches with hundreds
+            // of workgroups.
+            const uint32_t z = args.z;
+            uint32_t *flag = (uint32_t *)(red + (size_t)S * TILE_FLOATS); // (one tile per workgroup)
+            float *mine = args.partials + ((size_t)tile * z + zpart) * TILE_FLOATS + lane;
+#pragma unroll
+            for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+                for (int j = 0; j < TNW; ++j) {
+#pragma unroll
+                    for (int vv = 0; vv < VQ; ++vv) {
+                        __hip_atomic_store(mine + ((i * TNW + j) * 16 + (uint32_t)VQ * s + vv) * WAVE,
+                                           fin[i][j][vv], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+            }
+            __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); // vmcnt(0)
+            asm volatile("" ::: "memory");
+            __syncthreads();
+            if (threadIdx.x == 0u) {
+                *flag = __hip_atomic_fetch_add(&args.arrivals[tile], 1u, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __syncthreads();
+            const uint32_t arrived = __builtin_amdgcn_readfirstlane(*flag);
+            if (arrived != z - 1u) {
+                return;
+            }
+            asm volatile("" ::: "memory");
+            if (threadIdx.x == 0u) { // (every workgroup of the tile has counted itself)
+                __hip_atomic_store(&args.arrivals[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            const float *first = args.partials + (size_t)tile * z * TILE_FLOATS + lane;
+            for (uint32_t c = 0; c < z; ++c) { // in part order, whoever arrived last
+                const float *part = first + (size_t)c * TILE_FLOATS;
+#pragma unroll
+                for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+                    for (int j = 0; j < TNW; ++j) {
+#pragma unroll
+                        for (int vv = 0; vv < VQ; ++vv) {
+                            const float pv = __hip_atomic_load(
+                                part + ((i * TNW + j) * 16 + (uint32_t)VQ * s + vv) * WAVE, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT);
+                            fin[i][j][vv] = c == 0u ? pv : fin[i][j][vv] + pv;
+                        }
+                    }
                 }
             }
         }
@@ -463,101 +526,9 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
             }
         }
         return;
-    } else if constexpr (S > 1) {
-        if (s > 0u) {
-            float *mine = red + ((size_t)p * (S - 1) + (s - 1u)) * TILE_FLOATS;
-#pragma unroll
-            for (int i = 0; i < TMW; ++i) {
-#pragma unroll
-                for (int j = 0; j < TNW; ++j) {
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        mine[((i * TNW + j) * 16 + v) * WAVE + lane] = acc[i][j][v];
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        if (s > 0u) {
-            return;
-        }
-        for (int o = 0; o < S - 1; ++o) {
-            const float *other = red + ((size_t)p * (S - 1) + o) * TILE_FLOATS;
-#pragma unroll
-            for (int i = 0; i < TMW; ++i) {
-#pragma unroll
-                for (int j = 0; j < TNW; ++j) {
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        acc[i][j][v] += other[((i * TNW + j) * 16 + v) * WAVE + lane];
-                    }
-                }
-            }
-        }
     }
     if (!valid) {
         return;
-    }
-    if constexpr (ZS) {
-        // (one wave is left: the partial tiles go to memory and come back from it
-        // with device-scope accesses that bypass this XCD's L2, so all it takes to
-        // publish them is to wait for the stores before the arrival is counted)
-        const uint32_t z = args.z;
-        float *mine = args.partials + ((size_t)tile * z + zpart) * TILE_FLOATS + lane;
-#pragma unroll
-        for (int i = 0; i < TMW; ++i) {
-#pragma unroll
-            for (int j = 0; j < TNW; ++j) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    __hip_atomic_store(mine + ((i * TNW + j) * 16 + v) * WAVE, acc[i][j][v],
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-            }
-        }
-        // Every access to a partial tile is a device-scope atomic (sc1: it goes to
-        // and comes from memory past this XCD's L2), so no cache has to be written
-        // back or invalidated to publish them; what is needed is order. Producer:
-        // vmcnt(0) returns once the stores are acknowledged, and only then is the
-        // arrival counted. Consumer: the loads below are issued after the count
-        // has come back (the branch waits for it; vector memory instructions
-        // issue in order). The empty asm statements keep the compiler from
-        // moving the relaxed atomics across either point. Device-scope release
-        // and acquire fences in their place write back and invalidate the whole
-        // L2 under the other workgroups: measured 1.7 us per launch of 12-15 us
-        // (a layer of four such launches at 128 tokens 78.1 -> 81.5 us), and far
-        // more on launches with hundreds of workgroups.
-        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8)); // vmcnt(0)
-        asm volatile("" ::: "memory");
-        uint32_t arrived = 0;
-        if (lane == 0u) {
-            arrived = __hip_atomic_fetch_add(&args.arrivals[tile], 1u, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT);
-        }
-        arrived = __builtin_amdgcn_readfirstlane(arrived);
-        if (arrived != z - 1u) {
-            return;
-        }
-        asm volatile("" ::: "memory");
-        if (lane == 0u) {
-            __hip_atomic_store(&args.arrivals[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        const float *first = args.partials + (size_t)tile * z * TILE_FLOATS + lane;
-        for (uint32_t c = 0; c < z; ++c) {
-            const float *part = first + (size_t)c * TILE_FLOATS;
-#pragma unroll
-            for (int i = 0; i < TMW; ++i) {
-#pragma unroll
-                for (int j = 0; j < TNW; ++j) {
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const float pv = __hip_atomic_load(part + ((i * TNW + j) * 16 + v) * WAVE,
-                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        acc[i][j][v] = c == 0u ? pv : acc[i][j][v] + pv;
-                    }
-                }
-            }
-        }
     }
     // acc[v] of a 32x32 tile is (token 8*(v/4) + 4*half + v%4, row idx).
     if constexpr (GLU) {
@@ -1077,7 +1048,8 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
         args.z = z;
         args.partials = shared.partials;
         args.arrivals = shared.arrivals;
-        const size_t lds = (size_t)(S - 1) * TMW * TNW * 16 * WAVE * sizeof(float);
+        // (every wave's partial tile, and the word through which the arrival count reaches them)
+        const size_t lds = (size_t)S * TMW * TNW * 16 * WAVE * sizeof(float) + 16u;
         Q8_LAUNCH((gemm_mma_kernel<L, TMW, TNW, S, XA, true>), dim3(groups * z), dim3(256), lds,
                   stream, stop, args);
         return hipGetLastError();
@@ -1092,7 +1064,7 @@ inline hipError_t launch_mma_cfg(hipStream_t stream, hipEvent_t stop, const MmaP
                   stop, args);
         return hipGetLastError();
     }
-    const size_t lds = S > 1 ? (size_t)P * (S - 1) * TMW * TNW * 16 * WAVE * sizeof(float) : 0;
+    const size_t lds = S > 1 ? (size_t)P * S * TMW * TNW * 16 * WAVE * sizeof(float) : 0; // every wave's partial tile
     Q8_LAUNCH((gemm_mma_kernel<L, TMW, TNW, S, XA>), dim3(groups), dim3(256), lds, stream, stop,
               args);
     return hipGetLastError();
@@ -1157,7 +1129,7 @@ inline hipError_t launch_mma_split_cfg(hipStream_t stream, hipEvent_t stop, cons
             args.z = z;
             args.partials = shared.partials;
             args.arrivals = shared.arrivals;
-            const size_t lds = (size_t)(S - 1) * TNW * 16 * WAVE * sizeof(float);
+            const size_t lds = (size_t)S * TNW * 16 * WAVE * sizeof(float) + 16u;
             Q8_LAUNCH((gemm_mma_kernel<PACKED, 1, TNW, S, true, true, true>), dim3(groups * z), dim3(256),
                       lds, stream, stop, args);
             return hipGetLastError();
