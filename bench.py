@@ -353,6 +353,20 @@ def _bench_layer_with_operators(host, ctx, mats, M, flops_total, steps, warmup, 
             "tflops_f32_equivalent": flops_total * tokens / M / us / 1e6,
             "order": "rmsnorm -> q,k,v -> o(q) -> axpy -> rmsnorm -> gate,up -> silu_mul -> down -> axpy; "
                      "no attention"}
+    # Four such layers in one group at the engine's prefill chunk (the same weights four
+    # times over: what a model's layers cost each when they follow one another, where the
+    # residual update at the end of a layer rides in the next layer's first norm).
+    if M >= 128:
+        layers = 4
+        t = run_steps(host, ctx, layer(128) * layers, warmup, max(steps // 2, 1), grouped=True)
+        stats = step_stats(t, max(steps // 2, 1))
+        us = stats.get("median_us") or stats["mean_us"]
+        out["layer_chain_m128"] = {
+            "M": 128, "layers": layers, "us": us, "us_per_layer": us / layers,
+            "us_per_token": us / layers / 128,
+            "launches_per_layer": t.launches / max(steps // 2, 1) / layers,
+            "order": "four times (rmsnorm -> q,k,v -> o(q) -> axpy -> rmsnorm -> gate,up -> silu_mul -> down "
+                     "-> axpy) in one group; no attention"}
     keep += list(bufs.values()) + [wn]
 
 
