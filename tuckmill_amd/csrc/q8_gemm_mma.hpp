@@ -221,9 +221,12 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
         // K range is made of groups of four Q8_0 blocks, a group's weights are one
         // whole 128-byte line per row (four 16-byte loads per lane, issued
         // together) and its four scales one 8-byte load; the activations' pieces
-        // are whole lines as they are. The next group's weights and the
-        // activations of the next two blocks are on their way while a block is
-        // multiplied.
+        // are whole lines as they are. The next block's activations (and behind a
+        // group's last block the next group's weights) are asked for as soon as
+        // the block's operands are converted; more in flight than that costs the
+        // registers that let two workgroups share a CU (measured with two blocks
+        // of activations and two weight groups held: the gated pair at 128 tokens
+        // 17.7 us against 15.3, 4096 x 1024 with two row tiles 11.1 against 9.0).
         static_assert(L == PACKED, "split-form activations: sealed weights");
         const uint32_t groups = (blocks + 3u) >> 2;
         const uint32_t g_begin = (uint32_t)(((uint64_t)groups * kpart) / kparts);
@@ -277,69 +280,60 @@ __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs
                     }
                 }
             };
-            WGroup wg[2];
-            XBlock xb[2];
-            load_w(g_begin, wg[0]);
-            load_x(xkb_begin, xb[0]);
-            if (xkb_begin + 1u < xkb_end) {
-                load_x(xkb_begin + 1u, xb[1]);
-            }
-            for (uint32_t g0 = g_begin; g0 < g_end; g0 += 2u) {
+            WGroup wg;
+            XBlock xb;
+            load_w(g_begin, wg);
+            load_x(xkb_begin, xb);
+            for (uint32_t grp = g_begin; grp < g_end; ++grp) {
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const uint32_t grp = g0 + (uint32_t)u;
-                    if (grp >= g_end) { // (uniform over the wave)
+                for (int b = 0; b < 4; ++b) {
+                    const uint32_t kb = grp * 4u + (uint32_t)b;
+                    if (kb >= xkb_end) { // (uniform over the wave)
                         break;
                     }
-                    if (grp + 1u < g_end) {
-                        load_w(grp + 1u, wg[u ^ 1]);
+                    bf16x8_t wb[TNW][2], xp[TMW][3][2];
+                    float dsc[TNW];
+#pragma unroll
+                    for (int j = 0; j < TNW; ++j) {
+                        const uint32_t pair = b < 2 ? wg.sc[j].x : wg.sc[j].y;
+                        dsc[j] = f16_bits_to_f32(b % 2 ? pair >> 16 : pair & 0xffffu);
+                        wb[j][0] = sbytes_to_bf16x8(wg.q[j][b].x, wg.q[j][b].y);
+                        wb[j][1] = sbytes_to_bf16x8(wg.q[j][b].z, wg.q[j][b].w);
                     }
 #pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        const uint32_t kb = grp * 4u + (uint32_t)b;
-                        if (kb >= xkb_end) {
-                            break;
-                        }
-                        bf16x8_t wb[TNW][2], xp[TMW][3][2];
-                        float dsc[TNW];
+                    for (int i = 0; i < TMW; ++i) {
 #pragma unroll
-                        for (int j = 0; j < TNW; ++j) {
-                            const uint32_t pair = b < 2 ? wg[u].sc[j].x : wg[u].sc[j].y;
-                            dsc[j] = f16_bits_to_f32(b % 2 ? pair >> 16 : pair & 0xffffu);
-                            wb[j][0] = sbytes_to_bf16x8(wg[u].q[j][b].x, wg[u].q[j][b].y);
-                            wb[j][1] = sbytes_to_bf16x8(wg[u].q[j][b].z, wg[u].q[j][b].w);
-                        }
+                        for (int pc = 0; pc < 3; ++pc) {
 #pragma unroll
-                        for (int i = 0; i < TMW; ++i) {
-#pragma unroll
-                            for (int pc = 0; pc < 3; ++pc) {
-#pragma unroll
-                                for (int k2 = 0; k2 < 2; ++k2) {
-                                    xp[i][pc][k2] = __builtin_bit_cast(bf16x8_t, xb[b % 2].p[i][pc][k2]);
-                                }
+                            for (int k2 = 0; k2 < 2; ++k2) {
+                                xp[i][pc][k2] = __builtin_bit_cast(bf16x8_t, xb.p[i][pc][k2]);
                             }
                         }
-                        if (kb + 2u < xkb_end) {
-                            load_x(kb + 2u, xb[b % 2]);
-                        }
+                    }
+                    // the block's operands are converted: ask for the next ones
+                    if (b == 3 && grp + 1u < g_end) {
+                        load_w(grp + 1u, wg);
+                    }
+                    if (kb + 1u < xkb_end) {
+                        load_x(kb + 1u, xb);
+                    }
 #pragma unroll
-                        for (int i = 0; i < TMW; ++i) {
+                    for (int i = 0; i < TMW; ++i) {
 #pragma unroll
-                            for (int j = 0; j < TNW; ++j) {
-                                floatx16 sum = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
-                                                0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+                        for (int j = 0; j < TNW; ++j) {
+                            floatx16 sum = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
+                                            0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                                for (int piece = 2; piece >= 0; --piece) { // smallest pieces first
+                            for (int piece = 2; piece >= 0; --piece) { // smallest pieces first
 #pragma unroll
-                                    for (int k2 = 0; k2 < 2; ++k2) {
-                                        sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xp[i][piece][k2], wb[j][k2],
-                                                                                      sum, 0, 0, 0);
-                                    }
+                                for (int k2 = 0; k2 < 2; ++k2) {
+                                    sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xp[i][piece][k2], wb[j][k2],
+                                                                                  sum, 0, 0, 0);
                                 }
+                            }
 #pragma unroll
-                                for (int v = 0; v < 16; ++v) {
-                                    acc[i][j][v] = __builtin_fmaf(dsc[j], sum[v], acc[i][j][v]);
-                                }
+                            for (int v = 0; v < 16; ++v) {
+                                acc[i][j][v] = __builtin_fmaf(dsc[j], sum[v], acc[i][j][v]);
                             }
                         }
                     }
@@ -1123,7 +1117,8 @@ inline hipError_t launch_mma_split_cfg(hipStream_t stream, hipEvent_t stop, cons
                   stream, stop, args);
         return hipGetLastError();
     }
-    if constexpr (S == 4 && TNW == 1) if (shared.partials != nullptr && shared.arrivals != nullptr) {
+    if constexpr (S == 4) if (glu == nullptr && shared.partials != nullptr && shared.arrivals != nullptr) {
+        static_assert(256u * (uint32_t)TNW * 16u * WAVE <= MMA_SHARED_PARTIAL_FLOATS, "partial tiles");
         const uint32_t z = mma_shared_parts(tiles, min_blocks);
         if (z > 1u) {
             args.z = z;

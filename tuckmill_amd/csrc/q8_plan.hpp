@@ -107,12 +107,17 @@ inline MmaConfig pick_mma_config(const MmaProduct *prods, int n) {
 
 
 // The same kernel fed with activations in split form (gemm_mma_kernel<..., XP>):
-// always the 32-token tile. Two row tiles per wave once the launch has more than
-// two rounds of workgroups (the activations' pieces are then fetched once for
-// both: at 256 tokens 4096 x 1024 takes 18 us against 22, 6144 x 1024 26 against
-// 30; with fewer workgroups the narrow tile is ahead, 1024 x 2048 at 256 tokens 12
-// us against 18). A wave's share of K is made of whole groups of four blocks, so
-// K is split over four waves from 16 blocks on.
+// always the 32-token tile. A wave's share of K is made of whole groups of four
+// blocks, so K is split over four waves from 16 blocks on. Two row tiles per wave
+// (the activations' pieces are then fetched once for both) from more than 256
+// tiles of one, and from about 256 under a K of 96 blocks and more, where the
+// halved tile count lets two workgroups share each tile. Measured alone (us, one
+// row tile against two): 4096 x 1024 at 128 tokens 11.1 against 9.0, at 64 tokens
+// (256 tiles) 7.1 against 8.5, at 256 tokens 19.8 against 14.9; 6144 x 1024 at 64
+// tokens (384 tiles) 10.8 against 8.7, at 32 tokens (192 tiles) 6.9 against 8.3;
+// 1024 x 3072 at 256 tokens (256 tiles) 17.3 against 14.3, at 128 tokens (two
+// workgroups per tile either way) 11.1 against 11.9; 1024 x 2048 at 256 tokens
+// 11.4 against 11.7.
 inline MmaConfig pick_mma_split_config(const MmaProduct *prods, int n) {
     uint32_t min_blocks = 0xffffffffu;
     uint64_t tiles = 0;
@@ -124,10 +129,9 @@ inline MmaConfig pick_mma_split_config(const MmaProduct *prods, int n) {
     MmaConfig c;
     c.tmw = 1;
     c.s = min_blocks >= 16u ? 4 : (min_blocks >= 8u ? 2 : 1);
-    c.tnw = c.s == 4 && tiles >= 1024u ? 2 : 1;
+    c.tnw = c.s == 4 && (tiles > 256u || (tiles > 192u && min_blocks >= 96u)) ? 2 : 1;
     return c;
 }
-
 
 // ---- prefill GEMM on the bf16 matrix cores (q8_gemm_bf16x3.hpp) -------------
 
