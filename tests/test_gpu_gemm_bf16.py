@@ -378,7 +378,8 @@ def test_small_launches_behind_an_operator_read_its_split_form(ctx, kind, batch,
 
 @pytest.mark.parametrize("kind,batch,hid,ffn,in_place",
                          [("silu_mul", 128, 1024, 3072, False), ("gelu_tanh_mul", 100, 1056, 1120, False),
-                          ("silu_mul", 64, 1024, 3072, True), ("silu_mul", 40, 256, 512, False)])
+                          ("silu_mul", 64, 1024, 3072, True), ("silu_mul", 40, 256, 512, False),
+                          ("silu_mul", 256, 1024, 3072, False)])
 def test_the_gated_activation_rides_in_the_launch_of_gate_and_up(ctx, kind, batch, hid, ffn, in_place):
     # The feed-forward half of a layer at a small prefill size: norm, gate and up, the
     # gated activation, down. In one group that is three launches: gate and up with the
@@ -386,7 +387,11 @@ def test_the_gated_activation_rides_in_the_launch_of_gate_and_up(ctx, kind, batc
     # down projection. Every buffer comes out bit for bit as from the same operations in
     # two groups (norm, gate, up | activation, down), where the activation launches on
     # its own. In place (the activation over the gate's buffer) the raw gate is not kept,
-    # as with the operator on its own.
+    # as with the operator on its own. At 256 tokens gate and up alone have enough work for
+    # the staged kernel's 64-token tile; with the activation and the down projection behind
+    # them they take the small tiles with the activation fused in, and the results then
+    # agree with the two-group run to the products' tolerance, not bit for bit.
+    staged_apart = H.gemm_mma_launch_tile([(ffn, hid, batch)] * 2) != 0
     h = upload_new(ctx, S.make_activations(batch * hid, 31))
     wn = upload_new(ctx, (1.0 + 0.1 * S.make_activations(hid, 9)).astype(np.float32))
     xn = ctx.buffer(batch * hid * 4)
@@ -436,7 +441,19 @@ def test_the_gated_activation_rides_in_the_launch_of_gate_and_up(ctx, kind, batc
         fused = state()
         assert ctx.kernel_launches() == before + 3
         for i, (a, b) in enumerate(zip(apart, fused)):
-            assert np.array_equal(bits(a), bits(b)), f"attempt {attempt}, buffer {i}"
+            if staged_apart and i > 0:
+                scale = max(1.0, float(np.abs(a).max()))
+                assert np.abs(a - b).max() <= 2e-5 * scale, f"attempt {attempt}, buffer {i}"
+            else:
+                assert np.array_equal(bits(a), bits(b)), f"attempt {attempt}, buffer {i}"
+        if attempt == 0:
+            first = fused
+        else:
+            for i, (a, b) in enumerate(zip(first, fused)):
+                assert np.array_equal(bits(a), bits(b)), f"buffer {i} differs between two runs"
+    if staged_apart:
+        apart = first
+        raw_gate = first[1]
 
     x = apart[0]
     g_want = O.gemm_q8_0_f32(wg, ffn, hid, x, batch, threads=8)

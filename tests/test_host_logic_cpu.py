@@ -550,6 +550,39 @@ def test_small_prefill_launches_behind_their_operator_take_its_split_form(driver
         assert splits == ([False] * 4 if name == "raw" else [False, False, True, False]), shape(ls)
 
 
+def test_a_staged_gated_pair_up_to_256_tokens_takes_the_fused_small_tiles(driver):
+    """Gate and up of the 0.6B layer at 256 tokens have enough work for the staged bf16
+    kernel's 64-token tile when they stand alone. Behind their norm and in front of the
+    gated activation and a down projection that stays on the small tiles, the pair takes
+    the small tiles too, with the activation in its launch (three launches where four
+    stood); at 512 tokens (the large tile, a staged down projection) nothing changes."""
+    hid, ffn = 1024, 3072
+    lines = ["ctx main", f"buf nw {hid * 4}", f"buf h {512 * hid * 4}", f"buf xn {512 * hid * 4}",
+             f"buf act {512 * ffn * 4}", f"buf Yg {512 * ffn * 4}", f"buf Yu {512 * ffn * 4}",
+             f"buf Yd {512 * hid * 4}"]
+    for name, r, c in (("gate", ffn, hid), ("up", ffn, hid), ("down", hid, ffn)):
+        lines += [f"buf W{name} {r * (c // 32) * 34}", f"seal W{name} {r} {c}"]
+
+    def half(M):
+        return ["begin", f"rmsnorm h nw xn {M} {hid}", f"mma Wgate xn Yg {ffn} {hid} {M} 0 0",
+                f"mma Wup xn Yu {ffn} {hid} {M} 0 0", f"silu Yg Yu act {M * ffn}",
+                f"mma Wdown act Yd {hid} {ffn} {M} 0 0", "end", "fence"]
+
+    lines += ["fence", "mark alone", "begin", f"mma Wgate xn Yg {ffn} {hid} 256 0 0",
+              f"mma Wup xn Yu {ffn} {hid} 256 0 0", "end", "fence",
+              "mark m256"] + half(256) + ["mark m512"] + half(512) + ["stats"]
+    sec = sections(run_program(driver, lines))
+    (alone,) = launches_of(sec["alone"])
+    assert alone["variant"] == "bf16x3" and alone["p"][0] == 1
+    m256 = launches_of(sec["m256"])
+    assert [(l["k"], l.get("variant") or l["what"]) for l in m256] == \
+        [("single", "rmsnorm"), ("list", "mma_split"), ("list", "mma_split")], m256
+    assert "glu" in m256[1]["ops"][0] and m256[1]["split_out"] and m256[2]["xs_in_off"] == 256 * hid * 6
+    m512 = launches_of(sec["m512"])
+    assert [(l["k"], l.get("variant") or l["what"]) for l in m512] == \
+        [("single", "rmsnorm"), ("list", "bf16x3"), ("single", "silu_mul"), ("list", "bf16x3")], m512
+
+
 # ------------------------------------------------------------------ threads --
 
 def test_two_contexts_and_their_readers_on_four_threads_under_the_thread_sanitizer(tmp_path):
