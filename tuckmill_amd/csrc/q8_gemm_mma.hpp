@@ -125,10 +125,10 @@ __device__ __forceinline__ void mma_load_block(const WView<L> &wv, const float *
 //
 // GLU (with XP): the launch is the gate and the up projection of a gated unit
 // (same shape, same activations) and the activation behind them. A wave's two
-// accumulator tiles are the same 32 x 32 outputs of both; the wave that holds the
-// sums stores the projections, act(gate) * up and, for a product launched right
-// behind, its split form: one launch and one pass over the outputs in the place of
-// two. Every sum is formed as in the launch without the activation.
+// accumulator tiles are the same 32 x 32 outputs of both; where the sums are
+// finished, the projections, act(gate) * up and, for a product launched right
+// behind, its split form are stored: one launch and one pass over the outputs in
+// the place of two. Every sum is formed as in the launch without the activation.
 template <int L, int TMW, int TNW, int S, bool XA, bool ZS = false, bool XP = false, bool GLU = false>
 __global__ __launch_bounds__(256, XP ? 2 : 1) void gemm_mma_kernel(const MmaArgs args) {
     static_assert(!ZS || S == 4, "shared tiles: one tile per workgroup");
