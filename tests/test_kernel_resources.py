@@ -101,6 +101,27 @@ def test_bf16_gemm_keeps_its_results_in_vector_registers(resource_remarks):
         assert agprs == 0 and spill == 0 and occupancy >= 2, block
 
 
+# gemm_mma_kernel<sealed, 1 token tile, row tiles, K split, aligned, shared tiles, split-form input = true, gated pair>
+SPLIT_FORM_KERNEL = re.compile(
+    r"Function Name: _ZN2q815gemm_mma_kernelILi1ELi1ELi[12]ELi[124]ELb1ELb[01]ELb1ELb[01]EEE")
+
+
+def test_split_form_tiles_keep_two_workgroups_per_cu_without_spills(resource_remarks):
+    """The small tiles fed from the split form are bound by waiting for operands:
+    what hides it is waves side by side, not a deeper queue per wave. With two blocks
+    of activations and two weight groups held, the forms with two accumulator tiles
+    took all 256 registers and spilled (the gated pair at 128 tokens 17.7 us
+    against 15.3 with one of each)."""
+    blocks = _blocks(resource_remarks, SPLIT_FORM_KERNEL)
+    assert len(blocks) >= 8, "split-form instantiations of gemm_mma_kernel not found"
+    for block in blocks:
+        vgprs = int(re.search(r" VGPRs: (\d+)", block).group(1))
+        spill = int(re.search(r"VGPRs Spill: (\d+)", block).group(1))
+        scratch = int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", block).group(1))
+        occupancy = int(re.search(r"Occupancy \[waves/SIMD\]: (\d+)", block).group(1))
+        assert spill == 0 and scratch == 0 and vgprs <= 224 and occupancy >= 2, block
+
+
 # gemm_split_list_kernel<layout, waves, tokens per wave, aligned x, column tails, rows per step>
 SMALL_BATCH_KERNEL = re.compile(
     r"Function Name: _ZN2q822gemm_split_list_kernelILi[01]ELi\d+ELi\d+ELb[01]ELb[01]ELi[48]EEE")
