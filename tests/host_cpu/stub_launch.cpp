@@ -223,6 +223,11 @@ hipError_t tmdev::launch_list(hipStream_t stream, hipEvent_t stop, const Launch 
             die("bf16 launch: partial tiles do not fit the workspace");
         }
         out += ",\"presplit\":" + std::to_string(l.bx3_presplit);
+        bool small_batch = true; // up to 32 tokens: the f32 kernel's tiles fed from the split form
+        for (size_t i = 0; i < n; ++i) {
+            small_batch = small_batch && q8::bx3_small_batch_tiles(l.list[i]->batch);
+        }
+        out += std::string(",\"small_tiles\":") + (small_batch ? "true" : "false");
     }
     if (key.variant == V_MMA_SPLIT) { // every product reads the one split form the launch before has written
         if (!key.packed || l.bx3_inputs != 1 || l.bx3_presplit != 1u) {

@@ -14,7 +14,7 @@ from q8util import bits, norm_err, ref_scale, require_gpu, upload_new, weights_b
 
 pytestmark = pytest.mark.gpu
 
-M0 = H.GEMM_MMA_BF16_MIN_BATCH  # 17: one 64-token tile up to 64 tokens
+M0 = 17  # the least batch at which every sealed product is left to the matrix cores
 
 
 @pytest.fixture(scope="module")
@@ -65,6 +65,40 @@ def test_gaussian_products_within_1e5(ctx, rows, cols, batch):
     assert not got[:8].any(), "nothing before y_off"
     want = O.gemm_q8_0_f32(w, rows, cols, x, batch, threads=8)
     assert norm_err(got[8:].reshape(batch, rows), want) <= 1e-5
+    wb.free()
+
+
+# Up to 32 tokens a launch large enough for the bf16 matrix cores runs on 32-token tiles
+# behind the split pass, and from 9 tokens (34 M weights) or 5 (128 M and more) so does the
+# MFMA entry point over a product that is that large on its own. Ragged rows and a K of
+# 33 blocks; the smallest batches; a batch of 16 and of 32.
+@pytest.mark.parametrize("rows,cols,batch", [(33001, 1024, 9), (33001, 1024, 16), (33000, 1056, 32),
+                                             (131100, 1024, 5), (131100, 1024, 8), (66000, 2048, 12)])
+def test_large_products_at_few_tokens_within_1e5(ctx, rows, cols, batch):
+    assert H.gemm_mma_on_bf16(rows, cols, batch)
+    w = S.make_weights(rows, cols, 300 + batch)
+    wb = weights_buffer(ctx, w, rows, cols, True)
+    x = S.make_activations(batch * cols, 301)
+    before = ctx.kernel_launches()
+    got = product(ctx, wb, x, rows, cols, batch).reshape(batch, rows)
+    assert ctx.kernel_launches() == before + 2  # the split pass and the products
+    again = product(ctx, wb, x, rows, cols, batch).reshape(batch, rows)
+    assert np.array_equal(bits(got), bits(again))
+    tokens = sorted({0, batch - 1, batch // 2})
+    want = O.gemm_q8_0_f32(w, rows, cols, np.ascontiguousarray(x.reshape(batch, cols)[tokens]).ravel(),
+                           len(tokens), threads=8)
+    assert norm_err(got[tokens], want) <= 1e-5
+    # one token fewer than the rule asks for: the vector kernel, the GEMV's bits
+    if batch in (5, 9):
+        assert not H.gemm_mma_on_bf16(rows, cols, batch - 1)
+        small = product(ctx, wb, x[:(batch - 1) * cols], rows, cols, batch - 1).reshape(batch - 1, rows)
+        yb = ctx.buffer(rows * 4)
+        xb = upload_new(ctx, x[:cols])
+        ctx.q8_0_gemv(wb, xb, yb, rows, cols)
+        ctx.fence()
+        assert np.array_equal(bits(small[0]), bits(yb.download_f32(0, rows)))
+        xb.free()
+        yb.free()
     wb.free()
 
 

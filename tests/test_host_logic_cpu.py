@@ -479,7 +479,12 @@ def test_a_ragged_last_round_is_cut_off_as_a_tail_segment(driver):
              "mark m64", f"mma w x y {rows} {cols} 64 0 0", "fence",
              "mark m128", f"mma w x y {rows} {cols} 128 0 0", "fence",
              "mark m512", f"mma w x y {rows} {cols} 512 0 0", "fence", "stats"]
+    lines += ["mark m32", f"mma w x y {rows} {cols} 32 0 0", "fence", "mark m17", f"mma w x y {rows} {cols} 17 0 0",
+              "fence"]
     sec = sections(run_program(driver, lines))
+    for name in ("m32", "m17"):  # up to 32 tokens: the 32-token tiles behind the same split pass
+        (l,) = launches_of(sec[name])
+        assert l["variant"] == "bf16x3" and l["p"][0] == 1 and l["small_tiles"] is True, l
     for name in ("t128", "noalloc"):
         (l,) = launches_of(sec[name])
         assert l["variant"] == "bf16x3" and l["p"][0] == 2, l
@@ -489,6 +494,7 @@ def test_a_ragged_last_round_is_cut_off_as_a_tail_segment(driver):
     for name in ("m64", "m128", "m512"):
         (l,) = launches_of(sec[name])
         assert "tail" not in l and l["ops"][0]["chunks"] == 1
+        assert l["small_tiles"] is False  # (33 tokens and more: the staged kernel itself)
 
 
 def test_small_prefill_launches_behind_their_operator_take_its_split_form(driver):

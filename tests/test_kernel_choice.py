@@ -34,8 +34,10 @@ def test_which_products_take_the_bf16_matrix_cores():
         if name in ("q", "k", "v", "o"):
             assert not H.gemm_mma_on_bf16(rows, cols, 512)
     _, rows, cols = S.QWEN3_0_6B_LM_HEAD
-    assert H.gemm_mma_on_bf16(rows, cols, H.GEMM_MMA_BF16_MIN_BATCH)
+    assert H.gemm_mma_on_bf16(rows, cols, H.GEMM_MMA_BF16_MIN_BATCH)  # 155 M weights: from 5 tokens
     assert not H.gemm_mma_on_bf16(rows, cols, H.GEMM_MMA_BF16_MIN_BATCH - 1)
+    assert not H.gemm_mma_on_bf16(33000, 1024, 8) and H.gemm_mma_on_bf16(33000, 1024, 9)  # 34 M: from 9
+    assert not H.gemm_mma_on_bf16(6144, 2048, 16)  # 13 M: the vector kernel up to 16 tokens
     for _, rows, cols in S.SWEEP_2B:
         assert H.gemm_mma_on_bf16(rows, cols, 256)
     # 192 units of the small tile are the least that pays: q (128 units) stays on

@@ -569,6 +569,34 @@ inline uint32_t bx3_launch_tile(const Bx3Shape3 *shapes, int n) {
     return here_us_x100 < f32_us_x100 ? 64u : 0u;
 }
 
+// Up to 32 tokens half of the staged kernel's 64-token tile is padding, and its time
+// hardly depends on the batch. The launches it takes there (32 M weights and more)
+// run on the 32-token tiles of the f32 kernel fed from the split form instead
+// (gemm_mma_kernel<..., XP>), behind the same split pass. Measured, split pass
+// included, staged against small tiles: 151936 x 1024 at 17 / 32 tokens 80 us against
+// 53 / 57; 33000 x 1024 35 against 20 / 21; 262144 x 1152 at 32 tokens 136 against
+// 127; forty 2B-class matrices (6144 x 2048, 2048 x 6144) in one launch at 32 tokens
+// 277 against 231. From 33 tokens the small tiles need two token tiles and lose
+// (the forty matrices at 64 tokens 284 against 382).
+inline bool bx3_small_batch_tiles(uint32_t batch) { return batch <= 32u; }
+
+// Below 17 tokens the MFMA entry point over sealed weights of 1024 columns and more
+// normally runs the vector kernels (GEMV arithmetic). A large product does better on
+// the 32-token tiles above, whose time hardly depends on the batch, from 9 tokens
+// (32 M weights and more) or from 5 (128 M and more: the vocabulary projections).
+// Measured against the vector kernel, split pass included: 151936 x 1024 at 5 / 8 /
+// 12 / 16 tokens 72 / 70 / 125 / 129 us against 62; 262144 x 1152 at 8 / 16 tokens
+// 222 / 386 against about 120; 33000 x 1024 at 5 / 8 tokens 25 / 24 against 27 (not
+// taken), at 12 / 16 tokens 36 against 27.
+inline bool mma_small_batch_on_tiles(uint32_t rows, uint32_t cols, uint32_t batch) {
+    if (batch < 5u || batch > 16u) {
+        return false;
+    }
+    const Bx3Shape3 one{rows, cols, batch};
+    return (uint64_t)rows * cols >= (batch <= 8u ? (1ull << 27) : (1ull << 25)) &&
+           bx3_launch_tile(&one, 1) != 0u;
+}
+
 // A product on its own: its plan, and whether the kernel pays for it (`worth`).
 inline Bx3Plan bx3_plan(uint32_t rows, uint32_t cols, uint32_t batch, bool *worth) {
     const Bx3Shape3 one{rows, cols, batch};

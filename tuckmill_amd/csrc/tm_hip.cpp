@@ -391,7 +391,7 @@ int wait_pending(tm_hip_ctx *ctx, char *err, size_t cap) {
 // the same group gives the same bits every time, but a product's bits may depend
 // on what shares its launch (the entry point is tolerance-qualified,
 // native/metal/tm_metal.h:172-175; bit-identity claims belong to q8_0_gemm).
-constexpr uint32_t kBx3MinBatch = 17;
+constexpr uint32_t kBx3MinBatch = 5; // (below 17 only what q8::mma_small_batch_on_tiles lets through)
 constexpr uint64_t kBx3MaxPartialFloats = 1ull << 29; // 2 GiB of partial tiles per launch
 
 bool x_aligned_of(const Op &op) {
@@ -1314,6 +1314,8 @@ Op mma_op(tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y, uint32_t rows, u
     // Below this batch a 32-token MFMA tile is mostly padding and the vector
     // kernels (GEMV arithmetic, which is within any tolerance of itself) are
     // faster: 1 token -> the decode kernel, 2..16 -> the token-split kernel.
+    // (A large product is the exception: from 5 or 9 tokens it takes the 32-token
+    // tiles on the bf16 matrix cores, q8::mma_small_batch_on_tiles.)
     const bool small = w->alloc->packed && (batch == 1 || (batch <= 16 && cols >= 1024u));
     op.kind = small ? OP_GEMV_LIST : OP_MMA;
     op.a[0] = w->alloc;
@@ -1328,6 +1330,12 @@ Op mma_op(tm_hip_buffer *w, tm_hip_buffer *x, tm_hip_buffer *y, uint32_t rows, u
     op.y_off = y_off;
     op.packed = w->alloc->packed;
     op.what = "q8_0_gemm_mma";
+    if (small && q8::mma_small_batch_on_tiles(rows, cols, batch)) {
+        op.kind = OP_MMA;
+        if (!bx3_admissible(op) || !bx3_fits(op, 64u)) {
+            op.kind = OP_GEMV_LIST;
+        }
+    }
     return op;
 }
 

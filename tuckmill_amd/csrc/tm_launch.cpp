@@ -307,6 +307,19 @@ hipError_t launch_bx3_list(hipStream_t stream, hipEvent_t stop, const Launch &la
             return e;
         }
     }
+    bool small_batch = n <= q8::MMA_MAX_DESCS;
+    for (const Op *op : ops) {
+        small_batch = small_batch && q8::bx3_small_batch_tiles(op->batch);
+    }
+    if (small_batch) { // (no tail segments on the 64-token tile: one entry per product)
+        q8::MmaProduct small[q8::MMA_MAX_DESCS];
+        for (int i = 0; i < n; ++i) {
+            small[i] = q8::MmaProduct{prods[i].w, (const float *)prods[i].xs, prods[i].y, prods[i].rows,
+                                      prods[i].cols, prods[i].batch};
+        }
+        const q8::MmaShared shared{ws.mma_partials, ws.arrivals};
+        return q8::launch_gemm_mma_split_list(stream, stop, small, n, shared);
+    }
     return q8::launch_gemm_bf16x3_list(stream, stop, launch.key.p0 * 64u, prods, n,
                                        ws.partials, ws.arrivals);
 }

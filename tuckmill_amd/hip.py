@@ -27,8 +27,10 @@ GEMM_MMA_MAX_BATCH = 512
 PREFILL_BATCH = 128  # crates/tuckcore/src/engine/metal.rs:25 (the engine's prefill chunk)
 # From this batch on tm_hip_q8_0_gemm_mma over sealed weights with 16-byte aligned
 # activations may run on the bf16 matrix cores (activations split into three exact bf16
-# pieces), when the products of its launch are large enough together (gemm_mma_launch_tile).
-GEMM_MMA_BF16_MIN_BATCH = 17
+# pieces), when the products of its launch are large enough together (gemm_mma_launch_tile);
+# below 17 tokens only a product that is large on its own (gemm_mma_small_batch_on_tiles),
+# the others take the vector kernels there.
+GEMM_MMA_BF16_MIN_BATCH = 5
 
 
 def _bf16_units(rows: int, cols: int, batch: int, tokens: int):
@@ -108,8 +110,20 @@ def gemm_mma_on_bf16(rows: int, cols: int, batch: int, x_off: int = 0) -> bool:
     csrc/tm_hip.cpp; the limits on region sizes beyond 4 GiB are left out). In a
     dispatch group the products that share a launch decide together
     (gemm_mma_launch_tile)."""
+    if batch <= 16 and cols >= 1024 and not gemm_mma_small_batch_on_tiles(rows, cols, batch):
+        return False
     return (batch >= GEMM_MMA_BF16_MIN_BATCH and x_off % 4 == 0 and
             gemm_mma_bf16_plan(rows, cols, batch)[2])
+
+
+def gemm_mma_small_batch_on_tiles(rows: int, cols: int, batch: int) -> bool:
+    """Whether a sealed product of 5 to 16 tokens leaves the vector kernels for the
+    32-token tiles on the bf16 matrix cores (mirror of q8::mma_small_batch_on_tiles):
+    32 M weights and more from 9 tokens, 128 M and more from 5."""
+    if batch < 5 or batch > 16:
+        return False
+    return rows * cols >= (1 << 27 if batch <= 8 else 1 << 25) and \
+        gemm_mma_launch_tile([(rows, cols, batch)]) != 0
 
 
 NOALLOC_WORKSPACE_BYTES = 64 << 20  # TM_HIP_NOALLOC_WORKSPACE_BYTES
