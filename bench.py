@@ -722,7 +722,7 @@ def bench_sweep(host, ctx, steps, warmup, cpu=True, batches=None):
                           kernel="q8::gemv_i8_list_kernel (v_dot4)" if M <= 4
                           else "q8::gemm_i8_lds_kernel (v_mfma_i32_16x16x32_i8)")
             elif kind == TMH_GEMM_MMA and \
-                    (mb > 16 or all(H.gemm_mma_small_batch_on_tiles(r, c, mb) for _, r, c, _ in pool)) and \
+                    (mb >= 9 or all(H.gemm_mma_small_batch_on_tiles(r, c, mb) for _, r, c, _ in pool)) and \
                     H.gemm_mma_launch_tile([(r, c, mb) for _, r, c, _ in pool]):
                 # three bf16 products are issued per f32 one
                 pt.update(path=label + ": bf16 matrix cores, exact products",

@@ -102,6 +102,45 @@ def test_large_products_at_few_tokens_within_1e5(ctx, rows, cols, batch):
     wb.free()
 
 
+def test_few_token_products_that_are_large_together_share_the_small_tiles(ctx):
+    # Six products of 8 to 13 M weights each over two inputs at 12 tokens through the MFMA
+    # entry point: alone each runs the vector kernel (the GEMV's bits), in one group they are
+    # one split pass and one launch on the bf16 matrix cores.
+    batch = 12
+    shapes = [(6144, 2048), (6144, 2048), (4096, 2048), (2048, 6144), (2048, 6144), (2048, 6144)]
+    xs = {2048: S.make_activations(batch * 2048, 501), 6144: S.make_activations(batch * 6144, 502)}
+    xbs = {c: upload_new(ctx, x) for c, x in xs.items()}
+    mats = []
+    for i, (rows, cols) in enumerate(shapes):
+        w = S.make_weights(rows, cols, 510 + i)
+        mats.append((w, rows, cols, weights_buffer(ctx, w, rows, cols, True), ctx.buffer(batch * rows * 4)))
+    before = ctx.kernel_launches()
+    w, rows, cols, wb, yb = mats[0]
+    ctx.q8_0_gemm_mma(wb, xbs[cols], yb, rows, cols, batch, 0, 0)
+    ctx.fence()
+    assert ctx.kernel_launches() == before + 1
+    alone = yb.download_f32(0, batch * rows).copy()
+    runs = []
+    for attempt in range(2):
+        for m in mats:
+            m[4].zero(0, batch * m[1] * 4)
+        before = ctx.kernel_launches()
+        ctx.begin_group()
+        for w, rows, cols, wb, yb in mats:
+            ctx.q8_0_gemm_mma(wb, xbs[cols], yb, rows, cols, batch, 0, 0)
+        ctx.end_group()
+        ctx.fence()
+        assert ctx.kernel_launches() == before + 2
+        runs.append([m[4].download_f32(0, batch * m[1]).copy() for m in mats])
+    for i, (w, rows, cols, wb, yb) in enumerate(mats):
+        assert np.array_equal(bits(runs[0][i]), bits(runs[1][i])), f"product {i}"
+        want = O.gemm_q8_0_f32(w, rows, cols, xs[cols], batch, threads=8)
+        assert norm_err(runs[0][i].reshape(batch, rows), want) <= 1e-5, f"product {i}"
+    assert norm_err(alone.reshape(batch, shapes[0][0]), runs[0][0].reshape(batch, shapes[0][0])) <= 1e-5
+    for b in list(xbs.values()) + [m[3] for m in mats] + [m[4] for m in mats]:
+        b.free()
+
+
 def test_boundary_values_and_wide_ranges(ctx):
     # crates/metal/src/tests.rs:1169-1233 (boundary weights and inputs), and
     # activations that span 60 binades: every piece of the split is exact, so the

@@ -589,6 +589,33 @@ def test_a_staged_gated_pair_up_to_256_tokens_takes_the_fused_small_tiles(driver
         [("single", "rmsnorm"), ("list", "bf16x3"), ("single", "silu_mul"), ("list", "bf16x3")], m512
 
 
+def test_few_token_products_that_are_large_together_leave_the_vector_kernel(driver):
+    """Products of 13 M weights each at 16 tokens through the MFMA entry point: alone a
+    product stays on the token-split vector kernel (too small for the 32-token tiles to
+    pay), four of them in one group (50 M weights) go to the bf16 path's small tiles behind
+    one split pass. The same products through the exact entry point, or with a residual
+    update riding in the launch, stay where they are."""
+    rows, cols, M = 6144, 2048, 16
+    lines = ["ctx main", f"buf x {M * cols * 4}", f"buf h {M * rows * 4}"]
+    for i in range(4):
+        lines += [f"buf w{i} {rows * (cols // 32) * 34}", f"seal w{i} {rows} {cols}", f"buf y{i} {M * rows * 4}"]
+    lines += ["fence", "mark alone", f"mma w0 x y0 {rows} {cols} {M} 0 0", "fence",
+              "mark group", "begin"] + [f"mma w{i} x y{i} {rows} {cols} {M} 0 0" for i in range(4)] + ["end", "fence",
+              "mark exact", "begin"] + [f"gemm w{i} x y{i} {rows} {cols} {M} 0 0" for i in range(4)] + ["end", "fence",
+              "mark fused", "begin"] + [f"mma w{i} x y{i} {rows} {cols} {M} 0 0" for i in range(4)] + \
+             [f"axpy y3 h 1.0 {M * rows}", "end", "fence", "stats"]
+    sec = sections(run_program(driver, lines))
+    (alone,) = launches_of(sec["alone"])
+    assert alone["variant"] == "split"
+    (group,) = launches_of(sec["group"])
+    assert group["variant"] == "bf16x3" and group["p"][0] == 1 and group["small_tiles"] is True
+    assert len(group["ops"]) == 4 and group["presplit"] == 0
+    (exact,) = launches_of(sec["exact"])
+    assert exact["variant"] == "split"
+    fused = launches_of(sec["fused"])
+    assert fused[0]["variant"] == "split" and "residual" in fused[0]["ops"][3], fused
+
+
 # ------------------------------------------------------------------ threads --
 
 def test_two_contexts_and_their_readers_on_four_threads_under_the_thread_sanitizer(tmp_path):

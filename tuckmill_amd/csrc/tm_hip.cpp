@@ -839,6 +839,57 @@ void fuse_split_passes(std::vector<Launch> &plan) {
     }
 }
 
+// A launch of the token-split vector kernel whose products all came through the
+// MFMA entry point (tolerance-qualified: free to take another kernel) at 9 to 16
+// tokens, with 32 M weights and more between them, goes to the bf16 path instead,
+// where up to 32 tokens means 32-token tiles behind a split pass
+// (q8::bx3_small_batch_tiles): each product alone was too small for
+// q8::mma_small_batch_on_tiles, together they are not (forty 2B-class matrices at 16
+// tokens: 381 us on the vector kernel, about 210 there). Launches with operators fused
+// in stay as they are.
+void promote_small_batch_lists(std::vector<Launch> &plan) {
+    for (Launch &l : plan) {
+        if (l.single != nullptr || l.key.kind != OP_GEMV_LIST || l.key.variant != V_SPLIT || !l.key.packed ||
+            l.norm != nullptr || l.per_token || l.list.empty() || l.list.size() > (size_t)q8::BX3_MAX_DESCS) {
+            continue;
+        }
+        bool ok = true;
+        q8::Bx3Shape3 shapes[q8::BX3_MAX_DESCS];
+        const Op *input_of[q8::SPLIT_MAX_DESCS];
+        int n = 0, n_in = 0;
+        uint64_t xs_bytes = 0;
+        for (size_t i = 0; i < l.list.size() && ok; ++i) {
+            const Op &op = *l.list[i];
+            Op as_mma = op;
+            as_mma.kind = OP_MMA;
+            ok = strcmp(op.what, "q8_0_gemm_mma") == 0 && op.batch >= 9u && op.batch <= 16u &&
+                 l.residual[i] == nullptr && l.glu[i] == nullptr && bx3_admissible(as_mma) &&
+                 bx3_fits(as_mma, 64u);
+            shapes[n++] = q8::Bx3Shape3{op.rows, op.cols, op.batch};
+            int at = 0;
+            while (at < n_in && !same_input(*input_of[at], op)) {
+                ++at;
+            }
+            if (at == n_in) {
+                if (n_in == q8::SPLIT_MAX_DESCS) {
+                    ok = false;
+                    break;
+                }
+                input_of[n_in++] = &op;
+                xs_bytes += bx3_xs_bytes_of(op);
+            }
+        }
+        if (!ok || q8::bx3_launch_tile(shapes, n) != 64u) {
+            continue;
+        }
+        l.key = bx3_key(64u);
+        l.bx3_inputs = n_in;
+        l.bx3_xs_bytes = xs_bytes;
+        l.bx3_presplit = 0;
+        l.descs = (uint32_t)n;
+    }
+}
+
 // Plan the launches of a sequence of recorded operations. Consecutive
 // list-kernel products that neither read nor overwrite each other's outputs
 // share one launch; everything else launches on its own, in order.
@@ -1076,6 +1127,7 @@ std::vector<Launch> plan_launches(tm_hip_ctx *ctx, const std::vector<Op> &ops) {
         }
     }
     flush();
+    promote_small_batch_lists(plan);
     for (Launch &l : plan) {
         cut_bx3_launch(l);
     }

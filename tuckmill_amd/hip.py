@@ -119,7 +119,9 @@ def gemm_mma_on_bf16(rows: int, cols: int, batch: int, x_off: int = 0) -> bool:
 def gemm_mma_small_batch_on_tiles(rows: int, cols: int, batch: int) -> bool:
     """Whether a sealed product of 5 to 16 tokens leaves the vector kernels for the
     32-token tiles on the bf16 matrix cores (mirror of q8::mma_small_batch_on_tiles):
-    32 M weights and more from 9 tokens, 128 M and more from 5."""
+    32 M weights and more from 9 tokens, 128 M and more from 5. (From 9 tokens the
+    products of one launch that are that large together do so as well:
+    gemm_mma_launch_tile over the launch's shapes.)"""
     if batch < 5 or batch > 16:
         return False
     return rows * cols >= (1 << 27 if batch <= 8 else 1 << 25) and \
